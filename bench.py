@@ -1,0 +1,262 @@
+#!/usr/bin/env python3
+"""Benchmark of the decoding-attention hot path on one MI355X.
+
+Default run (one JSON line on stdout):
+  * primary workload — GQA decode, bf16, batch 64, 32 query / 8 KV heads, head_dim 128, seq_k 4096
+    (K/V packed [batch*seq_k, 8, 128], distinct V): one "step" = one call of the op;
+  * alongside — MLA decode, fp16, batch 64, 128 query heads over one 576-wide latent head, seq_k 4096,
+    V = K[..., :512];
+  * the CPU oracle timed on the host cores for the same primary workload (bounded sample).
+
+`value` is the achieved HBM rate of the primary workload: algorithmic bytes (Q, K, V, O once each +
+cu_seq_k) divided by the mean time of one call, inputs resident in HBM.  Calls are timed with events on the
+stream the kernels are launched on.  Working sets below 512 MB are rotated over several input copies so the
+256 MB Infinity Cache cannot serve them.
+
+`--sweep` prints the reference's two sweeps (batch sweep at seq_k 128, sequence sweep at batch 1, and the
+MLA equivalents) in the reference's log format
+(reference benchmarks/python/benchmark_decoding_attn.py:248-249, formulas :52-57).
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBPS = 8000.0      # MI355X HBM3E, published
+MFMA_PEAK_TFLOPS = 2500.0   # MI355X dense fp16/bf16 MFMA, published
+
+
+def _time_calls(torch, fn_list, steps, warmup):
+    """Mean and min milliseconds per call over `steps` calls, rotating over fn_list."""
+    n = len(fn_list)
+    for i in range(warmup):
+        fn_list[i % n]()
+    torch.cuda.synchronize()
+    start = torch.cuda.Event(enable_timing=True)
+    end = torch.cuda.Event(enable_timing=True)
+    start.record()
+    for i in range(steps):
+        fn_list[i % n]()
+    end.record()
+    torch.cuda.synchronize()
+    mean_ms = start.elapsed_time(end) / steps
+    # per-call minimum from a short individually-timed tail
+    mins = []
+    for i in range(min(steps, 10)):
+        s = torch.cuda.Event(enable_timing=True)
+        e = torch.cuda.Event(enable_timing=True)
+        s.record()
+        fn_list[i % n]()
+        e.record()
+        torch.cuda.synchronize()
+        mins.append(s.elapsed_time(e))
+    return mean_ms, min(mins)
+
+
+def _device_copies(torch, w, dev, min_total_bytes=768 << 20):
+    """Enough independent device copies of the inputs that consecutive calls cannot hit in the Infinity Cache."""
+    from decoding_attention_amd import workloads as wl
+
+    nbytes = wl.workload_bytes(w)
+    ncopies = 1 if nbytes >= (512 << 20) else max(2, -(-min_total_bytes // nbytes))
+    ncopies = min(ncopies, 64)
+    copies = []
+    for _ in range(ncopies):
+        wd = w.to(dev)
+        copies.append(wd if len(copies) == 0 else type(wd)(
+            wd.name, wd.q.clone(), wd.k.clone(), None if wd.v is None else wd.v.clone(), wd.cu_seq_k.clone(),
+            wd.max_seq_k, wd.dim_v, wd.is_alibi, wd.lengths))
+    return copies
+
+
+def measure(torch, w, steps, warmup):
+    from decoding_attention_amd import _lib, decoding_attn_fwd
+    from decoding_attention_amd import workloads as wl
+
+    dev = torch.device("cuda:0")
+    copies = _device_copies(torch, w, dev)
+    outs = []
+
+    def make(c):
+        def call():
+            outs[:] = [decoding_attn_fwd(c.q, c.k, c.v, c.cu_seq_k, c.max_seq_k, c.dim_v, c.is_alibi)]
+        return call
+
+    fns = [make(c) for c in copies]
+    mean_ms, min_ms = _time_calls(torch, fns, steps, warmup)
+    assert torch.isfinite(outs[0].float()).all()
+    nbytes = wl.workload_bytes(w)
+    flops = wl.workload_flops(w)
+    plan = _lib.plan(w.max_seq_k, w.batch, w.head_q, w.head_k, w.dim, w.dim_v)
+    return {
+        "workload": w.name,
+        "us_per_call": mean_ms * 1e3,
+        "us_per_call_min": min_ms * 1e3,
+        "algorithmic_bytes": nbytes,
+        "algorithmic_flops": flops,
+        "hbm_GBps": nbytes / (mean_ms * 1e-3) / 1e9,
+        "hbm_frac_of_peak": nbytes / (mean_ms * 1e-3) / 1e9 / HBM_PEAK_GBPS,
+        "tflops": flops / (mean_ms * 1e-3) / 1e12,
+        "mfma_frac_of_peak": flops / (mean_ms * 1e-3) / 1e12 / MFMA_PEAK_TFLOPS,
+        "input_copies_rotated": len(copies),
+        "plan": plan,
+    }
+
+
+def cpu_baseline(torch, w, budget_s=20.0):
+    """The CPU oracle on the host cores: one thread (what the reference's CPU path does) on as many whole
+    sequences of the workload as fit the time budget, scaled to the full batch when it is a subset."""
+    from decoding_attention_amd import workloads as wl
+    from oracle import oracle
+
+    def sub(nseq):
+        cu = w.cu_seq_k.tolist()
+        end = cu[nseq]
+        return (w.q[:nseq].contiguous(), w.k[:end].contiguous(), None if w.v is None else w.v[:end].contiguous(),
+                w.cu_seq_k[:nseq + 1].contiguous())
+
+    def run(nseq, threads):
+        q, k, v, cu = sub(nseq)
+        t0 = time.perf_counter()
+        oracle.attn_cpu(q, k, v, cu, w.max_seq_k, w.dim_v, w.is_alibi, nthreads=threads)
+        return time.perf_counter() - t0
+
+    t1 = run(1, 1)
+    nseq = int(max(1, min(w.batch, budget_s / max(t1, 1e-6))))
+    t = run(nseq, 1) if nseq > 1 else t1
+    full_s = t * w.batch / nseq
+    ncores = oracle.max_threads()
+    tm = run(min(w.batch, max(nseq, ncores)), ncores) * w.batch / min(w.batch, max(nseq, ncores))
+    nbytes = wl.workload_bytes(w)
+    return {
+        "value": nbytes / full_s / 1e12,
+        "unit": "TB/s",
+        "cores": 1,
+        "kind": "port",
+        "sample": f"{nseq} of {w.batch} sequences of {w.name}, single thread, {t:.2f} s measured"
+                  + ("" if nseq == w.batch else ", scaled linearly to the full batch (extrapolated)"),
+        "us_per_call": full_s * 1e6,
+        "all_cores": {"cores": ncores, "us_per_call": tm * 1e6, "value": nbytes / tm / 1e12},
+    }
+
+
+def run_default(args):
+    import torch
+
+    from decoding_attention_amd import workloads as wl
+
+    if not torch.cuda.is_available():
+        print("bench.py needs a GPU (no CPU fallback exists for the op)", file=sys.stderr)
+        return 2
+    gqa_w = wl.config_gqa_fixed(seed=0)
+    gqa = measure(torch, gqa_w, args.steps, args.warmup)
+    mla = None
+    if not args.no_mla:
+        mla = measure(torch, wl.config_mla(64, 4096), max(5, args.steps // 2), max(2, args.warmup // 2))
+    cpu = None if args.no_cpu else cpu_baseline(torch, gqa_w, args.cpu_budget)
+
+    line = {
+        "metric": "decode attn achieved HBM TB/s, GQA bf16 b64 seq_k 4096 (us/call and MLA fp16 b64 alongside)",
+        "value": gqa["hbm_GBps"] / 1e3,
+        "unit": "TB/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": gqa["us_per_call"] / 1e3,
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "bf16",
+        "data": "synthetic",
+        "config": {"workload": "GQA decode bf16, batch 64, 32 q heads / 8 kv heads, head_dim 128, seq_k 4096, "
+                               "packed K/V [262144, 8, 128], scale 1/sqrt(128), seed 0",
+                   "name": gqa["workload"], "plan": gqa["plan"]},
+        "us_per_call": gqa["us_per_call"],
+        "us_per_call_min": gqa["us_per_call_min"],
+        "pct_hbm_peak": 100.0 * gqa["hbm_frac_of_peak"],
+        "roofline": {"bound": "hbm", "achieved": gqa["hbm_GBps"], "peak": HBM_PEAK_GBPS, "unit": "GB/s",
+                     "frac": gqa["hbm_frac_of_peak"], "traffic": None,
+                     "kernel": "sweep kernel + split merge of one call (whole-call time)"},
+        "cpu_baseline": cpu,
+    }
+    if mla is not None:
+        line["mla"] = {
+            "workload": "MLA decode fp16, batch 64, 128 q heads / 1 latent kv head, dims 576/512, seq_k 4096, "
+                        "V = K[..., :512]",
+            "us_per_call": mla["us_per_call"], "us_per_call_min": mla["us_per_call_min"],
+            "hbm_TBps": mla["hbm_GBps"] / 1e3, "pct_hbm_peak": 100.0 * mla["hbm_frac_of_peak"],
+            "tflops": mla["tflops"], "pct_mfma_peak": 100.0 * mla["mfma_frac_of_peak"],
+            "algorithmic_bytes": mla["algorithmic_bytes"], "algorithmic_flops": mla["algorithmic_flops"],
+            "input_copies_rotated": mla["input_copies_rotated"], "plan": mla["plan"],
+            "roofline": {"bound": "hbm", "achieved": mla["hbm_GBps"], "peak": HBM_PEAK_GBPS, "unit": "GB/s",
+                         "frac": mla["hbm_frac_of_peak"], "traffic": None},
+            "roofline_mfma": {"bound": "mfma", "achieved": mla["tflops"], "peak": MFMA_PEAK_TFLOPS,
+                              "unit": "TFLOP/s", "frac": mla["mfma_frac_of_peak"]},
+        }
+    print(json.dumps(line))
+    return 0
+
+
+def run_sweep(args):
+    """The reference's sweeps, printed in its log format (one line per shape)."""
+    import torch
+
+    from decoding_attention_amd import workloads as wl
+
+    shapes = []
+    if args.sweep in ("mha", "all"):
+        shapes += [("mha-batch", wl.config_mha_sweep(b, 128)) for b in (1, 8, 32, 128, 512, 2048)]
+        shapes += [("mha-seq", wl.config_mha_sweep(1, s)) for s in (128, 512, 1536, 4096, 8192)]
+    if args.sweep in ("mla", "all"):
+        shapes += [("mla-batch", wl.config_mla(b, 4096)) for b in (1, 16, 64, 128)]
+        shapes += [("mla-seq", wl.config_mla(16, s)) for s in (512, 1024, 2048, 4096, 8192, 16384)]
+    if args.sweep in ("gqa", "all"):
+        shapes += [("gqa-varlen", wl.config_gqa_varlen()), ("gqa-fixed", wl.config_gqa_fixed()),
+                   ("mqa-alibi", wl.config_mqa_alibi())]
+    results = []
+    for tag, w in shapes:
+        r = measure(torch, w, args.steps, args.warmup)
+        ms = r["us_per_call"] / 1e3
+        sk = w.max_seq_k
+        ref_bytes = wl.reference_formula_bytes(w.batch, w.head_q, w.head_k, w.dim, w.dim_v, sk)
+        print(f"Decoding-Attention {w.batch}-{sk} profiling time: {ms:.4f} ms, throughput: {r['tflops']:.4f} TFLOPS, "
+              f"bandwidth: {ref_bytes / (ms * 1e-3) / 1e9:.3f} GB/s", flush=True)
+        print(f"    [{tag}] {w.name}: {r['us_per_call']:.1f} us/call (min {r['us_per_call_min']:.1f}), "
+              f"{r['hbm_GBps'] / 1e3:.3f} TB/s of real traffic = {100 * r['hbm_frac_of_peak']:.1f}% of "
+              f"{HBM_PEAK_GBPS / 1e3:.0f} TB/s, plan {r['plan']}", flush=True)
+        r["tag"] = tag
+        results.append(r)
+        del w
+    if args.json_out:
+        with open(args.json_out, "w") as f:
+            json.dump(results, f, indent=1)
+    return 0
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU oracle timing")
+    ap.add_argument("--no-mla", action="store_true", help="skip the MLA measurement")
+    ap.add_argument("--cpu-budget", type=float, default=15.0, help="seconds of single-thread CPU work to sample")
+    ap.add_argument("--sweep", choices=["mha", "mla", "gqa", "all"], help="print the reference's sweeps instead")
+    ap.add_argument("--json-out", help="with --sweep: also write the results as JSON")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py measures one GPU: the op has no multi-GPU path (sequences and KV heads shard without "
+              "communication); run with --gpus 1", file=sys.stderr)
+        return 2
+    if args.sweep:
+        return run_sweep(args)
+    return run_default(args)
+
+
+if __name__ == "__main__":
+    sys.exit(main())

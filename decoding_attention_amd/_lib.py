@@ -1,0 +1,78 @@
+"""ctypes binding of libdecoding_attn_hip.so (the C-ABI declared in include/decoding_attn_hip.h).
+
+The library is loaded from this package directory.  There is no fallback of any kind: if the
+shared object is missing the import of the op fails loudly with the build command to run.
+"""
+import ctypes
+import os
+
+PKG_DIR = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(PKG_DIR, "libdecoding_attn_hip.so")
+
+# Every symbol include/decoding_attn_hip.h declares.
+EXPORTED_SYMBOLS = (
+    "da_decoding_attn",
+    "da_decoding_attn_ex",
+    "da_workspace_bytes",
+    "da_plan",
+    "da_supported_head_dims",
+    "da_last_error",
+    "da_version",
+)
+
+DA_OK = 0
+DA_ERR_INVALID_ARGUMENT = 1
+DA_ERR_UNSUPPORTED = 2
+DA_ERR_WORKSPACE = 3
+DA_ERR_HIP = 4
+
+_lib = None
+
+
+class LibraryNotBuilt(ImportError):
+    pass
+
+
+def load():
+    """Load the shared library once and declare the prototypes."""
+    global _lib
+    if _lib is not None:
+        return _lib
+    if not os.path.exists(LIB_PATH):
+        raise LibraryNotBuilt(
+            f"{LIB_PATH} is missing: build it with `python -m decoding_attention_amd.build` "
+            "(hipcc, --offload-arch=gfx950). There is no CPU or PyTorch fallback.")
+    lib = ctypes.CDLL(LIB_PATH)
+    vp, sz, ci, cf = ctypes.c_void_p, ctypes.c_size_t, ctypes.c_int, ctypes.c_float
+    lib.da_decoding_attn.restype = ci
+    lib.da_decoding_attn.argtypes = [vp, vp, vp, vp, vp, sz, sz, sz, sz, sz, sz, ci, ci, vp]
+    lib.da_decoding_attn_ex.restype = ci
+    lib.da_decoding_attn_ex.argtypes = [vp, vp, vp, vp, vp, sz, sz, sz, sz, sz, sz, ci, ci, cf, vp, vp, sz, vp]
+    lib.da_workspace_bytes.restype = sz
+    lib.da_workspace_bytes.argtypes = [sz, sz, sz, sz, sz, sz]
+    ip = ctypes.POINTER(ci)
+    lib.da_plan.restype = ci
+    lib.da_plan.argtypes = [sz, sz, sz, sz, sz, sz, ci, ip, ip, ip, ip]
+    lib.da_supported_head_dims.restype = ci
+    lib.da_supported_head_dims.argtypes = [sz, sz]
+    lib.da_last_error.restype = ctypes.c_char_p
+    lib.da_last_error.argtypes = []
+    lib.da_version.restype = ci
+    lib.da_version.argtypes = []
+    _lib = lib
+    return lib
+
+
+def last_error() -> str:
+    return load().da_last_error().decode("utf-8", "replace")
+
+
+def plan(max_seq_k, batch, head_q, head_k, dim, dim_v, is_bf16=False):
+    """Launch plan for a shape: dict(kind, nsplit, chunk, heads_per_group)."""
+    lib = load()
+    kind, ns, ch, rt = ctypes.c_int(), ctypes.c_int(), ctypes.c_int(), ctypes.c_int()
+    rc = lib.da_plan(max_seq_k, batch, head_q, head_k, dim, dim_v, int(is_bf16), ctypes.byref(kind),
+                     ctypes.byref(ns), ctypes.byref(ch), ctypes.byref(rt))
+    if rc != DA_OK:
+        raise RuntimeError(f"da_plan failed ({rc}): {last_error()}")
+    return {"kind": kind.value, "nsplit": ns.value, "chunk": ch.value, "heads_per_group": rt.value}

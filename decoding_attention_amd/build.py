@@ -1,0 +1,70 @@
+"""Build libdecoding_attn_hip.so for gfx950 with hipcc (cross-compiles without a GPU).
+
+Usage: python -m decoding_attention_amd.build [--force]
+"""
+import concurrent.futures
+import os
+import subprocess
+import sys
+
+PKG_DIR = os.path.dirname(os.path.abspath(__file__))
+CSRC = os.path.join(PKG_DIR, "csrc")
+LIB_PATH = os.path.join(PKG_DIR, "libdecoding_attn_hip.so")
+OBJ_DIR = os.path.join(PKG_DIR, "build")
+
+SOURCES = [
+    "da_api.hip",
+    "da_sweep_d64.hip",
+    "da_sweep_d96.hip",
+    "da_sweep_d128.hip",
+    "da_sweep_d256.hip",
+    "da_sweep_d576.hip",
+    "da_mla.hip",
+]
+
+# packed-fp32 VALU forms are switched off on purpose: only scalar fp32 arithmetic is emitted.
+HIPCC_FLAGS = [
+    "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-Wall", "-Wextra",
+    "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+    "-Wno-unused-command-line-argument",
+]
+
+
+def _hipcc():
+    return os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
+
+
+def _compile(src):
+    obj = os.path.join(OBJ_DIR, os.path.splitext(src)[0] + ".o")
+    cmd = [_hipcc()] + HIPCC_FLAGS + ["-c", os.path.join(CSRC, src), "-o", obj]
+    if os.environ.get("DA_SAVE_TEMPS"):
+        cmd += ["-save-temps=obj"]
+    res = subprocess.run(cmd, capture_output=True, text=True)
+    if res.returncode != 0:
+        raise RuntimeError(f"hipcc failed for {src}:\n{res.stdout}\n{res.stderr}")
+    warn = "\n".join(ln for ln in res.stderr.splitlines() if "packed-fp32-ops" not in ln and ln.strip())
+    return obj, warn
+
+
+def build(force=True, verbose=False):
+    """Compile every translation unit and link the shared library.  Always compiles when force is set."""
+    if not force and os.path.exists(LIB_PATH):
+        return LIB_PATH
+    os.makedirs(OBJ_DIR, exist_ok=True)
+    with concurrent.futures.ThreadPoolExecutor(max_workers=min(8, len(SOURCES))) as ex:
+        results = list(ex.map(_compile, SOURCES))
+    objs = [r[0] for r in results]
+    if verbose:
+        for _, w in results:
+            if w:
+                print(w, file=sys.stderr)
+    cmd = [_hipcc(), "--offload-arch=gfx950", "-shared", "-fPIC", "-o", LIB_PATH] + objs
+    res = subprocess.run(cmd, capture_output=True, text=True)
+    if res.returncode != 0:
+        raise RuntimeError(f"link failed:\n{res.stdout}\n{res.stderr}")
+    return LIB_PATH
+
+
+if __name__ == "__main__":
+    path = build(force=True, verbose=True)
+    print(path)

@@ -1,0 +1,292 @@
+// C-ABI of libdecoding_attn_hip.so: argument checks, launch planning, workspace, dispatch.
+//
+// Stands where the reference's csrc/ops/decoding_attn.cpp does (set_dmha_fwd_params :13-62,
+// run_dmha_fwd :64-68, decoding_attn :70-76): derive strides from head counts, alias V onto K
+// when v is null, choose the kernel for (dtype, dim, dim_v), enqueue on the caller's stream.
+#include <hip/hip_runtime.h>
+
+#include <cmath>
+#include <cstdarg>
+#include <cstdio>
+#include <cstdlib>
+#include <map>
+#include <mutex>
+#include <string>
+#include <utility>
+
+#include "../../include/decoding_attn_hip.h"
+#include "da_mla.h"
+#include "da_sweep_launch.h"
+
+namespace {
+
+thread_local std::string g_last_error;
+
+int fail(int code, const char* fmt, ...) {
+    char buf[512];
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(buf, sizeof(buf), fmt, ap);
+    va_end(ap);
+    g_last_error = buf;
+    return code;
+}
+
+int env_int(const char* name, int dflt) {
+    const char* s = getenv(name);
+    if (!s || !*s) return dflt;
+    return atoi(s);
+}
+
+// Tunables, read once.  DA_TARGET_WGS: work-groups a launch should reach before the sequence
+// stops being split further; DA_MAX_CHUNK / DA_MIN_CHUNK: bounds on tokens per split.
+struct Tunables {
+    int target_wgs, max_chunk, min_chunk, force_kind;
+    Tunables() {
+        target_wgs = env_int("DA_TARGET_WGS", 1024);
+        max_chunk = env_int("DA_MAX_CHUNK", 1024);
+        min_chunk = env_int("DA_MIN_CHUNK", 256);
+        force_kind = env_int("DA_FORCE_KIND", 0);
+    }
+};
+const Tunables& tun() {
+    static Tunables t;
+    return t;
+}
+
+constexpr int kKindSweep = 1;
+constexpr int kKindMfma = 2;
+constexpr int kMaxSplits = 256;
+
+struct Plan {
+    int kind = 0;
+    int rt = 1;      // query heads per work-group
+    int groups = 1;  // work-groups per KV head
+    int nsplit = 1;
+    int chunk = 0;
+    size_t ws_bytes = 0;
+};
+
+bool supported_dims(size_t dim, size_t dim_v) {
+    return (dim == 64 && dim_v == 64) || (dim == 96 && dim_v == 96) || (dim == 128 && dim_v == 128) ||
+           (dim == 256 && dim_v == 256) || (dim == 576 && dim_v == 512);
+}
+
+int rows_per_trip(size_t dim) {
+    switch (dim) {
+        case 64: return da::sweep_rows_per_trip<64>();
+        case 96: return da::sweep_rows_per_trip<96>();
+        case 128: return da::sweep_rows_per_trip<128>();
+        case 256: return da::sweep_rows_per_trip<256>();
+        default: return da::sweep_rows_per_trip<576>();
+    }
+}
+
+Plan make_plan(size_t max_seq_k, size_t batch, size_t head_q, size_t head_k, size_t dim, size_t dim_v) {
+    Plan pl;
+    const int ratio = (int)(head_q / head_k);
+    int trip;
+    const bool mfma = da::mla_supported(dim, dim_v, ratio) && tun().force_kind != kKindSweep;
+    if (mfma) {
+        pl.kind = kKindMfma;
+        pl.rt = da::mla_heads_per_group(ratio);
+        trip = da::mla_rows_per_trip();
+    } else {
+        pl.kind = kKindSweep;
+        const int max_rt = dim > 256 ? 2 : 4;
+        pl.rt = ratio >= 3 ? 4 : ratio;  // 1, 2 or 4 (a group of 3 runs as 4 with one idle head)
+        if (pl.rt > max_rt) pl.rt = max_rt;
+        trip = rows_per_trip(dim);
+    }
+    pl.groups = (ratio + pl.rt - 1) / pl.rt;
+    const long long base = (long long)batch * (long long)head_k * pl.groups;
+    const int min_chunk = std::max(tun().min_chunk, trip);
+    long long want = base > 0 ? (tun().target_wgs + base - 1) / base : 1;
+    const long long by_len = std::max<long long>(1, (long long)max_seq_k / min_chunk);
+    long long by_cap = ((long long)max_seq_k + tun().max_chunk - 1) / std::max(1, tun().max_chunk);
+    long long ns = std::max(std::min(want, by_len), std::min(by_cap, by_len));
+    ns = std::max<long long>(1, std::min<long long>(ns, kMaxSplits));
+    long long chunk = ((long long)max_seq_k + ns - 1) / ns;
+    chunk = (chunk + trip - 1) / trip * trip;
+    if (chunk <= 0) chunk = trip;
+    ns = std::max<long long>(1, ((long long)max_seq_k + chunk - 1) / chunk);
+    pl.nsplit = (int)ns;
+    pl.chunk = (int)chunk;
+    pl.ws_bytes = pl.nsplit > 1 ? (size_t)batch * head_q * pl.nsplit * (dim_v + 2) * sizeof(float) : 0;
+    return pl;
+}
+
+struct CachedWs {
+    void* ptr = nullptr;
+    size_t bytes = 0;
+};
+std::mutex g_ws_mutex;
+std::map<std::pair<int, void*>, CachedWs> g_ws;
+
+// Workspace of the reference-signature entry point: one buffer per (device, stream), grown on demand.
+int cached_workspace(size_t bytes, hipStream_t stream, void** out) {
+    int dev = 0;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return fail(DA_ERR_HIP, "hipGetDevice: %s", hipGetErrorString(e));
+    std::lock_guard<std::mutex> lock(g_ws_mutex);
+    CachedWs& w = g_ws[std::make_pair(dev, (void*)stream)];
+    if (w.bytes < bytes) {
+        if (w.ptr) {
+            e = hipFree(w.ptr);  // waits for work that may still read it
+            w.ptr = nullptr;
+            w.bytes = 0;
+            if (e != hipSuccess) return fail(DA_ERR_HIP, "hipFree(workspace): %s", hipGetErrorString(e));
+        }
+        const size_t want = (bytes + (1u << 20) - 1) & ~((size_t)(1u << 20) - 1);
+        e = hipMalloc(&w.ptr, want);
+        if (e != hipSuccess) {
+            w.ptr = nullptr;
+            return fail(DA_ERR_HIP, "hipMalloc(workspace, %zu): %s", want, hipGetErrorString(e));
+        }
+        w.bytes = want;
+    }
+    *out = w.ptr;
+    return DA_OK;
+}
+
+bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+
+}  // namespace
+
+extern "C" {
+
+const char* da_last_error(void) { return g_last_error.c_str(); }
+
+int da_version(void) { return 100; }
+
+int da_supported_head_dims(size_t dim, size_t dim_v) { return supported_dims(dim, dim_v) ? 1 : 0; }
+
+int da_plan(size_t max_seq_k, size_t batch, size_t head_q, size_t head_k, size_t dim, size_t dim_v, int is_bf16,
+            int* kernel_kind, int* nsplit, int* chunk, int* heads_per_group) {
+    (void)is_bf16;
+    if (head_k == 0 || head_q % head_k != 0)
+        return fail(DA_ERR_INVALID_ARGUMENT, "head_q (%zu) must be a multiple of head_k (%zu)", head_q, head_k);
+    if (!supported_dims(dim, dim_v))
+        return fail(DA_ERR_UNSUPPORTED, "unsupported head dims (dim %zu, dim_v %zu)", dim, dim_v);
+    const Plan pl = make_plan(max_seq_k, batch, head_q, head_k, dim, dim_v);
+    if (kernel_kind) *kernel_kind = pl.kind;
+    if (nsplit) *nsplit = pl.nsplit;
+    if (chunk) *chunk = pl.chunk;
+    if (heads_per_group) *heads_per_group = pl.rt;
+    return DA_OK;
+}
+
+size_t da_workspace_bytes(size_t max_seq_k, size_t batch, size_t head_q, size_t head_k, size_t dim, size_t dim_v) {
+    if (head_k == 0 || head_q % head_k != 0 || !supported_dims(dim, dim_v)) return 0;
+    return make_plan(max_seq_k, batch, head_q, head_k, dim, dim_v).ws_bytes;
+}
+
+int da_decoding_attn_ex(const void* q, const void* k, const void* v, void* o, const int32_t* cu_seq_k,
+                        size_t max_seq_k, size_t batch, size_t head_q, size_t head_k, size_t dim, size_t dim_v,
+                        int is_alibi, int is_bf16, float softmax_scale, const float* alibi_slopes, void* workspace,
+                        size_t workspace_bytes, void* hip_stream) {
+    // the reference's checks (csrc/ops/decoding_attn.cpp:16-22) ...
+    if (!q) return fail(DA_ERR_INVALID_ARGUMENT, "q is null");
+    if (!k) return fail(DA_ERR_INVALID_ARGUMENT, "k is null");
+    if (!o) return fail(DA_ERR_INVALID_ARGUMENT, "o is null");
+    if (!cu_seq_k) return fail(DA_ERR_INVALID_ARGUMENT, "cu_seq_k is null");
+    if (head_k == 0 || head_q % head_k != 0)
+        return fail(DA_ERR_INVALID_ARGUMENT, "head_q (%zu) must be a multiple of head_k (%zu)", head_q, head_k);
+    if (dim > 576) return fail(DA_ERR_INVALID_ARGUMENT, "dim (%zu) must be <= 576", dim);
+    if (dim_v > 512) return fail(DA_ERR_INVALID_ARGUMENT, "dim_v (%zu) must be <= 512", dim_v);
+    // ... and the ones it leaves out
+    if (!supported_dims(dim, dim_v))
+        return fail(DA_ERR_UNSUPPORTED,
+                    "unsupported head dims (dim %zu, dim_v %zu): supported are (64,64) (96,96) (128,128) (256,256) "
+                    "(576,512)",
+                    dim, dim_v);
+    if (!aligned16(q) || !aligned16(k) || (v && !aligned16(v)))
+        return fail(DA_ERR_INVALID_ARGUMENT, "q, k and v must be 16-byte aligned");
+    if ((reinterpret_cast<uintptr_t>(o) & 1u) != 0) return fail(DA_ERR_INVALID_ARGUMENT, "o must be 2-byte aligned");
+    if (max_seq_k > (size_t)INT32_MAX || batch > 65535 * (size_t)64 || head_q > 65535)
+        return fail(DA_ERR_INVALID_ARGUMENT, "shape out of range (max_seq_k %zu, batch %zu, head_q %zu)", max_seq_k,
+                    batch, head_q);
+    if (batch == 0) return DA_OK;
+
+    hipStream_t stream = reinterpret_cast<hipStream_t>(hip_stream);
+    const Plan pl = make_plan(max_seq_k, batch, head_q, head_k, dim, dim_v);
+    if (batch > 65535) return fail(DA_ERR_INVALID_ARGUMENT, "batch (%zu) exceeds the grid limit 65535", batch);
+    if ((size_t)head_k * pl.groups > 65535)
+        return fail(DA_ERR_INVALID_ARGUMENT, "head_k * groups exceeds the grid limit 65535");
+
+    void* ws = nullptr;
+    if (pl.ws_bytes > 0) {
+        if (workspace) {
+            if (workspace_bytes < pl.ws_bytes)
+                return fail(DA_ERR_WORKSPACE, "workspace has %zu bytes, %zu needed", workspace_bytes, pl.ws_bytes);
+            if (!aligned16(workspace)) return fail(DA_ERR_INVALID_ARGUMENT, "workspace must be 16-byte aligned");
+            ws = workspace;
+        } else {
+            const int rc = cached_workspace(pl.ws_bytes, stream, &ws);
+            if (rc != DA_OK) return rc;
+        }
+    }
+
+    da::SweepParams sp;
+    sp.q = q;
+    sp.k = k;
+    // V absent: the values are the leading dim_v columns of each K row, read with K's pitch
+    // (reference csrc/ops/decoding_attn.cpp:30-37).
+    sp.v = v ? v : k;
+    sp.o = o;
+    sp.cu_seq_k = cu_seq_k;
+    sp.ws_o = reinterpret_cast<float*>(ws);
+    sp.ws_ml = ws ? reinterpret_cast<float*>(ws) + (size_t)batch * head_q * pl.nsplit * dim_v : nullptr;
+    sp.slopes = is_alibi ? alibi_slopes : nullptr;
+    sp.k_row = (int64_t)(head_k * dim);
+    sp.v_row = v ? (int64_t)(head_k * dim_v) : (int64_t)(head_k * dim);
+    sp.v_head = v ? (int)dim_v : (int)dim;
+    sp.head_q = (int)head_q;
+    sp.head_k = (int)head_k;
+    sp.ratio = (int)(head_q / head_k);
+    sp.groups = pl.groups;
+    sp.nsplit = pl.nsplit;
+    sp.chunk = pl.chunk;
+    const float scale = softmax_scale > 0.0f ? softmax_scale : (float)(1.0 / std::sqrt((double)dim));
+    sp.scale_log2 = scale * da::kLog2e;
+    sp.is_alibi = is_alibi ? 1 : 0;
+
+    const dim3 grid((unsigned)pl.nsplit, (unsigned)(head_k * pl.groups), (unsigned)batch);
+    hipError_t e;
+    if (pl.kind == kKindMfma) {
+        e = da::launch_mla(sp, is_bf16 != 0, pl.rt, grid, stream);
+    } else {
+        switch (dim) {
+            case 64: e = da::launch_sweep_d64(sp, is_bf16 != 0, pl.rt, grid, stream); break;
+            case 96: e = da::launch_sweep_d96(sp, is_bf16 != 0, pl.rt, grid, stream); break;
+            case 128: e = da::launch_sweep_d128(sp, is_bf16 != 0, pl.rt, grid, stream); break;
+            case 256: e = da::launch_sweep_d256(sp, is_bf16 != 0, pl.rt, grid, stream); break;
+            default: e = da::launch_sweep_d576(sp, is_bf16 != 0, pl.rt, grid, stream); break;
+        }
+    }
+    if (e != hipSuccess) return fail(DA_ERR_HIP, "sweep kernel launch: %s", hipGetErrorString(e));
+
+    if (pl.nsplit > 1) {
+        da::ReduceParams rp;
+        rp.o = o;
+        rp.cu_seq_k = cu_seq_k;
+        rp.ws_o = sp.ws_o;
+        rp.ws_ml = sp.ws_ml;
+        rp.head_q = (int)head_q;
+        rp.dim_v = (int)dim_v;
+        rp.nsplit = pl.nsplit;
+        rp.chunk = pl.chunk;
+        e = da::launch_reduce(rp, is_bf16 != 0, (int)(batch * head_q), stream);
+        if (e != hipSuccess) return fail(DA_ERR_HIP, "merge kernel launch: %s", hipGetErrorString(e));
+    }
+    return DA_OK;
+}
+
+int da_decoding_attn(const void* q, const void* k, const void* v, void* o, const int32_t* cu_seq_k, size_t max_seq_k,
+                     size_t batch, size_t head_q, size_t head_k, size_t dim, size_t dim_v, int is_alibi, int is_bf16,
+                     void* hip_stream) {
+    return da_decoding_attn_ex(q, k, v, o, cu_seq_k, max_seq_k, batch, head_q, head_k, dim, dim_v, is_alibi, is_bf16,
+                               0.0f, nullptr, nullptr, 0, hip_stream);
+}
+
+}  // extern "C"

@@ -1,0 +1,113 @@
+// Shared device helpers and launch parameter blocks for the gfx950 decoding-attention kernels.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace da {
+
+constexpr int kWave = 64;          // CDNA4 wavefront width
+constexpr float kLog2e = 1.4426950408889634f;
+constexpr float kNegBig = -1.0e30f;  // finite stand-in for -inf as the initial running maximum
+
+struct f16_tag {};
+struct bf16_tag {};
+
+typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
+typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+
+// Per-dtype element arithmetic on packed pairs held in a 32-bit register.
+template <typename Tag>
+struct Elem;
+
+template <>
+struct Elem<f16_tag> {
+    // acc + a.lo*b.lo + a.hi*b.hi with fp32 accumulation (v_dot2_f32_f16)
+    static __device__ __forceinline__ float dot2(uint32_t a, uint32_t b, float acc) {
+        return __builtin_amdgcn_fdot2(__builtin_bit_cast(f16x2, a), __builtin_bit_cast(f16x2, b), acc, false);
+    }
+    static __device__ __forceinline__ float lo(uint32_t a) { return (float)__builtin_bit_cast(f16x2, a)[0]; }
+    static __device__ __forceinline__ float hi(uint32_t a) { return (float)__builtin_bit_cast(f16x2, a)[1]; }
+    // round-to-nearest-even, the reference's __float2half
+    static __device__ __forceinline__ uint16_t from_f32(float f) {
+        _Float16 h = (_Float16)f;
+        return __builtin_bit_cast(uint16_t, h);
+    }
+};
+
+template <>
+struct Elem<bf16_tag> {
+    static __device__ __forceinline__ float dot2(uint32_t a, uint32_t b, float acc) {
+        return __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2, a), __builtin_bit_cast(bf16x2, b), acc,
+                                               false);
+    }
+    static __device__ __forceinline__ float lo(uint32_t a) { return __uint_as_float(a << 16); }
+    static __device__ __forceinline__ float hi(uint32_t a) { return __uint_as_float(a & 0xffff0000u); }
+    // round-to-nearest-even, the reference's __float2bfloat16
+    static __device__ __forceinline__ uint16_t from_f32(float f) {
+        uint32_t x = __float_as_uint(f);
+        if ((x & 0x7fffffffu) > 0x7f800000u) return (uint16_t)((x >> 16) | 0x40u);
+        x += 0x7fffu + ((x >> 16) & 1u);
+        return (uint16_t)(x >> 16);
+    }
+};
+
+__device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
+
+// Butterfly sum over groups of G adjacent lanes (G a power of two <= 16) with DPP lane
+// permutes; every lane of the group ends with the group's total.
+template <int G>
+__device__ __forceinline__ float group_sum(float x) {
+    if constexpr (G >= 2) {  // quad_perm [1,0,3,2]
+        x += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, x), 0xB1, 0xF, 0xF, true));
+    }
+    if constexpr (G >= 4) {  // quad_perm [2,3,0,1]
+        x += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, x), 0x4E, 0xF, 0xF, true));
+    }
+    if constexpr (G >= 8) {  // row_half_mirror: quads are uniform by now, so i -> 7-i swaps the two quads
+        x += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, x), 0x141, 0xF, 0xF, true));
+    }
+    if constexpr (G >= 16) {  // row_mirror: halves are uniform, i -> 15-i swaps them
+        x += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, x), 0x140, 0xF, 0xF, true));
+    }
+    return x;
+}
+
+// Argument block of the sweep kernels (passed by value).
+struct SweepParams {
+    const void* q;            // [batch, head_q, dim]
+    const void* k;            // [total_k, head_k, dim]
+    const void* v;            // [total_k, head_k, dim_v], or k when V is the leading columns of K
+    void* o;                  // [batch, head_q, dim_v]
+    const int32_t* cu_seq_k;  // [batch + 1]
+    float* ws_o;              // [batch, head_q, nsplit, dim_v] un-normalised partial outputs
+    float* ws_ml;             // [batch, head_q, nsplit, 2] running maximum (log2 units) and denominator
+    const float* slopes;      // [head_q] ALiBi slopes or null for the closed form
+    int64_t k_row;            // elements between consecutive tokens of K
+    int64_t v_row;            // same for V
+    int v_head;               // elements between KV heads of V
+    int head_q, head_k, ratio;
+    int groups;               // work-groups per KV head (ceil(ratio / heads per work-group))
+    int nsplit, chunk;        // sequence splits and tokens per split
+    float scale_log2;         // softmax scale * log2(e)
+    int is_alibi;
+};
+
+struct ReduceParams {
+    void* o;
+    const int32_t* cu_seq_k;
+    const float* ws_o;
+    const float* ws_ml;
+    int head_q, dim_v, nsplit, chunk;
+};
+
+__device__ __forceinline__ float alibi_slope_log2(const float* slopes, int h, int head_q) {
+    // closed form 2^(-8(h+1)/head_q); a slope array overrides it
+    float s = slopes ? slopes[h] : fast_exp2(-8.0f * (float)(h + 1) / (float)head_q);
+    return s * kLog2e;
+}
+
+}  // namespace da

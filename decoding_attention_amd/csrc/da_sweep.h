@@ -1,0 +1,277 @@
+// Single-query attention as a bandwidth-bound sweep over K and V (wave64, gfx950).
+//
+// One work-group of four wavefronts serves one (sequence, KV head, query-head group, sequence
+// split).  The RT query heads of the group sit in registers as packed 16-bit pairs and are
+// shared by every K row that is streamed, so a GQA/MQA group reads its K/V once.
+//
+// Lane layout: G adjacent lanes cooperate on one K (or V) row, each lane owning the 16-byte
+// chunks  g, g+G, g+2G, ...  of the row, so one load instruction covers 64/G rows with
+// G*16 contiguous bytes per row.  Each row slot (lane / G) keeps its own online-softmax
+// state (running maximum, denominator, un-normalised output) for the rows it has seen; the
+// states are merged once at the end (lane shuffles inside a wave, LDS across the four waves),
+// which keeps the streaming loop free of cross-lane traffic apart from the G-lane dot-product
+// butterfly.
+//
+// The work-group either finishes the row (nsplit == 1: divide, round to nearest even, store)
+// or writes an fp32 partial (un-normalised output, maximum, denominator) for the merge kernel.
+//
+// Follows the mathematics of the reference kernel (csrc/kernel/decoding_attn/
+// decoding_fwd_kernel.h:50-235) and its index rules (block_info.h:14-30), not its structure:
+// the reference keeps the whole score row in shared memory and streams K and V once per query
+// head.
+#pragma once
+#include "da_common.h"
+
+namespace da {
+
+template <typename Tag, int D, int DV, int G, int RT, int U>
+__global__ __launch_bounds__(256) void sweep_kernel(const SweepParams p) {
+    static_assert(D % (8 * G) == 0 && DV % (8 * G) == 0, "row must split into 16-byte chunks over G lanes");
+    constexpr int CPL = D / 8 / G;    // K chunks per lane
+    constexpr int CPLV = DV / 8 / G;  // V chunks per lane
+    constexpr int E = CPLV * 8;       // output columns per lane
+    constexpr int RPI = kWave / G;    // rows per load instruction
+    constexpr int NW = 4;             // waves per work-group
+    constexpr int TILE = RPI * U;     // rows per wave iteration
+    using EL = Elem<Tag>;
+
+    __shared__ float lds_acc[NW][RT][DV];
+    __shared__ float lds_ml[NW][RT][2];
+
+    const int lane = threadIdx.x & (kWave - 1);
+    const int wave = threadIdx.x / kWave;
+    const int g = lane % G;
+    const int slot = lane / G;
+
+    const int split = blockIdx.x;
+    const int hk = blockIdx.y / p.groups;
+    const int grp = blockIdx.y % p.groups;
+    const int b = blockIdx.z;
+
+    const int start = p.cu_seq_k[b];
+    const int len = p.cu_seq_k[b + 1] - start;
+    const int c0 = split * p.chunk;
+    const int c1 = (split == p.nsplit - 1) ? len : min(len, c0 + p.chunk);
+
+    const int h_base = hk * p.ratio + grp * RT;
+    const int nh = min(RT, p.ratio - grp * RT);  // live heads of this group
+
+    if (c0 >= c1) {
+        // Nothing to read.  An empty sequence still owns an output row: store zeros when this
+        // work-group is the one that would have finished it.
+        if (p.nsplit == 1) {
+            uint16_t* o = reinterpret_cast<uint16_t*>(p.o);
+            for (int idx = threadIdx.x; idx < nh * DV; idx += blockDim.x) {
+                const int r = idx / DV, col = idx % DV;
+                o[((size_t)b * p.head_q + h_base + r) * DV + col] = 0;
+            }
+        }
+        return;
+    }
+
+    // Query heads of the group, as packed pairs, at this lane's chunk positions.
+    uint4 qreg[RT][CPL];
+    float slope[RT];
+#pragma unroll
+    for (int r = 0; r < RT; ++r) {
+        const int h = h_base + min(r, nh - 1);
+        const uint16_t* qrow = reinterpret_cast<const uint16_t*>(p.q) + ((size_t)b * p.head_q + h) * D;
+#pragma unroll
+        for (int c = 0; c < CPL; ++c) qreg[r][c] = *reinterpret_cast<const uint4*>(qrow + (c * G + g) * 8);
+        slope[r] = p.is_alibi ? alibi_slope_log2(p.slopes, h, p.head_q) : 0.0f;
+    }
+
+    float m[RT], l[RT], acc[RT][E];
+#pragma unroll
+    for (int r = 0; r < RT; ++r) {
+        m[r] = kNegBig;
+        l[r] = 0.0f;
+#pragma unroll
+        for (int e = 0; e < E; ++e) acc[r][e] = 0.0f;
+    }
+
+    const uint16_t* kbase = reinterpret_cast<const uint16_t*>(p.k) + (size_t)start * p.k_row + (size_t)hk * D + g * 8;
+    const uint16_t* vbase =
+        reinterpret_cast<const uint16_t*>(p.v) + (size_t)start * p.v_row + (size_t)hk * p.v_head + g * 8;
+
+    const int ntiles = (c1 - c0 + TILE - 1) / TILE;
+    for (int t = wave; t < ntiles; t += NW) {
+        const int base = c0 + t * TILE + slot;
+        uint4 kreg[U][CPL];
+        uint4 vreg[U][CPLV];
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            const int j = min(base + u * RPI, c1 - 1);  // rows past the end re-read the last row and are masked
+            const uint16_t* kr = kbase + (size_t)j * p.k_row;
+#pragma unroll
+            for (int c = 0; c < CPL; ++c) kreg[u][c] = *reinterpret_cast<const uint4*>(kr + c * G * 8);
+        }
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            const int j = min(base + u * RPI, c1 - 1);
+            const uint16_t* vr = vbase + (size_t)j * p.v_row;
+#pragma unroll
+            for (int c = 0; c < CPLV; ++c) vreg[u][c] = *reinterpret_cast<const uint4*>(vr + c * G * 8);
+        }
+
+        // scores in log2 units
+        float s[U][RT];
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            const int j = base + u * RPI;
+#pragma unroll
+            for (int r = 0; r < RT; ++r) {
+                float d = 0.0f;
+#pragma unroll
+                for (int c = 0; c < CPL; ++c) {
+                    d = EL::dot2(qreg[r][c].x, kreg[u][c].x, d);
+                    d = EL::dot2(qreg[r][c].y, kreg[u][c].y, d);
+                    d = EL::dot2(qreg[r][c].z, kreg[u][c].z, d);
+                    d = EL::dot2(qreg[r][c].w, kreg[u][c].w, d);
+                }
+                d = group_sum<G>(d);
+                d = d * p.scale_log2 + slope[r] * (float)(j - (len - 1));
+                s[u][r] = (j < c1) ? d : -INFINITY;
+            }
+        }
+
+        // online softmax, one rescale per tile
+#pragma unroll
+        for (int r = 0; r < RT; ++r) {
+            float mn = m[r];
+#pragma unroll
+            for (int u = 0; u < U; ++u) mn = fmaxf(mn, s[u][r]);
+            const float alpha = fast_exp2(m[r] - mn);
+            m[r] = mn;
+            l[r] *= alpha;
+#pragma unroll
+            for (int e = 0; e < E; ++e) acc[r][e] *= alpha;
+#pragma unroll
+            for (int u = 0; u < U; ++u) {
+                s[u][r] = fast_exp2(s[u][r] - mn);
+                l[r] += s[u][r];
+            }
+        }
+
+        // O += P V
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+#pragma unroll
+            for (int c = 0; c < CPLV; ++c) {
+                float vf[8];
+                vf[0] = EL::lo(vreg[u][c].x);
+                vf[1] = EL::hi(vreg[u][c].x);
+                vf[2] = EL::lo(vreg[u][c].y);
+                vf[3] = EL::hi(vreg[u][c].y);
+                vf[4] = EL::lo(vreg[u][c].z);
+                vf[5] = EL::hi(vreg[u][c].z);
+                vf[6] = EL::lo(vreg[u][c].w);
+                vf[7] = EL::hi(vreg[u][c].w);
+#pragma unroll
+                for (int r = 0; r < RT; ++r) {
+#pragma unroll
+                    for (int e = 0; e < 8; ++e) acc[r][c * 8 + e] += s[u][r] * vf[e];
+                }
+            }
+        }
+    }
+
+    // Merge the row slots of this wave (lanes that own the same columns).
+#pragma unroll
+    for (int off = G; off < kWave; off <<= 1) {
+#pragma unroll
+        for (int r = 0; r < RT; ++r) {
+            const float mo = __shfl_xor(m[r], off);
+            const float lo = __shfl_xor(l[r], off);
+            const float mn = fmaxf(m[r], mo);
+            const float wa = fast_exp2(m[r] - mn);
+            const float wb = fast_exp2(mo - mn);
+            m[r] = mn;
+            l[r] = l[r] * wa + lo * wb;
+#pragma unroll
+            for (int e = 0; e < E; ++e) {
+                const float ao = __shfl_xor(acc[r][e], off);
+                acc[r][e] = acc[r][e] * wa + ao * wb;
+            }
+        }
+    }
+
+    if (slot == 0) {
+#pragma unroll
+        for (int r = 0; r < RT; ++r) {
+#pragma unroll
+            for (int c = 0; c < CPLV; ++c) {
+#pragma unroll
+                for (int e = 0; e < 8; ++e) lds_acc[wave][r][(c * G + g) * 8 + e] = acc[r][c * 8 + e];
+            }
+            if (g == 0) {
+                lds_ml[wave][r][0] = m[r];
+                lds_ml[wave][r][1] = l[r];
+            }
+        }
+    }
+    __syncthreads();
+
+    // Merge the four waves in a fixed order and finish.
+    for (int idx = threadIdx.x; idx < nh * DV; idx += blockDim.x) {
+        const int r = idx / DV, col = idx % DV;
+        float mm = lds_ml[0][r][0];
+#pragma unroll
+        for (int w = 1; w < NW; ++w) mm = fmaxf(mm, lds_ml[w][r][0]);
+        float num = 0.0f, den = 0.0f;
+#pragma unroll
+        for (int w = 0; w < NW; ++w) {
+            const float wt = fast_exp2(lds_ml[w][r][0] - mm);
+            num += wt * lds_acc[w][r][col];
+            den += wt * lds_ml[w][r][1];
+        }
+        const int h = h_base + r;
+        if (p.nsplit == 1) {
+            reinterpret_cast<uint16_t*>(p.o)[((size_t)b * p.head_q + h) * DV + col] = EL::from_f32(num / den);
+        } else {
+            const size_t part = ((size_t)b * p.head_q + h) * p.nsplit + split;
+            p.ws_o[part * DV + col] = num;
+            if (col == 0) {
+                p.ws_ml[part * 2 + 0] = mm;
+                p.ws_ml[part * 2 + 1] = den;
+            }
+        }
+    }
+}
+
+// Second pass: merge the per-split partials of one (sequence, query head) in split order.
+template <typename Tag>
+__global__ __launch_bounds__(128) void reduce_kernel(const ReduceParams p) {
+    using EL = Elem<Tag>;
+    __shared__ float wts[256];
+    __shared__ float s_den;
+    const int b = blockIdx.x / p.head_q;
+    const int h = blockIdx.x % p.head_q;
+    const int len = p.cu_seq_k[b + 1] - p.cu_seq_k[b];
+    int ns = 0;
+    if (len > 0) ns = min(p.nsplit, (len + p.chunk - 1) / p.chunk);
+    const size_t part0 = ((size_t)b * p.head_q + h) * p.nsplit;
+    uint16_t* orow = reinterpret_cast<uint16_t*>(p.o) + ((size_t)b * p.head_q + h) * p.dim_v;
+    if (ns == 0) {
+        for (int col = threadIdx.x; col < p.dim_v; col += blockDim.x) orow[col] = 0;
+        return;
+    }
+    float mm = kNegBig;
+    for (int s = 0; s < ns; ++s) mm = fmaxf(mm, p.ws_ml[(part0 + s) * 2]);
+    for (int s = threadIdx.x; s < ns; s += blockDim.x) wts[s] = fast_exp2(p.ws_ml[(part0 + s) * 2] - mm);
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        float den = 0.0f;
+        for (int s = 0; s < ns; ++s) den += wts[s] * p.ws_ml[(part0 + s) * 2 + 1];
+        s_den = den;
+    }
+    __syncthreads();
+    const float inv = 1.0f / s_den;
+    for (int col = threadIdx.x; col < p.dim_v; col += blockDim.x) {
+        float num = 0.0f;
+        for (int s = 0; s < ns; ++s) num += wts[s] * p.ws_o[(part0 + s) * p.dim_v + col];
+        orow[col] = EL::from_f32(num * inv);
+    }
+}
+
+}  // namespace da

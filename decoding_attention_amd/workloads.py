@@ -1,0 +1,141 @@
+"""Seeded synthetic workloads and the work formulas used to report them.
+
+Inputs are drawn on the CPU from ``torch.Generator().manual_seed(seed)`` in the fixed
+order q, k, v, lengths as fp32 N(0,1) and then cast (round-to-nearest-even) to
+fp16/bf16, so a CPU checker and the GPU kernel see identical bits whatever the device.
+
+The packed layout is the reference's: q [batch, head_q, dim], k [total_k, head_k, dim],
+v [total_k, head_k, dim_v] or None for the latent (MLA) form where V is the first
+dim_v columns of K, and cu_seq_k = int32 prefix offsets built as in the reference's
+``get_cu_seq`` (reference tests/test_decoding_attn.py:23-31).
+"""
+from dataclasses import dataclass
+from typing import List, Optional
+
+import torch
+
+
+@dataclass
+class Workload:
+    name: str
+    q: torch.Tensor
+    k: torch.Tensor
+    v: Optional[torch.Tensor]
+    cu_seq_k: torch.Tensor
+    max_seq_k: int
+    dim_v: int
+    is_alibi: bool
+    lengths: List[int]
+
+    @property
+    def batch(self):
+        return self.q.shape[0]
+
+    @property
+    def head_q(self):
+        return self.q.shape[1]
+
+    @property
+    def head_k(self):
+        return self.k.shape[1]
+
+    @property
+    def dim(self):
+        return self.q.shape[2]
+
+    def to(self, device):
+        return Workload(self.name, self.q.to(device), self.k.to(device),
+                        None if self.v is None else self.v.to(device), self.cu_seq_k.to(device),
+                        self.max_seq_k, self.dim_v, self.is_alibi, self.lengths)
+
+
+def get_cu_seq(seqs: torch.Tensor) -> torch.Tensor:
+    """[batch] lengths -> [batch+1] int32 prefix offsets with a leading zero."""
+    return torch.nn.functional.pad(seqs.cumsum(dim=0, dtype=torch.int32), (1, 0))
+
+
+def make_workload(batch, head_q, head_k, dim, dim_v, seq_k, dtype, *, seed=0, varlen=False, latent=None,
+                  is_alibi=False, name=None, min_len=1) -> Workload:
+    """Build one workload.
+
+    ``seq_k`` is the common length, or the inclusive upper bound of uniform random lengths
+    when ``varlen`` is set.  ``latent`` (default: dim != dim_v) makes V alias K[..., :dim_v].
+    """
+    if latent is None:
+        latent = dim != dim_v
+    g = torch.Generator(device="cpu").manual_seed(seed)
+    if varlen:
+        # lengths are drawn last in the stream order, but are needed first to size K/V;
+        # use a generator forked from the same seed so that the order stays reproducible.
+        gl = torch.Generator(device="cpu").manual_seed(seed + 0x5EED)
+        lens = torch.randint(min_len, seq_k + 1, (batch,), generator=gl, dtype=torch.int32)
+    else:
+        lens = torch.full((batch,), seq_k, dtype=torch.int32)
+    total_k = int(lens.sum().item())
+    q = torch.randn(batch, head_q, dim, generator=g, dtype=torch.float32).to(dtype)
+    k = torch.randn(total_k, head_k, dim, generator=g, dtype=torch.float32).to(dtype)
+    v = None
+    if not latent:
+        v = torch.randn(total_k, head_k, dim_v, generator=g, dtype=torch.float32).to(dtype)
+    cu = get_cu_seq(lens)
+    max_seq_k = int(lens.max().item()) if batch > 0 else 0
+    if name is None:
+        name = f"b{batch}_hq{head_q}_hk{head_k}_d{dim}_dv{dim_v}_sk{seq_k}{'_var' if varlen else ''}_" \
+               f"{'bf16' if dtype == torch.bfloat16 else 'fp16'}{'_alibi' if is_alibi else ''}"
+    return Workload(name, q, k, v, cu, max_seq_k, dim_v, is_alibi, [int(x) for x in lens.tolist()])
+
+
+# The five benchmark configurations (fixed shapes; sweeps take the swept value as an argument).
+def config_mha_cpu_case(seed=0):
+    return make_workload(1, 32, 32, 128, 128, 128, torch.float16, seed=seed, name="C0_mha_fp16_b1_sk128")
+
+
+def config_mha_sweep(batch, seq_k, seed=0):
+    return make_workload(batch, 32, 32, 128, 128, seq_k, torch.float16, seed=seed,
+                         name=f"C1_mha_fp16_b{batch}_sk{seq_k}")
+
+
+def config_gqa_varlen(seed=0, batch=64, max_len=8192):
+    return make_workload(batch, 32, 8, 128, 128, max_len, torch.bfloat16, seed=seed, varlen=True,
+                         name=f"C2_gqa_bf16_b{batch}_varlen{max_len}")
+
+
+def config_gqa_fixed(seed=0, batch=64, seq_k=4096):
+    return make_workload(batch, 32, 8, 128, 128, seq_k, torch.bfloat16, seed=seed,
+                         name=f"C2_gqa_bf16_b{batch}_sk{seq_k}")
+
+
+def config_mqa_alibi(seed=0, batch=32, seq_k=4096):
+    return make_workload(batch, 32, 1, 128, 128, seq_k, torch.float16, seed=seed, is_alibi=True,
+                         name=f"C3_mqa_fp16_alibi_b{batch}_sk{seq_k}")
+
+
+def config_mla(batch, seq_k, seed=0, dtype=torch.float16, head_q=128):
+    return make_workload(batch, head_q, 1, 576, 512, seq_k, dtype, seed=seed, latent=True,
+                         name=f"C4_mla_{'bf16' if dtype == torch.bfloat16 else 'fp16'}_b{batch}_sk{seq_k}")
+
+
+def algorithmic_bytes(batch, head_q, head_k, dim, dim_v, total_k, v_distinct, elem_bytes=2) -> int:
+    """HBM bytes the operation must move: Q, K, (V if it is its own buffer), O once each, plus cu_seq_k."""
+    elems = batch * head_q * dim + total_k * head_k * dim + batch * head_q * dim_v
+    if v_distinct:
+        elems += total_k * head_k * dim_v
+    return elem_bytes * elems + 4 * (batch + 1)
+
+
+def algorithmic_flops(head_q, dim, dim_v, total_k) -> int:
+    """2 * sum(len) * head_q * (dim + dim_v), the reference's count (csrc/common/tester.h:270)."""
+    return 2 * total_k * head_q * (dim + dim_v)
+
+
+def reference_formula_bytes(batch, head_q, head_k, dim, dim_v, seq_k, elem_bytes=2) -> int:
+    """The reference's bandwidth numerator (csrc/common/tester.h:273-276); it leaves V out."""
+    return elem_bytes * (batch * head_q * dim + batch * seq_k * head_k * dim + batch * head_q * dim_v)
+
+
+def workload_bytes(w: Workload) -> int:
+    return algorithmic_bytes(w.batch, w.head_q, w.head_k, w.dim, w.dim_v, int(w.k.shape[0]), w.v is not None)
+
+
+def workload_flops(w: Workload) -> int:
+    return algorithmic_flops(w.head_q, w.dim, w.dim_v, int(w.k.shape[0]))

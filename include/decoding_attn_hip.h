@@ -1,0 +1,108 @@
+/*
+ * C-ABI of libdecoding_attn_hip.so — single-query ("decoding") attention for MI355X (gfx950).
+ *
+ *   O[b,h,:] = softmax_j( scale * <Q[b,h,:], K[cu[b]+j, h/ratio, :]> + slope_h * (j - (len_b - 1)) ) . V[cu[b]+j, h/ratio, :]
+ *
+ * for MHA / GQA / MQA (dim == dim_v in {64, 96, 128, 256}) and the latent MLA form
+ * (dim 576, dim_v 512, v == NULL: V is the first 512 columns of every K row).
+ *
+ * All pointers are device pointers unless said otherwise; every call only enqueues work on
+ * `hip_stream` (a hipStream_t passed as void*, NULL = the default stream) and returns without
+ * synchronising.  Functions return 0 on success and a DA_ERR_* code otherwise; the message is
+ * available from da_last_error() on the calling thread.  Nothing here calls exit().
+ */
+#ifndef DECODING_ATTN_HIP_H_
+#define DECODING_ATTN_HIP_H_
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define DA_OK 0
+#define DA_ERR_INVALID_ARGUMENT 1 /* null pointer, misaligned pointer, head_q % head_k != 0, dim > 576, dim_v > 512 */
+#define DA_ERR_UNSUPPORTED 2      /* (dim, dim_v) pair outside the supported set */
+#define DA_ERR_WORKSPACE 3        /* caller workspace smaller than da_workspace_bytes() */
+#define DA_ERR_HIP 4              /* a HIP runtime call failed */
+
+/*
+ * Replaces the reference's
+ *   void decoding_attn(void *q, void *k, void *v, void *o, int *cu_seq_k, size_t max_seq_k, size_t batch,
+ *                      size_t head_q, size_t head_k, size_t dim, size_t dim_v, bool is_alibi, bool is_bf16,
+ *                      cudaStream_t stream)                         (reference csrc/ops/decoding_attn.h:29-30,
+ *                                                                    csrc/ops/decoding_attn.cpp:70-76)
+ * Same argument order and meaning; softmax scale is 1/sqrt(dim) (decoding_attn.cpp:54) and the ALiBi slope of
+ * head h is 2^(-8(h+1)/head_q) (csrc/kernel/decoding_attn/block_info.h:21).
+ *   q [batch, head_q, dim]; k [total_k, head_k, dim]; v [total_k, head_k, dim_v] or NULL (MLA);
+ *   o [batch, head_q, dim_v]; cu_seq_k [batch + 1] int32 prefix offsets; q/k/v 16-byte aligned.
+ * Split-sequence partials live in a workspace the library keeps per (device, stream) and grows on demand
+ * (growth calls hipMalloc; steady-state calls allocate nothing).  Use da_decoding_attn_ex to bring your own.
+ */
+int da_decoding_attn(const void *q, const void *k, const void *v, void *o, const int32_t *cu_seq_k, size_t max_seq_k,
+                     size_t batch, size_t head_q, size_t head_k, size_t dim, size_t dim_v, int is_alibi, int is_bf16,
+                     void *hip_stream);
+
+/*
+ * Same operation with the two constants of the reference exposed as arguments and a caller-owned workspace.
+ * Extends reference csrc/ops/decoding_attn.cpp:13-62 (set_dmha_fwd_params), which hard-codes both.
+ *   softmax_scale  <= 0 selects 1/sqrt(dim)
+ *   alibi_slopes   device float[head_q] or NULL for the closed form; read only when is_alibi != 0
+ *   workspace      device buffer of at least da_workspace_bytes(...) bytes, 16-byte aligned, or NULL to use the
+ *                  library's cached one
+ */
+int da_decoding_attn_ex(const void *q, const void *k, const void *v, void *o, const int32_t *cu_seq_k,
+                        size_t max_seq_k, size_t batch, size_t head_q, size_t head_k, size_t dim, size_t dim_v,
+                        int is_alibi, int is_bf16, float softmax_scale, const float *alibi_slopes, void *workspace,
+                        size_t workspace_bytes, void *hip_stream);
+
+/*
+ * Bytes of workspace da_decoding_attn_ex needs for this shape (0 when the sequence is not split).
+ * No counterpart in the reference, whose kernel never splits a sequence
+ * (csrc/kernel/decoding_attn/decoding_fwd_launch_template.h:12-31).
+ */
+size_t da_workspace_bytes(size_t max_seq_k, size_t batch, size_t head_q, size_t head_k, size_t dim, size_t dim_v);
+
+/*
+ * Launch plan the library would use for this shape, for tests and benchmarks:
+ *   kernel_kind 1 = VALU sweep, 2 = MFMA sweep (grouped heads / latent); nsplit = sequence splits;
+ *   chunk = tokens per split; heads_per_group = query heads one work-group serves.
+ * Any output pointer may be NULL.  Returns DA_ERR_UNSUPPORTED for an unsupported (dim, dim_v).
+ * Mirrors the role of the reference's per-head-dim tile choice (csrc/kernel/decoding_attn/decoding_fwd_hd*.cu).
+ */
+int da_plan(size_t max_seq_k, size_t batch, size_t head_q, size_t head_k, size_t dim, size_t dim_v, int is_bf16,
+            int *kernel_kind, int *nsplit, int *chunk, int *heads_per_group);
+
+/* 1 when (dim, dim_v) is a supported pair: the reference's DA_HEADDIM_SWITCH set (csrc/common/common.h:73-96). */
+int da_supported_head_dims(size_t dim, size_t dim_v);
+
+/* Message of the last failing call on this thread (never NULL).  Replaces the reference's log-and-exit
+ * DA_CHECK / DA_CHECK_CUDART_ERROR macros (csrc/common/common.h:17-49). */
+const char *da_last_error(void);
+
+/* Library version, major * 10000 + minor * 100 + patch (reference decoding_attn/__init__.py:15 holds "0.1.0"). */
+int da_version(void);
+
+#ifdef __cplusplus
+} /* extern "C" */
+
+/*
+ * C++ convenience overload with the reference's exact name and parameter list (reference
+ * csrc/ops/decoding_attn.h:29-30), the stream being a HIP stream.  Defined inline so that the shared
+ * library itself exports C symbols only.  Throws nothing; on failure it prints da_last_error() to stderr
+ * and returns (the reference would exit the process).
+ */
+#include <stdio.h>
+struct ihipStream_t;
+inline void decoding_attn(void *q, void *k, void *v, void *o, int *cu_seq_k, size_t max_seq_k, size_t batch,
+                          size_t head_q, size_t head_k, size_t dim, size_t dim_v, bool is_alibi, bool is_bf16,
+                          ihipStream_t *stream) {
+    if (da_decoding_attn(q, k, v, o, cu_seq_k, max_seq_k, batch, head_q, head_k, dim, dim_v, is_alibi ? 1 : 0,
+                         is_bf16 ? 1 : 0, (void *)stream) != DA_OK) {
+        fprintf(stderr, "decoding_attn: %s\n", da_last_error());
+    }
+}
+#endif
+
+#endif /* DECODING_ATTN_HIP_H_ */

@@ -1,0 +1,272 @@
+"""GPU parity: the HIP path, called through the C-ABI, against the CPU oracle on the same seeded inputs.
+
+Tolerances: max-abs <= 2e-3 (fp16) / 1e-2 (bf16) against the oracle's fp32-accumulated result, and the
+reference's own bar (mean-abs <= 5e-3, reference tests/test_decoding_attn.py:94,128) against its rounded
+output.  The case matrices re-author the reference's pytest grids (tests/test_decoding_attn.py:61-66,97-103)
+and add what they leave out: variable lengths, ALiBi, MQA, empty and ragged sequences.
+"""
+import pytest
+import torch
+
+from decoding_attention_amd import _lib, decoding_attn_fwd, fwd
+from decoding_attention_amd import workloads as wl
+from gpu_util import TOL, check_against_oracle, run_hip, run_oracle, sub_workload
+
+pytestmark = pytest.mark.gpu
+DTYPES = [torch.float16, torch.bfloat16]
+
+
+def _name(dtype):
+    return "bf16" if dtype == torch.bfloat16 else "fp16"
+
+
+def test_config0_mha_cpu_case():
+    w = wl.config_mha_cpu_case()
+    check_against_oracle(w, run_hip(w))
+
+
+@pytest.mark.parametrize("dtype", DTYPES, ids=_name)
+@pytest.mark.parametrize("seq_k", [1, 128, 512])
+@pytest.mark.parametrize("batch", [1, 2, 16])
+@pytest.mark.parametrize("dim", [64, 96, 128, 256])
+@pytest.mark.parametrize("head_k", [8, 32])
+@pytest.mark.parametrize("head_q", [32, 64])
+def test_reference_grid_mha_gqa(head_q, head_k, dim, batch, seq_k, dtype):
+    w = wl.make_workload(batch, head_q, head_k, dim, dim, seq_k, dtype, seed=head_q + head_k + dim + batch + seq_k)
+    check_against_oracle(w, run_hip(w))
+
+
+@pytest.mark.parametrize("dtype", DTYPES, ids=_name)
+@pytest.mark.parametrize("seq_k", [1, 128, 512])
+@pytest.mark.parametrize("batch", [1, 2, 16])
+@pytest.mark.parametrize("head_q", [16, 32, 64, 128])
+def test_reference_grid_mla(head_q, batch, seq_k, dtype):
+    w = wl.config_mla(batch, seq_k, seed=head_q + batch + seq_k, dtype=dtype, head_q=head_q)
+    check_against_oracle(w, run_hip(w))
+
+
+@pytest.mark.parametrize("batch,seq_k", [(1, 128), (8, 128), (32, 128), (1, 512), (1, 1536), (1, 4096), (1, 8192)])
+def test_config1_mha_sweep_points(batch, seq_k):
+    w = wl.config_mha_sweep(batch, seq_k)
+    check_against_oracle(w, run_hip(w))
+
+
+def test_config2_gqa_varlen_scaled():
+    w = wl.config_gqa_varlen(seed=1, batch=16, max_len=2048)
+    check_against_oracle(w, run_hip(w))
+
+
+def test_config2_gqa_varlen_full_size_spot_checked():
+    w = wl.config_gqa_varlen(seed=0)
+    o = run_hip(w)
+    assert torch.isfinite(o.float()).all()
+    order = sorted(range(w.batch), key=lambda b: w.lengths[b])
+    rows = [order[0], order[1], order[len(order) // 2], order[-1]]  # shortest, median, longest
+    sub = sub_workload(w, rows)
+    _, ref32 = run_oracle(sub)
+    assert (o[rows].float() - ref32).abs().max().item() <= TOL[torch.bfloat16]
+
+
+def test_config2_gqa_fixed_4096_spot_checked():
+    w = wl.config_gqa_fixed(seed=0)
+    o = run_hip(w)
+    rows = [0, 31, 63]
+    _, ref32 = run_oracle(sub_workload(w, rows))
+    assert (o[rows].float() - ref32).abs().max().item() <= TOL[torch.bfloat16]
+
+
+def test_config3_mqa_alibi_scaled_and_full():
+    w = wl.config_mqa_alibi(seed=2, batch=4, seq_k=1024)
+    check_against_oracle(w, run_hip(w))
+    w = wl.config_mqa_alibi(seed=0)
+    o = run_hip(w)
+    rows = [0, 17]
+    _, ref32 = run_oracle(sub_workload(w, rows))
+    assert (o[rows].float() - ref32).abs().max().item() <= TOL[torch.float16]
+
+
+@pytest.mark.parametrize("batch,seq_k", [(1, 4096), (16, 512), (2, 16384)])
+def test_config4_mla_points(batch, seq_k):
+    w = wl.config_mla(batch, seq_k)
+    o = run_hip(w)
+    rows = [0] if batch == 1 else [0, batch - 1]
+    sub = sub_workload(w, rows)
+    _, ref32 = run_oracle(sub)
+    assert (o[rows].float() - ref32).abs().max().item() <= TOL[torch.float16]
+
+
+def test_config4_mla_b64_full_size_spot_checked():
+    w = wl.config_mla(64, 4096)
+    o = run_hip(w)
+    assert torch.isfinite(o.float()).all()
+    rows = [5, 63]
+    _, ref32 = run_oracle(sub_workload(w, rows))
+    assert (o[rows].float() - ref32).abs().max().item() <= TOL[torch.float16]
+
+
+@pytest.mark.parametrize("dtype", DTYPES, ids=_name)
+@pytest.mark.parametrize("hq,hk", [(8, 8), (8, 4), (12, 4), (8, 1), (32, 1), (20, 4), (48, 8)])
+def test_head_group_shapes(hq, hk, dtype):
+    """Group sizes 1, 2, 3, 4, 5, 6, 8, 32 (3, 5 and 6 leave a partly idle work-group)."""
+    w = wl.make_workload(3, hq, hk, 128, 128, 333, dtype, seed=hq * 7 + hk, varlen=True)
+    check_against_oracle(w, run_hip(w))
+
+
+@pytest.mark.parametrize("dim", [64, 96, 128, 256])
+def test_ragged_lengths_with_empty_and_single(dim):
+    lens = torch.tensor([0, 1, 2, 63, 64, 65, 127, 129, 0, 700, 1, 0], dtype=torch.int32)
+    g = torch.Generator().manual_seed(dim)
+    total = int(lens.sum())
+    q = torch.randn(len(lens), 8, dim, generator=g).to(torch.float16)
+    k = torch.randn(total, 2, dim, generator=g).to(torch.float16)
+    v = torch.randn(total, 2, dim, generator=g).to(torch.float16)
+    w = wl.Workload("ragged", q, k, v, wl.get_cu_seq(lens), int(lens.max()), dim, False, lens.tolist())
+    o = run_hip(w)
+    check_against_oracle(w, o)
+    for b, n in enumerate(lens.tolist()):
+        if n == 0:
+            assert (o[b].float() == 0).all()  # documented: an empty sequence yields zeros
+        if n == 1:
+            start = int(w.cu_seq_k[b])
+            assert torch.equal(o[b].view(torch.int16), v[start].repeat_interleave(4, dim=0).view(torch.int16))
+
+
+def test_ragged_mla_with_empty():
+    lens = torch.tensor([0, 1, 65, 300, 0, 1031], dtype=torch.int32)
+    g = torch.Generator().manual_seed(5)
+    total = int(lens.sum())
+    q = torch.randn(len(lens), 128, 576, generator=g).to(torch.bfloat16)
+    k = torch.randn(total, 1, 576, generator=g).to(torch.bfloat16)
+    w = wl.Workload("ragged_mla", q, k, None, wl.get_cu_seq(lens), int(lens.max()), 512, False, lens.tolist())
+    o = run_hip(w)
+    check_against_oracle(w, o)
+    assert (o[0].float() == 0).all() and (o[4].float() == 0).all()
+    assert torch.equal(o[1, 7].view(torch.int16), k[0, 0, :512].view(torch.int16))
+
+
+def test_split_and_unsplit_agree():
+    """One sequence alone is split many ways; inside a large batch it is not.  Both must match the oracle
+    and each other."""
+    big = wl.make_workload(256, 32, 8, 128, 128, 2048, torch.float16, seed=21)
+    p_big = _lib.plan(2048, 256, 32, 8, 128, 128)
+    o_big = run_hip(big)
+    one = sub_workload(big, [3])
+    p_one = _lib.plan(2048, 1, 32, 8, 128, 128)
+    assert p_one["nsplit"] > p_big["nsplit"]
+    o_one = run_hip(one)
+    _, ref32 = run_oracle(one)
+    assert (o_one.float() - ref32).abs().max().item() <= TOL[torch.float16]
+    assert (o_big[3:4].float() - ref32).abs().max().item() <= TOL[torch.float16]
+    assert (o_big[3:4].float() - o_one.float()).abs().max().item() <= 1e-3
+
+
+def test_repeated_calls_are_bit_identical():
+    for w in (wl.config_mha_sweep(1, 4096), wl.config_mla(2, 1024), wl.config_gqa_varlen(seed=4, batch=8, max_len=1024)):
+        a = run_hip(w)
+        b = run_hip(w)
+        assert torch.equal(a.view(torch.int16), b.view(torch.int16))
+
+
+def test_alibi_default_and_custom_slopes():
+    w = wl.make_workload(3, 16, 4, 128, 128, 777, torch.float16, seed=31, varlen=True, is_alibi=True)
+    check_against_oracle(w, run_hip(w))
+    slopes = torch.linspace(0.01, 0.7, 16, dtype=torch.float32)
+    o = run_hip(w, alibi_slopes=slopes.cuda())
+    check_against_oracle(w, o, alibi_slopes=slopes.numpy())
+    w2 = wl.make_workload(2, 128, 1, 576, 512, 300, torch.float16, seed=32, is_alibi=True, latent=True)
+    check_against_oracle(w2, run_hip(w2))
+
+
+def test_softmax_scale_argument():
+    w = wl.make_workload(2, 8, 2, 64, 64, 200, torch.bfloat16, seed=33)
+    o = run_hip(w, softmax_scale=0.3)
+    check_against_oracle(w, o, softmax_scale=0.3)
+
+
+def test_max_seq_k_larger_than_needed_and_output_argument():
+    w = wl.make_workload(4, 32, 8, 128, 128, 300, torch.float16, seed=34, varlen=True)
+    dev = torch.device("cuda:0")
+    wd = w.to(dev)
+    o_buf = torch.full((4, 32, 128), 7.0, dtype=torch.float16, device=dev)
+    out = fwd(wd.q, wd.k, wd.v, o_buf, wd.cu_seq_k, 5000, 128, False)
+    torch.cuda.synchronize()
+    assert out.data_ptr() == o_buf.data_ptr()
+    check_against_oracle(w, out.cpu())
+
+
+def test_non_contiguous_inputs_are_copied_not_misread():
+    w = wl.make_workload(2, 8, 8, 64, 64, 50, torch.float16, seed=35)
+    dev = torch.device("cuda:0")
+    k_wide = torch.zeros(100, 8, 128, dtype=torch.float16, device=dev)
+    k_wide[:, :, :64] = w.k.to(dev)
+    k_view = k_wide[:, :, :64]          # unit last stride, but not dense: the reference would mis-read it
+    v_t = w.v.to(dev).transpose(0, 1).contiguous().transpose(0, 1)  # last stride 1, rows permuted in memory
+    o = decoding_attn_fwd(w.q.to(dev), k_view, v_t, w.cu_seq_k.to(dev), 50, 64, False)
+    torch.cuda.synchronize()
+    check_against_oracle(w, o.cpu())
+
+
+def test_non_default_stream():
+    w = wl.config_mha_sweep(1, 2048)
+    dev = torch.device("cuda:0")
+    wd = w.to(dev)
+    s = torch.cuda.Stream()
+    s.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(s):
+        o = decoding_attn_fwd(wd.q, wd.k, wd.v, wd.cu_seq_k, wd.max_seq_k, 128, False)
+    s.synchronize()
+    check_against_oracle(w, o.cpu())
+
+
+def test_reference_signature_entry_point_with_library_workspace():
+    """da_decoding_attn (the reference's argument list, library-owned workspace) on a split shape."""
+    lib = _lib.load()
+    w = wl.config_mha_sweep(1, 4096)
+    assert _lib.plan(4096, 1, 32, 32, 128, 128)["nsplit"] > 1
+    dev = torch.device("cuda:0")
+    wd = w.to(dev)
+    o = torch.empty(1, 32, 128, dtype=torch.float16, device=dev)
+    for _ in range(2):
+        rc = lib.da_decoding_attn(wd.q.data_ptr(), wd.k.data_ptr(), wd.v.data_ptr(), o.data_ptr(),
+                                  wd.cu_seq_k.data_ptr(), 4096, 1, 32, 32, 128, 128, 0, 0,
+                                  torch.cuda.current_stream().cuda_stream)
+        assert rc == 0, _lib.last_error()
+    torch.cuda.synchronize()
+    check_against_oracle(w, o.cpu())
+
+
+def test_gpu_side_argument_errors():
+    lib = _lib.load()
+    dev = torch.device("cuda:0")
+    w = wl.config_mha_sweep(1, 4096).to(dev)
+    o = torch.empty(1, 32, 128, dtype=torch.float16, device=dev)
+    small = torch.empty(64, dtype=torch.uint8, device=dev)
+    rc = lib.da_decoding_attn_ex(w.q.data_ptr(), w.k.data_ptr(), w.v.data_ptr(), o.data_ptr(), w.cu_seq_k.data_ptr(),
+                                 4096, 1, 32, 32, 128, 128, 0, 0, 0.0, None, small.data_ptr(), 64, None)
+    assert rc == _lib.DA_ERR_WORKSPACE and "workspace" in _lib.last_error()
+    with pytest.raises(RuntimeError, match="one query token per sequence"):
+        fwd(torch.cat([w.q, w.q]), w.k, w.v, None, w.cu_seq_k, 4096, 128, False)
+    with pytest.raises(RuntimeError, match="shape"):
+        fwd(w.q, w.k, w.v[:-1], None, w.cu_seq_k, 4096, 128, False)
+    with pytest.raises(RuntimeError, match="unsupported head dims"):
+        fwd(w.q[..., :80].contiguous(), w.k[..., :80].contiguous(), None, None, w.cu_seq_k, 4096, 80, False)
+    with pytest.raises(RuntimeError, match="batch size must be positive"):
+        fwd(w.q[:0], w.k, w.v, None, w.cu_seq_k[:1], 4096, 128, False)
+
+
+def test_full_size_properties_gqa():
+    """Size-independent properties at the benchmark shape: q = 0 gives the mean of V; constant V comes back."""
+    dev = torch.device("cuda:0")
+    b, hq, hk, d, sk = 64, 32, 8, 128, 4096
+    g = torch.Generator().manual_seed(41)
+    k = torch.randn(b * sk, hk, d, generator=g).to(torch.bfloat16).to(dev)
+    v = torch.randn(b * sk, hk, d, generator=g).to(torch.bfloat16).to(dev)
+    cu = wl.get_cu_seq(torch.full((b,), sk, dtype=torch.int32)).to(dev)
+    q0 = torch.zeros(b, hq, d, dtype=torch.bfloat16, device=dev)
+    o = decoding_attn_fwd(q0, k, v, cu, sk, d, False).float()
+    mean_v = v.float().reshape(b, sk, hk, d).mean(dim=1).repeat_interleave(hq // hk, dim=1)
+    assert (o - mean_v).abs().max().item() <= 2e-3  # |mean| ~ 0.016, bf16 rounding step there is 6e-5
+    q = torch.randn(b, hq, d, generator=g).to(torch.bfloat16).to(dev)
+    vc = torch.full_like(v, 0.375)
+    o = decoding_attn_fwd(q, k, vc, cu, sk, d, False).float()
+    assert (o - 0.375).abs().max().item() <= 2e-3

@@ -1,0 +1,113 @@
+"""CPU-side checks: the shared library loads and exports the declared C-ABI, argument validation returns
+the documented codes before anything touches a GPU, the launch planner is self-consistent, and the Python
+face rejects what the reference's binding rejects (reference csrc/torch/decoding_torch.cpp:24-74)."""
+import ctypes
+import os
+import re
+
+import pytest
+import torch
+
+from decoding_attention_amd import _lib, interface
+from decoding_attention_amd import workloads as wl
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+LEGAL = [(64, 64), (96, 96), (128, 128), (256, 256), (576, 512)]
+
+
+def test_header_symbols_are_exported():
+    text = open(os.path.join(ROOT, "include", "decoding_attn_hip.h")).read()
+    c_part = text.split('#ifdef __cplusplus\n} /* extern "C" */')[0]
+    declared = set(re.findall(r"\b(da_[a-z_0-9]+)\s*\(", c_part))
+    assert declared == set(_lib.EXPORTED_SYMBOLS)
+    lib = ctypes.CDLL(_lib.LIB_PATH)
+    for name in declared:
+        assert getattr(lib, name) is not None
+
+
+def test_version_and_supported_dims():
+    lib = _lib.load()
+    assert lib.da_version() == 100
+    for d in (32, 64, 96, 128, 192, 256, 512, 576):
+        for dv in (64, 96, 128, 256, 512, 576):
+            assert bool(lib.da_supported_head_dims(d, dv)) == ((d, dv) in LEGAL)
+
+
+def _call_ex(lib, q=16, k=16, v=16, o=16, cu=16, max_seq_k=8, batch=1, hq=4, hk=4, d=64, dv=64):
+    return lib.da_decoding_attn_ex(q, k, v, o, cu, max_seq_k, batch, hq, hk, d, dv, 0, 0, 0.0, None, None, 0, None)
+
+
+def test_argument_errors_without_gpu():
+    lib = _lib.load()
+    assert _call_ex(lib, q=None) == _lib.DA_ERR_INVALID_ARGUMENT and "q is null" in _lib.last_error()
+    assert _call_ex(lib, k=None) == _lib.DA_ERR_INVALID_ARGUMENT
+    assert _call_ex(lib, o=None) == _lib.DA_ERR_INVALID_ARGUMENT
+    assert _call_ex(lib, cu=None) == _lib.DA_ERR_INVALID_ARGUMENT
+    assert _call_ex(lib, hq=6, hk=4) == _lib.DA_ERR_INVALID_ARGUMENT and "multiple" in _lib.last_error()
+    assert _call_ex(lib, d=640, dv=64) == _lib.DA_ERR_INVALID_ARGUMENT
+    assert _call_ex(lib, d=576, dv=576) == _lib.DA_ERR_INVALID_ARGUMENT
+    assert _call_ex(lib, d=80, dv=80) == _lib.DA_ERR_UNSUPPORTED and "unsupported" in _lib.last_error()
+    assert _call_ex(lib, d=128, dv=64) == _lib.DA_ERR_UNSUPPORTED
+    assert _call_ex(lib, q=24) == _lib.DA_ERR_INVALID_ARGUMENT and "aligned" in _lib.last_error()
+    assert _call_ex(lib, batch=0) == _lib.DA_OK  # nothing to do, nothing launched
+
+
+@pytest.mark.parametrize("d,dv", LEGAL)
+@pytest.mark.parametrize("batch", [1, 16, 64, 2048])
+@pytest.mark.parametrize("sk", [1, 128, 1536, 4096, 16384])
+def test_plan_is_consistent(d, dv, batch, sk):
+    hq, hk = (128, 1) if d == 576 else (32, 8)
+    p = _lib.plan(sk, batch, hq, hk, d, dv)
+    assert p["kind"] in (1, 2)
+    assert 1 <= p["nsplit"] <= 256
+    assert p["nsplit"] * p["chunk"] >= sk
+    assert (p["nsplit"] - 1) * p["chunk"] < max(sk, 1)
+    ws = _lib.load().da_workspace_bytes(sk, batch, hq, hk, d, dv)
+    assert ws == (0 if p["nsplit"] == 1 else batch * hq * p["nsplit"] * (dv + 2) * 4)
+
+
+def test_plan_rejects_bad_shapes():
+    with pytest.raises(RuntimeError):
+        _lib.plan(128, 1, 6, 4, 64, 64)
+    with pytest.raises(RuntimeError):
+        _lib.plan(128, 1, 4, 4, 80, 80)
+
+
+def test_python_face_checks_cpu_inputs():
+    w = wl.make_workload(2, 4, 2, 64, 64, 8, torch.float16)
+    with pytest.raises(RuntimeError, match="GPU"):
+        interface.decoding_attn_fwd(w.q, w.k, w.v, w.cu_seq_k, 8, 64, False)
+    with pytest.raises(RuntimeError, match="FP16 and BF16"):
+        interface.fwd(w.q.float(), w.k.float(), None, None, w.cu_seq_k, 8, 64, False)
+    with pytest.raises(RuntimeError, match="same dtype"):
+        interface.fwd(w.q, w.k.to(torch.bfloat16), None, None, w.cu_seq_k, 8, 64, False)
+    with pytest.raises(RuntimeError, match="int32"):
+        interface.fwd(w.q, w.k, None, None, w.cu_seq_k.long(), 8, 64, False)
+
+
+def test_drop_in_package_name():
+    import decoding_attn
+
+    assert decoding_attn.decoding_attn_fwd is interface.decoding_attn_fwd
+    assert decoding_attn.__version__ == "0.1.0"
+
+
+def test_work_formulas():
+    # figures quoted for the benchmark configurations
+    assert wl.algorithmic_bytes(1, 32, 32, 128, 128, 128, True) == 2 * (4096 + 2 * 128 * 4096 + 4096) + 8
+    gqa = wl.algorithmic_bytes(64, 32, 8, 128, 128, 64 * 4096, True)
+    assert abs(gqa - 1074.8e6) < 0.1e6
+    mla = wl.algorithmic_bytes(64, 128, 1, 576, 512, 64 * 4096, False)
+    assert abs(mla - 319.8e6) < 0.1e6
+    assert wl.algorithmic_flops(128, 576, 512, 64 * 4096) == 2 * 64 * 4096 * 128 * 1088
+    assert wl.reference_formula_bytes(1, 32, 32, 128, 128, 128) == 2 * (4096 + 128 * 4096 + 4096)
+
+
+def test_workloads_are_reproducible():
+    a = wl.config_gqa_varlen(seed=3, batch=4, max_len=64)
+    b = wl.config_gqa_varlen(seed=3, batch=4, max_len=64)
+    assert a.lengths == b.lengths and torch.equal(a.k.view(torch.int16), b.k.view(torch.int16))
+    assert a.cu_seq_k.tolist()[-1] == sum(a.lengths) == a.k.shape[0]
+    assert 1 <= min(a.lengths) and max(a.lengths) <= 64 and a.max_seq_k == max(a.lengths)
+    m = wl.config_mla(2, 16)
+    assert m.v is None and m.q.shape == (2, 128, 576) and m.dim_v == 512
