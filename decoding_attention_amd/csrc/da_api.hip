@@ -41,9 +41,10 @@ int env_int(const char* name, int dflt) {
 // Tunables, read once.  DA_TARGET_WGS: work-groups a launch should reach before the sequence
 // stops being split further; DA_MAX_CHUNK / DA_MIN_CHUNK: bounds on tokens per split.
 struct Tunables {
-    int target_wgs, max_chunk, min_chunk, force_kind;
+    int target_wgs, mfma_target_wgs, max_chunk, min_chunk, force_kind;
     Tunables() {
         target_wgs = env_int("DA_TARGET_WGS", 1024);
+        mfma_target_wgs = env_int("DA_MFMA_TARGET_WGS", 256);
         max_chunk = env_int("DA_MAX_CHUNK", 1024);
         min_chunk = env_int("DA_MIN_CHUNK", 256);
         force_kind = env_int("DA_FORCE_KIND", 0);
@@ -82,15 +83,19 @@ int rows_per_trip(size_t dim) {
     }
 }
 
-Plan make_plan(size_t max_seq_k, size_t batch, size_t head_q, size_t head_k, size_t dim, size_t dim_v) {
+// v_distinct: V is its own buffer (the MFMA kernel reads V out of the K tile, so it needs the aliased form).
+Plan make_plan(size_t max_seq_k, size_t batch, size_t head_q, size_t head_k, size_t dim, size_t dim_v,
+               bool v_distinct) {
     Plan pl;
     const int ratio = (int)(head_q / head_k);
     int trip;
-    const bool mfma = da::mla_supported(dim, dim_v, ratio) && tun().force_kind != kKindSweep;
+    int target_wgs = tun().target_wgs;
+    const bool mfma = !v_distinct && da::mla_supported(dim, dim_v, ratio) && tun().force_kind != kKindSweep;
     if (mfma) {
         pl.kind = kKindMfma;
         pl.rt = da::mla_heads_per_group(ratio);
         trip = da::mla_rows_per_trip();
+        target_wgs = tun().mfma_target_wgs;  // one 4-wave work-group fills a CU
     } else {
         pl.kind = kKindSweep;
         const int max_rt = dim > 256 ? 2 : 4;
@@ -101,9 +106,11 @@ Plan make_plan(size_t max_seq_k, size_t batch, size_t head_q, size_t head_k, siz
     pl.groups = (ratio + pl.rt - 1) / pl.rt;
     const long long base = (long long)batch * (long long)head_k * pl.groups;
     const int min_chunk = std::max(tun().min_chunk, trip);
-    long long want = base > 0 ? (tun().target_wgs + base - 1) / base : 1;
+    long long want = base > 0 ? (target_wgs + base - 1) / base : 1;
     const long long by_len = std::max<long long>(1, (long long)max_seq_k / min_chunk);
-    long long by_cap = ((long long)max_seq_k + tun().max_chunk - 1) / std::max(1, tun().max_chunk);
+    // sweep work-groups are also kept short so that ragged batches balance; the MFMA kernel's partials are too
+    // large (heads x dim_v floats per split) to split more than occupancy asks for
+    long long by_cap = mfma ? 1 : ((long long)max_seq_k + tun().max_chunk - 1) / std::max(1, tun().max_chunk);
     long long ns = std::max(std::min(want, by_len), std::min(by_cap, by_len));
     ns = std::max<long long>(1, std::min<long long>(ns, kMaxSplits));
     long long chunk = ((long long)max_seq_k + ns - 1) / ns;
@@ -168,7 +175,7 @@ int da_plan(size_t max_seq_k, size_t batch, size_t head_q, size_t head_k, size_t
         return fail(DA_ERR_INVALID_ARGUMENT, "head_q (%zu) must be a multiple of head_k (%zu)", head_q, head_k);
     if (!supported_dims(dim, dim_v))
         return fail(DA_ERR_UNSUPPORTED, "unsupported head dims (dim %zu, dim_v %zu)", dim, dim_v);
-    const Plan pl = make_plan(max_seq_k, batch, head_q, head_k, dim, dim_v);
+    const Plan pl = make_plan(max_seq_k, batch, head_q, head_k, dim, dim_v, false);
     if (kernel_kind) *kernel_kind = pl.kind;
     if (nsplit) *nsplit = pl.nsplit;
     if (chunk) *chunk = pl.chunk;
@@ -178,7 +185,9 @@ int da_plan(size_t max_seq_k, size_t batch, size_t head_q, size_t head_k, size_t
 
 size_t da_workspace_bytes(size_t max_seq_k, size_t batch, size_t head_q, size_t head_k, size_t dim, size_t dim_v) {
     if (head_k == 0 || head_q % head_k != 0 || !supported_dims(dim, dim_v)) return 0;
-    return make_plan(max_seq_k, batch, head_q, head_k, dim, dim_v).ws_bytes;
+    const size_t a = make_plan(max_seq_k, batch, head_q, head_k, dim, dim_v, false).ws_bytes;
+    const size_t b = make_plan(max_seq_k, batch, head_q, head_k, dim, dim_v, true).ws_bytes;
+    return a > b ? a : b;
 }
 
 int da_decoding_attn_ex(const void* q, const void* k, const void* v, void* o, const int32_t* cu_seq_k,
@@ -203,14 +212,13 @@ int da_decoding_attn_ex(const void* q, const void* k, const void* v, void* o, co
     if (!aligned16(q) || !aligned16(k) || (v && !aligned16(v)))
         return fail(DA_ERR_INVALID_ARGUMENT, "q, k and v must be 16-byte aligned");
     if ((reinterpret_cast<uintptr_t>(o) & 1u) != 0) return fail(DA_ERR_INVALID_ARGUMENT, "o must be 2-byte aligned");
-    if (max_seq_k > (size_t)INT32_MAX || batch > 65535 * (size_t)64 || head_q > 65535)
-        return fail(DA_ERR_INVALID_ARGUMENT, "shape out of range (max_seq_k %zu, batch %zu, head_q %zu)", max_seq_k,
-                    batch, head_q);
+    if (max_seq_k > (size_t)INT32_MAX || batch > 65535 || head_q > 65535)
+        return fail(DA_ERR_INVALID_ARGUMENT, "shape out of range (max_seq_k %zu, batch %zu, head_q %zu; grid limit 65535)",
+                    max_seq_k, batch, head_q);
     if (batch == 0) return DA_OK;
 
     hipStream_t stream = reinterpret_cast<hipStream_t>(hip_stream);
-    const Plan pl = make_plan(max_seq_k, batch, head_q, head_k, dim, dim_v);
-    if (batch > 65535) return fail(DA_ERR_INVALID_ARGUMENT, "batch (%zu) exceeds the grid limit 65535", batch);
+    const Plan pl = make_plan(max_seq_k, batch, head_q, head_k, dim, dim_v, v != nullptr);
     if ((size_t)head_k * pl.groups > 65535)
         return fail(DA_ERR_INVALID_ARGUMENT, "head_k * groups exceeds the grid limit 65535");
 

@@ -1,7 +1,387 @@
+// MFMA sweep for many query heads over one KV head whose values are the leading columns of
+// the keys (the latent MLA form: 128 heads, key width 576, value width 512).
+//
+// One work-group serves one (sequence, head group of up to 128 heads, sequence split).  Each of
+// its wavefronts owns 32 query heads: their Q rows stay in registers as MFMA B-operands
+// (36 k-steps x 4 VGPRs), their un-normalised output O^T[512 x 32] stays in 16 accumulator
+// tiles (256 registers), so one wavefront per SIMD uses the whole 512-register budget.
+//
+// K tiles of 32 tokens stream HBM -> LDS with direct-to-LDS loads (no register staging),
+// three buffers deep.  A tile is read from LDS twice and from HBM once:
+//   S^T[32 tok x 32 heads] = K_tile . Q^T      K rows as A-operands, ds_read_b128
+//   O^T[512 x 32 heads]   += V_tile^T . P^T    V = K[:, :512]; the A-operand needs 8 tokens of
+//                                              one column per lane, delivered by the LDS
+//                                              transpose read ds_read_b64_tr_b16
+// The score tile leaves the MFMA with one head per lane (column n = lane % 32) and 16 tokens
+// per lane, so the online softmax is lane-local but for one exchange between the two
+// half-waves, and the probabilities feed the second MFMA as its B-operand without any lane
+// movement (the token <-> k-index permutation is applied to V's rows instead).
+//
+// LDS rows are padded by 16 bytes (pitch 1168) which makes both read patterns conflict-free.
+//
+// Mathematics as in the reference kernel (csrc/kernel/decoding_attn/decoding_fwd_kernel.h:50-235
+// with the latent aliasing of csrc/ops/decoding_attn.cpp:30-37); the structure is unrelated.
 #include "da_mla.h"
+
+#include <mutex>
+
 namespace da {
-bool mla_supported(size_t, size_t, int) { return false; }
-int mla_heads_per_group(int) { return 1; }
-int mla_rows_per_trip() { return 64; }
-hipError_t launch_mla(const SweepParams&, bool, int, dim3, hipStream_t) { return hipErrorNotSupported; }
+
+namespace {
+
+constexpr int kTile = 32;  // tokens per LDS tile
+constexpr int kNBuf = 3;   // LDS tile buffers (two tiles in flight behind the one being read)
+constexpr float kLazy = 8.0f;  // the running maximum moves only when exceeded by this much (log2 units)
+
+typedef short s16x4 __attribute__((__vector_size__(4 * sizeof(short))));
+
+template <typename Tag>
+struct Mma;
+template <>
+struct Mma<f16_tag> {
+    typedef f16x8 vec8;
+    static __device__ __forceinline__ f32x16 mma(vec8 a, vec8 b, f32x16 c) {
+        return __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c, 0, 0, 0);
+    }
+    // same product with the accumulator pinned to ordinary VGPRs (the score tile: the accumulation
+    // registers are all taken by the output tiles)
+    static __device__ __forceinline__ void mma_v(vec8 a, vec8 b, f32x16& c) {
+        asm("v_mfma_f32_32x32x16_f16 %0, %1, %2, %0" : "+v"(c) : "v"(a), "v"(b));
+    }
+    static __device__ __forceinline__ void mma_v0(vec8 a, vec8 b, f32x16& c) {  // c = a.b
+        asm("v_mfma_f32_32x32x16_f16 %0, %1, %2, 0" : "=v"(c) : "v"(a), "v"(b));
+    }
+    static __device__ __forceinline__ vec8 pack8(const float* x) {
+        vec8 v;
+#pragma unroll
+        for (int j = 0; j < 8; ++j) v[j] = (_Float16)x[j];
+        return v;
+    }
+};
+template <>
+struct Mma<bf16_tag> {
+    typedef bf16x8 vec8;
+    static __device__ __forceinline__ f32x16 mma(vec8 a, vec8 b, f32x16 c) {
+        return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0);
+    }
+    static __device__ __forceinline__ void mma_v(vec8 a, vec8 b, f32x16& c) {
+        asm("v_mfma_f32_32x32x16_bf16 %0, %1, %2, %0" : "+v"(c) : "v"(a), "v"(b));
+    }
+    static __device__ __forceinline__ void mma_v0(vec8 a, vec8 b, f32x16& c) {
+        asm("v_mfma_f32_32x32x16_bf16 %0, %1, %2, 0" : "=v"(c) : "v"(a), "v"(b));
+    }
+    static __device__ __forceinline__ vec8 pack8(const float* x) {
+        vec8 v;
+#pragma unroll
+        for (int j = 0; j < 8; ++j) v[j] = (__bf16)x[j];
+        return v;
+    }
+};
+
+// 16 bytes per lane from global memory straight into LDS at lds_off + lane * 16 (lds_off is
+// wave-uniform).  Issued from assembly so that the wait for it is placed by hand: the
+// compiler would otherwise drain every outstanding load before the next LDS read.
+__device__ __forceinline__ void lds_dma16(const void* gptr, uint32_t lds_off) {
+    const uint32_t off = __builtin_amdgcn_readfirstlane(lds_off);
+    asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off" ::"v"(gptr), "s"(off) : "memory");
+}
+
+// x *= alpha for an MFMA accumulator element that lives in an accumulation register.  Written as
+// assembly on the AGPR so that the (rare) rescale path does not pull the 256 accumulators of a
+// wave into ordinary VGPRs around the whole loop.
+__device__ __forceinline__ void scale_acc(float& x, float alpha) {
+    float tmp;
+    asm volatile("v_accvgpr_read_b32 %1, %0\n\tv_mul_f32 %1, %1, %2\n\ts_nop 0\n\tv_accvgpr_write_b32 %0, %1"
+                 : "+a"(x), "=&v"(tmp)
+                 : "v"(alpha));
+}
+
+template <int N>
+__device__ __forceinline__ void wait_vmcnt() {
+    asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory");
+}
+
+template <typename Tag, int D, int DV, int NWV>
+__global__ __launch_bounds__(64 * NWV) void mfma_latent_kernel(const SweepParams p) {
+    using MM = Mma<Tag>;
+    using vec8 = typename MM::vec8;
+    using EL = Elem<Tag>;
+    constexpr int PITCH = D * 2 + 16;                    // bytes per LDS row
+    constexpr int SPR = PITCH / 16;                      // 16-byte slots per row
+    constexpr int NINSTR = (kTile * SPR + 63) / 64;      // load instructions per tile (whole work-group)
+    constexpr int BUF = NINSTR * 1024;                   // bytes per tile buffer
+    constexpr int NLW = (NINSTR + NWV - 1) / NWV;        // load instructions per tile per wave
+    constexpr int KS = D / 16;                           // k-steps of Q K^T
+    constexpr int CT = DV / 32;                          // 32-column tiles of the output
+    static_assert(D % 16 == 0 && DV % 32 == 0 && DV <= D, "shape");
+
+    extern __shared__ __attribute__((aligned(1024))) uint8_t smem[];  // kNBuf * BUF, then 1 KiB that absorbs surplus loads
+    const uint32_t smem_off = (uint32_t)(uintptr_t)smem;
+
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int half = lane >> 5;
+    const int n = lane & 31;
+
+    const int split = blockIdx.x;
+    const int hk = blockIdx.y / p.groups;
+    const int grp = blockIdx.y % p.groups;
+    const int b = blockIdx.z;
+
+    const int start = p.cu_seq_k[b];
+    const int len = p.cu_seq_k[b + 1] - start;
+    const int c0 = split * p.chunk;
+    const int c1 = (split == p.nsplit - 1) ? len : min(len, c0 + p.chunk);
+
+    const int wg_heads = min(32 * NWV, p.ratio - grp * 32 * NWV);  // live heads of this work-group
+    const int nh = max(0, min(32, wg_heads - wave * 32));          // live heads of this wave
+    const int h_base = hk * p.ratio + grp * 32 * NWV + wave * 32;
+    uint16_t* const o16 = reinterpret_cast<uint16_t*>(p.o);
+
+    if (c0 >= c1) {
+        if (p.nsplit == 1 && n < nh) {
+            for (int col = half; col < DV; col += 2) o16[((size_t)b * p.head_q + h_base + n) * DV + col] = 0;
+        }
+        return;
+    }
+
+    // Q rows of this wave's heads as B-operands: lane (n, half) holds Q[head n][ks*16 + half*8 .. +8)
+    const int hq = min(h_base + min(n, max(nh, 1) - 1), p.head_q - 1);
+    vec8 qf[KS];
+    {
+        const uint16_t* qrow = reinterpret_cast<const uint16_t*>(p.q) + ((size_t)b * p.head_q + hq) * D + half * 8;
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks) qf[ks] = __builtin_bit_cast(vec8, *reinterpret_cast<const uint4*>(qrow + ks * 16));
+    }
+    const float slope = p.is_alibi ? alibi_slope_log2(p.slopes, hq, p.head_q) : 0.0f;
+
+    f32x16 acc[CT];
+#pragma unroll
+    for (int c = 0; c < CT; ++c)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) acc[c][r] = 0.0f;
+    float m = kNegBig, l = 0.0f;
+
+    const uint8_t* const kbytes =
+        reinterpret_cast<const uint8_t*>(p.k) + ((size_t)start * p.k_row + (size_t)hk * D) * 2;
+    const size_t k_row_bytes = (size_t)p.k_row * 2;
+
+    // Stage the tile that starts at token tok0 into buffer `buf`.  Every wave always issues exactly
+    // NLW loads, so the hand-placed vmcnt waits below count the same on every wave; loads that fall
+    // outside the tile land in the spare KiB, rows past the end re-read the last valid row.
+    auto issue_tile = [&](int tok0, int buf) {
+#pragma unroll
+        for (int q = 0; q < NLW; ++q) {
+            const int i = wave + NWV * q;
+            const uint32_t dst = smem_off + ((i < NINSTR) ? (uint32_t)(buf * BUF + i * 1024) : (uint32_t)(kNBuf * BUF));
+            const int slot = min(i, NINSTR - 1) * 64 + lane;
+            int row = slot / SPR;
+            int ch = slot - row * SPR;
+            if (ch == SPR - 1) ch = 0;  // the pad slot: any valid bytes
+            row = min(row, kTile - 1);
+            const int tok = min(tok0 + row, c1 - 1);
+            lds_dma16(kbytes + (size_t)tok * k_row_bytes + ch * 16, dst);
+        }
+    };
+
+    const int ntiles = (c1 - c0 + kTile - 1) / kTile;
+    issue_tile(c0, 0);
+    if (ntiles > 1) issue_tile(c0 + kTile, 1);
+
+    // per-lane LDS byte offsets of the two read patterns (relative to the tile buffer)
+    const uint32_t k_rd = smem_off + n * PITCH + half * 16;
+    const uint32_t v_rd =
+        smem_off + (half * 4 + ((lane & 15) >> 2)) * PITCH + (((lane >> 4) & 1) * 16 + (lane & 3) * 4) * 2;
+    typedef __attribute__((address_space(3))) const uint4* lds_u4;
+    typedef __attribute__((address_space(3))) s16x4* lds_s4;
+    typedef short s16x8 __attribute__((__vector_size__(8 * sizeof(short))));
+
+    const float bias0 = slope * (float)(half * 4 - (len - 1));  // ALiBi: slope * (token - (len - 1)), split in lane and tile parts
+    int buf = 0;       // buffer that holds tile t
+    int buf_next = 2;  // buffer that receives tile t + 2
+    for (int t = 0; t < ntiles; ++t) {
+        if (t + 1 < ntiles)
+            wait_vmcnt<NLW>();  // tile t landed; tile t+1 may still be in flight
+        else
+            wait_vmcnt<0>();
+        __syncthreads();  // every wave's share of tile t is in LDS, and every wave is done with tile t-1
+        if (t + 2 < ntiles) issue_tile(c0 + (t + 2) * kTile, buf_next);
+
+        const int tok0 = c0 + t * kTile;
+        // tile base addresses, made opaque so that the constant offsets below stay in the instructions'
+        // offset fields instead of being folded into per-read address arithmetic
+        uint32_t kaddr = k_rd + buf * BUF;
+        uint32_t vaddr = v_rd + buf * BUF;
+        asm volatile("" : "+v"(kaddr), "+v"(vaddr));
+        buf = (buf == kNBuf - 1) ? 0 : buf + 1;
+        buf_next = (buf_next == kNBuf - 1) ? 0 : buf_next + 1;
+
+        // S^T = K_tile . Q^T : rows = tokens, columns = heads.  K fragments are read KPD steps ahead.
+        f32x16 s;
+        {
+            constexpr int KPD = 4;
+            vec8 kf[KPD];
+#pragma unroll
+            for (int i = 0; i < KPD; ++i) kf[i] = __builtin_bit_cast(vec8, *(lds_u4)(uintptr_t)(kaddr + i * 32));
+#pragma unroll
+            for (int ks = 0; ks < KS; ++ks) {
+                const vec8 a = kf[ks % KPD];
+                if (ks + KPD < KS) kf[ks % KPD] = __builtin_bit_cast(vec8, *(lds_u4)(uintptr_t)(kaddr + (ks + KPD) * 32));
+                if (ks == 0)
+                    MM::mma_v0(a, qf[ks], s);
+                else
+                    MM::mma_v(a, qf[ks], s);
+            }
+            // the compiler does not see the matrix instructions inside the assembly: cover the
+            // result latency of the last one before anything reads the scores (the scores pass
+            // through this statement, so no reader can be scheduled ahead of it)
+            asm volatile("s_nop 15\n\ts_nop 7" : "+v"(s));
+        }
+
+        // online softmax for head n over this lane's 16 tokens; token of register r: tok0 + (r/4)*8 + half*4 + r%4
+        float pv[16];
+        float mx = -INFINITY;
+        const bool tail = tok0 + kTile > c1;
+        if (p.is_alibi || tail) {
+            const float b0 = bias0 + slope * (float)tok0;
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                const int off = (r >> 2) * 8 + (r & 3);
+                const float x = s[r] * p.scale_log2 + (b0 + slope * (float)off);
+                pv[r] = (tok0 + half * 4 + off) < c1 ? x : -INFINITY;
+                mx = fmaxf(mx, pv[r]);
+            }
+        } else {
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                pv[r] = s[r] * p.scale_log2;
+                mx = fmaxf(mx, pv[r]);
+            }
+        }
+        mx = fmaxf(mx, __shfl_xor(mx, 32));
+        const bool up = mx > m + kLazy;
+        if (__any(up)) {
+            const float mn = up ? mx : m;
+            const float alpha = fast_exp2(m - mn);
+            m = mn;
+            l *= alpha;
+#pragma unroll
+            for (int c = 0; c < CT; ++c)
+#pragma unroll
+                for (int r = 0; r < 16; ++r) {
+                    float x = acc[c][r];
+                    scale_acc(x, alpha);
+                    acc[c][r] = x;
+                }
+        }
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+            pv[r] = fast_exp2(pv[r] - m);
+            l += pv[r];
+        }
+        vec8 pf[2];
+        pf[0] = MM::pack8(pv);
+        pf[1] = MM::pack8(pv + 8);
+
+        // O^T += V_tile^T . P^T : rows = value columns, columns = heads.  V fragments are read VPD steps ahead.
+        {
+            constexpr int VPD = 3;
+            constexpr int NV = CT * 2;  // (column tile, k-step) pairs, column tile major
+            s16x4 vlo[VPD], vhi[VPD];
+            auto rd = [&](int i, s16x4& lo, s16x4& hi) {
+                const int c = i >> 1, s2 = i & 1;
+                lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s4)(uintptr_t)(vaddr + c * 64 + (s2 * 16) * PITCH));
+                hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s4)(uintptr_t)(vaddr + c * 64 + (s2 * 16 + 8) * PITCH));
+            };
+#pragma unroll
+            for (int i = 0; i < VPD; ++i) rd(i, vlo[i], vhi[i]);
+#pragma unroll
+            for (int i = 0; i < NV; ++i) {
+                const s16x8 both = __builtin_shufflevector(vlo[i % VPD], vhi[i % VPD], 0, 1, 2, 3, 4, 5, 6, 7);
+                if (i + VPD < NV) rd(i + VPD, vlo[i % VPD], vhi[i % VPD]);
+                acc[i >> 1] = MM::mma(__builtin_bit_cast(vec8, both), pf[i & 1], acc[i >> 1]);
+            }
+        }
+    }
+
+    // finish: the two half-waves hold partial denominators over disjoint tokens
+    const float l_tot = l + __shfl_xor(l, 32);
+    if (n < nh) {
+        const int h = h_base + n;
+        if (p.nsplit == 1) {
+            const float inv = 1.0f / l_tot;
+            uint16_t* orow = o16 + ((size_t)b * p.head_q + h) * DV;
+#pragma unroll
+            for (int c = 0; c < CT; ++c)
+#pragma unroll
+                for (int r4 = 0; r4 < 4; ++r4) {
+                    const int col = c * 32 + r4 * 8 + half * 4;
+                    ushort4 w;
+                    w.x = EL::from_f32(acc[c][r4 * 4 + 0] * inv);
+                    w.y = EL::from_f32(acc[c][r4 * 4 + 1] * inv);
+                    w.z = EL::from_f32(acc[c][r4 * 4 + 2] * inv);
+                    w.w = EL::from_f32(acc[c][r4 * 4 + 3] * inv);
+                    *reinterpret_cast<ushort4*>(orow + col) = w;
+                }
+        } else {
+            const size_t part = ((size_t)b * p.head_q + h) * p.nsplit + split;
+            float* wrow = p.ws_o + part * DV;
+#pragma unroll
+            for (int c = 0; c < CT; ++c)
+#pragma unroll
+                for (int r4 = 0; r4 < 4; ++r4) {
+                    const int col = c * 32 + r4 * 8 + half * 4;
+                    float4 w = make_float4(acc[c][r4 * 4 + 0], acc[c][r4 * 4 + 1], acc[c][r4 * 4 + 2], acc[c][r4 * 4 + 3]);
+                    *reinterpret_cast<float4*>(wrow + col) = w;
+                }
+            if (half == 0) {
+                p.ws_ml[part * 2 + 0] = m;
+                p.ws_ml[part * 2 + 1] = l_tot;
+            }
+        }
+    }
+}
+
+template <int D>
+constexpr size_t lds_bytes() {
+    return (size_t)kNBuf * (((kTile * ((D * 2 + 16) / 16) + 63) / 64) * 1024) + 1024;
+}
+
+template <typename Tag, int D, int DV, int NWV>
+hipError_t launch_one(const SweepParams& p, dim3 grid, hipStream_t stream) {
+    static std::once_flag once;
+    static hipError_t attr_err = hipSuccess;
+    auto kern = mfma_latent_kernel<Tag, D, DV, NWV>;
+    std::call_once(once, [&] {
+        attr_err = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                       (int)lds_bytes<D>());
+    });
+    if (attr_err != hipSuccess) return attr_err;
+    hipLaunchKernelGGL(kern, grid, dim3(64 * NWV), lds_bytes<D>(), stream, p);
+    return hipGetLastError();
+}
+
+template <typename Tag>
+hipError_t launch_tag(const SweepParams& p, int rt, dim3 grid, hipStream_t stream) {
+    switch (rt) {
+        case 32: return launch_one<Tag, 576, 512, 1>(p, grid, stream);
+        case 64: return launch_one<Tag, 576, 512, 2>(p, grid, stream);
+        case 96: return launch_one<Tag, 576, 512, 3>(p, grid, stream);
+        case 128: return launch_one<Tag, 576, 512, 4>(p, grid, stream);
+        default: return hipErrorInvalidValue;
+    }
+}
+
+}  // namespace
+
+bool mla_supported(size_t dim, size_t dim_v, int ratio) { return dim == 576 && dim_v == 512 && ratio >= 1; }
+
+int mla_heads_per_group(int ratio) { return std::min(128, (ratio + 31) / 32 * 32); }
+
+int mla_rows_per_trip() { return kTile; }
+
+hipError_t launch_mla(const SweepParams& p, bool is_bf16, int rt, dim3 grid, hipStream_t stream) {
+    return is_bf16 ? launch_tag<bf16_tag>(p, rt, grid, stream) : launch_tag<f16_tag>(p, rt, grid, stream);
+}
+
 }  // namespace da

@@ -63,7 +63,9 @@ def test_plan_is_consistent(d, dv, batch, sk):
     assert p["nsplit"] * p["chunk"] >= sk
     assert (p["nsplit"] - 1) * p["chunk"] < max(sk, 1)
     ws = _lib.load().da_workspace_bytes(sk, batch, hq, hk, d, dv)
-    assert ws == (0 if p["nsplit"] == 1 else batch * hq * p["nsplit"] * (dv + 2) * 4)
+    need = 0 if p["nsplit"] == 1 else batch * hq * p["nsplit"] * (dv + 2) * 4
+    # (576, 512) also covers the plan used when V is passed as its own buffer
+    assert ws >= need if d == 576 else ws == need
 
 
 def test_plan_rejects_bad_shapes():
