@@ -153,8 +153,23 @@ def run_default(args):
     if not torch.cuda.is_available():
         print("bench.py needs a GPU (no CPU fallback exists for the op)", file=sys.stderr)
         return 2
+    if args.calibrate_copy:
+        # a device-to-device copy of known size, so that a profiler's FETCH_SIZE / WRITE_SIZE counters can be scaled
+        src = torch.empty(1 << 30, dtype=torch.uint8, device="cuda:0").fill_(1)
+        dst = torch.empty_like(src)
+        for _ in range(3):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        del src, dst
     gqa_w = wl.config_gqa_fixed(seed=0)
+    if args.only == "mla":
+        mla = measure(torch, wl.config_mla(64, 4096), args.steps, args.warmup)
+        print(json.dumps({"only": "mla", **mla}))
+        return 0
     gqa = measure(torch, gqa_w, args.steps, args.warmup)
+    if args.only == "gqa":
+        print(json.dumps({"only": "gqa", **gqa}))
+        return 0
     mla = None
     if not args.no_mla:
         mla = measure(torch, wl.config_mla(64, 4096), max(5, args.steps // 2), max(2, args.warmup // 2))
@@ -245,6 +260,10 @@ def main():
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU oracle timing")
     ap.add_argument("--no-mla", action="store_true", help="skip the MLA measurement")
+    ap.add_argument("--only", choices=["gqa", "mla"], help="measure one workload only and print its record "
+                    "(for profiler runs)")
+    ap.add_argument("--calibrate-copy", action="store_true", help="first run three 1 GiB device copies (a known "
+                    "traffic figure for scaling profiler byte counters)")
     ap.add_argument("--cpu-budget", type=float, default=15.0, help="seconds of single-thread CPU work to sample")
     ap.add_argument("--sweep", choices=["mha", "mla", "gqa", "all"], help="print the reference's sweeps instead")
     ap.add_argument("--json-out", help="with --sweep: also write the results as JSON")

@@ -20,6 +20,7 @@ SOURCES = [
     "da_sweep_d256.hip",
     "da_sweep_d576.hip",
     "da_mla.hip",
+    "da_gqa_mfma.hip",
 ]
 
 # packed-fp32 VALU forms are switched off on purpose: only scalar fp32 arithmetic is emitted.

@@ -15,6 +15,7 @@
 #include <utility>
 
 #include "../../include/decoding_attn_hip.h"
+#include "da_gqa_mfma.h"
 #include "da_mla.h"
 #include "da_sweep_launch.h"
 
@@ -41,13 +42,15 @@ int env_int(const char* name, int dflt) {
 // Tunables, read once.  DA_TARGET_WGS: work-groups a launch should reach before the sequence
 // stops being split further; DA_MAX_CHUNK / DA_MIN_CHUNK: bounds on tokens per split.
 struct Tunables {
-    int target_wgs, mfma_target_wgs, max_chunk, min_chunk, force_kind;
+    int target_wgs, mfma_target_wgs, max_chunk, min_chunk, force_kind, group_min_ratio, wave_per_head;
     Tunables() {
         target_wgs = env_int("DA_TARGET_WGS", 1024);
         mfma_target_wgs = env_int("DA_MFMA_TARGET_WGS", 256);
         max_chunk = env_int("DA_MAX_CHUNK", 1024);
         min_chunk = env_int("DA_MIN_CHUNK", 256);
         force_kind = env_int("DA_FORCE_KIND", 0);
+        wave_per_head = env_int("DA_WAVE_PER_HEAD", 1);
+        group_min_ratio = env_int("DA_GROUP_MIN_RATIO", 3);  // smallest head group that takes the grouped MFMA sweep
     }
 };
 const Tunables& tun() {
@@ -57,6 +60,7 @@ const Tunables& tun() {
 
 constexpr int kKindSweep = 1;
 constexpr int kKindMfma = 2;
+constexpr int kKindGroup = 3;
 constexpr int kMaxSplits = 256;
 
 struct Plan {
@@ -66,6 +70,7 @@ struct Plan {
     int nsplit = 1;
     int chunk = 0;
     size_t ws_bytes = 0;
+    bool wave_per_head = false;  // grouped kernel: the four waves of a work-group take four KV heads
 };
 
 bool supported_dims(size_t dim, size_t dim_v) {
@@ -96,6 +101,11 @@ Plan make_plan(size_t max_seq_k, size_t batch, size_t head_q, size_t head_k, siz
         pl.rt = da::mla_heads_per_group(ratio);
         trip = da::mla_rows_per_trip();
         target_wgs = tun().mfma_target_wgs;  // one 4-wave work-group fills a CU
+    } else if (dim <= 256 && ratio >= tun().group_min_ratio && tun().force_kind != kKindSweep) {
+        pl.kind = kKindGroup;
+        pl.rt = ratio > 16 ? 32 : 16;
+        pl.wave_per_head = head_k % 4 == 0 && tun().wave_per_head;
+        trip = pl.wave_per_head ? da::kGqaTile : 4 * da::kGqaTile;
     } else {
         pl.kind = kKindSweep;
         const int max_rt = dim > 256 ? 2 : 4;
@@ -104,7 +114,7 @@ Plan make_plan(size_t max_seq_k, size_t batch, size_t head_q, size_t head_k, siz
         trip = rows_per_trip(dim);
     }
     pl.groups = (ratio + pl.rt - 1) / pl.rt;
-    const long long base = (long long)batch * (long long)head_k * pl.groups;
+    const long long base = (long long)batch * (long long)(pl.wave_per_head ? head_k / 4 : head_k) * pl.groups;
     const int min_chunk = std::max(tun().min_chunk, trip);
     long long want = base > 0 ? (target_wgs + base - 1) / base : 1;
     const long long by_len = std::max<long long>(1, (long long)max_seq_k / min_chunk);
@@ -259,10 +269,13 @@ int da_decoding_attn_ex(const void* q, const void* k, const void* v, void* o, co
     sp.scale_log2 = scale * da::kLog2e;
     sp.is_alibi = is_alibi ? 1 : 0;
 
-    const dim3 grid((unsigned)pl.nsplit, (unsigned)(head_k * pl.groups), (unsigned)batch);
+    const dim3 grid((unsigned)pl.nsplit, (unsigned)((pl.wave_per_head ? head_k / 4 : head_k) * pl.groups),
+                    (unsigned)batch);
     hipError_t e;
     if (pl.kind == kKindMfma) {
         e = da::launch_mla(sp, is_bf16 != 0, pl.rt, grid, stream);
+    } else if (pl.kind == kKindGroup) {
+        e = da::launch_gqa_mfma(sp, is_bf16 != 0, (int)dim, pl.rt, pl.wave_per_head, grid, stream);
     } else {
         switch (dim) {
             case 64: e = da::launch_sweep_d64(sp, is_bf16 != 0, pl.rt, grid, stream); break;

@@ -104,6 +104,20 @@ struct ReduceParams {
     int head_q, dim_v, nsplit, chunk;
 };
 
+// An empty sequence still owns output rows: when the sequence is not split, its work-group stores zeros for
+// its heads (n_ranges runs of nheads consecutive heads, range_stride apart); otherwise the merge kernel does.
+template <int DV>
+__device__ __forceinline__ void zero_rows(const SweepParams& p, int b, int h_first, int nheads, int n_ranges,
+                                          int range_stride) {
+    uint16_t* const o16 = reinterpret_cast<uint16_t*>(p.o);
+    for (int it = threadIdx.x; it < n_ranges * nheads * DV; it += blockDim.x) {
+        const int col = it % DV;
+        const int hh = (it / DV) % nheads;
+        const int rg = it / (DV * nheads);
+        o16[((size_t)b * p.head_q + h_first + rg * range_stride + hh) * DV + col] = 0;
+    }
+}
+
 __device__ __forceinline__ float alibi_slope_log2(const float* slopes, int h, int head_q) {
     // closed form 2^(-8(h+1)/head_q); a slope array overrides it
     float s = slopes ? slopes[h] : fast_exp2(-8.0f * (float)(h + 1) / (float)head_q);

@@ -1,0 +1,381 @@
+// Single-query attention for a group of query heads that share one KV head (GQA / MQA), with
+// both contractions on the matrix cores so that the sweep stays bandwidth-bound for any group
+// size (wave64, gfx950).
+//
+// One work-group of four wavefronts serves one (sequence, KV head, group of up to 16*NT query
+// heads, sequence split).  Wavefronts do not share data while streaming: each takes every
+// fourth 32-token tile of the split and keeps its own online-softmax state; the four states
+// are merged through LDS at the end.  Per tile and wavefront:
+//
+//   K rows go from global memory straight into MFMA A-operand layout (16-byte loads: lane
+//   (n, g) takes bytes [(ks*4+g)*16, +16) of row n, so one instruction reads 64 contiguous
+//   bytes of 16 rows), and  S^T[16 tok x 16 heads] = K . Q^T  accumulates over D/32 k-steps
+//   of v_mfma_f32_16x16x32 with the Q rows held in registers as B-operands.
+//
+//   The score tile leaves the MFMA with one head per lane (column n) and 4 tokens per lane, so
+//   the online softmax is lane-local except for the maximum across the four 16-lane groups,
+//   and two score tiles (32 tokens) are exactly one B-operand of the second product.
+//
+//   V rows are loaded coalesced, parked in a wave-private LDS tile, and read back transposed
+//   (ds_read_b64_tr_b16: 8 tokens of one column per lane) as the A-operand of
+//   O^T[DV x 16 heads] += V^T . P^T.
+//
+// Mathematics as in the reference kernel (csrc/kernel/decoding_attn/decoding_fwd_kernel.h:50-235,
+// head mapping block_info.h:14-30); the reference streams K and V once per query head on CUDA
+// cores and keeps the whole score row in shared memory.
+#pragma once
+#include "da_common.h"
+
+namespace da {
+
+typedef short s16x4_t __attribute__((__vector_size__(4 * sizeof(short))));
+typedef short s16x8_t __attribute__((__vector_size__(8 * sizeof(short))));
+
+template <typename Tag>
+struct Mma16;
+template <>
+struct Mma16<f16_tag> {
+    typedef f16x8 vec8;
+    static __device__ __forceinline__ f32x4 mma(vec8 a, vec8 b, f32x4 c) {
+        return __builtin_amdgcn_mfma_f32_16x16x32_f16(a, b, c, 0, 0, 0);
+    }
+    static __device__ __forceinline__ vec8 pack8(const float* x) {
+        vec8 v;
+#pragma unroll
+        for (int j = 0; j < 8; ++j) v[j] = (_Float16)x[j];
+        return v;
+    }
+};
+template <>
+struct Mma16<bf16_tag> {
+    typedef bf16x8 vec8;
+    static __device__ __forceinline__ f32x4 mma(vec8 a, vec8 b, f32x4 c) {
+        return __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, c, 0, 0, 0);
+    }
+    static __device__ __forceinline__ vec8 pack8(const float* x) {
+        vec8 v;
+#pragma unroll
+        for (int j = 0; j < 8; ++j) v[j] = (__bf16)x[j];
+        return v;
+    }
+};
+
+constexpr int kGqaTile = 32;  // tokens per wave iteration
+
+template <int DV>
+constexpr int gqa_v_pitch() { return DV * 2 + 32; }  // LDS row pitch of the V tile: conflict-free transposed reads
+
+template <int DV>
+constexpr size_t gqa_lds_bytes(int nt) {
+    // V tiles of the four waves, reused for the final merge ([4][heads][DV] floats + (m, l))
+    const size_t vt = 4 * (size_t)kGqaTile * gqa_v_pitch<DV>();
+    const size_t mg = 4 * (size_t)(16 * nt) * (DV + 2) * sizeof(float);
+    return vt > mg ? vt : mg;
+}
+
+// WH (wave per head): the four wavefronts of a work-group take four consecutive KV heads over the same
+// tokens, so together they read whole [token][4 heads][D] rows (1 KiB contiguous for D = 128) at about the
+// same time, which HBM serves measurably faster than four streams of 256-byte pieces; no merge is needed.
+// Otherwise (head_k not a multiple of 4) the wavefronts split the tokens of one KV head and merge at the end.
+// MINW: wavefronts per SIMD the register allocation must leave room for (2 caps the kernel at 256 registers
+// and keeps the accumulators in ordinary VGPRs, so the rescale needs no accumulation-register copies).
+template <typename Tag, int D, int DV, int NT, bool PREFETCH, bool WH, int MINW>
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(MINW))) void gqa_mfma_kernel(const SweepParams p) {
+    using MM = Mma16<Tag>;
+    using vec8 = typename MM::vec8;
+    using EL = Elem<Tag>;
+    constexpr int KS = D / 32;      // k-steps of Q K^T
+    constexpr int CT = DV / 16;     // 16-column tiles of the output
+    constexpr int CPR = DV / 8;     // 16-byte chunks per V row
+    constexpr int NVI = kGqaTile * CPR / 64;  // V load instructions per tile
+    constexpr int VP = gqa_v_pitch<DV>();
+    constexpr int NW = WH ? 1 : 4;  // wavefronts that share the tokens of one KV head
+    constexpr int HG = 16 * NT;     // query heads per KV head and work-group
+    constexpr float kLazy = 8.0f;   // the running maximum moves only when exceeded by this much (log2 units)
+    static_assert(D % 32 == 0 && DV % 16 == 0 && (kGqaTile * CPR) % 64 == 0, "shape");
+
+    extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
+
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int n = lane & 15;
+    const int g = lane >> 4;
+
+    const int split = blockIdx.x;
+    const int hk = WH ? (blockIdx.y / p.groups) * 4 + wave : blockIdx.y / p.groups;
+    const int grp = blockIdx.y % p.groups;
+    const int b = blockIdx.z;
+    const int tw = WH ? 0 : wave;  // this wave's position among the waves that share the tokens
+
+    const int start = p.cu_seq_k[b];
+    const int len = p.cu_seq_k[b + 1] - start;
+    const int c0 = split * p.chunk;
+    const int c1 = (split == p.nsplit - 1) ? len : min(len, c0 + p.chunk);
+
+    const int h_base = hk * p.ratio + grp * HG;
+    const int nh = min(HG, p.ratio - grp * HG);  // live heads of this group
+    uint16_t* const o16 = reinterpret_cast<uint16_t*>(p.o);
+
+    if (c0 >= c1) {
+        // every wave of the work-group sees the same (sequence, split), so they all leave together; the
+        // work-group covers NR runs of nh heads, one per KV head
+        constexpr int NR = WH ? 4 : 1;
+        const int wg_h_first = (WH ? (blockIdx.y / p.groups) * 4 : hk) * p.ratio + grp * HG;
+        if (p.nsplit == 1) zero_rows<DV>(p, b, wg_h_first, nh, NR, p.ratio);
+        return;
+    }
+
+    // Q rows as B-operands: lane (n, g) holds Q[head nt*16+n][(ks*4+g)*8 .. +8)
+    vec8 qf[NT][KS];
+    float slope[NT];
+#pragma unroll
+    for (int nt = 0; nt < NT; ++nt) {
+        const int h = h_base + min(nt * 16 + n, nh - 1);
+        const uint16_t* qrow = reinterpret_cast<const uint16_t*>(p.q) + ((size_t)b * p.head_q + h) * D + g * 8;
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks) qf[nt][ks] = __builtin_bit_cast(vec8, *reinterpret_cast<const uint4*>(qrow + ks * 32));
+        slope[nt] = p.is_alibi ? alibi_slope_log2(p.slopes, h, p.head_q) : 0.0f;
+    }
+
+    f32x4 acc[NT][CT];
+    float m[NT], l[NT];
+#pragma unroll
+    for (int nt = 0; nt < NT; ++nt) {
+        m[nt] = kNegBig;
+        l[nt] = 0.0f;
+#pragma unroll
+        for (int ct = 0; ct < CT; ++ct) acc[nt][ct] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+    }
+
+    // wave-uniform byte bases (scalar registers) and 32-bit per-lane byte offsets
+    const uint8_t* const kbytes =
+        reinterpret_cast<const uint8_t*>(p.k) + ((size_t)start * p.k_row + (size_t)hk * D) * 2;
+    const uint8_t* const vbytes =
+        reinterpret_cast<const uint8_t*>(p.v) + ((size_t)start * p.v_row + (size_t)hk * p.v_head) * 2;
+    const uint32_t k_row_b = (uint32_t)p.k_row * 2, v_row_b = (uint32_t)p.v_row * 2;
+
+    // wave-private V tile in LDS
+    uint8_t* const vt = smem + wave * (kGqaTile * VP);
+    // transposed-read address of this lane: 16-lane group g reads rows g*4 .. g*4+3 (and +16), 16 columns
+    const uint8_t* const v_rd = vt + (g * 4 + (n >> 2)) * VP + (n & 3) * 8;
+    typedef __attribute__((address_space(3))) s16x4_t* lds_s4;
+
+    // One tile in registers: K in A-operand layout [16-token tile][k-step], V row-major chunks.  There is a
+    // single register set: the loads of the next tile are issued as soon as this tile's registers are free
+    // (V once it is parked in LDS, K once the score MFMAs have read it), so they fly during the rest of the
+    // tile's work without doubling the register footprint.
+    struct TileRegs {
+        uint4 k[2][KS];
+        uint4 v[NVI];
+    };
+    TileRegs tr;
+
+    auto load_k = [&](int tok0, TileRegs& r) __attribute__((always_inline)) {
+        const uint8_t* const base = kbytes + (size_t)tok0 * k_row_b;
+        const int last = c1 - 1 - tok0;  // rows past the end re-read the last row and are masked
+#pragma unroll
+        for (int mt = 0; mt < 2; ++mt) {
+            const uint32_t off = (uint32_t)min(mt * 16 + n, last) * k_row_b + g * 16;
+#pragma unroll
+            for (int ks = 0; ks < KS; ++ks) r.k[mt][ks] = *reinterpret_cast<const uint4*>(base + off + ks * 64);
+        }
+    };
+    auto load_v = [&](int tok0, TileRegs& r) __attribute__((always_inline)) {
+        const uint8_t* const base = vbytes + (size_t)tok0 * v_row_b;
+        const int last = c1 - 1 - tok0;
+#pragma unroll
+        for (int i = 0; i < NVI; ++i) {
+            const int slot = i * 64 + lane;
+            const int row = slot / CPR, ch = slot % CPR;
+            const uint32_t off = (uint32_t)min(row, last) * v_row_b + ch * 16;
+            r.v[i] = *reinterpret_cast<const uint4*>(base + off);
+        }
+    };
+
+    const int ntiles = (c1 - c0 + kGqaTile - 1) / kGqaTile;
+    if (tw < ntiles) {
+        load_v(c0 + tw * kGqaTile, tr);
+        load_k(c0 + tw * kGqaTile, tr);
+    }
+
+    for (int t = tw; t < ntiles; t += NW) {
+        const int tok0 = c0 + t * kGqaTile;
+        const bool more = t + NW < ntiles;
+        const int tok_next = tok0 + NW * kGqaTile;
+
+        // park V in LDS (row-major, padded pitch), then refill the V registers
+#pragma unroll
+        for (int i = 0; i < NVI; ++i) {
+            const int slot = i * 64 + lane;
+            const int row = slot / CPR, ch = slot % CPR;
+            *reinterpret_cast<uint4*>(vt + row * VP + ch * 16) = tr.v[i];
+        }
+        if (PREFETCH && more) load_v(tok_next, tr);
+
+        // S^T = K . Q^T for the two 16-token tiles, then refill the K registers
+        f32x4 s[2][NT];
+#pragma unroll
+        for (int mt = 0; mt < 2; ++mt)
+#pragma unroll
+            for (int nt = 0; nt < NT; ++nt) {
+                f32x4 c = {0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+                for (int ks = 0; ks < KS; ++ks) c = MM::mma(__builtin_bit_cast(vec8, tr.k[mt][ks]), qf[nt][ks], c);
+                s[mt][nt] = c;
+            }
+        if (PREFETCH && more) load_k(tok_next, tr);
+
+        // online softmax; token of s[mt][nt][r]: tok0 + mt*16 + g*4 + r, head nt*16 + n
+        vec8 pf[NT];
+        const bool tail = tok0 + kGqaTile > c1;
+#pragma unroll
+        for (int nt = 0; nt < NT; ++nt) {
+            float x[8];
+            float mx = -INFINITY;
+            if (p.is_alibi || tail) {
+#pragma unroll
+                for (int mt = 0; mt < 2; ++mt)
+#pragma unroll
+                    for (int r = 0; r < 4; ++r) {
+                        const int tok = tok0 + mt * 16 + g * 4 + r;
+                        float v = s[mt][nt][r] * p.scale_log2 + slope[nt] * (float)(tok - (len - 1));
+                        if (tok >= c1) v = -INFINITY;
+                        x[mt * 4 + r] = v;
+                        mx = fmaxf(mx, v);
+                    }
+            } else {
+#pragma unroll
+                for (int mt = 0; mt < 2; ++mt)
+#pragma unroll
+                    for (int r = 0; r < 4; ++r) {
+                        x[mt * 4 + r] = s[mt][nt][r] * p.scale_log2;
+                        mx = fmaxf(mx, x[mt * 4 + r]);
+                    }
+            }
+            mx = fmaxf(mx, __shfl_xor(mx, 16));
+            mx = fmaxf(mx, __shfl_xor(mx, 32));
+            const bool up = mx > m[nt] + kLazy;
+            if (__any(up)) {
+                const float mn = up ? mx : m[nt];
+                const float alpha = fast_exp2(m[nt] - mn);
+                m[nt] = mn;
+                l[nt] *= alpha;
+#pragma unroll
+                for (int ct = 0; ct < CT; ++ct) acc[nt][ct] *= alpha;
+            }
+#pragma unroll
+            for (int j = 0; j < 8; ++j) {
+                x[j] = fast_exp2(x[j] - m[nt]);
+                l[nt] += x[j];
+            }
+            pf[nt] = MM::pack8(x);  // k index j <-> token g*4+j (j<4), 16+g*4+(j-4) (j>=4)
+        }
+
+        // O^T += V^T . P^T
+#pragma unroll
+        for (int ct = 0; ct < CT; ++ct) {
+            const s16x4_t lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s4)(v_rd + ct * 32));
+            const s16x4_t hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s4)(v_rd + ct * 32 + 16 * VP));
+            const s16x8_t both = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+            const vec8 a = __builtin_bit_cast(vec8, both);
+#pragma unroll
+            for (int nt = 0; nt < NT; ++nt) acc[nt][ct] = MM::mma(a, pf[nt], acc[nt][ct]);
+        }
+
+        if (!PREFETCH && more) {
+            load_v(tok_next, tr);
+            load_k(tok_next, tr);
+        }
+    }
+
+    // denominators: each 16-lane group summed its own tokens
+#pragma unroll
+    for (int nt = 0; nt < NT; ++nt) {
+        l[nt] += __shfl_xor(l[nt], 16);
+        l[nt] += __shfl_xor(l[nt], 32);
+    }
+
+    if constexpr (WH) {
+        // every wave owns its heads outright: finish from registers.  acc[nt][ct][r] is head nt*16+n,
+        // column ct*16 + g*4 + r.
+#pragma unroll
+        for (int nt = 0; nt < NT; ++nt) {
+            const int hh = nt * 16 + n;
+            if (hh < nh) {
+                const int h = h_base + hh;
+                if (p.nsplit == 1) {
+                    const float inv = 1.0f / l[nt];
+                    uint16_t* orow = o16 + ((size_t)b * p.head_q + h) * DV + g * 4;
+#pragma unroll
+                    for (int ct = 0; ct < CT; ++ct) {
+                        ushort4 w;
+                        w.x = EL::from_f32(acc[nt][ct][0] * inv);
+                        w.y = EL::from_f32(acc[nt][ct][1] * inv);
+                        w.z = EL::from_f32(acc[nt][ct][2] * inv);
+                        w.w = EL::from_f32(acc[nt][ct][3] * inv);
+                        *reinterpret_cast<ushort4*>(orow + ct * 16) = w;
+                    }
+                } else {
+                    const size_t part = ((size_t)b * p.head_q + h) * p.nsplit + split;
+                    float* wrow = p.ws_o + part * DV + g * 4;
+#pragma unroll
+                    for (int ct = 0; ct < CT; ++ct) *reinterpret_cast<f32x4*>(wrow + ct * 16) = acc[nt][ct];
+                    if (g == 0) {
+                        p.ws_ml[part * 2 + 0] = m[nt];
+                        p.ws_ml[part * 2 + 1] = l[nt];
+                    }
+                }
+            }
+        }
+        return;
+    }
+
+    // merge the four waves through LDS (the V tiles are dead by now)
+    constexpr int MW = 4;
+    __syncthreads();
+    float* const lds_acc = reinterpret_cast<float*>(smem);                 // [MW][HG][DV]
+    float* const lds_ml = lds_acc + MW * HG * DV;                          // [MW][HG][2]
+#pragma unroll
+    for (int nt = 0; nt < NT; ++nt) {
+        const int hh = nt * 16 + n;
+#pragma unroll
+        for (int ct = 0; ct < CT; ++ct)
+            *reinterpret_cast<f32x4*>(lds_acc + ((size_t)wave * HG + hh) * DV + ct * 16 + g * 4) = acc[nt][ct];
+        if (g == 0) {
+            lds_ml[(wave * HG + hh) * 2 + 0] = m[nt];
+            lds_ml[(wave * HG + hh) * 2 + 1] = l[nt];
+        }
+    }
+    __syncthreads();
+
+    for (int idx = threadIdx.x; idx < nh * DV; idx += blockDim.x) {
+        const int r = idx / DV, col = idx % DV;
+        float mm = lds_ml[(0 * HG + r) * 2];
+#pragma unroll
+        for (int w = 1; w < MW; ++w) mm = fmaxf(mm, lds_ml[(w * HG + r) * 2]);
+        float num = 0.0f, den = 0.0f;
+#pragma unroll
+        for (int w = 0; w < MW; ++w) {
+            const float wt = fast_exp2(lds_ml[(w * HG + r) * 2] - mm);
+            num += wt * lds_acc[((size_t)w * HG + r) * DV + col];
+            den += wt * lds_ml[(w * HG + r) * 2 + 1];
+        }
+        const int h = h_base + r;
+        if (p.nsplit == 1) {
+            o16[((size_t)b * p.head_q + h) * DV + col] = EL::from_f32(num / den);
+        } else {
+            const size_t part = ((size_t)b * p.head_q + h) * p.nsplit + split;
+            p.ws_o[part * DV + col] = num;
+            if (col == 0) {
+                p.ws_ml[part * 2 + 0] = mm;
+                p.ws_ml[part * 2 + 1] = den;
+            }
+        }
+    }
+}
+
+// wave_per_head selects the WH form; the grid's y extent must then count groups of four KV heads.
+hipError_t launch_gqa_mfma(const SweepParams& p, bool is_bf16, int dim, int heads_per_group, bool wave_per_head,
+                           dim3 grid, hipStream_t stream);
+
+}  // namespace da

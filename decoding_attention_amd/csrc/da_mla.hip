@@ -139,9 +139,7 @@ __global__ __launch_bounds__(64 * NWV) void mfma_latent_kernel(const SweepParams
     uint16_t* const o16 = reinterpret_cast<uint16_t*>(p.o);
 
     if (c0 >= c1) {
-        if (p.nsplit == 1 && n < nh) {
-            for (int col = half; col < DV; col += 2) o16[((size_t)b * p.head_q + h_base + n) * DV + col] = 0;
-        }
+        if (p.nsplit == 1) zero_rows<DV>(p, b, hk * p.ratio + grp * 32 * NWV, wg_heads, 1, 0);
         return;
     }
 

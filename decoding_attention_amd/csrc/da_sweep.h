@@ -57,15 +57,9 @@ __global__ __launch_bounds__(256) void sweep_kernel(const SweepParams p) {
     const int nh = min(RT, p.ratio - grp * RT);  // live heads of this group
 
     if (c0 >= c1) {
-        // Nothing to read.  An empty sequence still owns an output row: store zeros when this
-        // work-group is the one that would have finished it.
-        if (p.nsplit == 1) {
-            uint16_t* o = reinterpret_cast<uint16_t*>(p.o);
-            for (int idx = threadIdx.x; idx < nh * DV; idx += blockDim.x) {
-                const int r = idx / DV, col = idx % DV;
-                o[((size_t)b * p.head_q + h_base + r) * DV + col] = 0;
-            }
-        }
+        // Nothing to read.  An empty sequence still owns output rows (the merge kernel writes them
+        // when the sequence is split).
+        if (p.nsplit == 1) zero_rows<DV>(p, b, h_base, nh, 1, 0);
         return;
     }
 

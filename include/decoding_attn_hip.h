@@ -66,7 +66,7 @@ size_t da_workspace_bytes(size_t max_seq_k, size_t batch, size_t head_q, size_t 
 
 /*
  * Launch plan the library would use for this shape, for tests and benchmarks:
- *   kernel_kind 1 = VALU sweep, 2 = MFMA sweep (grouped heads / latent); nsplit = sequence splits;
+ *   kernel_kind 1 = VALU sweep, 2 = latent (MLA) MFMA sweep, 3 = grouped-head MFMA sweep; nsplit = sequence splits;
  *   chunk = tokens per split; heads_per_group = query heads one work-group serves.
  * Any output pointer may be NULL.  Returns DA_ERR_UNSUPPORTED for an unsupported (dim, dim_v).
  * Mirrors the role of the reference's per-head-dim tile choice (csrc/kernel/decoding_attn/decoding_fwd_hd*.cu).
