@@ -113,3 +113,12 @@ def test_workloads_are_reproducible():
     assert 1 <= min(a.lengths) and max(a.lengths) <= 64 and a.max_seq_k == max(a.lengths)
     m = wl.config_mla(2, 16)
     assert m.v is None and m.q.shape == (2, 128, 576) and m.dim_v == 512
+
+
+def test_torch_extension_module_exports_fwd():
+    """The PyTorch-ROCm extension (the counterpart of the reference's `decoding_attn_cuda`) loads and exposes `fwd`
+    with the reference's argument names (reference csrc/torch/decoding_torch.cpp:82-85)."""
+    ext = interface._extension()
+    doc = ext.fwd.__doc__
+    for name in ("q", "k", "v_", "o_", "cu_seq_k", "max_seq_k", "dim_v", "is_alibi"):
+        assert name + ":" in doc
