@@ -29,6 +29,9 @@ if ROOT not in sys.path:
 
 HBM_PEAK_GBPS = 8000.0      # MI355X HBM3E, published
 MFMA_PEAK_TFLOPS = 2500.0   # MI355X dense fp16/bf16 MFMA, published
+# HBM bytes per call from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of `bench.py --only gqa|mla`, each counter
+# scaled by what it reads for a 1 GiB device copy (profiles/*_hbm_traffic.md); valid for the default launch plan.
+MEASURED_TRAFFIC_BYTES = {"gqa": 1098235904, "mla": None}
 
 
 def _time_calls(torch, fn_list, steps, warmup):
@@ -195,8 +198,8 @@ def run_default(args):
         "us_per_call_min": gqa["us_per_call_min"],
         "pct_hbm_peak": 100.0 * gqa["hbm_frac_of_peak"],
         "roofline": {"bound": "hbm", "achieved": gqa["hbm_GBps"], "peak": HBM_PEAK_GBPS, "unit": "GB/s",
-                     "frac": gqa["hbm_frac_of_peak"], "traffic": None,
-                     "kernel": "sweep kernel + split merge of one call (whole-call time)"},
+                     "frac": gqa["hbm_frac_of_peak"], "traffic": MEASURED_TRAFFIC_BYTES["gqa"],
+                     "kernel": "gqa_mfma_kernel + reduce_kernel of one call (whole-call time)"},
         "cpu_baseline": cpu,
     }
     if mla is not None:
@@ -209,7 +212,7 @@ def run_default(args):
             "algorithmic_bytes": mla["algorithmic_bytes"], "algorithmic_flops": mla["algorithmic_flops"],
             "input_copies_rotated": mla["input_copies_rotated"], "plan": mla["plan"],
             "roofline": {"bound": "hbm", "achieved": mla["hbm_GBps"], "peak": HBM_PEAK_GBPS, "unit": "GB/s",
-                         "frac": mla["hbm_frac_of_peak"], "traffic": None},
+                         "frac": mla["hbm_frac_of_peak"], "traffic": MEASURED_TRAFFIC_BYTES["mla"]},
             "roofline_mfma": {"bound": "mfma", "achieved": mla["tflops"], "peak": MFMA_PEAK_TFLOPS,
                               "unit": "TFLOP/s", "frac": mla["mfma_frac_of_peak"]},
         }
