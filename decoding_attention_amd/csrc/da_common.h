@@ -3,6 +3,8 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include <type_traits>
+
 namespace da {
 
 constexpr int kWave = 64;          // CDNA4 wavefront width
@@ -56,6 +58,16 @@ struct Elem<bf16_tag> {
 };
 
 __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
+
+// f(integral_constant<int, B>), ..., f(integral_constant<int, E-1>): a loop whose index is a constant
+// expression in the body (needed for instruction offset fields and wait counts in inline assembly).
+template <int B, int E, typename F>
+__device__ __forceinline__ void static_for(F&& f) {
+    if constexpr (B < E) {
+        f(std::integral_constant<int, B>{});
+        static_for<B + 1, E>(f);
+    }
+}
 
 // Butterfly sum over groups of G adjacent lanes (G a power of two <= 16) with DPP lane
 // permutes; every lane of the group ends with the group's total.

@@ -17,7 +17,14 @@
 // half-waves, and the probabilities feed the second MFMA as its B-operand without any lane
 // movement (the token <-> k-index permutation is applied to V's rows instead).
 //
-// LDS rows are padded by 16 bytes (pitch 1168) which makes both read patterns conflict-free.
+// LDS tile layout.  A tile buffer has two regions: the 512 value columns of the 32 rows (1 KiB per row) and
+// the remaining 64 key columns (128 B per row).  One direct-to-LDS load instruction fills exactly one row of
+// the first region (or eight rows of the second), so its source is a wave-uniform row address plus a per-lane
+// chunk offset.  Inside a row the 16-byte chunks are XOR-swizzled with the row index --
+//   first region:  chunk c of row r at c ^ ((r & 3) << 2 | (r >> 2) & 3)
+//   second region: chunk c of row r at c ^ ((r >> 1) & 7)
+// -- which makes both read patterns (16 rows x one chunk for K, 4 rows x 64 bytes for V^T) conflict-free, and
+// because XOR commutes with the per-step chunk offsets every read address is one per-lane base XOR a constant.
 //
 // Mathematics as in the reference kernel (csrc/kernel/decoding_attn/decoding_fwd_kernel.h:50-235
 // with the latent aliasing of csrc/ops/decoding_attn.cpp:30-37); the structure is unrelated.
@@ -32,6 +39,8 @@ namespace {
 constexpr int kTile = 32;  // tokens per LDS tile
 constexpr int kNBuf = 3;   // LDS tile buffers (two tiles in flight behind the one being read)
 constexpr float kLazy = 8.0f;  // the running maximum moves only when exceeded by this much (log2 units)
+constexpr int kKPD = 8;  // K fragments read from LDS ahead of the MFMA that uses them
+constexpr int kVPD = 6;  // V^T fragment pairs read ahead
 
 typedef short s16x4 __attribute__((__vector_size__(4 * sizeof(short))));
 
@@ -46,10 +55,10 @@ struct Mma<f16_tag> {
     // same product with the accumulator pinned to ordinary VGPRs (the score tile: the accumulation
     // registers are all taken by the output tiles)
     static __device__ __forceinline__ void mma_v(vec8 a, vec8 b, f32x16& c) {
-        asm("v_mfma_f32_32x32x16_f16 %0, %1, %2, %0" : "+v"(c) : "v"(a), "v"(b));
+        asm volatile("v_mfma_f32_32x32x16_f16 %0, %1, %2, %0" : "+v"(c) : "v"(a), "v"(b));
     }
     static __device__ __forceinline__ void mma_v0(vec8 a, vec8 b, f32x16& c) {  // c = a.b
-        asm("v_mfma_f32_32x32x16_f16 %0, %1, %2, 0" : "=v"(c) : "v"(a), "v"(b));
+        asm volatile("v_mfma_f32_32x32x16_f16 %0, %1, %2, 0" : "=v"(c) : "v"(a), "v"(b));
     }
     static __device__ __forceinline__ vec8 pack8(const float* x) {
         vec8 v;
@@ -65,10 +74,10 @@ struct Mma<bf16_tag> {
         return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0);
     }
     static __device__ __forceinline__ void mma_v(vec8 a, vec8 b, f32x16& c) {
-        asm("v_mfma_f32_32x32x16_bf16 %0, %1, %2, %0" : "+v"(c) : "v"(a), "v"(b));
+        asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, %0" : "+v"(c) : "v"(a), "v"(b));
     }
     static __device__ __forceinline__ void mma_v0(vec8 a, vec8 b, f32x16& c) {
-        asm("v_mfma_f32_32x32x16_bf16 %0, %1, %2, 0" : "=v"(c) : "v"(a), "v"(b));
+        asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, 0" : "=v"(c) : "v"(a), "v"(b));
     }
     static __device__ __forceinline__ vec8 pack8(const float* x) {
         vec8 v;
@@ -81,9 +90,15 @@ struct Mma<bf16_tag> {
 // 16 bytes per lane from global memory straight into LDS at lds_off + lane * 16 (lds_off is
 // wave-uniform).  Issued from assembly so that the wait for it is placed by hand: the
 // compiler would otherwise drain every outstanding load before the next LDS read.
-__device__ __forceinline__ void lds_dma16(const void* gptr, uint32_t lds_off) {
+// The source address is a wave-uniform 64-bit base plus a 32-bit per-lane byte offset.
+__device__ __forceinline__ void lds_dma16(const void* gbase, uint32_t lane_off, uint32_t lds_off) {
     const uint32_t off = __builtin_amdgcn_readfirstlane(lds_off);
-    asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off" ::"v"(gptr), "s"(off) : "memory");
+    const uintptr_t b = reinterpret_cast<uintptr_t>(gbase);
+    // readfirstlane returns a signed int: go through uint32_t so that the low word is not sign-extended
+    const uint64_t base = (uint64_t)(uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)b) |
+                          ((uint64_t)(uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)(b >> 32)) << 32);
+    asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1" ::"v"(lane_off), "s"(base), "s"(off)
+                 : "memory");
 }
 
 // x *= alpha for an MFMA accumulator element that lives in an accumulation register.  Written as
@@ -96,6 +111,32 @@ __device__ __forceinline__ void scale_acc(float& x, float alpha) {
                  : "v"(alpha));
 }
 
+// LDS reads issued from assembly, in program order and with hand-placed waits.  Left to itself the compiler
+// sinks these reads next to their use to save registers (the kernel sits at the register limit), which leaves
+// one or two reads in flight; a single wavefront per SIMD then stalls on LDS latency before every MFMA.
+template <int OFF, typename V>
+__device__ __forceinline__ void lds_read_b128(V& dst, uint32_t addr) {
+    asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(dst) : "v"(addr), "n"(OFF));
+}
+template <int OFF>
+__device__ __forceinline__ void lds_read_tr16_b64(s16x4& dst, uint32_t addr) {
+    asm volatile("ds_read_b64_tr_b16 %0, %1 offset:%2" : "=v"(dst) : "v"(addr), "n"(OFF));
+}
+// Wait until at most N LDS reads are outstanding; the operands pass through so that no consumer of them can
+// be scheduled ahead of the wait.
+template <int N, typename V>
+__device__ __forceinline__ void wait_lgkm(V& x) {
+    asm volatile("s_waitcnt lgkmcnt(%1)" : "+v"(x) : "n"(N));
+}
+template <int N, typename V>
+__device__ __forceinline__ void wait_lgkm(V& x, V& y) {
+    asm volatile("s_waitcnt lgkmcnt(%2)" : "+v"(x), "+v"(y) : "n"(N));
+}
+
+// Chunk swizzles of the two tile regions (see the header comment).
+__device__ __forceinline__ int swz_a(int r) { return ((r & 3) << 2) | ((r >> 2) & 3); }
+__device__ __forceinline__ int swz_b(int r) { return (r >> 1) & 7; }
+
 template <int N>
 __device__ __forceinline__ void wait_vmcnt() {
     asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory");
@@ -106,16 +147,19 @@ __global__ __launch_bounds__(64 * NWV) void mfma_latent_kernel(const SweepParams
     using MM = Mma<Tag>;
     using vec8 = typename MM::vec8;
     using EL = Elem<Tag>;
-    constexpr int PITCH = D * 2 + 16;                    // bytes per LDS row
-    constexpr int SPR = PITCH / 16;                      // 16-byte slots per row
-    constexpr int NINSTR = (kTile * SPR + 63) / 64;      // load instructions per tile (whole work-group)
-    constexpr int BUF = NINSTR * 1024;                   // bytes per tile buffer
-    constexpr int NLW = (NINSTR + NWV - 1) / NWV;        // load instructions per tile per wave
+    static_assert(D == 576 && DV == 512 && (NWV == 1 || NWV == 2 || NWV == 4), "tile layout is specific to (576, 512)");
+    constexpr int ROW_A = DV * 2;                        // bytes per row, region A (value columns)
+    constexpr int ROW_B = (D - DV) * 2;                  // bytes per row, region B (remaining key columns)
+    constexpr int OFF_B = kTile * ROW_A;                 // region B starts here
+    constexpr int BUF = kTile * D * 2;                   // bytes per tile buffer
+    constexpr int NLA = kTile / NWV;                     // region-A load instructions per tile per wave (one row each)
+    constexpr int NLB = (kTile / 8) / NWV;               // region-B load instructions per tile per wave (eight rows each)
+    constexpr int NLW = NLA + NLB;                       // load instructions per tile per wave
     constexpr int KS = D / 16;                           // k-steps of Q K^T
     constexpr int CT = DV / 32;                          // 32-column tiles of the output
     static_assert(D % 16 == 0 && DV % 32 == 0 && DV <= D, "shape");
 
-    extern __shared__ __attribute__((aligned(1024))) uint8_t smem[];  // kNBuf * BUF, then 1 KiB that absorbs surplus loads
+    extern __shared__ __attribute__((aligned(1024))) uint8_t smem[];  // kNBuf * BUF
     const uint32_t smem_off = (uint32_t)(uintptr_t)smem;
 
     const int lane = threadIdx.x & 63;
@@ -164,32 +208,49 @@ __global__ __launch_bounds__(64 * NWV) void mfma_latent_kernel(const SweepParams
         reinterpret_cast<const uint8_t*>(p.k) + ((size_t)start * p.k_row + (size_t)hk * D) * 2;
     const size_t k_row_bytes = (size_t)p.k_row * 2;
 
-    // Stage the tile that starts at token tok0 into buffer `buf`.  Every wave always issues exactly
-    // NLW loads, so the hand-placed vmcnt waits below count the same on every wave; loads that fall
-    // outside the tile land in the spare KiB, rows past the end re-read the last valid row.
+    // Stage the tile that starts at token tok0 into buffer `buf`.  Rows past the end of the split re-read the
+    // last valid row (they are masked later).  Every wave always issues exactly NLW loads, so the hand-placed
+    // vmcnt waits count the same on every wave.
+    const uint32_t lane16 = lane * 16;
+    const int rb = lane >> 3;  // region B: row within the group of eight, chunk lane & 7
     auto issue_tile = [&](int tok0, int buf) {
+        const uint8_t* const base = kbytes + (size_t)tok0 * k_row_bytes;
+        const int last = c1 - 1 - tok0;
 #pragma unroll
-        for (int q = 0; q < NLW; ++q) {
-            const int i = wave + NWV * q;
-            const uint32_t dst = smem_off + ((i < NINSTR) ? (uint32_t)(buf * BUF + i * 1024) : (uint32_t)(kNBuf * BUF));
-            const int slot = min(i, NINSTR - 1) * 64 + lane;
-            int row = slot / SPR;
-            int ch = slot - row * SPR;
-            if (ch == SPR - 1) ch = 0;  // the pad slot: any valid bytes
-            row = min(row, kTile - 1);
-            const int tok = min(tok0 + row, c1 - 1);
-            lds_dma16(kbytes + (size_t)tok * k_row_bytes + ch * 16, dst);
+        for (int q = 0; q < NLA; ++q) {
+            const int row = wave + NWV * q;  // wave-uniform
+            lds_dma16(base, (uint32_t)min(row, last) * (uint32_t)k_row_bytes + (lane16 ^ (uint32_t)(swz_a(row) * 16)),
+                      smem_off + (uint32_t)(buf * BUF + row * ROW_A));
+        }
+#pragma unroll
+        for (int q = 0; q < NLB; ++q) {
+            const int j = wave + NWV * q;
+            const int row = j * 8 + rb;
+            lds_dma16(base, (uint32_t)min(row, last) * (uint32_t)k_row_bytes +
+                                (uint32_t)(DV * 2 + (((lane & 7) ^ swz_b(row)) * 16)),
+                      smem_off + (uint32_t)(buf * BUF + OFF_B + j * 1024));
         }
     };
 
     const int ntiles = (c1 - c0 + kTile - 1) / kTile;
     issue_tile(c0, 0);
     if (ntiles > 1) issue_tile(c0 + kTile, 1);
+    // Make the compiler settle its own wait for the Q loads here, before the loop.  It cannot see the
+    // direct-to-LDS loads, so a wait for Q placed inside the loop would count down to vmcnt(0) on every trip
+    // and drain the tiles in flight.
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) asm volatile("" : "+v"(qf[ks]));
 
-    // per-lane LDS byte offsets of the two read patterns (relative to the tile buffer)
-    const uint32_t k_rd = smem_off + n * PITCH + half * 16;
-    const uint32_t v_rd =
-        smem_off + (half * 4 + ((lane & 15) >> 2)) * PITCH + (((lane >> 4) & 1) * 16 + (lane & 3) * 4) * 2;
+    // Per-lane LDS read bases (buffer 0); per-step chunk offsets are XORed in, the rest is instruction offset.
+    // K rows: lane (n, half) reads chunk 2 ks + half of row n.
+    //   ks < 32: (base_a ^ 32 (ks & 7)) + 256 (ks >> 3)        ks >= 32: base_b ^ 32 (ks - 32)
+    const uint32_t base_a = smem_off + n * ROW_A + ((swz_a(n) ^ half) * 16);
+    const uint32_t base_b = smem_off + OFF_B + n * ROW_B + ((swz_b(n) ^ half) * 16);
+    // V^T: as a source lane of the transpose read this lane addresses row half*4 + q (+16 s2, +8 for the second
+    // read), 8 bytes at chunk 4 c + 2 b1 + b0 of it, q = (lane & 15) >> 2, b1 = lane bit 4, b0 = lane bit 1:
+    //   (base_v ^ (64 c | 32 hi)) + 16 KiB s2 + 8 KiB hi
+    const uint32_t base_v = smem_off + (half * 4 + ((lane & 15) >> 2)) * ROW_A + 64 * ((lane & 15) >> 2) +
+                            16 * ((2 * ((lane >> 4) & 1) + ((lane >> 1) & 1)) ^ half) + 8 * (lane & 1);
     typedef __attribute__((address_space(3))) const uint4* lds_u4;
     typedef __attribute__((address_space(3))) s16x4* lds_s4;
     typedef short s16x8 __attribute__((__vector_size__(8 * sizeof(short))));
@@ -208,28 +269,37 @@ __global__ __launch_bounds__(64 * NWV) void mfma_latent_kernel(const SweepParams
         const int tok0 = c0 + t * kTile;
         // tile base addresses, made opaque so that the constant offsets below stay in the instructions'
         // offset fields instead of being folded into per-read address arithmetic
-        uint32_t kaddr = k_rd + buf * BUF;
-        uint32_t vaddr = v_rd + buf * BUF;
-        asm volatile("" : "+v"(kaddr), "+v"(vaddr));
+        const uint32_t ta = base_a + buf * BUF, tb = base_b + buf * BUF, tv = base_v + buf * BUF;
+        uint32_t kaddr[8], kaddr_b[4];
+#pragma unroll
+        for (int j = 0; j < 8; ++j) kaddr[j] = ta ^ (32 * j);
+#pragma unroll
+        for (int j = 0; j < 4; ++j) kaddr_b[j] = tb ^ (32 * j);
         buf = (buf == kNBuf - 1) ? 0 : buf + 1;
         buf_next = (buf_next == kNBuf - 1) ? 0 : buf_next + 1;
 
-        // S^T = K_tile . Q^T : rows = tokens, columns = heads.  K fragments are read KPD steps ahead.
+        // S^T = K_tile . Q^T : rows = tokens, columns = heads.  K fragments are read kKPD steps ahead.
         f32x16 s;
         {
-            constexpr int KPD = 4;
+            constexpr int KPD = kKPD;
             vec8 kf[KPD];
-#pragma unroll
-            for (int i = 0; i < KPD; ++i) kf[i] = __builtin_bit_cast(vec8, *(lds_u4)(uintptr_t)(kaddr + i * 32));
-#pragma unroll
-            for (int ks = 0; ks < KS; ++ks) {
-                const vec8 a = kf[ks % KPD];
-                if (ks + KPD < KS) kf[ks % KPD] = __builtin_bit_cast(vec8, *(lds_u4)(uintptr_t)(kaddr + (ks + KPD) * 32));
-                if (ks == 0)
-                    MM::mma_v0(a, qf[ks], s);
+            static_for<0, KPD>([&](auto ic) {
+                constexpr int i = decltype(ic)::value;
+                lds_read_b128<(i >> 3) * 256>(kf[i], kaddr[i & 7]);
+            });
+            static_for<0, KS>([&](auto ic) {
+                constexpr int ks = decltype(ic)::value;
+                constexpr int left = KS - 1 - ks;  // reads issued after the one this step consumes
+                wait_lgkm<(left < KPD - 1 ? left : KPD - 1)>(kf[ks % KPD]);
+                if constexpr (ks == 0)
+                    MM::mma_v0(kf[ks % KPD], qf[ks], s);
                 else
-                    MM::mma_v(a, qf[ks], s);
-            }
+                    MM::mma_v(kf[ks % KPD], qf[ks], s);
+                if constexpr (ks + KPD < 32)
+                    lds_read_b128<((ks + KPD) >> 3) * 256>(kf[ks % KPD], kaddr[(ks + KPD) & 7]);
+                else if constexpr (ks + KPD < KS)
+                    lds_read_b128<0>(kf[ks % KPD], kaddr_b[ks + KPD - 32]);
+            });
             // the compiler does not see the matrix instructions inside the assembly: cover the
             // result latency of the last one before anything reads the scores (the scores pass
             // through this statement, so no reader can be scheduled ahead of it)
@@ -281,24 +351,30 @@ __global__ __launch_bounds__(64 * NWV) void mfma_latent_kernel(const SweepParams
         pf[0] = MM::pack8(pv);
         pf[1] = MM::pack8(pv + 8);
 
-        // O^T += V_tile^T . P^T : rows = value columns, columns = heads.  V fragments are read VPD steps ahead.
+        // O^T += V_tile^T . P^T : rows = value columns, columns = heads.  V fragment pairs are read kVPD steps ahead.
         {
-            constexpr int VPD = 3;
+            constexpr int VPD = kVPD;
             constexpr int NV = CT * 2;  // (column tile, k-step) pairs, column tile major
+            static_assert(2 * (VPD - 1) <= 15, "lgkmcnt is a 4-bit counter");
             s16x4 vlo[VPD], vhi[VPD];
-            auto rd = [&](int i, s16x4& lo, s16x4& hi) {
-                const int c = i >> 1, s2 = i & 1;
-                lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s4)(uintptr_t)(vaddr + c * 64 + (s2 * 16) * PITCH));
-                hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s4)(uintptr_t)(vaddr + c * 64 + (s2 * 16 + 8) * PITCH));
-            };
-#pragma unroll
-            for (int i = 0; i < VPD; ++i) rd(i, vlo[i], vhi[i]);
-#pragma unroll
-            for (int i = 0; i < NV; ++i) {
+            static_for<0, VPD>([&](auto ic) {
+                constexpr int i = decltype(ic)::value;
+                constexpr int c = i >> 1, s2 = i & 1;
+                lds_read_tr16_b64<s2 * 16 * ROW_A>(vlo[i], tv ^ (64 * c));
+                lds_read_tr16_b64<s2 * 16 * ROW_A + 8 * ROW_A>(vhi[i], tv ^ (64 * c + 32));
+            });
+            static_for<0, NV>([&](auto ic) {
+                constexpr int i = decltype(ic)::value;
+                constexpr int left = NV - 1 - i;
+                wait_lgkm<2 * (left < VPD - 1 ? left : VPD - 1)>(vlo[i % VPD], vhi[i % VPD]);
                 const s16x8 both = __builtin_shufflevector(vlo[i % VPD], vhi[i % VPD], 0, 1, 2, 3, 4, 5, 6, 7);
-                if (i + VPD < NV) rd(i + VPD, vlo[i % VPD], vhi[i % VPD]);
                 acc[i >> 1] = MM::mma(__builtin_bit_cast(vec8, both), pf[i & 1], acc[i >> 1]);
-            }
+                if constexpr (i + VPD < NV) {
+                    constexpr int c = (i + VPD) >> 1, s2 = (i + VPD) & 1;
+                    lds_read_tr16_b64<s2 * 16 * ROW_A>(vlo[i % VPD], tv ^ (64 * c));
+                    lds_read_tr16_b64<s2 * 16 * ROW_A + 8 * ROW_A>(vhi[i % VPD], tv ^ (64 * c + 32));
+                }
+            });
         }
     }
 
@@ -342,7 +418,7 @@ __global__ __launch_bounds__(64 * NWV) void mfma_latent_kernel(const SweepParams
 
 template <int D>
 constexpr size_t lds_bytes() {
-    return (size_t)kNBuf * (((kTile * ((D * 2 + 16) / 16) + 63) / 64) * 1024) + 1024;
+    return (size_t)kNBuf * kTile * D * 2;
 }
 
 template <typename Tag, int D, int DV, int NWV>
@@ -364,7 +440,6 @@ hipError_t launch_tag(const SweepParams& p, int rt, dim3 grid, hipStream_t strea
     switch (rt) {
         case 32: return launch_one<Tag, 576, 512, 1>(p, grid, stream);
         case 64: return launch_one<Tag, 576, 512, 2>(p, grid, stream);
-        case 96: return launch_one<Tag, 576, 512, 3>(p, grid, stream);
         case 128: return launch_one<Tag, 576, 512, 4>(p, grid, stream);
         default: return hipErrorInvalidValue;
     }
@@ -374,7 +449,7 @@ hipError_t launch_tag(const SweepParams& p, int rt, dim3 grid, hipStream_t strea
 
 bool mla_supported(size_t dim, size_t dim_v, int ratio) { return dim == 576 && dim_v == 512 && ratio >= 1; }
 
-int mla_heads_per_group(int ratio) { return std::min(128, (ratio + 31) / 32 * 32); }
+int mla_heads_per_group(int ratio) { return ratio <= 32 ? 32 : (ratio <= 64 ? 64 : 128); }
 
 int mla_rows_per_trip() { return kTile; }
 
