@@ -95,7 +95,7 @@ def measure(torch, w, steps, warmup):
     assert torch.isfinite(outs[0].float()).all()
     nbytes = wl.workload_bytes(w)
     flops = wl.workload_flops(w)
-    plan = _lib.plan(w.max_seq_k, w.batch, w.head_q, w.head_k, w.dim, w.dim_v)
+    plan = _lib.plan(w.max_seq_k, w.batch, w.head_q, w.head_k, w.dim, w.dim_v, total_k=int(w.k.shape[0]))
     return {
         "workload": w.name,
         "us_per_call": mean_ms * 1e3,

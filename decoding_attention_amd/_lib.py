@@ -47,12 +47,12 @@ def load():
     lib.da_decoding_attn.restype = ci
     lib.da_decoding_attn.argtypes = [vp, vp, vp, vp, vp, sz, sz, sz, sz, sz, sz, ci, ci, vp]
     lib.da_decoding_attn_ex.restype = ci
-    lib.da_decoding_attn_ex.argtypes = [vp, vp, vp, vp, vp, sz, sz, sz, sz, sz, sz, ci, ci, cf, vp, vp, sz, vp]
+    lib.da_decoding_attn_ex.argtypes = [vp, vp, vp, vp, vp, sz, sz, sz, sz, sz, sz, ci, ci, cf, vp, sz, vp, sz, vp]
     lib.da_workspace_bytes.restype = sz
-    lib.da_workspace_bytes.argtypes = [sz, sz, sz, sz, sz, sz]
+    lib.da_workspace_bytes.argtypes = [sz, sz, sz, sz, sz, sz, sz]
     ip = ctypes.POINTER(ci)
     lib.da_plan.restype = ci
-    lib.da_plan.argtypes = [sz, sz, sz, sz, sz, sz, ci, ip, ip, ip, ip]
+    lib.da_plan.argtypes = [sz, sz, sz, sz, sz, sz, ci, sz, ip, ip, ip, ip]
     lib.da_supported_head_dims.restype = ci
     lib.da_supported_head_dims.argtypes = [sz, sz]
     lib.da_last_error.restype = ctypes.c_char_p
@@ -67,11 +67,11 @@ def last_error() -> str:
     return load().da_last_error().decode("utf-8", "replace")
 
 
-def plan(max_seq_k, batch, head_q, head_k, dim, dim_v, is_bf16=False):
+def plan(max_seq_k, batch, head_q, head_k, dim, dim_v, is_bf16=False, total_k=0):
     """Launch plan for a shape: dict(kind, nsplit, chunk, heads_per_group)."""
     lib = load()
     kind, ns, ch, rt = ctypes.c_int(), ctypes.c_int(), ctypes.c_int(), ctypes.c_int()
-    rc = lib.da_plan(max_seq_k, batch, head_q, head_k, dim, dim_v, int(is_bf16), ctypes.byref(kind),
+    rc = lib.da_plan(max_seq_k, batch, head_q, head_k, dim, dim_v, int(is_bf16), int(total_k), ctypes.byref(kind),
                      ctypes.byref(ns), ctypes.byref(ch), ctypes.byref(rt))
     if rc != DA_OK:
         raise RuntimeError(f"da_plan failed ({rc}): {last_error()}")

@@ -42,12 +42,13 @@ int env_int(const char* name, int dflt) {
 // Tunables, read once.  DA_TARGET_WGS: work-groups a launch should reach before the sequence
 // stops being split further; DA_MAX_CHUNK / DA_MIN_CHUNK: bounds on tokens per split.
 struct Tunables {
-    int target_wgs, mfma_target_wgs, max_chunk, min_chunk, force_kind, group_min_ratio, wave_per_head;
+    int target_wgs, mfma_target_wgs, max_chunk, min_chunk, ragged_chunk, force_kind, group_min_ratio, wave_per_head;
     Tunables() {
         target_wgs = env_int("DA_TARGET_WGS", 1024);
         mfma_target_wgs = env_int("DA_MFMA_TARGET_WGS", 256);
         max_chunk = env_int("DA_MAX_CHUNK", 1024);
-        min_chunk = env_int("DA_MIN_CHUNK", 256);
+        min_chunk = env_int("DA_MIN_CHUNK", 512);
+        ragged_chunk = env_int("DA_RAGGED_CHUNK", 256);  // tokens per split when the lengths are known to be ragged
         force_kind = env_int("DA_FORCE_KIND", 0);
         wave_per_head = env_int("DA_WAVE_PER_HEAD", 1);
         group_min_ratio = env_int("DA_GROUP_MIN_RATIO", 3);  // smallest head group that takes the grouped MFMA sweep
@@ -89,8 +90,11 @@ int rows_per_trip(size_t dim) {
 }
 
 // v_distinct: V is its own buffer (the MFMA kernel reads V out of the K tile, so it needs the aliased form).
+// total_k: sum of the key lengths if the caller knows it (0 = unknown).  The planner never reads cu_seq_k (that
+// would need a device synchronisation); when total_k shows that the batch is ragged it cuts the sequences into
+// shorter splits so that the work-groups, whose number is sized for max_seq_k, balance.
 Plan make_plan(size_t max_seq_k, size_t batch, size_t head_q, size_t head_k, size_t dim, size_t dim_v,
-               bool v_distinct) {
+               bool v_distinct, size_t total_k) {
     Plan pl;
     const int ratio = (int)(head_q / head_k);
     int trip;
@@ -115,12 +119,19 @@ Plan make_plan(size_t max_seq_k, size_t batch, size_t head_q, size_t head_k, siz
     }
     pl.groups = (ratio + pl.rt - 1) / pl.rt;
     const long long base = (long long)batch * (long long)(pl.wave_per_head ? head_k / 4 : head_k) * pl.groups;
-    const int min_chunk = std::max(tun().min_chunk, trip);
+    const bool ragged = total_k > 0 && (long long)total_k * 10 < (long long)batch * (long long)max_seq_k * 9;
+    int min_chunk = std::max(mfma ? 256 : tun().min_chunk, trip);
+    if (!mfma) {
+        // 512-token splits run best; go down to 256 only when that is needed to give every CU a work-group
+        if (base * std::max<long long>(1, (long long)max_seq_k / min_chunk) < 256) min_chunk = std::max(std::min(min_chunk, 256), trip);
+        if (ragged) min_chunk = std::max(std::min(min_chunk, tun().ragged_chunk), trip);
+    }
     long long want = base > 0 ? (target_wgs + base - 1) / base : 1;
     const long long by_len = std::max<long long>(1, (long long)max_seq_k / min_chunk);
-    // sweep work-groups are also kept short so that ragged batches balance; the MFMA kernel's partials are too
-    // large (heads x dim_v floats per split) to split more than occupancy asks for
-    long long by_cap = mfma ? 1 : ((long long)max_seq_k + tun().max_chunk - 1) / std::max(1, tun().max_chunk);
+    // sweep work-groups are also kept short (shorter still for a ragged batch); the latent MFMA kernel's partials
+    // are too large (heads x dim_v floats per split) to split more than occupancy asks for
+    const int max_chunk = std::max(1, ragged ? tun().ragged_chunk : tun().max_chunk);
+    long long by_cap = mfma ? 1 : ((long long)max_seq_k + max_chunk - 1) / max_chunk;
     long long ns = std::max(std::min(want, by_len), std::min(by_cap, by_len));
     ns = std::max<long long>(1, std::min<long long>(ns, kMaxSplits));
     long long chunk = ((long long)max_seq_k + ns - 1) / ns;
@@ -179,13 +190,13 @@ int da_version(void) { return 100; }
 int da_supported_head_dims(size_t dim, size_t dim_v) { return supported_dims(dim, dim_v) ? 1 : 0; }
 
 int da_plan(size_t max_seq_k, size_t batch, size_t head_q, size_t head_k, size_t dim, size_t dim_v, int is_bf16,
-            int* kernel_kind, int* nsplit, int* chunk, int* heads_per_group) {
+            size_t total_k, int* kernel_kind, int* nsplit, int* chunk, int* heads_per_group) {
     (void)is_bf16;
     if (head_k == 0 || head_q % head_k != 0)
         return fail(DA_ERR_INVALID_ARGUMENT, "head_q (%zu) must be a multiple of head_k (%zu)", head_q, head_k);
     if (!supported_dims(dim, dim_v))
         return fail(DA_ERR_UNSUPPORTED, "unsupported head dims (dim %zu, dim_v %zu)", dim, dim_v);
-    const Plan pl = make_plan(max_seq_k, batch, head_q, head_k, dim, dim_v, false);
+    const Plan pl = make_plan(max_seq_k, batch, head_q, head_k, dim, dim_v, false, total_k);
     if (kernel_kind) *kernel_kind = pl.kind;
     if (nsplit) *nsplit = pl.nsplit;
     if (chunk) *chunk = pl.chunk;
@@ -193,17 +204,18 @@ int da_plan(size_t max_seq_k, size_t batch, size_t head_q, size_t head_k, size_t
     return DA_OK;
 }
 
-size_t da_workspace_bytes(size_t max_seq_k, size_t batch, size_t head_q, size_t head_k, size_t dim, size_t dim_v) {
+size_t da_workspace_bytes(size_t max_seq_k, size_t batch, size_t head_q, size_t head_k, size_t dim, size_t dim_v,
+                          size_t total_k) {
     if (head_k == 0 || head_q % head_k != 0 || !supported_dims(dim, dim_v)) return 0;
-    const size_t a = make_plan(max_seq_k, batch, head_q, head_k, dim, dim_v, false).ws_bytes;
-    const size_t b = make_plan(max_seq_k, batch, head_q, head_k, dim, dim_v, true).ws_bytes;
+    const size_t a = make_plan(max_seq_k, batch, head_q, head_k, dim, dim_v, false, total_k).ws_bytes;
+    const size_t b = make_plan(max_seq_k, batch, head_q, head_k, dim, dim_v, true, total_k).ws_bytes;
     return a > b ? a : b;
 }
 
 int da_decoding_attn_ex(const void* q, const void* k, const void* v, void* o, const int32_t* cu_seq_k,
                         size_t max_seq_k, size_t batch, size_t head_q, size_t head_k, size_t dim, size_t dim_v,
-                        int is_alibi, int is_bf16, float softmax_scale, const float* alibi_slopes, void* workspace,
-                        size_t workspace_bytes, void* hip_stream) {
+                        int is_alibi, int is_bf16, float softmax_scale, const float* alibi_slopes, size_t total_k,
+                        void* workspace, size_t workspace_bytes, void* hip_stream) {
     // the reference's checks (csrc/ops/decoding_attn.cpp:16-22) ...
     if (!q) return fail(DA_ERR_INVALID_ARGUMENT, "q is null");
     if (!k) return fail(DA_ERR_INVALID_ARGUMENT, "k is null");
@@ -228,7 +240,7 @@ int da_decoding_attn_ex(const void* q, const void* k, const void* v, void* o, co
     if (batch == 0) return DA_OK;
 
     hipStream_t stream = reinterpret_cast<hipStream_t>(hip_stream);
-    const Plan pl = make_plan(max_seq_k, batch, head_q, head_k, dim, dim_v, v != nullptr);
+    const Plan pl = make_plan(max_seq_k, batch, head_q, head_k, dim, dim_v, v != nullptr, total_k);
     if ((size_t)head_k * pl.groups > 65535)
         return fail(DA_ERR_INVALID_ARGUMENT, "head_k * groups exceeds the grid limit 65535");
 
@@ -307,7 +319,7 @@ int da_decoding_attn(const void* q, const void* k, const void* v, void* o, const
                      size_t batch, size_t head_q, size_t head_k, size_t dim, size_t dim_v, int is_alibi, int is_bf16,
                      void* hip_stream) {
     return da_decoding_attn_ex(q, k, v, o, cu_seq_k, max_seq_k, batch, head_q, head_k, dim, dim_v, is_alibi, is_bf16,
-                               0.0f, nullptr, nullptr, 0, hip_stream);
+                               0.0f, nullptr, 0, nullptr, 0, hip_stream);
 }
 
 }  // extern "C"

@@ -233,39 +233,53 @@ __global__ __launch_bounds__(256) void sweep_kernel(const SweepParams p) {
     }
 }
 
-// Second pass: merge the per-split partials of one (sequence, query head) in split order.
+// Second pass: merge the per-split partials in split order.  One thread per (sequence, query head, group of four
+// output columns); the partials of four splits are fetched together so that their latencies overlap.
 template <typename Tag>
-__global__ __launch_bounds__(128) void reduce_kernel(const ReduceParams p) {
+__global__ __launch_bounds__(256) void reduce_kernel(const ReduceParams p, int rows) {
     using EL = Elem<Tag>;
-    __shared__ float wts[256];
-    __shared__ float s_den;
-    const int b = blockIdx.x / p.head_q;
-    const int h = blockIdx.x % p.head_q;
+    const int nc4 = p.dim_v >> 2;
+    const int gid = blockIdx.x * 256 + threadIdx.x;
+    const int row = gid / nc4;  // (sequence, head) index
+    const int c4 = gid - row * nc4;
+    if (row >= rows) return;
+    const int b = row / p.head_q;
     const int len = p.cu_seq_k[b + 1] - p.cu_seq_k[b];
     int ns = 0;
     if (len > 0) ns = min(p.nsplit, (len + p.chunk - 1) / p.chunk);
-    const size_t part0 = ((size_t)b * p.head_q + h) * p.nsplit;
-    uint16_t* orow = reinterpret_cast<uint16_t*>(p.o) + ((size_t)b * p.head_q + h) * p.dim_v;
-    if (ns == 0) {
-        for (int col = threadIdx.x; col < p.dim_v; col += blockDim.x) orow[col] = 0;
-        return;
-    }
+    const size_t part0 = (size_t)row * p.nsplit;
+    const float2* const ml = reinterpret_cast<const float2*>(p.ws_ml) + part0;
+    const float4* const src = reinterpret_cast<const float4*>(p.ws_o + part0 * p.dim_v) + c4;
     float mm = kNegBig;
-    for (int s = 0; s < ns; ++s) mm = fmaxf(mm, p.ws_ml[(part0 + s) * 2]);
-    for (int s = threadIdx.x; s < ns; s += blockDim.x) wts[s] = fast_exp2(p.ws_ml[(part0 + s) * 2] - mm);
-    __syncthreads();
-    if (threadIdx.x == 0) {
-        float den = 0.0f;
-        for (int s = 0; s < ns; ++s) den += wts[s] * p.ws_ml[(part0 + s) * 2 + 1];
-        s_den = den;
+    for (int s = 0; s < ns; ++s) mm = fmaxf(mm, ml[s].x);
+    float4 num = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+    float den = 0.0f;
+    for (int s0 = 0; s0 < ns; s0 += 4) {
+        float2 e[4];
+        float4 x[4];
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+            const int s = min(s0 + u, ns - 1);
+            e[u] = ml[s];
+            x[u] = src[(size_t)s * nc4];
+        }
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+            const float w = (s0 + u < ns) ? fast_exp2(e[u].x - mm) : 0.0f;
+            den += w * e[u].y;
+            num.x += w * x[u].x;
+            num.y += w * x[u].y;
+            num.z += w * x[u].z;
+            num.w += w * x[u].w;
+        }
     }
-    __syncthreads();
-    const float inv = 1.0f / s_den;
-    for (int col = threadIdx.x; col < p.dim_v; col += blockDim.x) {
-        float num = 0.0f;
-        for (int s = 0; s < ns; ++s) num += wts[s] * p.ws_o[(part0 + s) * p.dim_v + col];
-        orow[col] = EL::from_f32(num * inv);
-    }
+    const float inv = ns > 0 ? 1.0f / den : 0.0f;  // an empty sequence yields a zero row
+    ushort4 r;
+    r.x = EL::from_f32(num.x * inv);
+    r.y = EL::from_f32(num.y * inv);
+    r.z = EL::from_f32(num.z * inv);
+    r.w = EL::from_f32(num.w * inv);
+    *reinterpret_cast<ushort4*>(reinterpret_cast<uint16_t*>(p.o) + (size_t)row * p.dim_v + c4 * 4) = r;
 }
 
 }  // namespace da

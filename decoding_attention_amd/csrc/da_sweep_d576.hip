@@ -5,10 +5,13 @@ hipError_t launch_sweep_d576(const SweepParams& p, bool is_bf16, int rt, dim3 gr
     return launch_sweep_dim<576, 512, 2>(p, is_bf16, rt, grid, stream);
 }
 hipError_t launch_reduce(const ReduceParams& p, bool is_bf16, int blocks, hipStream_t stream) {
+    // `blocks` counts (sequence, head) rows; one thread per four output columns
+    const long long threads = (long long)blocks * (p.dim_v / 4);
+    const dim3 grid((unsigned)((threads + 255) / 256));
     if (is_bf16)
-        hipLaunchKernelGGL((reduce_kernel<bf16_tag>), dim3(blocks), dim3(128), 0, stream, p);
+        hipLaunchKernelGGL((reduce_kernel<bf16_tag>), grid, dim3(256), 0, stream, p, blocks);
     else
-        hipLaunchKernelGGL((reduce_kernel<f16_tag>), dim3(blocks), dim3(128), 0, stream, p);
+        hipLaunchKernelGGL((reduce_kernel<f16_tag>), grid, dim3(256), 0, stream, p, blocks);
     return hipGetLastError();
 }
 }  // namespace da

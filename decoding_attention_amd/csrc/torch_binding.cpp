@@ -103,15 +103,16 @@ at::Tensor dmha_fwd(const at::Tensor &q, const at::Tensor &k, const std::optiona
     c10::hip::HIPGuardMasqueradingAsCUDA guard(q.device());
     hipStream_t stream = c10::hip::getCurrentHIPStreamMasqueradingAsCUDA(q.device().index()).stream();
 
+    // k.size(0) is the sum of the key lengths: a free host-side hint for sizing the sequence splits
     const size_t ws_bytes = da_workspace_bytes((size_t)max_seq_k, (size_t)batch, (size_t)head_q, (size_t)head_k,
-                                               (size_t)dim, (size_t)dim_v);
+                                               (size_t)dim, (size_t)dim_v, (size_t)total_k);
     at::Tensor ws;  // from torch's stream-aware caching allocator
     if (ws_bytes > 0) ws = torch::empty({(int64_t)ws_bytes}, q.options().dtype(torch::kUInt8));
 
     const int rc = da_decoding_attn_ex(
         q.data_ptr(), k.data_ptr(), v_ptr, o.data_ptr(), cu_seq_k.data_ptr<int32_t>(), (size_t)max_seq_k,
         (size_t)batch, (size_t)head_q, (size_t)head_k, (size_t)dim, (size_t)dim_v, is_alibi ? 1 : 0, is_bf16 ? 1 : 0,
-        softmax_scale.has_value() ? (float)softmax_scale.value() : 0.0f, slopes_ptr,
+        softmax_scale.has_value() ? (float)softmax_scale.value() : 0.0f, slopes_ptr, (size_t)total_k,
         ws_bytes > 0 ? ws.data_ptr() : nullptr, ws_bytes, (void *)stream);
     TORCH_CHECK(rc == DA_OK, "decoding_attn failed (", rc, "): ", da_last_error());
     return o;

@@ -49,30 +49,35 @@ int da_decoding_attn(const void *q, const void *k, const void *v, void *o, const
  * Extends reference csrc/ops/decoding_attn.cpp:13-62 (set_dmha_fwd_params), which hard-codes both.
  *   softmax_scale  <= 0 selects 1/sqrt(dim)
  *   alibi_slopes   device float[head_q] or NULL for the closed form; read only when is_alibi != 0
+ *   total_k        number of key tokens (cu_seq_k[batch]) if the caller knows it on the host, else 0.  Only a
+ *                  hint: a batch that is much shorter than batch * max_seq_k is cut into shorter sequence splits
+ *                  so that it balances; results do not depend on it.  Pass the same value to da_workspace_bytes.
  *   workspace      device buffer of at least da_workspace_bytes(...) bytes, 16-byte aligned, or NULL to use the
  *                  library's cached one
  */
 int da_decoding_attn_ex(const void *q, const void *k, const void *v, void *o, const int32_t *cu_seq_k,
                         size_t max_seq_k, size_t batch, size_t head_q, size_t head_k, size_t dim, size_t dim_v,
-                        int is_alibi, int is_bf16, float softmax_scale, const float *alibi_slopes, void *workspace,
-                        size_t workspace_bytes, void *hip_stream);
+                        int is_alibi, int is_bf16, float softmax_scale, const float *alibi_slopes, size_t total_k,
+                        void *workspace, size_t workspace_bytes, void *hip_stream);
 
 /*
  * Bytes of workspace da_decoding_attn_ex needs for this shape (0 when the sequence is not split).
  * No counterpart in the reference, whose kernel never splits a sequence
  * (csrc/kernel/decoding_attn/decoding_fwd_launch_template.h:12-31).
  */
-size_t da_workspace_bytes(size_t max_seq_k, size_t batch, size_t head_q, size_t head_k, size_t dim, size_t dim_v);
+size_t da_workspace_bytes(size_t max_seq_k, size_t batch, size_t head_q, size_t head_k, size_t dim, size_t dim_v,
+                          size_t total_k);
 
 /*
  * Launch plan the library would use for this shape, for tests and benchmarks:
  *   kernel_kind 1 = VALU sweep, 2 = latent (MLA) MFMA sweep, 3 = grouped-head MFMA sweep; nsplit = sequence splits;
- *   chunk = tokens per split; heads_per_group = query heads one work-group serves.
+ *   chunk = tokens per split; heads_per_group = query heads one work-group serves; total_k as for
+ *   da_decoding_attn_ex (0 = unknown).
  * Any output pointer may be NULL.  Returns DA_ERR_UNSUPPORTED for an unsupported (dim, dim_v).
  * Mirrors the role of the reference's per-head-dim tile choice (csrc/kernel/decoding_attn/decoding_fwd_hd*.cu).
  */
 int da_plan(size_t max_seq_k, size_t batch, size_t head_q, size_t head_k, size_t dim, size_t dim_v, int is_bf16,
-            int *kernel_kind, int *nsplit, int *chunk, int *heads_per_group);
+            size_t total_k, int *kernel_kind, int *nsplit, int *chunk, int *heads_per_group);
 
 /* 1 when (dim, dim_v) is a supported pair: the reference's DA_HEADDIM_SWITCH set (csrc/common/common.h:73-96). */
 int da_supported_head_dims(size_t dim, size_t dim_v);

@@ -235,6 +235,27 @@ def test_reference_signature_entry_point_with_library_workspace():
     check_against_oracle(w, o.cpu())
 
 
+def test_total_k_hint_changes_the_plan_not_the_result():
+    """A ragged batch through da_decoding_attn_ex with and without the token-count hint; both match the oracle."""
+    lib = _lib.load()
+    dev = torch.device("cuda:0")
+    b = 64
+    w = wl.make_workload(b, 32, 8, 128, 128, 2048, torch.bfloat16, seed=11, varlen=True)
+    total, sk = int(w.k.shape[0]), int(w.max_seq_k)
+    assert _lib.plan(sk, b, 32, 8, 128, 128, True, total)["chunk"] < _lib.plan(sk, b, 32, 8, 128, 128, True)["chunk"]
+    wd = w.to(dev)
+    for hint in (0, total):
+        n = lib.da_workspace_bytes(sk, b, 32, 8, 128, 128, hint)
+        ws = torch.empty(n, dtype=torch.uint8, device=dev)
+        o = torch.full((b, 32, 128), float("nan"), dtype=torch.bfloat16, device=dev)
+        rc = lib.da_decoding_attn_ex(wd.q.data_ptr(), wd.k.data_ptr(), wd.v.data_ptr(), o.data_ptr(),
+                                     wd.cu_seq_k.data_ptr(), sk, b, 32, 8, 128, 128, 0, 1, 0.0, None, hint,
+                                     ws.data_ptr(), n, None)
+        assert rc == 0, _lib.last_error()
+        torch.cuda.synchronize()
+        check_against_oracle(w, o.cpu())
+
+
 def test_gpu_side_argument_errors():
     lib = _lib.load()
     dev = torch.device("cuda:0")
@@ -242,7 +263,7 @@ def test_gpu_side_argument_errors():
     o = torch.empty(1, 32, 128, dtype=torch.float16, device=dev)
     small = torch.empty(64, dtype=torch.uint8, device=dev)
     rc = lib.da_decoding_attn_ex(w.q.data_ptr(), w.k.data_ptr(), w.v.data_ptr(), o.data_ptr(), w.cu_seq_k.data_ptr(),
-                                 4096, 1, 32, 32, 128, 128, 0, 0, 0.0, None, small.data_ptr(), 64, None)
+                                 4096, 1, 32, 32, 128, 128, 0, 0, 0.0, None, 0, small.data_ptr(), 64, None)
     assert rc == _lib.DA_ERR_WORKSPACE and "workspace" in _lib.last_error()
     with pytest.raises(RuntimeError, match="one query token per sequence"):
         fwd(torch.cat([w.q, w.q]), w.k, w.v, None, w.cu_seq_k, 4096, 128, False)

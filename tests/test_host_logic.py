@@ -34,7 +34,7 @@ def test_version_and_supported_dims():
 
 
 def _call_ex(lib, q=16, k=16, v=16, o=16, cu=16, max_seq_k=8, batch=1, hq=4, hk=4, d=64, dv=64):
-    return lib.da_decoding_attn_ex(q, k, v, o, cu, max_seq_k, batch, hq, hk, d, dv, 0, 0, 0.0, None, None, 0, None)
+    return lib.da_decoding_attn_ex(q, k, v, o, cu, max_seq_k, batch, hq, hk, d, dv, 0, 0, 0.0, None, 0, None, 0, None)
 
 
 def test_argument_errors_without_gpu():
@@ -62,10 +62,23 @@ def test_plan_is_consistent(d, dv, batch, sk):
     assert 1 <= p["nsplit"] <= 256
     assert p["nsplit"] * p["chunk"] >= sk
     assert (p["nsplit"] - 1) * p["chunk"] < max(sk, 1)
-    ws = _lib.load().da_workspace_bytes(sk, batch, hq, hk, d, dv)
+    ws = _lib.load().da_workspace_bytes(sk, batch, hq, hk, d, dv, 0)
     need = 0 if p["nsplit"] == 1 else batch * hq * p["nsplit"] * (dv + 2) * 4
     # (576, 512) also covers the plan used when V is passed as its own buffer
     assert ws >= need if d == 576 else ws == need
+
+
+def test_plan_total_k_hint_only_shortens_splits_of_ragged_batches():
+    """The token-count hint changes the split size of a ragged batch only, and never the kernel kind."""
+    sk, batch = 8192, 64
+    base = _lib.plan(sk, batch, 32, 8, 128, 128)
+    full = _lib.plan(sk, batch, 32, 8, 128, 128, total_k=batch * sk)
+    ragged = _lib.plan(sk, batch, 32, 8, 128, 128, total_k=batch * sk // 2)
+    assert full == base
+    assert ragged["kind"] == base["kind"] and ragged["chunk"] < base["chunk"]
+    assert ragged["nsplit"] * ragged["chunk"] >= sk
+    ws = _lib.load().da_workspace_bytes(sk, batch, 32, 8, 128, 128, batch * sk // 2)
+    assert ws == batch * 32 * ragged["nsplit"] * (128 + 2) * 4
 
 
 def test_plan_rejects_bad_shapes():
