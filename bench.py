@@ -31,11 +31,13 @@ HBM_PEAK_GBPS = 8000.0      # MI355X HBM3E, published
 MFMA_PEAK_TFLOPS = 2500.0   # MI355X dense fp16/bf16 MFMA, published
 # HBM bytes per call from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of `bench.py --only gqa|mla`, each counter
 # scaled by what it reads for a 1 GiB device copy (profiles/*_hbm_traffic.md); valid for the default launch plan.
-MEASURED_TRAFFIC_BYTES = {"gqa": 1098235904, "mla": None}
+MEASURED_TRAFFIC_BYTES = {"gqa": 1098235904, "mla": 488047616}
 
 
 def _time_calls(torch, fn_list, steps, warmup):
-    """Mean and min milliseconds per call over `steps` calls, rotating over fn_list."""
+    """Mean milliseconds per call over `steps` back-to-back calls, rotating over fn_list, and the fastest of a few
+    calls timed one by one with a host synchronisation after each (that one includes the launch gap between the
+    sweep and the merge kernel, so it can exceed the back-to-back mean)."""
     n = len(fn_list)
     for i in range(warmup):
         fn_list[i % n]()
@@ -99,7 +101,7 @@ def measure(torch, w, steps, warmup):
     return {
         "workload": w.name,
         "us_per_call": mean_ms * 1e3,
-        "us_per_call_min": min_ms * 1e3,
+        "us_isolated_call_min": min_ms * 1e3,
         "algorithmic_bytes": nbytes,
         "algorithmic_flops": flops,
         "hbm_GBps": nbytes / (mean_ms * 1e-3) / 1e9,
@@ -195,7 +197,7 @@ def run_default(args):
                                "packed K/V [262144, 8, 128], scale 1/sqrt(128), seed 0",
                    "name": gqa["workload"], "plan": gqa["plan"]},
         "us_per_call": gqa["us_per_call"],
-        "us_per_call_min": gqa["us_per_call_min"],
+        "us_isolated_call_min": gqa["us_isolated_call_min"],
         "pct_hbm_peak": 100.0 * gqa["hbm_frac_of_peak"],
         "roofline": {"bound": "hbm", "achieved": gqa["hbm_GBps"], "peak": HBM_PEAK_GBPS, "unit": "GB/s",
                      "frac": gqa["hbm_frac_of_peak"], "traffic": MEASURED_TRAFFIC_BYTES["gqa"],
@@ -206,7 +208,7 @@ def run_default(args):
         line["mla"] = {
             "workload": "MLA decode fp16, batch 64, 128 q heads / 1 latent kv head, dims 576/512, seq_k 4096, "
                         "V = K[..., :512]",
-            "us_per_call": mla["us_per_call"], "us_per_call_min": mla["us_per_call_min"],
+            "us_per_call": mla["us_per_call"], "us_isolated_call_min": mla["us_isolated_call_min"],
             "hbm_TBps": mla["hbm_GBps"] / 1e3, "pct_hbm_peak": 100.0 * mla["hbm_frac_of_peak"],
             "tflops": mla["tflops"], "pct_mfma_peak": 100.0 * mla["mfma_frac_of_peak"],
             "algorithmic_bytes": mla["algorithmic_bytes"], "algorithmic_flops": mla["algorithmic_flops"],
@@ -244,7 +246,7 @@ def run_sweep(args):
         ref_bytes = wl.reference_formula_bytes(w.batch, w.head_q, w.head_k, w.dim, w.dim_v, sk)
         print(f"Decoding-Attention {w.batch}-{sk} profiling time: {ms:.4f} ms, throughput: {r['tflops']:.4f} TFLOPS, "
               f"bandwidth: {ref_bytes / (ms * 1e-3) / 1e9:.3f} GB/s", flush=True)
-        print(f"    [{tag}] {w.name}: {r['us_per_call']:.1f} us/call (min {r['us_per_call_min']:.1f}), "
+        print(f"    [{tag}] {w.name}: {r['us_per_call']:.1f} us/call (min {r['us_isolated_call_min']:.1f}), "
               f"{r['hbm_GBps'] / 1e3:.3f} TB/s of real traffic = {100 * r['hbm_frac_of_peak']:.1f}% of "
               f"{HBM_PEAK_GBPS / 1e3:.0f} TB/s, plan {r['plan']}", flush=True)
         r["tag"] = tag
