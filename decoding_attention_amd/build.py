@@ -66,6 +66,28 @@ def build(force=True, verbose=False):
     return LIB_PATH
 
 
+CLI_SRC = os.path.join(PKG_DIR, "bench_cli", "benchmark_decoding_attn.cpp")
+CLI_PATH = os.path.join(PKG_DIR, "bench_cli", "benchmark_decoding_attn")
+
+
+def build_cli(force=True):
+    """Compile the benchmark executable (host code only) against the in-tree library."""
+    if not force and os.path.exists(CLI_PATH):
+        return CLI_PATH
+    if not os.path.exists(LIB_PATH):
+        build(force=True)
+    rocm = os.environ.get("ROCM_PATH", "/opt/rocm")
+    include = os.path.join(os.path.dirname(PKG_DIR), "include")
+    cmd = [os.environ.get("CXX", "g++"), "-O2", "-std=c++17", "-Wall", "-Wextra", "-fopenmp", "-D__HIP_PLATFORM_AMD__=1",
+           f"-I{include}", f"-I{rocm}/include", CLI_SRC, "-o", CLI_PATH, f"-L{PKG_DIR}", "-ldecoding_attn_hip",
+           f"-L{rocm}/lib", "-lamdhip64", "-Wl,-rpath,$ORIGIN/..", f"-Wl,-rpath,{rocm}/lib"]
+    res = subprocess.run(cmd, capture_output=True, text=True)
+    if res.returncode != 0:
+        raise RuntimeError(f"building the benchmark executable failed:\n{res.stdout}\n{res.stderr}")
+    return CLI_PATH
+
+
 if __name__ == "__main__":
     path = build(force=True, verbose=True)
     print(path)
+    print(build_cli(force=True))

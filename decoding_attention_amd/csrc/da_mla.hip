@@ -159,7 +159,7 @@ __global__ __launch_bounds__(64 * NWV) void mfma_latent_kernel(const SweepParams
     constexpr int CT = DV / 32;                          // 32-column tiles of the output
     static_assert(D % 16 == 0 && DV % 32 == 0 && DV <= D, "shape");
 
-    extern __shared__ __attribute__((aligned(1024))) uint8_t smem[];  // kNBuf * BUF
+    extern __shared__ __attribute__((aligned(1024))) uint8_t smem[];  // max(kNBuf, NWV) * BUF
     const uint32_t smem_off = (uint32_t)(uintptr_t)smem;
 
     const int lane = threadIdx.x & 63;
@@ -167,10 +167,23 @@ __global__ __launch_bounds__(64 * NWV) void mfma_latent_kernel(const SweepParams
     const int half = lane >> 5;
     const int n = lane & 31;
 
-    const int split = blockIdx.x;
-    const int hk = blockIdx.y / p.groups;
-    const int grp = blockIdx.y % p.groups;
-    const int b = blockIdx.z;
+    // Work-groups are handed to the eight XCDs round-robin by linear id, and each XCD has its own L2.  Renumber
+    // so that the sequence splits of one (sequence, head group) run on one XCD: they read the same Q block, which
+    // then leaves HBM once instead of once per split.
+    int split = blockIdx.x, by = blockIdx.y, b = blockIdx.z;
+    {
+        const int outer_n = gridDim.y * gridDim.z;
+        if (gridDim.x > 1 && outer_n % 8 == 0) {
+            const int lin = blockIdx.x + gridDim.x * (blockIdx.y + gridDim.y * blockIdx.z);
+            const int slot = lin >> 3;
+            split = slot % (int)gridDim.x;
+            const int outer = (slot / (int)gridDim.x) * 8 + (lin & 7);
+            by = outer % (int)gridDim.y;
+            b = outer / (int)gridDim.y;
+        }
+    }
+    const int hk = by / p.groups;
+    const int grp = by % p.groups;
 
     const int start = p.cu_seq_k[b];
     const int len = p.cu_seq_k[b + 1] - start;
@@ -187,14 +200,44 @@ __global__ __launch_bounds__(64 * NWV) void mfma_latent_kernel(const SweepParams
         return;
     }
 
-    // Q rows of this wave's heads as B-operands: lane (n, half) holds Q[head n][ks*16 + half*8 .. +8)
-    const int hq = min(h_base + min(n, max(nh, 1) - 1), p.head_q - 1);
+    // Q rows of this wave's heads as B-operands: lane (n, half) holds Q[head n][ks*16 + half*8 .. +8).  Loading
+    // that layout straight from global memory costs 36 instructions of 32-byte pieces per wave; instead the
+    // wave's 32 x 576 block of Q is staged like a K tile (whole-row direct-to-LDS loads, same swizzle, into the
+    // wave's own buffer) and read back with the K-row read pattern, which is the same operand layout.
+    const int q_last = max(nh, 1) - 1;
+    const int hq = min(h_base + min(n, q_last), p.head_q - 1);
+    const uint32_t lane16 = lane * 16;
+    const int rb = lane >> 3;  // region B: row within the group of eight, chunk lane & 7
     vec8 qf[KS];
     {
-        const uint16_t* qrow = reinterpret_cast<const uint16_t*>(p.q) + ((size_t)b * p.head_q + hq) * D + half * 8;
-#pragma unroll
-        for (int ks = 0; ks < KS; ++ks) qf[ks] = __builtin_bit_cast(vec8, *reinterpret_cast<const uint4*>(qrow + ks * 16));
+        const uint8_t* const qb = reinterpret_cast<const uint8_t*>(p.q) + (size_t)b * p.head_q * (D * 2);
+        const uint32_t qbuf = smem_off + wave * BUF;
+        static_for<0, kTile>([&](auto rc) {
+            constexpr int row = decltype(rc)::value;
+            const int head = min(h_base + min(row, q_last), p.head_q - 1);  // wave-uniform
+            lds_dma16(qb, (uint32_t)head * (uint32_t)(D * 2) + (lane16 ^ (uint32_t)(swz_a(row) * 16)),
+                      qbuf + (uint32_t)(row * ROW_A));
+        });
+        static_for<0, kTile / 8>([&](auto jc) {
+            constexpr int j = decltype(jc)::value;
+            const int row = j * 8 + rb;
+            const int head = min(h_base + min(row, q_last), p.head_q - 1);
+            lds_dma16(qb, (uint32_t)head * (uint32_t)(D * 2) + (uint32_t)(DV * 2 + (((lane & 7) ^ swz_b(row)) * 16)),
+                      qbuf + (uint32_t)(OFF_B + j * 1024));
+        });
+        wait_vmcnt<0>();
+        const uint32_t qa = qbuf + n * ROW_A + ((swz_a(n) ^ half) * 16);
+        const uint32_t qbb = qbuf + OFF_B + n * ROW_B + ((swz_b(n) ^ half) * 16);
+        static_for<0, KS>([&](auto ic) {
+            constexpr int ks = decltype(ic)::value;
+            if constexpr (ks < 32)
+                lds_read_b128<(ks >> 3) * 256>(qf[ks], qa ^ (uint32_t)(32 * (ks & 7)));
+            else
+                lds_read_b128<0>(qf[ks], qbb ^ (uint32_t)(32 * (ks - 32)));
+            if constexpr (ks % 12 == 11) wait_lgkm<0>(qf[ks]);  // the counter of outstanding reads is 4 bits wide
+        });
     }
+    __syncthreads();  // the tile buffers are free for K once every wave has its Q in registers
     const float slope = p.is_alibi ? alibi_slope_log2(p.slopes, hq, p.head_q) : 0.0f;
 
     f32x16 acc[CT];
@@ -211,8 +254,6 @@ __global__ __launch_bounds__(64 * NWV) void mfma_latent_kernel(const SweepParams
     // Stage the tile that starts at token tok0 into buffer `buf`.  Rows past the end of the split re-read the
     // last valid row (they are masked later).  Every wave always issues exactly NLW loads, so the hand-placed
     // vmcnt waits count the same on every wave.
-    const uint32_t lane16 = lane * 16;
-    const int rb = lane >> 3;  // region B: row within the group of eight, chunk lane & 7
     auto issue_tile = [&](int tok0, int buf) {
         const uint8_t* const base = kbytes + (size_t)tok0 * k_row_bytes;
         const int last = c1 - 1 - tok0;
@@ -416,9 +457,10 @@ __global__ __launch_bounds__(64 * NWV) void mfma_latent_kernel(const SweepParams
     }
 }
 
-template <int D>
+// kNBuf tile buffers; the prologue stages each wave's Q block in a buffer of its own.
+template <int D, int NWV>
 constexpr size_t lds_bytes() {
-    return (size_t)kNBuf * kTile * D * 2;
+    return (size_t)(kNBuf > NWV ? kNBuf : NWV) * kTile * D * 2;
 }
 
 template <typename Tag, int D, int DV, int NWV>
@@ -428,10 +470,11 @@ hipError_t launch_one(const SweepParams& p, dim3 grid, hipStream_t stream) {
     auto kern = mfma_latent_kernel<Tag, D, DV, NWV>;
     std::call_once(once, [&] {
         attr_err = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
-                                       (int)lds_bytes<D>());
+                                       (int)lds_bytes<D, NWV>());
     });
     if (attr_err != hipSuccess) return attr_err;
-    hipLaunchKernelGGL(kern, grid, dim3(64 * NWV), lds_bytes<D>(), stream, p);
+    constexpr size_t lds = lds_bytes<D, NWV>();
+    hipLaunchKernelGGL(kern, grid, dim3(64 * NWV), lds, stream, p);
     return hipGetLastError();
 }
 
