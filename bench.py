@@ -79,7 +79,7 @@ def _device_copies(torch, w, dev, min_total_bytes=768 << 20):
     return copies
 
 
-def measure(torch, w, steps, warmup):
+def measure(torch, w, steps, warmup, page_size=0):
     from decoding_attention_amd import _lib, decoding_attn_fwd
     from decoding_attention_amd import workloads as wl
 
@@ -88,6 +88,17 @@ def measure(torch, w, steps, warmup):
     outs = []
 
     def make(c):
+        if page_size:
+            from decoding_attention_amd import decoding_attn_paged_fwd
+
+            pk = wl.to_pages(w, page_size, seed=len(outs)).to(dev)
+            total = int(w.k.shape[0])
+
+            def call_paged():
+                outs[:] = [decoding_attn_paged_fwd(c.q, pk.k_pages, pk.v_pages, pk.block_table, pk.seq_lens,
+                                                   c.max_seq_k, c.dim_v, c.is_alibi, total_k=total)]
+            return call_paged
+
         def call():
             outs[:] = [decoding_attn_fwd(c.q, c.k, c.v, c.cu_seq_k, c.max_seq_k, c.dim_v, c.is_alibi)]
         return call
@@ -238,9 +249,12 @@ def run_sweep(args):
     if args.sweep in ("gqa", "all"):
         shapes += [("gqa-varlen", wl.config_gqa_varlen()), ("gqa-fixed", wl.config_gqa_fixed()),
                    ("mqa-alibi", wl.config_mqa_alibi())]
+    if args.sweep == "paged":  # the two benchmark shapes over shuffled 64-token pages, beside the packed layout
+        for w in (wl.config_gqa_fixed(), wl.config_mla(64, 4096)):
+            shapes += [("packed", w), ("paged-64", w)]
     results = []
     for tag, w in shapes:
-        r = measure(torch, w, args.steps, args.warmup)
+        r = measure(torch, w, args.steps, args.warmup, page_size=64 if tag == "paged-64" else 0)
         ms = r["us_per_call"] / 1e3
         sk = w.max_seq_k
         ref_bytes = wl.reference_formula_bytes(w.batch, w.head_q, w.head_k, w.dim, w.dim_v, sk)
@@ -270,7 +284,8 @@ def main():
     ap.add_argument("--calibrate-copy", action="store_true", help="first run three 1 GiB device copies (a known "
                     "traffic figure for scaling profiler byte counters)")
     ap.add_argument("--cpu-budget", type=float, default=15.0, help="seconds of single-thread CPU work to sample")
-    ap.add_argument("--sweep", choices=["mha", "mla", "gqa", "all"], help="print the reference's sweeps instead")
+    ap.add_argument("--sweep", choices=["mha", "mla", "gqa", "all", "paged"], help="print the reference's sweeps instead "
+                    "(paged: the two benchmark shapes over a paged K/V cache)")
     ap.add_argument("--json-out", help="with --sweep: also write the results as JSON")
     args = ap.parse_args()
     if args.gpus != 1:

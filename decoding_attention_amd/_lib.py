@@ -14,6 +14,8 @@ EXPORTED_SYMBOLS = (
     "da_decoding_attn",
     "da_decoding_attn_ex",
     "da_workspace_bytes",
+    "da_decoding_attn_paged",
+    "da_workspace_bytes_paged",
     "da_plan",
     "da_supported_head_dims",
     "da_last_error",
@@ -50,6 +52,11 @@ def load():
     lib.da_decoding_attn_ex.argtypes = [vp, vp, vp, vp, vp, sz, sz, sz, sz, sz, sz, ci, ci, cf, vp, sz, vp, sz, vp]
     lib.da_workspace_bytes.restype = sz
     lib.da_workspace_bytes.argtypes = [sz, sz, sz, sz, sz, sz, sz]
+    lib.da_decoding_attn_paged.restype = ci
+    lib.da_decoding_attn_paged.argtypes = [vp, vp, vp, vp, vp, vp, sz, sz, sz, sz, sz, sz, sz, sz, sz, sz, ci, ci, cf,
+                                           vp, sz, vp, sz, vp]
+    lib.da_workspace_bytes_paged.restype = sz
+    lib.da_workspace_bytes_paged.argtypes = [sz, sz, sz, sz, sz, sz, sz, sz]
     ip = ctypes.POINTER(ci)
     lib.da_plan.restype = ci
     lib.da_plan.argtypes = [sz, sz, sz, sz, sz, sz, ci, sz, ip, ip, ip, ip]

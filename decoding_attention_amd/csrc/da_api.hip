@@ -93,19 +93,22 @@ int rows_per_trip(size_t dim) {
 // total_k: sum of the key lengths if the caller knows it (0 = unknown).  The planner never reads cu_seq_k (that
 // would need a device synchronisation); when total_k shows that the batch is ragged it cuts the sequences into
 // shorter splits so that the work-groups, whose number is sized for max_seq_k, balance.
+// tiles_contiguous: every aligned run of 32 tokens is contiguous in memory (always true for the packed layout; for
+// paged K/V only when a page holds a multiple of 32 tokens).  The two MFMA kernels fetch whole tiles and need it.
 Plan make_plan(size_t max_seq_k, size_t batch, size_t head_q, size_t head_k, size_t dim, size_t dim_v,
-               bool v_distinct, size_t total_k) {
+               bool v_distinct, size_t total_k, bool tiles_contiguous = true) {
     Plan pl;
     const int ratio = (int)(head_q / head_k);
     int trip;
     int target_wgs = tun().target_wgs;
-    const bool mfma = !v_distinct && da::mla_supported(dim, dim_v, ratio) && tun().force_kind != kKindSweep;
+    const bool force_sweep = tun().force_kind == kKindSweep || !tiles_contiguous;
+    const bool mfma = !v_distinct && da::mla_supported(dim, dim_v, ratio) && !force_sweep;
     if (mfma) {
         pl.kind = kKindMfma;
         pl.rt = da::mla_heads_per_group(ratio);
         trip = da::mla_rows_per_trip();
         target_wgs = tun().mfma_target_wgs;  // one 4-wave work-group fills a CU
-    } else if (dim <= 256 && ratio >= tun().group_min_ratio && tun().force_kind != kKindSweep) {
+    } else if (dim <= 256 && ratio >= tun().group_min_ratio && !force_sweep) {
         pl.kind = kKindGroup;
         pl.rt = ratio > 16 ? 32 : 16;
         pl.wave_per_head = head_k % 4 == 0 && tun().wave_per_head;
@@ -212,15 +215,35 @@ size_t da_workspace_bytes(size_t max_seq_k, size_t batch, size_t head_q, size_t 
     return a > b ? a : b;
 }
 
-int da_decoding_attn_ex(const void* q, const void* k, const void* v, void* o, const int32_t* cu_seq_k,
-                        size_t max_seq_k, size_t batch, size_t head_q, size_t head_k, size_t dim, size_t dim_v,
-                        int is_alibi, int is_bf16, float softmax_scale, const float* alibi_slopes, size_t total_k,
-                        void* workspace, size_t workspace_bytes, void* hip_stream) {
+size_t da_workspace_bytes_paged(size_t max_seq_k, size_t batch, size_t head_q, size_t head_k, size_t dim, size_t dim_v,
+                                size_t total_k, size_t page_size) {
+    if (head_k == 0 || head_q % head_k != 0 || !supported_dims(dim, dim_v)) return 0;
+    const bool contiguous = page_size % 32 == 0;
+    const size_t a = make_plan(max_seq_k, batch, head_q, head_k, dim, dim_v, false, total_k, contiguous).ws_bytes;
+    const size_t b = make_plan(max_seq_k, batch, head_q, head_k, dim, dim_v, true, total_k, contiguous).ws_bytes;
+    return a > b ? a : b;
+}
+
+}  // extern "C"
+
+namespace {
+
+// Page-pool description of paged K/V; table == nullptr means the packed layout.
+struct Paging {
+    const int32_t* table = nullptr;
+    const int32_t* seq_lens = nullptr;
+    size_t page_size = 0, max_blocks = 0, k_page = 0, v_page = 0;
+};
+
+int run_attention(const void* q, const void* k, const void* v, void* o, const int32_t* cu_seq_k, const Paging& pg,
+                  size_t max_seq_k, size_t batch, size_t head_q, size_t head_k, size_t dim, size_t dim_v,
+                  int is_alibi, int is_bf16, float softmax_scale, const float* alibi_slopes, size_t total_k,
+                  void* workspace, size_t workspace_bytes, void* hip_stream) {
     // the reference's checks (csrc/ops/decoding_attn.cpp:16-22) ...
     if (!q) return fail(DA_ERR_INVALID_ARGUMENT, "q is null");
     if (!k) return fail(DA_ERR_INVALID_ARGUMENT, "k is null");
     if (!o) return fail(DA_ERR_INVALID_ARGUMENT, "o is null");
-    if (!cu_seq_k) return fail(DA_ERR_INVALID_ARGUMENT, "cu_seq_k is null");
+    if (!pg.table && !cu_seq_k) return fail(DA_ERR_INVALID_ARGUMENT, "cu_seq_k is null");
     if (head_k == 0 || head_q % head_k != 0)
         return fail(DA_ERR_INVALID_ARGUMENT, "head_q (%zu) must be a multiple of head_k (%zu)", head_q, head_k);
     if (dim > 576) return fail(DA_ERR_INVALID_ARGUMENT, "dim (%zu) must be <= 576", dim);
@@ -240,7 +263,8 @@ int da_decoding_attn_ex(const void* q, const void* k, const void* v, void* o, co
     if (batch == 0) return DA_OK;
 
     hipStream_t stream = reinterpret_cast<hipStream_t>(hip_stream);
-    const Plan pl = make_plan(max_seq_k, batch, head_q, head_k, dim, dim_v, v != nullptr, total_k);
+    const bool tiles_contiguous = !pg.table || pg.page_size % 32 == 0;
+    const Plan pl = make_plan(max_seq_k, batch, head_q, head_k, dim, dim_v, v != nullptr, total_k, tiles_contiguous);
     if ((size_t)head_k * pl.groups > 65535)
         return fail(DA_ERR_INVALID_ARGUMENT, "head_k * groups exceeds the grid limit 65535");
 
@@ -280,6 +304,13 @@ int da_decoding_attn_ex(const void* q, const void* k, const void* v, void* o, co
     const float scale = softmax_scale > 0.0f ? softmax_scale : (float)(1.0 / std::sqrt((double)dim));
     sp.scale_log2 = scale * da::kLog2e;
     sp.is_alibi = is_alibi ? 1 : 0;
+    sp.block_table = pg.table;
+    sp.seq_lens = pg.seq_lens;
+    sp.page_shift = 0;
+    while (pg.table && ((size_t)1 << sp.page_shift) < pg.page_size) ++sp.page_shift;
+    sp.max_blocks = (int)pg.max_blocks;
+    sp.k_page = (int64_t)pg.k_page;
+    sp.v_page = v ? (int64_t)pg.v_page : (int64_t)pg.k_page;
 
     const dim3 grid((unsigned)pl.nsplit, (unsigned)((pl.wave_per_head ? head_k / 4 : head_k) * pl.groups),
                     (unsigned)batch);
@@ -303,6 +334,7 @@ int da_decoding_attn_ex(const void* q, const void* k, const void* v, void* o, co
         da::ReduceParams rp;
         rp.o = o;
         rp.cu_seq_k = cu_seq_k;
+        rp.seq_lens = pg.seq_lens;
         rp.ws_o = sp.ws_o;
         rp.ws_ml = sp.ws_ml;
         rp.head_q = (int)head_q;
@@ -313,6 +345,52 @@ int da_decoding_attn_ex(const void* q, const void* k, const void* v, void* o, co
         if (e != hipSuccess) return fail(DA_ERR_HIP, "merge kernel launch: %s", hipGetErrorString(e));
     }
     return DA_OK;
+}
+
+}  // namespace
+
+extern "C" {
+
+int da_decoding_attn_ex(const void* q, const void* k, const void* v, void* o, const int32_t* cu_seq_k,
+                        size_t max_seq_k, size_t batch, size_t head_q, size_t head_k, size_t dim, size_t dim_v,
+                        int is_alibi, int is_bf16, float softmax_scale, const float* alibi_slopes, size_t total_k,
+                        void* workspace, size_t workspace_bytes, void* hip_stream) {
+    return run_attention(q, k, v, o, cu_seq_k, Paging{}, max_seq_k, batch, head_q, head_k, dim, dim_v, is_alibi,
+                         is_bf16, softmax_scale, alibi_slopes, total_k, workspace, workspace_bytes, hip_stream);
+}
+
+int da_decoding_attn_paged(const void* q, const void* k_pages, const void* v_pages, void* o,
+                           const int32_t* block_table, const int32_t* seq_lens, size_t max_seq_k, size_t batch,
+                           size_t head_q, size_t head_k, size_t dim, size_t dim_v, size_t page_size,
+                           size_t max_blocks_per_seq, size_t k_page_stride, size_t v_page_stride, int is_alibi,
+                           int is_bf16, float softmax_scale, const float* alibi_slopes, size_t total_k,
+                           void* workspace, size_t workspace_bytes, void* hip_stream) {
+    if (!block_table) return fail(DA_ERR_INVALID_ARGUMENT, "block_table is null");
+    if (!seq_lens) return fail(DA_ERR_INVALID_ARGUMENT, "seq_lens is null");
+    if (page_size == 0 || (page_size & (page_size - 1)) != 0 || page_size > ((size_t)1 << 20))
+        return fail(DA_ERR_INVALID_ARGUMENT, "page_size (%zu) must be a power of two", page_size);
+    if (max_blocks_per_seq * page_size < max_seq_k)
+        return fail(DA_ERR_INVALID_ARGUMENT, "block table rows (%zu pages of %zu tokens) cannot hold max_seq_k %zu",
+                    max_blocks_per_seq, page_size, max_seq_k);
+    if (max_blocks_per_seq > (size_t)INT32_MAX)
+        return fail(DA_ERR_INVALID_ARGUMENT, "max_blocks_per_seq (%zu) out of range", max_blocks_per_seq);
+    if (k_page_stride < page_size * head_k * dim || k_page_stride % 8 != 0)
+        return fail(DA_ERR_INVALID_ARGUMENT,
+                    "k_page_stride (%zu elements) must be a multiple of 8 and at least page_size * head_k * dim",
+                    k_page_stride);
+    if (v_pages && (v_page_stride < page_size * head_k * dim_v || v_page_stride % 8 != 0))
+        return fail(DA_ERR_INVALID_ARGUMENT,
+                    "v_page_stride (%zu elements) must be a multiple of 8 and at least page_size * head_k * dim_v",
+                    v_page_stride);
+    Paging pg;
+    pg.table = block_table;
+    pg.seq_lens = seq_lens;
+    pg.page_size = page_size;
+    pg.max_blocks = max_blocks_per_seq;
+    pg.k_page = k_page_stride;
+    pg.v_page = v_page_stride;
+    return run_attention(q, k_pages, v_pages, o, nullptr, pg, max_seq_k, batch, head_q, head_k, dim, dim_v, is_alibi,
+                         is_bf16, softmax_scale, alibi_slopes, total_k, workspace, workspace_bytes, hip_stream);
 }
 
 int da_decoding_attn(const void* q, const void* k, const void* v, void* o, const int32_t* cu_seq_k, size_t max_seq_k,

@@ -106,15 +106,57 @@ struct SweepParams {
     int nsplit, chunk;        // sequence splits and tokens per split
     float scale_log2;         // softmax scale * log2(e)
     int is_alibi;
+    // Paged K/V (block_table != null): k and v are page pools [pages, page_size, head_k, dim(_v)], token j of
+    // sequence b is row j % page_size of page block_table[b, j / page_size]; cu_seq_k is null and seq_lens
+    // gives the lengths.  page_size is a power of two.
+    const int32_t* block_table;  // [batch, max_blocks]
+    const int32_t* seq_lens;     // [batch]
+    int page_shift, max_blocks;
+    int64_t k_page, v_page;      // elements between consecutive pages of K and of V
 };
 
 struct ReduceParams {
     void* o;
     const int32_t* cu_seq_k;
+    const int32_t* seq_lens;  // lengths when cu_seq_k is null (paged K/V)
     const float* ws_o;
     const float* ws_ml;
     int head_q, dim_v, nsplit, chunk;
 };
+
+// First token (row of the packed K/V buffers) and length of sequence b; paged sequences start at row 0 of their
+// own pages.
+__device__ __forceinline__ void seq_range(const SweepParams& p, int b, int& start, int& len) {
+    if (p.block_table) {
+        start = 0;
+        len = p.seq_lens[b];
+    } else {
+        start = p.cu_seq_k[b];
+        len = p.cu_seq_k[b + 1] - start;
+    }
+}
+
+// Element offsets (head 0, column 0) of token j of sequence b in the K and V buffers.  The lookup comes in two
+// steps so that a kernel can fetch the page id early and do the arithmetic when it needs the address.
+struct RowRef {
+    int64_t k, v;
+};
+__device__ __forceinline__ int page_of(const SweepParams& p, int b, int j) {
+    if (p.block_table == nullptr) return 0;
+    // The table is read through the constant address space: nothing writes it while the kernel runs, and that
+    // lets a wave-uniform lookup become a scalar load even after assembly statements that clobber memory.
+    typedef const int32_t __attribute__((address_space(4))) * const_i32;
+    const const_i32 table = (const_i32)(uintptr_t)p.block_table;
+    return table[(int64_t)b * p.max_blocks + (j >> p.page_shift)];
+}
+__device__ __forceinline__ RowRef row_in_page(const SweepParams& p, int start, int j, int page) {
+    if (p.block_table == nullptr) return {(int64_t)(start + j) * p.k_row, (int64_t)(start + j) * p.v_row};
+    const int r = j & ((1 << p.page_shift) - 1);
+    return {(int64_t)page * p.k_page + (int64_t)r * p.k_row, (int64_t)page * p.v_page + (int64_t)r * p.v_row};
+}
+__device__ __forceinline__ RowRef row_ref(const SweepParams& p, int b, int start, int j) {
+    return row_in_page(p, start, j, page_of(p, b, j));
+}
 
 // An empty sequence still owns output rows: when the sequence is not split, its work-group stores zeros for
 // its heads (n_ranges runs of nheads consecutive heads, range_stride apart); otherwise the merge kernel does.

@@ -107,8 +107,8 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(MINW))) voi
     const int b = blockIdx.z;
     const int tw = WH ? 0 : wave;  // this wave's position among the waves that share the tokens
 
-    const int start = p.cu_seq_k[b];
-    const int len = p.cu_seq_k[b + 1] - start;
+    int start, len;
+    seq_range(p, b, start, len);
     const int c0 = split * p.chunk;
     const int c1 = (split == p.nsplit - 1) ? len : min(len, c0 + p.chunk);
 
@@ -148,10 +148,10 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(MINW))) voi
     }
 
     // wave-uniform byte bases (scalar registers) and 32-bit per-lane byte offsets
-    const uint8_t* const kbytes =
-        reinterpret_cast<const uint8_t*>(p.k) + ((size_t)start * p.k_row + (size_t)hk * D) * 2;
-    const uint8_t* const vbytes =
-        reinterpret_cast<const uint8_t*>(p.v) + ((size_t)start * p.v_row + (size_t)hk * p.v_head) * 2;
+    // (a tile of kGqaTile tokens is contiguous: it starts at a multiple of kGqaTile within the sequence, and pages
+    // of paged K/V hold a multiple of kGqaTile tokens, so one row_ref per tile locates it)
+    const uint8_t* const kbytes = reinterpret_cast<const uint8_t*>(p.k) + (size_t)hk * D * 2;
+    const uint8_t* const vbytes = reinterpret_cast<const uint8_t*>(p.v) + (size_t)hk * p.v_head * 2;
     const uint32_t k_row_b = (uint32_t)p.k_row * 2, v_row_b = (uint32_t)p.v_row * 2;
 
     // wave-private V tile in LDS
@@ -171,7 +171,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(MINW))) voi
     TileRegs tr;
 
     auto load_k = [&](int tok0, TileRegs& r) __attribute__((always_inline)) {
-        const uint8_t* const base = kbytes + (size_t)tok0 * k_row_b;
+        const uint8_t* const base = kbytes + row_ref(p, b, start, tok0).k * 2;
         const int last = c1 - 1 - tok0;  // rows past the end re-read the last row and are masked
 #pragma unroll
         for (int mt = 0; mt < 2; ++mt) {
@@ -181,7 +181,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(MINW))) voi
         }
     };
     auto load_v = [&](int tok0, TileRegs& r) __attribute__((always_inline)) {
-        const uint8_t* const base = vbytes + (size_t)tok0 * v_row_b;
+        const uint8_t* const base = vbytes + row_ref(p, b, start, tok0).v * 2;
         const int last = c1 - 1 - tok0;
 #pragma unroll
         for (int i = 0; i < NVI; ++i) {

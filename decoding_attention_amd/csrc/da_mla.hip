@@ -185,8 +185,8 @@ __global__ __launch_bounds__(64 * NWV) void mfma_latent_kernel(const SweepParams
     const int hk = by / p.groups;
     const int grp = by % p.groups;
 
-    const int start = p.cu_seq_k[b];
-    const int len = p.cu_seq_k[b + 1] - start;
+    int start, len;
+    seq_range(p, b, start, len);
     const int c0 = split * p.chunk;
     const int c1 = (split == p.nsplit - 1) ? len : min(len, c0 + p.chunk);
 
@@ -247,15 +247,16 @@ __global__ __launch_bounds__(64 * NWV) void mfma_latent_kernel(const SweepParams
         for (int r = 0; r < 16; ++r) acc[c][r] = 0.0f;
     float m = kNegBig, l = 0.0f;
 
-    const uint8_t* const kbytes =
-        reinterpret_cast<const uint8_t*>(p.k) + ((size_t)start * p.k_row + (size_t)hk * D) * 2;
+    const uint8_t* const kbytes = reinterpret_cast<const uint8_t*>(p.k) + (size_t)hk * D * 2;
     const size_t k_row_bytes = (size_t)p.k_row * 2;
 
     // Stage the tile that starts at token tok0 into buffer `buf`.  Rows past the end of the split re-read the
     // last valid row (they are masked later).  Every wave always issues exactly NLW loads, so the hand-placed
     // vmcnt waits count the same on every wave.
-    auto issue_tile = [&](int tok0, int buf) {
-        const uint8_t* const base = kbytes + (size_t)tok0 * k_row_bytes;
+    // `row0` is the tile's first row as row_ref() gives it (a tile never straddles pages of paged K/V: pages hold
+    // a multiple of kTile tokens and tiles start at multiples of kTile).
+    auto issue_tile = [&](int tok0, int64_t row0, int buf) {
+        const uint8_t* const base = kbytes + row0 * 2;
         const int last = c1 - 1 - tok0;
 #pragma unroll
         for (int q = 0; q < NLA; ++q) {
@@ -274,8 +275,10 @@ __global__ __launch_bounds__(64 * NWV) void mfma_latent_kernel(const SweepParams
     };
 
     const int ntiles = (c1 - c0 + kTile - 1) / kTile;
-    issue_tile(c0, 0);
-    if (ntiles > 1) issue_tile(c0 + kTile, 1);
+    issue_tile(c0, row_ref(p, b, start, c0).k, 0);
+    if (ntiles > 1) issue_tile(c0 + kTile, row_ref(p, b, start, c0 + kTile).k, 1);
+    // page of the tile after those, fetched one trip ahead of its use (a scalar load for paged K/V)
+    int page_ahead = ntiles > 2 ? page_of(p, b, c0 + 2 * kTile) : 0;
     // Make the compiler settle its own wait for the Q loads here, before the loop.  It cannot see the
     // direct-to-LDS loads, so a wait for Q placed inside the loop would count down to vmcnt(0) on every trip
     // and drain the tiles in flight.
@@ -305,7 +308,9 @@ __global__ __launch_bounds__(64 * NWV) void mfma_latent_kernel(const SweepParams
         else
             wait_vmcnt<0>();
         __syncthreads();  // every wave's share of tile t is in LDS, and every wave is done with tile t-1
-        if (t + 2 < ntiles) issue_tile(c0 + (t + 2) * kTile, buf_next);
+        if (t + 2 < ntiles)
+            issue_tile(c0 + (t + 2) * kTile, row_in_page(p, start, c0 + (t + 2) * kTile, page_ahead).k, buf_next);
+        if (t + 3 < ntiles) page_ahead = page_of(p, b, c0 + (t + 3) * kTile);
 
         const int tok0 = c0 + t * kTile;
         // tile base addresses, made opaque so that the constant offsets below stay in the instructions'

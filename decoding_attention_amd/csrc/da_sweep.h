@@ -48,8 +48,8 @@ __global__ __launch_bounds__(256) void sweep_kernel(const SweepParams p) {
     const int grp = blockIdx.y % p.groups;
     const int b = blockIdx.z;
 
-    const int start = p.cu_seq_k[b];
-    const int len = p.cu_seq_k[b + 1] - start;
+    int start, len;
+    seq_range(p, b, start, len);
     const int c0 = split * p.chunk;
     const int c1 = (split == p.nsplit - 1) ? len : min(len, c0 + p.chunk);
 
@@ -84,26 +84,28 @@ __global__ __launch_bounds__(256) void sweep_kernel(const SweepParams p) {
         for (int e = 0; e < E; ++e) acc[r][e] = 0.0f;
     }
 
-    const uint16_t* kbase = reinterpret_cast<const uint16_t*>(p.k) + (size_t)start * p.k_row + (size_t)hk * D + g * 8;
-    const uint16_t* vbase =
-        reinterpret_cast<const uint16_t*>(p.v) + (size_t)start * p.v_row + (size_t)hk * p.v_head + g * 8;
+    // rows are addressed one by one (row_ref), so paged K/V of any page size costs one table lookup per row
+    const uint16_t* kbase = reinterpret_cast<const uint16_t*>(p.k) + (size_t)hk * D + g * 8;
+    const uint16_t* vbase = reinterpret_cast<const uint16_t*>(p.v) + (size_t)hk * p.v_head + g * 8;
 
     const int ntiles = (c1 - c0 + TILE - 1) / TILE;
     for (int t = wave; t < ntiles; t += NW) {
         const int base = c0 + t * TILE + slot;
         uint4 kreg[U][CPL];
         uint4 vreg[U][CPLV];
+        RowRef rr[U];
+#pragma unroll
+        for (int u = 0; u < U; ++u)  // rows past the end re-read the last row and are masked
+            rr[u] = row_ref(p, b, start, min(base + u * RPI, c1 - 1));
 #pragma unroll
         for (int u = 0; u < U; ++u) {
-            const int j = min(base + u * RPI, c1 - 1);  // rows past the end re-read the last row and are masked
-            const uint16_t* kr = kbase + (size_t)j * p.k_row;
+            const uint16_t* kr = kbase + rr[u].k;
 #pragma unroll
             for (int c = 0; c < CPL; ++c) kreg[u][c] = *reinterpret_cast<const uint4*>(kr + c * G * 8);
         }
 #pragma unroll
         for (int u = 0; u < U; ++u) {
-            const int j = min(base + u * RPI, c1 - 1);
-            const uint16_t* vr = vbase + (size_t)j * p.v_row;
+            const uint16_t* vr = vbase + rr[u].v;
 #pragma unroll
             for (int c = 0; c < CPLV; ++c) vreg[u][c] = *reinterpret_cast<const uint4*>(vr + c * G * 8);
         }
@@ -244,7 +246,7 @@ __global__ __launch_bounds__(256) void reduce_kernel(const ReduceParams p, int r
     const int c4 = gid - row * nc4;
     if (row >= rows) return;
     const int b = row / p.head_q;
-    const int len = p.cu_seq_k[b + 1] - p.cu_seq_k[b];
+    const int len = p.cu_seq_k ? p.cu_seq_k[b + 1] - p.cu_seq_k[b] : p.seq_lens[b];
     int ns = 0;
     if (len > 0) ns = min(p.nsplit, (len + p.chunk - 1) / p.chunk);
     const size_t part0 = (size_t)row * p.nsplit;

@@ -118,6 +118,105 @@ at::Tensor dmha_fwd(const at::Tensor &q, const at::Tensor &k, const std::optiona
     return o;
 }
 
+// Paged K/V: k_pages [pages, page_size, head_k, dim] and v_pages [pages, page_size, head_k, dim_v] (or none: the
+// values are the first dim_v columns of each K row), dense within a page, any stride between pages (so the two
+// halves of a combined [pages, 2, page_size, head_k, dim] pool can be passed as views).
+at::Tensor dmha_fwd_paged(const at::Tensor &q, const at::Tensor &k_pages, const std::optional<at::Tensor> &v_pages_,
+                          const std::optional<at::Tensor> &o_, const at::Tensor &block_table,
+                          const at::Tensor &seq_lens, const int64_t max_seq_k, const int64_t dim_v, const bool is_alibi,
+                          const std::optional<double> softmax_scale, const std::optional<at::Tensor> &alibi_slopes,
+                          const int64_t total_k) {
+    auto q_dtype = q.dtype();
+    TORCH_CHECK(q_dtype == torch::kFloat16 || q_dtype == torch::kBFloat16,
+                "Decoding-Attention only support FP16 and BF16 data type");
+    const bool is_bf16 = q_dtype == torch::kBFloat16;
+    TORCH_CHECK(k_pages.dtype() == q_dtype, "query and key must have the same dtype");
+    TORCH_CHECK(block_table.dtype() == torch::kInt32, "block_table must have dtype int32");
+    TORCH_CHECK(seq_lens.dtype() == torch::kInt32, "seq_lens must have dtype int32");
+    DA_CHECK_DEVICE(q);
+    DA_CHECK_DEVICE(k_pages);
+    DA_CHECK_DEVICE(block_table);
+    DA_CHECK_DEVICE(seq_lens);
+    TORCH_CHECK(k_pages.device() == q.device() && block_table.device() == q.device() && seq_lens.device() == q.device(),
+                "q, k_pages, block_table and seq_lens must share a device");
+    TORCH_CHECK(q.dim() == 3, "q must have three dimensions (batch, heads, dim)");
+    TORCH_CHECK(k_pages.dim() == 4, "k_pages must have four dimensions (pages, page_size, heads, dim)");
+    TORCH_CHECK(block_table.dim() == 2, "block_table must have two dimensions (batch, max_blocks)");
+    DA_CHECK_CONTIGUOUS(q);
+    DA_CHECK_CONTIGUOUS(block_table);
+    DA_CHECK_CONTIGUOUS(seq_lens);
+
+    const int64_t batch = q.size(0), head_q = q.size(1), dim = q.size(2);
+    const int64_t page_size = k_pages.size(1), head_k = k_pages.size(2);
+    TORCH_CHECK(batch > 0, "batch size must be positive");
+    TORCH_CHECK(k_pages.size(3) == dim, "k_pages must have q's head dim");
+    TORCH_CHECK(head_q % head_k == 0, "number of heads in key/value must divide number of heads in query");
+    DA_CHECK_SHAPE(seq_lens, batch);
+    TORCH_CHECK(block_table.size(0) == batch, "block_table must have one row per sequence");
+    TORCH_CHECK(da_supported_head_dims((size_t)dim, (size_t)dim_v) == 1, "unsupported head dims (dim ", dim,
+                ", dim_v ", dim_v, "): supported are (64,64) (96,96) (128,128) (256,256) (576,512)");
+    auto page_dense = [](const at::Tensor &t) {
+        return t.stride(3) == 1 && t.stride(2) == t.size(3) && t.stride(1) == t.size(2) * t.size(3);
+    };
+    TORCH_CHECK(page_dense(k_pages), "k_pages must be dense within a page");
+
+    const void *v_ptr = nullptr;
+    int64_t v_stride = 0;
+    if (v_pages_.has_value()) {
+        const at::Tensor &v = v_pages_.value();
+        TORCH_CHECK(v.dtype() == q_dtype, "query and value must have the same dtype");
+        DA_CHECK_DEVICE(v);
+        TORCH_CHECK(v.device() == q.device(), "v_pages must be on q's device");
+        TORCH_CHECK(v.dim() == 4 && v.size(0) == k_pages.size(0) && v.size(1) == page_size && v.size(2) == head_k &&
+                        v.size(3) == dim_v,
+                    "v_pages must have shape (pages, page_size, head_k, dim_v)");
+        TORCH_CHECK(page_dense(v), "v_pages must be dense within a page");
+        v_ptr = v.data_ptr();
+        v_stride = v.stride(0);
+    } else {
+        TORCH_CHECK(dim_v <= dim, "without v the values are the first dim_v columns of k: dim_v must not exceed dim");
+    }
+
+    at::Tensor o;
+    if (o_.has_value()) {
+        o = o_.value();
+        TORCH_CHECK(o.dtype() == q_dtype, "Output must have the same dtype as inputs");
+        DA_CHECK_DEVICE(o);
+        TORCH_CHECK(o.device() == q.device(), "o must be on q's device");
+        DA_CHECK_SHAPE(o, batch, head_q, dim_v);
+        DA_CHECK_CONTIGUOUS(o);
+    } else {
+        o = torch::empty({batch, head_q, dim_v}, q.options());
+    }
+
+    const float *slopes_ptr = nullptr;
+    if (alibi_slopes.has_value()) {
+        const at::Tensor &s = alibi_slopes.value();
+        TORCH_CHECK(s.dtype() == torch::kFloat32 && s.is_cuda() && s.device() == q.device() && s.is_contiguous() &&
+                        s.numel() == head_q,
+                    "alibi_slopes must be a contiguous float32 GPU tensor of head_q values");
+        slopes_ptr = s.data_ptr<float>();
+    }
+
+    c10::hip::HIPGuardMasqueradingAsCUDA guard(q.device());
+    hipStream_t stream = c10::hip::getCurrentHIPStreamMasqueradingAsCUDA(q.device().index()).stream();
+
+    const size_t hint = total_k > 0 ? (size_t)total_k : 0;
+    const size_t ws_bytes = da_workspace_bytes_paged((size_t)max_seq_k, (size_t)batch, (size_t)head_q, (size_t)head_k,
+                                                     (size_t)dim, (size_t)dim_v, hint, (size_t)page_size);
+    at::Tensor ws;
+    if (ws_bytes > 0) ws = torch::empty({(int64_t)ws_bytes}, q.options().dtype(torch::kUInt8));
+
+    const int rc = da_decoding_attn_paged(
+        q.data_ptr(), k_pages.data_ptr(), v_ptr, o.data_ptr(), block_table.data_ptr<int32_t>(),
+        seq_lens.data_ptr<int32_t>(), (size_t)max_seq_k, (size_t)batch, (size_t)head_q, (size_t)head_k, (size_t)dim,
+        (size_t)dim_v, (size_t)page_size, (size_t)block_table.size(1), (size_t)k_pages.stride(0), (size_t)v_stride,
+        is_alibi ? 1 : 0, is_bf16 ? 1 : 0, softmax_scale.has_value() ? (float)softmax_scale.value() : 0.0f, slopes_ptr,
+        hint, ws_bytes > 0 ? ws.data_ptr() : nullptr, ws_bytes, (void *)stream);
+    TORCH_CHECK(rc == DA_OK, "decoding_attn (paged) failed (", rc, "): ", da_last_error());
+    return o;
+}
+
 }  // namespace
 
 PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
@@ -126,4 +225,9 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
           pybind11::arg("o_"), pybind11::arg("cu_seq_k"), pybind11::arg("max_seq_k"), pybind11::arg("dim_v"),
           pybind11::arg("is_alibi"), pybind11::arg("softmax_scale") = pybind11::none(),
           pybind11::arg("alibi_slopes") = pybind11::none());
+    m.def("fwd_paged", &dmha_fwd_paged, "Forward pass over a paged K/V cache", pybind11::arg("q"),
+          pybind11::arg("k_pages"), pybind11::arg("v_pages_"), pybind11::arg("o_"), pybind11::arg("block_table"),
+          pybind11::arg("seq_lens"), pybind11::arg("max_seq_k"), pybind11::arg("dim_v"), pybind11::arg("is_alibi"),
+          pybind11::arg("softmax_scale") = pybind11::none(), pybind11::arg("alibi_slopes") = pybind11::none(),
+          pybind11::arg("total_k") = 0);
 }

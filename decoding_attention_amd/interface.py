@@ -67,3 +67,30 @@ def decoding_attn_fwd(q: torch.Tensor, k: torch.Tensor, v: Optional[torch.Tensor
     q, k, v = [maybe_contiguous(x) for x in (q, k, v)]
     return fwd(q, k, v, None, cu_seq_k, max_seq_k, dim_v, is_alibi, softmax_scale=softmax_scale,
                alibi_slopes=alibi_slopes)
+
+
+def decoding_attn_paged_fwd(q: torch.Tensor, k_pages: torch.Tensor, v_pages: Optional[torch.Tensor],
+                            block_table: torch.Tensor, seq_lens: torch.Tensor, max_seq_k: int, dim_v: int,
+                            is_alibi: bool, *, softmax_scale: Optional[float] = None,
+                            alibi_slopes: Optional[torch.Tensor] = None, total_k: int = 0,
+                            out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """
+    The same attention over a paged K/V cache (no counterpart in the reference; the layouts are those of the
+    libraries its benchmark compares against, reference benchmarks/python/benchmark_decoding_attn.py:129-151,182-187).
+
+    Arguments:
+        q: [batch, head_q, dim], torch.float16 / torch.bfloat16; one query token per sequence.
+        k_pages: [pages, page_size, head_k, dim] page pool, dense within a page (any stride between pages).
+        v_pages: [pages, page_size, head_k, dim_v] or None for MLA (values are k_pages[..., :dim_v]).
+        block_table: [batch, max_blocks], torch.int32 page ids of each sequence in token order.
+        seq_lens: [batch], torch.int32 key tokens of each sequence.
+        max_seq_k: upper bound of seq_lens (a host integer: nothing here synchronises with the device).
+        page_size (from k_pages.shape[1]) must be a power of two.
+        total_k (keyword only): sum of seq_lens if the host knows it; only a hint for sizing sequence splits.
+    Return:
+        o: [batch, head_q, dim_v], same dtype as q.
+    """
+    q = maybe_contiguous(q)
+    return _extension().fwd_paged(q, k_pages, v_pages, out, block_table, seq_lens, int(max_seq_k), int(dim_v),
+                                  bool(is_alibi), None if softmax_scale is None else float(softmax_scale),
+                                  alibi_slopes, int(total_k))

@@ -86,6 +86,64 @@ def make_workload(batch, head_q, head_k, dim, dim_v, seq_k, dtype, *, seed=0, va
 
 
 # The five benchmark configurations (fixed shapes; sweeps take the swept value as an argument).
+@dataclass
+class PagedKV:
+    """A packed workload's K/V scattered into page pools (see `to_pages`)."""
+    k_pages: torch.Tensor               # [pages, page_size, head_k, dim] (a view of `pool` when combined)
+    v_pages: Optional[torch.Tensor]     # [pages, page_size, head_k, dim_v] or None (latent form)
+    block_table: torch.Tensor           # int32 [batch, max_blocks]
+    seq_lens: torch.Tensor              # int32 [batch]
+    page_size: int
+    pool: Optional[torch.Tensor] = None  # [pages, 2, page_size, head_k, dim] when combined
+
+    def to(self, device):
+        if self.pool is not None:
+            pool = self.pool.to(device)
+            return PagedKV(pool[:, 0], pool[:, 1], self.block_table.to(device), self.seq_lens.to(device),
+                           self.page_size, pool)
+        return PagedKV(self.k_pages.to(device), None if self.v_pages is None else self.v_pages.to(device),
+                       self.block_table.to(device), self.seq_lens.to(device), self.page_size)
+
+
+def to_pages(w: Workload, page_size: int, *, seed=0, combined=False, spare_pages=3) -> PagedKV:
+    """Scatter the packed K/V of `w` into page pools with shuffled page ids.
+
+    Unused pages, the unused tail of each sequence's last page and unused block-table entries are poisoned (NaN
+    rows, page id -1 replaced by an out-of-sequence valid id) so that a kernel that reads past a sequence's end
+    shows up in the output.  combined=True builds one [pages, 2, page_size, head_k, dim] pool (K and V interleaved
+    per page, dim == dim_v) and returns its two halves as views.
+    """
+    g = torch.Generator(device="cpu").manual_seed(seed)
+    lens = w.lengths
+    blocks = [(n + page_size - 1) // page_size for n in lens]
+    max_blocks = max(1, max(blocks))
+    n_pages = sum(blocks) + spare_pages
+    order = torch.randperm(n_pages, generator=g).tolist()
+    nan = float("nan")
+    if combined:
+        assert w.v is not None and w.dim == w.dim_v
+        pool = torch.full((n_pages, 2, page_size, w.head_k, w.dim), nan, dtype=w.k.dtype)
+        k_pages, v_pages = pool[:, 0], pool[:, 1]
+    else:
+        pool = None
+        k_pages = torch.full((n_pages, page_size, w.head_k, w.dim), nan, dtype=w.k.dtype)
+        v_pages = None if w.v is None else torch.full((n_pages, page_size, w.head_k, w.dim_v), nan, dtype=w.k.dtype)
+    # unused table entries point at a spare (all-NaN) page
+    table = torch.full((w.batch, max_blocks), order[-1], dtype=torch.int32)
+    cu = w.cu_seq_k.tolist()
+    nxt = 0
+    for b, n in enumerate(lens):
+        for i in range(blocks[b]):
+            page = order[nxt]
+            nxt += 1
+            table[b, i] = page
+            lo, hi = cu[b] + i * page_size, min(cu[b] + (i + 1) * page_size, cu[b] + n)
+            k_pages[page, :hi - lo] = w.k[lo:hi]
+            if v_pages is not None:
+                v_pages[page, :hi - lo] = w.v[lo:hi]
+    return PagedKV(k_pages, v_pages, table, torch.tensor(lens, dtype=torch.int32), page_size, pool)
+
+
 def config_mha_cpu_case(seed=0):
     return make_workload(1, 32, 32, 128, 128, 128, torch.float16, seed=seed, name="C0_mha_fp16_b1_sk128")
 

@@ -69,6 +69,33 @@ size_t da_workspace_bytes(size_t max_seq_k, size_t batch, size_t head_q, size_t 
                           size_t total_k);
 
 /*
+ * The same attention over a paged K/V cache: K and V live in page pools and each sequence lists its pages.
+ * The reference has no paged path of its own; these are the layouts of the libraries it is benchmarked against
+ * (benchmarks/python/benchmark_decoding_attn.py:129-151: a [pages, 2, page_size, head_k, dim] pool with one index
+ * array per batch; :182-187: a [blocks, 64, 1, 576] latent pool with a [batch, max_blocks] block table).
+ *
+ *   k_pages        [num_pages, page_size, head_k, dim], consecutive pages k_page_stride elements apart
+ *   v_pages        [num_pages, page_size, head_k, dim_v], pages v_page_stride elements apart, or NULL when V is the
+ *                  first dim_v columns of each K row (MLA).  A combined [pages, 2, page_size, head_k, dim] pool is
+ *                  k_pages = pool, v_pages = pool + page_size * head_k * dim, both strides 2 * page_size * head_k * dim.
+ *   block_table    device, int32 [batch, max_blocks_per_seq]: page ids of each sequence in token order; entries
+ *                  past ceil(seq_lens[b] / page_size) are not read
+ *   seq_lens       device, int32 [batch]: key tokens of each sequence (0 gives zero output rows)
+ *   page_size      tokens per page, a power of two.  Multiples of 32 run on the same kernels as the packed layout;
+ *                  smaller pages are served by the VALU sweep with one table lookup per row.
+ * The remaining arguments are those of da_decoding_attn_ex; workspace size from da_workspace_bytes_paged.
+ */
+int da_decoding_attn_paged(const void *q, const void *k_pages, const void *v_pages, void *o,
+                           const int32_t *block_table, const int32_t *seq_lens, size_t max_seq_k, size_t batch,
+                           size_t head_q, size_t head_k, size_t dim, size_t dim_v, size_t page_size,
+                           size_t max_blocks_per_seq, size_t k_page_stride, size_t v_page_stride, int is_alibi,
+                           int is_bf16, float softmax_scale, const float *alibi_slopes, size_t total_k,
+                           void *workspace, size_t workspace_bytes, void *hip_stream);
+
+size_t da_workspace_bytes_paged(size_t max_seq_k, size_t batch, size_t head_q, size_t head_k, size_t dim,
+                                size_t dim_v, size_t total_k, size_t page_size);
+
+/*
  * Launch plan the library would use for this shape, for tests and benchmarks:
  *   kernel_kind 1 = VALU sweep, 2 = latent (MLA) MFMA sweep, 3 = grouped-head MFMA sweep; nsplit = sequence splits;
  *   chunk = tokens per split; heads_per_group = query heads one work-group serves; total_k as for
