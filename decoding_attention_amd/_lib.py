@@ -16,6 +16,9 @@ EXPORTED_SYMBOLS = (
     "da_workspace_bytes",
     "da_decoding_attn_paged",
     "da_workspace_bytes_paged",
+    "da_decoding_attn_fp8kv",
+    "da_decoding_attn_paged_fp8kv",
+    "da_workspace_bytes_fp8kv",
     "da_plan",
     "da_supported_head_dims",
     "da_last_error",
@@ -57,6 +60,14 @@ def load():
                                            vp, sz, vp, sz, vp]
     lib.da_workspace_bytes_paged.restype = sz
     lib.da_workspace_bytes_paged.argtypes = [sz, sz, sz, sz, sz, sz, sz, sz]
+    lib.da_decoding_attn_fp8kv.restype = ci
+    lib.da_decoding_attn_fp8kv.argtypes = [vp, vp, vp, vp, vp, sz, sz, sz, sz, sz, sz, ci, ci, cf, vp, vp, vp, sz, vp, sz,
+                                           vp]
+    lib.da_decoding_attn_paged_fp8kv.restype = ci
+    lib.da_decoding_attn_paged_fp8kv.argtypes = [vp, vp, vp, vp, vp, vp, sz, sz, sz, sz, sz, sz, sz, sz, sz, sz, ci, ci,
+                                                 cf, vp, vp, vp, sz, vp, sz, vp]
+    lib.da_workspace_bytes_fp8kv.restype = sz
+    lib.da_workspace_bytes_fp8kv.argtypes = [sz, sz, sz, sz, sz, sz, sz, sz]
     ip = ctypes.POINTER(ci)
     lib.da_plan.restype = ci
     lib.da_plan.argtypes = [sz, sz, sz, sz, sz, sz, ci, sz, ip, ip, ip, ip]

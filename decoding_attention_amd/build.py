@@ -21,6 +21,8 @@ SOURCES = [
     "da_sweep_d576.hip",
     "da_mla.hip",
     "da_gqa_mfma.hip",
+    "da_sweep_kv8.hip",
+    "da_gqa_mfma_kv8.hip",
 ]
 
 # packed-fp32 VALU forms are switched off on purpose: only scalar fp32 arithmetic is emitted.

@@ -95,20 +95,21 @@ int rows_per_trip(size_t dim) {
 // shorter splits so that the work-groups, whose number is sized for max_seq_k, balance.
 // tiles_contiguous: every aligned run of 32 tokens is contiguous in memory (always true for the packed layout; for
 // paged K/V only when a page holds a multiple of 32 tokens).  The two MFMA kernels fetch whole tiles and need it.
+// kv_fp8: K/V are FP8; the latent MFMA kernel has no FP8 form and the grouped kernel needs dim % 64 == 0.
 Plan make_plan(size_t max_seq_k, size_t batch, size_t head_q, size_t head_k, size_t dim, size_t dim_v,
-               bool v_distinct, size_t total_k, bool tiles_contiguous = true) {
+               bool v_distinct, size_t total_k, bool tiles_contiguous = true, bool kv_fp8 = false) {
     Plan pl;
     const int ratio = (int)(head_q / head_k);
     int trip;
     int target_wgs = tun().target_wgs;
     const bool force_sweep = tun().force_kind == kKindSweep || !tiles_contiguous;
-    const bool mfma = !v_distinct && da::mla_supported(dim, dim_v, ratio) && !force_sweep;
+    const bool mfma = !v_distinct && !kv_fp8 && da::mla_supported(dim, dim_v, ratio) && !force_sweep;
     if (mfma) {
         pl.kind = kKindMfma;
         pl.rt = da::mla_heads_per_group(ratio);
         trip = da::mla_rows_per_trip();
         target_wgs = tun().mfma_target_wgs;  // one 4-wave work-group fills a CU
-    } else if (dim <= 256 && ratio >= tun().group_min_ratio && !force_sweep) {
+    } else if (dim <= 256 && ratio >= tun().group_min_ratio && !force_sweep && (!kv_fp8 || dim % 64 == 0)) {
         pl.kind = kKindGroup;
         pl.rt = ratio > 16 ? 32 : 16;
         pl.wave_per_head = head_k % 4 == 0 && tun().wave_per_head;
@@ -224,6 +225,15 @@ size_t da_workspace_bytes_paged(size_t max_seq_k, size_t batch, size_t head_q, s
     return a > b ? a : b;
 }
 
+size_t da_workspace_bytes_fp8kv(size_t max_seq_k, size_t batch, size_t head_q, size_t head_k, size_t dim,
+                                size_t dim_v, size_t total_k, size_t page_size) {
+    if (head_k == 0 || head_q % head_k != 0 || !supported_dims(dim, dim_v)) return 0;
+    const bool contiguous = page_size == 0 || page_size % 32 == 0;
+    const size_t a = make_plan(max_seq_k, batch, head_q, head_k, dim, dim_v, false, total_k, contiguous, true).ws_bytes;
+    const size_t b = make_plan(max_seq_k, batch, head_q, head_k, dim, dim_v, true, total_k, contiguous, true).ws_bytes;
+    return a > b ? a : b;
+}
+
 }  // extern "C"
 
 namespace {
@@ -235,8 +245,15 @@ struct Paging {
     size_t page_size = 0, max_blocks = 0, k_page = 0, v_page = 0;
 };
 
+// Element format of K/V: 16-bit like Q, or FP8 (e4m3) with per-KV-head de-quantisation factors (null = 1).
+struct KvFormat {
+    bool fp8 = false;
+    const float* k_scale = nullptr;
+    const float* v_scale = nullptr;
+};
+
 int run_attention(const void* q, const void* k, const void* v, void* o, const int32_t* cu_seq_k, const Paging& pg,
-                  size_t max_seq_k, size_t batch, size_t head_q, size_t head_k, size_t dim, size_t dim_v,
+                  const KvFormat& kf, size_t max_seq_k, size_t batch, size_t head_q, size_t head_k, size_t dim, size_t dim_v,
                   int is_alibi, int is_bf16, float softmax_scale, const float* alibi_slopes, size_t total_k,
                   void* workspace, size_t workspace_bytes, void* hip_stream) {
     // the reference's checks (csrc/ops/decoding_attn.cpp:16-22) ...
@@ -264,7 +281,7 @@ int run_attention(const void* q, const void* k, const void* v, void* o, const in
 
     hipStream_t stream = reinterpret_cast<hipStream_t>(hip_stream);
     const bool tiles_contiguous = !pg.table || pg.page_size % 32 == 0;
-    const Plan pl = make_plan(max_seq_k, batch, head_q, head_k, dim, dim_v, v != nullptr, total_k, tiles_contiguous);
+    const Plan pl = make_plan(max_seq_k, batch, head_q, head_k, dim, dim_v, v != nullptr, total_k, tiles_contiguous, kf.fp8);
     if ((size_t)head_k * pl.groups > 65535)
         return fail(DA_ERR_INVALID_ARGUMENT, "head_k * groups exceeds the grid limit 65535");
 
@@ -304,6 +321,8 @@ int run_attention(const void* q, const void* k, const void* v, void* o, const in
     const float scale = softmax_scale > 0.0f ? softmax_scale : (float)(1.0 / std::sqrt((double)dim));
     sp.scale_log2 = scale * da::kLog2e;
     sp.is_alibi = is_alibi ? 1 : 0;
+    sp.k_scale = kf.k_scale;
+    sp.v_scale = kf.v_scale;
     sp.block_table = pg.table;
     sp.seq_lens = pg.seq_lens;
     sp.page_shift = 0;
@@ -315,7 +334,12 @@ int run_attention(const void* q, const void* k, const void* v, void* o, const in
     const dim3 grid((unsigned)pl.nsplit, (unsigned)((pl.wave_per_head ? head_k / 4 : head_k) * pl.groups),
                     (unsigned)batch);
     hipError_t e;
-    if (pl.kind == kKindMfma) {
+    if (kf.fp8) {
+        if (pl.kind == kKindGroup)
+            e = da::launch_gqa_mfma_kv8(sp, is_bf16 != 0, (int)dim, pl.rt, pl.wave_per_head, grid, stream);
+        else
+            e = da::launch_sweep_kv8(sp, is_bf16 != 0, (int)dim, pl.rt, grid, stream);
+    } else if (pl.kind == kKindMfma) {
         e = da::launch_mla(sp, is_bf16 != 0, pl.rt, grid, stream);
     } else if (pl.kind == kKindGroup) {
         e = da::launch_gqa_mfma(sp, is_bf16 != 0, (int)dim, pl.rt, pl.wave_per_head, grid, stream);
@@ -347,24 +371,9 @@ int run_attention(const void* q, const void* k, const void* v, void* o, const in
     return DA_OK;
 }
 
-}  // namespace
-
-extern "C" {
-
-int da_decoding_attn_ex(const void* q, const void* k, const void* v, void* o, const int32_t* cu_seq_k,
-                        size_t max_seq_k, size_t batch, size_t head_q, size_t head_k, size_t dim, size_t dim_v,
-                        int is_alibi, int is_bf16, float softmax_scale, const float* alibi_slopes, size_t total_k,
-                        void* workspace, size_t workspace_bytes, void* hip_stream) {
-    return run_attention(q, k, v, o, cu_seq_k, Paging{}, max_seq_k, batch, head_q, head_k, dim, dim_v, is_alibi,
-                         is_bf16, softmax_scale, alibi_slopes, total_k, workspace, workspace_bytes, hip_stream);
-}
-
-int da_decoding_attn_paged(const void* q, const void* k_pages, const void* v_pages, void* o,
-                           const int32_t* block_table, const int32_t* seq_lens, size_t max_seq_k, size_t batch,
-                           size_t head_q, size_t head_k, size_t dim, size_t dim_v, size_t page_size,
-                           size_t max_blocks_per_seq, size_t k_page_stride, size_t v_page_stride, int is_alibi,
-                           int is_bf16, float softmax_scale, const float* alibi_slopes, size_t total_k,
-                           void* workspace, size_t workspace_bytes, void* hip_stream) {
+int check_paging(const int32_t* block_table, const int32_t* seq_lens, size_t max_seq_k, size_t head_k, size_t dim,
+                 size_t dim_v, size_t page_size, size_t max_blocks_per_seq, size_t k_page_stride, size_t v_page_stride,
+                 bool has_v, Paging* pg) {
     if (!block_table) return fail(DA_ERR_INVALID_ARGUMENT, "block_table is null");
     if (!seq_lens) return fail(DA_ERR_INVALID_ARGUMENT, "seq_lens is null");
     if (page_size == 0 || (page_size & (page_size - 1)) != 0 || page_size > ((size_t)1 << 20))
@@ -374,23 +383,82 @@ int da_decoding_attn_paged(const void* q, const void* k_pages, const void* v_pag
                     max_blocks_per_seq, page_size, max_seq_k);
     if (max_blocks_per_seq > (size_t)INT32_MAX)
         return fail(DA_ERR_INVALID_ARGUMENT, "max_blocks_per_seq (%zu) out of range", max_blocks_per_seq);
-    if (k_page_stride < page_size * head_k * dim || k_page_stride % 8 != 0)
+    // a multiple of 16 elements keeps every row 16-byte aligned for 16-bit and for FP8 elements alike
+    if (k_page_stride < page_size * head_k * dim || k_page_stride % 16 != 0)
         return fail(DA_ERR_INVALID_ARGUMENT,
-                    "k_page_stride (%zu elements) must be a multiple of 8 and at least page_size * head_k * dim",
+                    "k_page_stride (%zu elements) must be a multiple of 16 and at least page_size * head_k * dim",
                     k_page_stride);
-    if (v_pages && (v_page_stride < page_size * head_k * dim_v || v_page_stride % 8 != 0))
+    if (has_v && (v_page_stride < page_size * head_k * dim_v || v_page_stride % 16 != 0))
         return fail(DA_ERR_INVALID_ARGUMENT,
-                    "v_page_stride (%zu elements) must be a multiple of 8 and at least page_size * head_k * dim_v",
+                    "v_page_stride (%zu elements) must be a multiple of 16 and at least page_size * head_k * dim_v",
                     v_page_stride);
-    Paging pg;
-    pg.table = block_table;
-    pg.seq_lens = seq_lens;
-    pg.page_size = page_size;
-    pg.max_blocks = max_blocks_per_seq;
-    pg.k_page = k_page_stride;
-    pg.v_page = v_page_stride;
-    return run_attention(q, k_pages, v_pages, o, nullptr, pg, max_seq_k, batch, head_q, head_k, dim, dim_v, is_alibi,
+    pg->table = block_table;
+    pg->seq_lens = seq_lens;
+    pg->page_size = page_size;
+    pg->max_blocks = max_blocks_per_seq;
+    pg->k_page = k_page_stride;
+    pg->v_page = v_page_stride;
+    return DA_OK;
+}
+
+}  // namespace
+
+extern "C" {
+
+int da_decoding_attn_ex(const void* q, const void* k, const void* v, void* o, const int32_t* cu_seq_k,
+                        size_t max_seq_k, size_t batch, size_t head_q, size_t head_k, size_t dim, size_t dim_v,
+                        int is_alibi, int is_bf16, float softmax_scale, const float* alibi_slopes, size_t total_k,
+                        void* workspace, size_t workspace_bytes, void* hip_stream) {
+    return run_attention(q, k, v, o, cu_seq_k, Paging{}, KvFormat{}, max_seq_k, batch, head_q, head_k, dim, dim_v, is_alibi,
                          is_bf16, softmax_scale, alibi_slopes, total_k, workspace, workspace_bytes, hip_stream);
+}
+
+int da_decoding_attn_paged(const void* q, const void* k_pages, const void* v_pages, void* o,
+                           const int32_t* block_table, const int32_t* seq_lens, size_t max_seq_k, size_t batch,
+                           size_t head_q, size_t head_k, size_t dim, size_t dim_v, size_t page_size,
+                           size_t max_blocks_per_seq, size_t k_page_stride, size_t v_page_stride, int is_alibi,
+                           int is_bf16, float softmax_scale, const float* alibi_slopes, size_t total_k,
+                           void* workspace, size_t workspace_bytes, void* hip_stream) {
+    Paging pg;
+    const int rc = check_paging(block_table, seq_lens, max_seq_k, head_k, dim, dim_v, page_size, max_blocks_per_seq,
+                                k_page_stride, v_page_stride, v_pages != nullptr, &pg);
+    if (rc != DA_OK) return rc;
+    return run_attention(q, k_pages, v_pages, o, nullptr, pg, KvFormat{}, max_seq_k, batch, head_q, head_k, dim, dim_v,
+                         is_alibi, is_bf16, softmax_scale, alibi_slopes, total_k, workspace, workspace_bytes,
+                         hip_stream);
+}
+
+int da_decoding_attn_fp8kv(const void* q, const void* k8, const void* v8, void* o, const int32_t* cu_seq_k,
+                           size_t max_seq_k, size_t batch, size_t head_q, size_t head_k, size_t dim, size_t dim_v,
+                           int is_alibi, int is_bf16, float softmax_scale, const float* alibi_slopes,
+                           const float* k_scale, const float* v_scale, size_t total_k, void* workspace,
+                           size_t workspace_bytes, void* hip_stream) {
+    KvFormat kf;
+    kf.fp8 = true;
+    kf.k_scale = k_scale;
+    kf.v_scale = v_scale;
+    return run_attention(q, k8, v8, o, cu_seq_k, Paging{}, kf, max_seq_k, batch, head_q, head_k, dim, dim_v, is_alibi,
+                         is_bf16, softmax_scale, alibi_slopes, total_k, workspace, workspace_bytes, hip_stream);
+}
+
+int da_decoding_attn_paged_fp8kv(const void* q, const void* k_pages, const void* v_pages, void* o,
+                                 const int32_t* block_table, const int32_t* seq_lens, size_t max_seq_k, size_t batch,
+                                 size_t head_q, size_t head_k, size_t dim, size_t dim_v, size_t page_size,
+                                 size_t max_blocks_per_seq, size_t k_page_stride, size_t v_page_stride, int is_alibi,
+                                 int is_bf16, float softmax_scale, const float* alibi_slopes, const float* k_scale,
+                                 const float* v_scale, size_t total_k, void* workspace, size_t workspace_bytes,
+                                 void* hip_stream) {
+    Paging pg;
+    const int rc = check_paging(block_table, seq_lens, max_seq_k, head_k, dim, dim_v, page_size, max_blocks_per_seq,
+                                k_page_stride, v_page_stride, v_pages != nullptr, &pg);
+    if (rc != DA_OK) return rc;
+    KvFormat kf;
+    kf.fp8 = true;
+    kf.k_scale = k_scale;
+    kf.v_scale = v_scale;
+    return run_attention(q, k_pages, v_pages, o, nullptr, pg, kf, max_seq_k, batch, head_q, head_k, dim, dim_v,
+                         is_alibi, is_bf16, softmax_scale, alibi_slopes, total_k, workspace, workspace_bytes,
+                         hip_stream);
 }
 
 int da_decoding_attn(const void* q, const void* k, const void* v, void* o, const int32_t* cu_seq_k, size_t max_seq_k,

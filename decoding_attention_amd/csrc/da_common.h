@@ -59,6 +59,25 @@ struct Elem<bf16_tag> {
 
 __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
 
+// Eight FP8 (OCP e4m3) values -> eight 16-bit elements of the compute type.  Both conversions are exact (e4m3
+// has 3 mantissa bits and |x| <= 448), so an FP8 K/V cache feeds the same arithmetic as a 16-bit one.
+template <typename Tag>
+__device__ __forceinline__ uint4 fp8x8_to_16(uint2 w) {
+    uint4 r;
+    if constexpr (std::is_same<Tag, f16_tag>::value) {
+        r.x = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_f16_fp8((int)w.x, 1.0f, false));
+        r.y = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_f16_fp8((int)w.x, 1.0f, true));
+        r.z = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_f16_fp8((int)w.y, 1.0f, false));
+        r.w = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_f16_fp8((int)w.y, 1.0f, true));
+    } else {
+        r.x = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8((int)w.x, 1.0f, false));
+        r.y = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8((int)w.x, 1.0f, true));
+        r.z = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8((int)w.y, 1.0f, false));
+        r.w = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8((int)w.y, 1.0f, true));
+    }
+    return r;
+}
+
 // f(integral_constant<int, B>), ..., f(integral_constant<int, E-1>): a loop whose index is a constant
 // expression in the body (needed for instruction offset fields and wait counts in inline assembly).
 template <int B, int E, typename F>
@@ -113,7 +132,13 @@ struct SweepParams {
     const int32_t* seq_lens;     // [batch]
     int page_shift, max_blocks;
     int64_t k_page, v_page;      // elements between consecutive pages of K and of V
+    // De-quantisation factors of an FP8 K/V cache, one per KV head (null = 1): K = k_scale[hk] * fp8 value.
+    // The kernels fold k_scale into the softmax scale and v_scale into the final normalisation.
+    const float* k_scale;
+    const float* v_scale;
 };
+
+__device__ __forceinline__ float head_scale(const float* scales, int hk) { return scales ? scales[hk] : 1.0f; }
 
 struct ReduceParams {
     void* o;

@@ -79,7 +79,10 @@ constexpr size_t gqa_lds_bytes(int nt) {
 // Otherwise (head_k not a multiple of 4) the wavefronts split the tokens of one KV head and merge at the end.
 // MINW: wavefronts per SIMD the register allocation must leave room for (2 caps the kernel at 256 registers
 // and keeps the accumulators in ordinary VGPRs, so the rescale needs no accumulation-register copies).
-template <typename Tag, int D, int DV, int NT, bool PREFETCH, bool WH, int MINW>
+// KV8: K and V hold FP8 (e4m3) elements.  Loads stay 16 bytes per lane (sixteen elements: the k indices of two
+// consecutive k-steps, so the Q fragments are gathered with the matching index order) and the elements are
+// converted exactly to the compute type on their way into the matrix instruction (K) or the LDS tile (V).
+template <typename Tag, int D, int DV, int NT, bool PREFETCH, bool WH, int MINW, bool KV8 = false>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(MINW))) void gqa_mfma_kernel(const SweepParams p) {
     using MM = Mma16<Tag>;
     using vec8 = typename MM::vec8;
@@ -92,7 +95,12 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(MINW))) voi
     constexpr int NW = WH ? 1 : 4;  // wavefronts that share the tokens of one KV head
     constexpr int HG = 16 * NT;     // query heads per KV head and work-group
     constexpr float kLazy = 8.0f;   // the running maximum moves only when exceeded by this much (log2 units)
+    constexpr int KB = KV8 ? 1 : 2;                 // bytes per K/V element
+    constexpr int KSR = KV8 ? KS / 2 : KS;          // K registers (16 bytes) per 16-token tile
+    constexpr int CPRL = KV8 ? DV / 16 : CPR;       // 16-byte chunks per V row as loaded
+    constexpr int NVR = kGqaTile * CPRL / 64;       // V registers (16 bytes) per tile
     static_assert(D % 32 == 0 && DV % 16 == 0 && (kGqaTile * CPR) % 64 == 0, "shape");
+    static_assert(!KV8 || (D % 64 == 0 && (kGqaTile * CPRL) % 64 == 0), "FP8 K/V: two k-steps per 16-byte load");
 
     extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
 
@@ -131,9 +139,13 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(MINW))) voi
 #pragma unroll
     for (int nt = 0; nt < NT; ++nt) {
         const int h = h_base + min(nt * 16 + n, nh - 1);
-        const uint16_t* qrow = reinterpret_cast<const uint16_t*>(p.q) + ((size_t)b * p.head_q + h) * D + g * 8;
+        const uint16_t* qrow = reinterpret_cast<const uint16_t*>(p.q) + ((size_t)b * p.head_q + h) * D;
 #pragma unroll
-        for (int ks = 0; ks < KS; ++ks) qf[nt][ks] = __builtin_bit_cast(vec8, *reinterpret_cast<const uint4*>(qrow + ks * 32));
+        for (int ks = 0; ks < KS; ++ks) {
+            // k indices this lane contributes to k-step ks: those of the K fragment it will hold
+            const int at = KV8 ? (ks >> 1) * 64 + g * 16 + (ks & 1) * 8 : ks * 32 + g * 8;
+            qf[nt][ks] = __builtin_bit_cast(vec8, *reinterpret_cast<const uint4*>(qrow + at));
+        }
         slope[nt] = p.is_alibi ? alibi_slope_log2(p.slopes, h, p.head_q) : 0.0f;
     }
 
@@ -150,9 +162,11 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(MINW))) voi
     // wave-uniform byte bases (scalar registers) and 32-bit per-lane byte offsets
     // (a tile of kGqaTile tokens is contiguous: it starts at a multiple of kGqaTile within the sequence, and pages
     // of paged K/V hold a multiple of kGqaTile tokens, so one row_ref per tile locates it)
-    const uint8_t* const kbytes = reinterpret_cast<const uint8_t*>(p.k) + (size_t)hk * D * 2;
-    const uint8_t* const vbytes = reinterpret_cast<const uint8_t*>(p.v) + (size_t)hk * p.v_head * 2;
-    const uint32_t k_row_b = (uint32_t)p.k_row * 2, v_row_b = (uint32_t)p.v_row * 2;
+    const uint8_t* const kbytes = reinterpret_cast<const uint8_t*>(p.k) + (size_t)hk * D * KB;
+    const uint8_t* const vbytes = reinterpret_cast<const uint8_t*>(p.v) + (size_t)hk * p.v_head * KB;
+    const uint32_t k_row_b = (uint32_t)p.k_row * KB, v_row_b = (uint32_t)p.v_row * KB;
+    const float sl = p.scale_log2 * head_scale(p.k_scale, hk);  // score scale, log2 units
+    const float vs = head_scale(p.v_scale, hk);
 
     // wave-private V tile in LDS
     uint8_t* const vt = smem + wave * (kGqaTile * VP);
@@ -165,28 +179,28 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(MINW))) voi
     // (V once it is parked in LDS, K once the score MFMAs have read it), so they fly during the rest of the
     // tile's work without doubling the register footprint.
     struct TileRegs {
-        uint4 k[2][KS];
-        uint4 v[NVI];
+        uint4 k[2][KSR];
+        uint4 v[NVR];
     };
     TileRegs tr;
 
     auto load_k = [&](int tok0, TileRegs& r) __attribute__((always_inline)) {
-        const uint8_t* const base = kbytes + row_ref(p, b, start, tok0).k * 2;
+        const uint8_t* const base = kbytes + row_ref(p, b, start, tok0).k * KB;
         const int last = c1 - 1 - tok0;  // rows past the end re-read the last row and are masked
 #pragma unroll
         for (int mt = 0; mt < 2; ++mt) {
             const uint32_t off = (uint32_t)min(mt * 16 + n, last) * k_row_b + g * 16;
 #pragma unroll
-            for (int ks = 0; ks < KS; ++ks) r.k[mt][ks] = *reinterpret_cast<const uint4*>(base + off + ks * 64);
+            for (int ks = 0; ks < KSR; ++ks) r.k[mt][ks] = *reinterpret_cast<const uint4*>(base + off + ks * 64);
         }
     };
     auto load_v = [&](int tok0, TileRegs& r) __attribute__((always_inline)) {
-        const uint8_t* const base = vbytes + row_ref(p, b, start, tok0).v * 2;
+        const uint8_t* const base = vbytes + row_ref(p, b, start, tok0).v * KB;
         const int last = c1 - 1 - tok0;
 #pragma unroll
-        for (int i = 0; i < NVI; ++i) {
+        for (int i = 0; i < NVR; ++i) {
             const int slot = i * 64 + lane;
-            const int row = slot / CPR, ch = slot % CPR;
+            const int row = slot / CPRL, ch = slot % CPRL;
             const uint32_t off = (uint32_t)min(row, last) * v_row_b + ch * 16;
             r.v[i] = *reinterpret_cast<const uint4*>(base + off);
         }
@@ -205,10 +219,16 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(MINW))) voi
 
         // park V in LDS (row-major, padded pitch), then refill the V registers
 #pragma unroll
-        for (int i = 0; i < NVI; ++i) {
+        for (int i = 0; i < NVR; ++i) {
             const int slot = i * 64 + lane;
-            const int row = slot / CPR, ch = slot % CPR;
-            *reinterpret_cast<uint4*>(vt + row * VP + ch * 16) = tr.v[i];
+            const int row = slot / CPRL, ch = slot % CPRL;
+            if constexpr (KV8) {  // sixteen FP8 elements become 32 bytes of the 16-bit tile
+                *reinterpret_cast<uint4*>(vt + row * VP + ch * 32) = fp8x8_to_16<Tag>(make_uint2(tr.v[i].x, tr.v[i].y));
+                *reinterpret_cast<uint4*>(vt + row * VP + ch * 32 + 16) =
+                    fp8x8_to_16<Tag>(make_uint2(tr.v[i].z, tr.v[i].w));
+            } else {
+                *reinterpret_cast<uint4*>(vt + row * VP + ch * 16) = tr.v[i];
+            }
         }
         if (PREFETCH && more) load_v(tok_next, tr);
 
@@ -220,7 +240,16 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(MINW))) voi
             for (int nt = 0; nt < NT; ++nt) {
                 f32x4 c = {0.0f, 0.0f, 0.0f, 0.0f};
 #pragma unroll
-                for (int ks = 0; ks < KS; ++ks) c = MM::mma(__builtin_bit_cast(vec8, tr.k[mt][ks]), qf[nt][ks], c);
+                for (int ks = 0; ks < KS; ++ks) {
+                    uint4 kfrag;
+                    if constexpr (KV8) {
+                        const uint4 w = tr.k[mt][ks >> 1];
+                        kfrag = fp8x8_to_16<Tag>((ks & 1) ? make_uint2(w.z, w.w) : make_uint2(w.x, w.y));
+                    } else {
+                        kfrag = tr.k[mt][ks];
+                    }
+                    c = MM::mma(__builtin_bit_cast(vec8, kfrag), qf[nt][ks], c);
+                }
                 s[mt][nt] = c;
             }
         if (PREFETCH && more) load_k(tok_next, tr);
@@ -238,7 +267,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(MINW))) voi
 #pragma unroll
                     for (int r = 0; r < 4; ++r) {
                         const int tok = tok0 + mt * 16 + g * 4 + r;
-                        float v = s[mt][nt][r] * p.scale_log2 + slope[nt] * (float)(tok - (len - 1));
+                        float v = s[mt][nt][r] * sl + slope[nt] * (float)(tok - (len - 1));
                         if (tok >= c1) v = -INFINITY;
                         x[mt * 4 + r] = v;
                         mx = fmaxf(mx, v);
@@ -248,7 +277,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(MINW))) voi
                 for (int mt = 0; mt < 2; ++mt)
 #pragma unroll
                     for (int r = 0; r < 4; ++r) {
-                        x[mt * 4 + r] = s[mt][nt][r] * p.scale_log2;
+                        x[mt * 4 + r] = s[mt][nt][r] * sl;
                         mx = fmaxf(mx, x[mt * 4 + r]);
                     }
             }
@@ -304,7 +333,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(MINW))) voi
             if (hh < nh) {
                 const int h = h_base + hh;
                 if (p.nsplit == 1) {
-                    const float inv = 1.0f / l[nt];
+                    const float inv = vs / l[nt];
                     uint16_t* orow = o16 + ((size_t)b * p.head_q + h) * DV + g * 4;
 #pragma unroll
                     for (int ct = 0; ct < CT; ++ct) {
@@ -319,7 +348,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(MINW))) voi
                     const size_t part = ((size_t)b * p.head_q + h) * p.nsplit + split;
                     float* wrow = p.ws_o + part * DV + g * 4;
 #pragma unroll
-                    for (int ct = 0; ct < CT; ++ct) *reinterpret_cast<f32x4*>(wrow + ct * 16) = acc[nt][ct];
+                    for (int ct = 0; ct < CT; ++ct) *reinterpret_cast<f32x4*>(wrow + ct * 16) = acc[nt][ct] * vs;
                     if (g == 0) {
                         p.ws_ml[part * 2 + 0] = m[nt];
                         p.ws_ml[part * 2 + 1] = l[nt];
@@ -362,10 +391,10 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(MINW))) voi
         }
         const int h = h_base + r;
         if (p.nsplit == 1) {
-            o16[((size_t)b * p.head_q + h) * DV + col] = EL::from_f32(num / den);
+            o16[((size_t)b * p.head_q + h) * DV + col] = EL::from_f32(num * vs / den);
         } else {
             const size_t part = ((size_t)b * p.head_q + h) * p.nsplit + split;
-            p.ws_o[part * DV + col] = num;
+            p.ws_o[part * DV + col] = num * vs;
             if (col == 0) {
                 p.ws_ml[part * 2 + 0] = mm;
                 p.ws_ml[part * 2 + 1] = den;
@@ -377,5 +406,8 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(MINW))) voi
 // wave_per_head selects the WH form; the grid's y extent must then count groups of four KV heads.
 hipError_t launch_gqa_mfma(const SweepParams& p, bool is_bf16, int dim, int heads_per_group, bool wave_per_head,
                            dim3 grid, hipStream_t stream);
+// the same with FP8 (e4m3) K and V; dim must be a multiple of 64
+hipError_t launch_gqa_mfma_kv8(const SweepParams& p, bool is_bf16, int dim, int heads_per_group, bool wave_per_head,
+                               dim3 grid, hipStream_t stream);
 
 }  // namespace da

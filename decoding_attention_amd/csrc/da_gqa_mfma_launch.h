@@ -1,0 +1,54 @@
+// Launch helpers of the grouped-head MFMA sweep, shared by the translation units that instantiate it (16-bit
+// K/V in da_gqa_mfma.hip, FP8 K/V in da_gqa_mfma_kv8.hip; two units so that the two sets compile in parallel).
+#pragma once
+#include "da_gqa_mfma.h"
+
+#include <mutex>
+
+namespace da {
+
+namespace gqa_launch {
+
+template <typename Tag, int D, int NT, bool WH, bool KV8>
+hipError_t launch_one(const SweepParams& p, dim3 grid, hipStream_t stream) {
+    constexpr bool kPrefetch = D <= 128;
+    constexpr int kMinWaves = (D <= 128 && (NT == 1 || D <= 64)) ? 2 : 1;
+    auto kern = gqa_mfma_kernel<Tag, D, D, NT, kPrefetch, WH, kMinWaves, KV8>;
+    const size_t lds = gqa_lds_bytes<D>(NT);
+    static std::once_flag once;
+    static hipError_t attr_err = hipSuccess;
+    std::call_once(once, [&] {
+        if (lds > 48 * 1024)
+            attr_err = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
+                                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+    });
+    if (attr_err != hipSuccess) return attr_err;
+    hipLaunchKernelGGL(kern, grid, dim3(256), lds, stream, p);
+    return hipGetLastError();
+}
+
+template <typename Tag, int D, bool KV8>
+hipError_t launch_dim(const SweepParams& p, int heads_per_group, bool wh, dim3 grid, hipStream_t stream) {
+    if (heads_per_group == 16)
+        return wh ? launch_one<Tag, D, 1, true, KV8>(p, grid, stream) : launch_one<Tag, D, 1, false, KV8>(p, grid, stream);
+    if (heads_per_group == 32)
+        return wh ? launch_one<Tag, D, 2, true, KV8>(p, grid, stream) : launch_one<Tag, D, 2, false, KV8>(p, grid, stream);
+    return hipErrorInvalidValue;
+}
+
+template <typename Tag, bool KV8>
+hipError_t launch_tag(const SweepParams& p, int dim, int heads_per_group, bool wh, dim3 grid, hipStream_t stream) {
+    switch (dim) {
+        case 64: return launch_dim<Tag, 64, KV8>(p, heads_per_group, wh, grid, stream);
+        case 96:
+            if constexpr (!KV8) return launch_dim<Tag, 96, false>(p, heads_per_group, wh, grid, stream);
+            return hipErrorInvalidValue;  // FP8 loads pair up k-steps: head dims that are multiples of 64 only
+        case 128: return launch_dim<Tag, 128, KV8>(p, heads_per_group, wh, grid, stream);
+        case 256: return launch_dim<Tag, 256, KV8>(p, heads_per_group, wh, grid, stream);
+        default: return hipErrorInvalidValue;
+    }
+}
+
+}  // namespace gqa_launch
+
+}  // namespace da

@@ -24,7 +24,8 @@
 
 namespace da {
 
-template <typename Tag, int D, int DV, int G, int RT, int U>
+// KV8: K and V hold FP8 (e4m3) elements, converted exactly to the compute type as they are loaded.
+template <typename Tag, int D, int DV, int G, int RT, int U, bool KV8 = false>
 __global__ __launch_bounds__(256) void sweep_kernel(const SweepParams p) {
     static_assert(D % (8 * G) == 0 && DV % (8 * G) == 0, "row must split into 16-byte chunks over G lanes");
     constexpr int CPL = D / 8 / G;    // K chunks per lane
@@ -33,6 +34,7 @@ __global__ __launch_bounds__(256) void sweep_kernel(const SweepParams p) {
     constexpr int RPI = kWave / G;    // rows per load instruction
     constexpr int NW = 4;             // waves per work-group
     constexpr int TILE = RPI * U;     // rows per wave iteration
+    constexpr int KB = KV8 ? 1 : 2;   // bytes per K/V element
     using EL = Elem<Tag>;
 
     __shared__ float lds_acc[NW][RT][DV];
@@ -85,8 +87,16 @@ __global__ __launch_bounds__(256) void sweep_kernel(const SweepParams p) {
     }
 
     // rows are addressed one by one (row_ref), so paged K/V of any page size costs one table lookup per row
-    const uint16_t* kbase = reinterpret_cast<const uint16_t*>(p.k) + (size_t)hk * D + g * 8;
-    const uint16_t* vbase = reinterpret_cast<const uint16_t*>(p.v) + (size_t)hk * p.v_head + g * 8;
+    const uint8_t* kbase = reinterpret_cast<const uint8_t*>(p.k) + ((size_t)hk * D + g * 8) * KB;
+    const uint8_t* vbase = reinterpret_cast<const uint8_t*>(p.v) + ((size_t)hk * p.v_head + g * 8) * KB;
+    const float sl = p.scale_log2 * head_scale(p.k_scale, hk);  // score scale, log2 units
+    const float vs = head_scale(p.v_scale, hk);
+    auto load8 = [](const uint8_t* ptr) __attribute__((always_inline)) {  // eight elements as 16-bit pairs
+        if constexpr (KV8)
+            return fp8x8_to_16<Tag>(*reinterpret_cast<const uint2*>(ptr));
+        else
+            return *reinterpret_cast<const uint4*>(ptr);
+    };
 
     const int ntiles = (c1 - c0 + TILE - 1) / TILE;
     for (int t = wave; t < ntiles; t += NW) {
@@ -99,15 +109,15 @@ __global__ __launch_bounds__(256) void sweep_kernel(const SweepParams p) {
             rr[u] = row_ref(p, b, start, min(base + u * RPI, c1 - 1));
 #pragma unroll
         for (int u = 0; u < U; ++u) {
-            const uint16_t* kr = kbase + rr[u].k;
+            const uint8_t* kr = kbase + rr[u].k * KB;
 #pragma unroll
-            for (int c = 0; c < CPL; ++c) kreg[u][c] = *reinterpret_cast<const uint4*>(kr + c * G * 8);
+            for (int c = 0; c < CPL; ++c) kreg[u][c] = load8(kr + c * G * 8 * KB);
         }
 #pragma unroll
         for (int u = 0; u < U; ++u) {
-            const uint16_t* vr = vbase + rr[u].v;
+            const uint8_t* vr = vbase + rr[u].v * KB;
 #pragma unroll
-            for (int c = 0; c < CPLV; ++c) vreg[u][c] = *reinterpret_cast<const uint4*>(vr + c * G * 8);
+            for (int c = 0; c < CPLV; ++c) vreg[u][c] = load8(vr + c * G * 8 * KB);
         }
 
         // scores in log2 units
@@ -126,7 +136,7 @@ __global__ __launch_bounds__(256) void sweep_kernel(const SweepParams p) {
                     d = EL::dot2(qreg[r][c].w, kreg[u][c].w, d);
                 }
                 d = group_sum<G>(d);
-                d = d * p.scale_log2 + slope[r] * (float)(j - (len - 1));
+                d = d * sl + slope[r] * (float)(j - (len - 1));
                 s[u][r] = (j < c1) ? d : -INFINITY;
             }
         }
@@ -223,10 +233,10 @@ __global__ __launch_bounds__(256) void sweep_kernel(const SweepParams p) {
         }
         const int h = h_base + r;
         if (p.nsplit == 1) {
-            reinterpret_cast<uint16_t*>(p.o)[((size_t)b * p.head_q + h) * DV + col] = EL::from_f32(num / den);
+            reinterpret_cast<uint16_t*>(p.o)[((size_t)b * p.head_q + h) * DV + col] = EL::from_f32(num * vs / den);
         } else {
             const size_t part = ((size_t)b * p.head_q + h) * p.nsplit + split;
-            p.ws_o[part * DV + col] = num;
+            p.ws_o[part * DV + col] = num * vs;
             if (col == 0) {
                 p.ws_ml[part * 2 + 0] = mm;
                 p.ws_ml[part * 2 + 1] = den;

@@ -13,26 +13,26 @@ template <> struct SweepTile<128> { static constexpr int G = 8,  U = 4; };
 template <> struct SweepTile<256> { static constexpr int G = 16, U = 4; };
 template <> struct SweepTile<576> { static constexpr int G = 8,  U = 1; };
 
-template <typename Tag, int D, int DV, int RT>
+template <typename Tag, int D, int DV, int RT, bool KV8 = false>
 inline hipError_t launch_sweep_rt(const SweepParams& p, dim3 grid, hipStream_t stream) {
     constexpr int G = SweepTile<D>::G, U = SweepTile<D>::U;
-    hipLaunchKernelGGL((sweep_kernel<Tag, D, DV, G, RT, U>), grid, dim3(256), 0, stream, p);
+    hipLaunchKernelGGL((sweep_kernel<Tag, D, DV, G, RT, U, KV8>), grid, dim3(256), 0, stream, p);
     return hipGetLastError();
 }
 
-template <int D, int DV, int MAXRT>
+template <int D, int DV, int MAXRT, bool KV8 = false>
 inline hipError_t launch_sweep_dim(const SweepParams& p, bool is_bf16, int rt, dim3 grid, hipStream_t stream) {
     if (is_bf16) {
-        if (rt == 1) return launch_sweep_rt<bf16_tag, D, DV, 1>(p, grid, stream);
-        if (rt == 2) return launch_sweep_rt<bf16_tag, D, DV, 2>(p, grid, stream);
+        if (rt == 1) return launch_sweep_rt<bf16_tag, D, DV, 1, KV8>(p, grid, stream);
+        if (rt == 2) return launch_sweep_rt<bf16_tag, D, DV, 2, KV8>(p, grid, stream);
         if constexpr (MAXRT >= 4) {
-            if (rt == 4) return launch_sweep_rt<bf16_tag, D, DV, 4>(p, grid, stream);
+            if (rt == 4) return launch_sweep_rt<bf16_tag, D, DV, 4, KV8>(p, grid, stream);
         }
     } else {
-        if (rt == 1) return launch_sweep_rt<f16_tag, D, DV, 1>(p, grid, stream);
-        if (rt == 2) return launch_sweep_rt<f16_tag, D, DV, 2>(p, grid, stream);
+        if (rt == 1) return launch_sweep_rt<f16_tag, D, DV, 1, KV8>(p, grid, stream);
+        if (rt == 2) return launch_sweep_rt<f16_tag, D, DV, 2, KV8>(p, grid, stream);
         if constexpr (MAXRT >= 4) {
-            if (rt == 4) return launch_sweep_rt<f16_tag, D, DV, 4>(p, grid, stream);
+            if (rt == 4) return launch_sweep_rt<f16_tag, D, DV, 4, KV8>(p, grid, stream);
         }
     }
     return hipErrorInvalidValue;
@@ -46,6 +46,8 @@ hipError_t launch_sweep_d96(const SweepParams& p, bool is_bf16, int rt, dim3 gri
 hipError_t launch_sweep_d128(const SweepParams& p, bool is_bf16, int rt, dim3 grid, hipStream_t stream);
 hipError_t launch_sweep_d256(const SweepParams& p, bool is_bf16, int rt, dim3 grid, hipStream_t stream);
 hipError_t launch_sweep_d576(const SweepParams& p, bool is_bf16, int rt, dim3 grid, hipStream_t stream);
+// the VALU sweep over an FP8 (e4m3) K/V cache, any supported (dim, dim_v)
+hipError_t launch_sweep_kv8(const SweepParams& p, bool is_bf16, int dim, int rt, dim3 grid, hipStream_t stream);
 hipError_t launch_reduce(const ReduceParams& p, bool is_bf16, int blocks, hipStream_t stream);
 
 }  // namespace da

@@ -22,15 +22,35 @@ namespace {
     TORCH_CHECK(x.sizes() == torch::IntArrayRef({__VA_ARGS__}), #x " must have shape (" #__VA_ARGS__ ")")
 #define DA_CHECK_CONTIGUOUS(x) TORCH_CHECK(x.is_contiguous(), #x " must be contiguous")
 
+// K/V element format: the 16-bit type of q, or FP8 (e4m3) with optional per-KV-head de-quantisation factors.
+bool is_fp8_kv(const at::Tensor &q, const at::Tensor &k) {
+    if (k.dtype() == torch::kFloat8_e4m3fn) return true;
+    TORCH_CHECK(k.dtype() == q.dtype(), "query and key must have the same dtype (or the key cache is float8_e4m3fn)");
+    return false;
+}
+
+const float *scale_ptr(const std::optional<at::Tensor> &t, const at::Tensor &q, int64_t head_k, const char *name,
+                       bool fp8) {
+    if (!t.has_value()) return nullptr;
+    TORCH_CHECK(fp8, name, " applies to a float8_e4m3fn K/V cache only");
+    const at::Tensor &s = t.value();
+    TORCH_CHECK(s.dtype() == torch::kFloat32 && s.is_cuda() && s.device() == q.device() && s.is_contiguous() &&
+                    s.numel() == head_k,
+                name, " must be a contiguous float32 GPU tensor of head_k values");
+    return s.data_ptr<float>();
+}
+
 at::Tensor dmha_fwd(const at::Tensor &q, const at::Tensor &k, const std::optional<at::Tensor> &v_,
                     const std::optional<at::Tensor> &o_, const at::Tensor &cu_seq_k, const int64_t max_seq_k,
                     const int64_t dim_v, const bool is_alibi, const std::optional<double> softmax_scale,
-                    const std::optional<at::Tensor> &alibi_slopes) {
+                    const std::optional<at::Tensor> &alibi_slopes, const std::optional<at::Tensor> &k_scale,
+                    const std::optional<at::Tensor> &v_scale) {
     auto q_dtype = q.dtype();
     TORCH_CHECK(q_dtype == torch::kFloat16 || q_dtype == torch::kBFloat16,
                 "Decoding-Attention only support FP16 and BF16 data type");
     const bool is_bf16 = q_dtype == torch::kBFloat16;
-    TORCH_CHECK(k.dtype() == q_dtype, "query and key must have the same dtype");
+    const bool fp8 = is_fp8_kv(q, k);
+    const auto kv_dtype = k.dtype();
     TORCH_CHECK(cu_seq_k.dtype() == torch::kInt32, "cu_seq_k must have dtype int32");
 
     DA_CHECK_DEVICE(q);
@@ -66,7 +86,7 @@ at::Tensor dmha_fwd(const at::Tensor &q, const at::Tensor &k, const std::optiona
     const void *v_ptr = nullptr;
     if (v_.has_value()) {
         const at::Tensor &v = v_.value();
-        TORCH_CHECK(v.dtype() == q_dtype, "query and value must have the same dtype");
+        TORCH_CHECK(v.dtype() == kv_dtype, "key and value must have the same dtype");
         DA_CHECK_DEVICE(v);
         TORCH_CHECK(v.device() == q.device(), "v must be on q's device");
         TORCH_CHECK(v.stride(-1) == 1, "value must have contiguous last dimension");
@@ -103,17 +123,29 @@ at::Tensor dmha_fwd(const at::Tensor &q, const at::Tensor &k, const std::optiona
     c10::hip::HIPGuardMasqueradingAsCUDA guard(q.device());
     hipStream_t stream = c10::hip::getCurrentHIPStreamMasqueradingAsCUDA(q.device().index()).stream();
 
+    const float *k_scale_ptr = scale_ptr(k_scale, q, head_k, "k_scale", fp8);
+    const float *v_scale_ptr = scale_ptr(v_scale, q, head_k, "v_scale", fp8);
+
     // k.size(0) is the sum of the key lengths: a free host-side hint for sizing the sequence splits
-    const size_t ws_bytes = da_workspace_bytes((size_t)max_seq_k, (size_t)batch, (size_t)head_q, (size_t)head_k,
-                                               (size_t)dim, (size_t)dim_v, (size_t)total_k);
+    const size_t ws_bytes =
+        fp8 ? da_workspace_bytes_fp8kv((size_t)max_seq_k, (size_t)batch, (size_t)head_q, (size_t)head_k, (size_t)dim,
+                                       (size_t)dim_v, (size_t)total_k, 0)
+            : da_workspace_bytes((size_t)max_seq_k, (size_t)batch, (size_t)head_q, (size_t)head_k, (size_t)dim,
+                                 (size_t)dim_v, (size_t)total_k);
     at::Tensor ws;  // from torch's stream-aware caching allocator
     if (ws_bytes > 0) ws = torch::empty({(int64_t)ws_bytes}, q.options().dtype(torch::kUInt8));
 
-    const int rc = da_decoding_attn_ex(
-        q.data_ptr(), k.data_ptr(), v_ptr, o.data_ptr(), cu_seq_k.data_ptr<int32_t>(), (size_t)max_seq_k,
-        (size_t)batch, (size_t)head_q, (size_t)head_k, (size_t)dim, (size_t)dim_v, is_alibi ? 1 : 0, is_bf16 ? 1 : 0,
-        softmax_scale.has_value() ? (float)softmax_scale.value() : 0.0f, slopes_ptr, (size_t)total_k,
-        ws_bytes > 0 ? ws.data_ptr() : nullptr, ws_bytes, (void *)stream);
+    const float scale = softmax_scale.has_value() ? (float)softmax_scale.value() : 0.0f;
+    const int rc =
+        fp8 ? da_decoding_attn_fp8kv(q.data_ptr(), k.data_ptr(), v_ptr, o.data_ptr(), cu_seq_k.data_ptr<int32_t>(),
+                                     (size_t)max_seq_k, (size_t)batch, (size_t)head_q, (size_t)head_k, (size_t)dim,
+                                     (size_t)dim_v, is_alibi ? 1 : 0, is_bf16 ? 1 : 0, scale, slopes_ptr, k_scale_ptr,
+                                     v_scale_ptr, (size_t)total_k, ws_bytes > 0 ? ws.data_ptr() : nullptr, ws_bytes,
+                                     (void *)stream)
+            : da_decoding_attn_ex(q.data_ptr(), k.data_ptr(), v_ptr, o.data_ptr(), cu_seq_k.data_ptr<int32_t>(),
+                                  (size_t)max_seq_k, (size_t)batch, (size_t)head_q, (size_t)head_k, (size_t)dim,
+                                  (size_t)dim_v, is_alibi ? 1 : 0, is_bf16 ? 1 : 0, scale, slopes_ptr,
+                                  (size_t)total_k, ws_bytes > 0 ? ws.data_ptr() : nullptr, ws_bytes, (void *)stream);
     TORCH_CHECK(rc == DA_OK, "decoding_attn failed (", rc, "): ", da_last_error());
     return o;
 }
@@ -125,12 +157,14 @@ at::Tensor dmha_fwd_paged(const at::Tensor &q, const at::Tensor &k_pages, const 
                           const std::optional<at::Tensor> &o_, const at::Tensor &block_table,
                           const at::Tensor &seq_lens, const int64_t max_seq_k, const int64_t dim_v, const bool is_alibi,
                           const std::optional<double> softmax_scale, const std::optional<at::Tensor> &alibi_slopes,
-                          const int64_t total_k) {
+                          const int64_t total_k, const std::optional<at::Tensor> &k_scale,
+                          const std::optional<at::Tensor> &v_scale) {
     auto q_dtype = q.dtype();
     TORCH_CHECK(q_dtype == torch::kFloat16 || q_dtype == torch::kBFloat16,
                 "Decoding-Attention only support FP16 and BF16 data type");
     const bool is_bf16 = q_dtype == torch::kBFloat16;
-    TORCH_CHECK(k_pages.dtype() == q_dtype, "query and key must have the same dtype");
+    const bool fp8 = is_fp8_kv(q, k_pages);
+    const auto kv_dtype = k_pages.dtype();
     TORCH_CHECK(block_table.dtype() == torch::kInt32, "block_table must have dtype int32");
     TORCH_CHECK(seq_lens.dtype() == torch::kInt32, "seq_lens must have dtype int32");
     DA_CHECK_DEVICE(q);
@@ -164,7 +198,7 @@ at::Tensor dmha_fwd_paged(const at::Tensor &q, const at::Tensor &k_pages, const 
     int64_t v_stride = 0;
     if (v_pages_.has_value()) {
         const at::Tensor &v = v_pages_.value();
-        TORCH_CHECK(v.dtype() == q_dtype, "query and value must have the same dtype");
+        TORCH_CHECK(v.dtype() == kv_dtype, "key and value must have the same dtype");
         DA_CHECK_DEVICE(v);
         TORCH_CHECK(v.device() == q.device(), "v_pages must be on q's device");
         TORCH_CHECK(v.dim() == 4 && v.size(0) == k_pages.size(0) && v.size(1) == page_size && v.size(2) == head_k &&
@@ -201,18 +235,31 @@ at::Tensor dmha_fwd_paged(const at::Tensor &q, const at::Tensor &k_pages, const 
     c10::hip::HIPGuardMasqueradingAsCUDA guard(q.device());
     hipStream_t stream = c10::hip::getCurrentHIPStreamMasqueradingAsCUDA(q.device().index()).stream();
 
+    const float *k_scale_ptr = scale_ptr(k_scale, q, head_k, "k_scale", fp8);
+    const float *v_scale_ptr = scale_ptr(v_scale, q, head_k, "v_scale", fp8);
     const size_t hint = total_k > 0 ? (size_t)total_k : 0;
-    const size_t ws_bytes = da_workspace_bytes_paged((size_t)max_seq_k, (size_t)batch, (size_t)head_q, (size_t)head_k,
-                                                     (size_t)dim, (size_t)dim_v, hint, (size_t)page_size);
+    const size_t ws_bytes =
+        fp8 ? da_workspace_bytes_fp8kv((size_t)max_seq_k, (size_t)batch, (size_t)head_q, (size_t)head_k, (size_t)dim,
+                                       (size_t)dim_v, hint, (size_t)page_size)
+            : da_workspace_bytes_paged((size_t)max_seq_k, (size_t)batch, (size_t)head_q, (size_t)head_k, (size_t)dim,
+                                       (size_t)dim_v, hint, (size_t)page_size);
     at::Tensor ws;
     if (ws_bytes > 0) ws = torch::empty({(int64_t)ws_bytes}, q.options().dtype(torch::kUInt8));
 
-    const int rc = da_decoding_attn_paged(
-        q.data_ptr(), k_pages.data_ptr(), v_ptr, o.data_ptr(), block_table.data_ptr<int32_t>(),
-        seq_lens.data_ptr<int32_t>(), (size_t)max_seq_k, (size_t)batch, (size_t)head_q, (size_t)head_k, (size_t)dim,
-        (size_t)dim_v, (size_t)page_size, (size_t)block_table.size(1), (size_t)k_pages.stride(0), (size_t)v_stride,
-        is_alibi ? 1 : 0, is_bf16 ? 1 : 0, softmax_scale.has_value() ? (float)softmax_scale.value() : 0.0f, slopes_ptr,
-        hint, ws_bytes > 0 ? ws.data_ptr() : nullptr, ws_bytes, (void *)stream);
+    const float scale = softmax_scale.has_value() ? (float)softmax_scale.value() : 0.0f;
+    const int rc =
+        fp8 ? da_decoding_attn_paged_fp8kv(
+                  q.data_ptr(), k_pages.data_ptr(), v_ptr, o.data_ptr(), block_table.data_ptr<int32_t>(),
+                  seq_lens.data_ptr<int32_t>(), (size_t)max_seq_k, (size_t)batch, (size_t)head_q, (size_t)head_k,
+                  (size_t)dim, (size_t)dim_v, (size_t)page_size, (size_t)block_table.size(1),
+                  (size_t)k_pages.stride(0), (size_t)v_stride, is_alibi ? 1 : 0, is_bf16 ? 1 : 0, scale, slopes_ptr,
+                  k_scale_ptr, v_scale_ptr, hint, ws_bytes > 0 ? ws.data_ptr() : nullptr, ws_bytes, (void *)stream)
+            : da_decoding_attn_paged(
+                  q.data_ptr(), k_pages.data_ptr(), v_ptr, o.data_ptr(), block_table.data_ptr<int32_t>(),
+                  seq_lens.data_ptr<int32_t>(), (size_t)max_seq_k, (size_t)batch, (size_t)head_q, (size_t)head_k,
+                  (size_t)dim, (size_t)dim_v, (size_t)page_size, (size_t)block_table.size(1),
+                  (size_t)k_pages.stride(0), (size_t)v_stride, is_alibi ? 1 : 0, is_bf16 ? 1 : 0, scale, slopes_ptr,
+                  hint, ws_bytes > 0 ? ws.data_ptr() : nullptr, ws_bytes, (void *)stream);
     TORCH_CHECK(rc == DA_OK, "decoding_attn (paged) failed (", rc, "): ", da_last_error());
     return o;
 }
@@ -224,10 +271,12 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
     m.def("fwd", &dmha_fwd, "Forward pass", pybind11::arg("q"), pybind11::arg("k"), pybind11::arg("v_"),
           pybind11::arg("o_"), pybind11::arg("cu_seq_k"), pybind11::arg("max_seq_k"), pybind11::arg("dim_v"),
           pybind11::arg("is_alibi"), pybind11::arg("softmax_scale") = pybind11::none(),
-          pybind11::arg("alibi_slopes") = pybind11::none());
+          pybind11::arg("alibi_slopes") = pybind11::none(), pybind11::arg("k_scale") = pybind11::none(),
+          pybind11::arg("v_scale") = pybind11::none());
     m.def("fwd_paged", &dmha_fwd_paged, "Forward pass over a paged K/V cache", pybind11::arg("q"),
           pybind11::arg("k_pages"), pybind11::arg("v_pages_"), pybind11::arg("o_"), pybind11::arg("block_table"),
           pybind11::arg("seq_lens"), pybind11::arg("max_seq_k"), pybind11::arg("dim_v"), pybind11::arg("is_alibi"),
           pybind11::arg("softmax_scale") = pybind11::none(), pybind11::arg("alibi_slopes") = pybind11::none(),
-          pybind11::arg("total_k") = 0);
+          pybind11::arg("total_k") = 0, pybind11::arg("k_scale") = pybind11::none(),
+          pybind11::arg("v_scale") = pybind11::none());
 }

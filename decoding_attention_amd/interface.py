@@ -41,15 +41,17 @@ def maybe_contiguous(x):
 
 def fwd(q: torch.Tensor, k: torch.Tensor, v_: Optional[torch.Tensor], o_: Optional[torch.Tensor],
         cu_seq_k: torch.Tensor, max_seq_k: int, dim_v: int, is_alibi: bool, *,
-        softmax_scale: Optional[float] = None, alibi_slopes: Optional[torch.Tensor] = None) -> torch.Tensor:
+        softmax_scale: Optional[float] = None, alibi_slopes: Optional[torch.Tensor] = None,
+        k_scale: Optional[torch.Tensor] = None, v_scale: Optional[torch.Tensor] = None) -> torch.Tensor:
     """The extension's `fwd` (same role as the reference's `decoding_attn_cuda.fwd`)."""
     return _extension().fwd(q, k, v_, o_, cu_seq_k, int(max_seq_k), int(dim_v), bool(is_alibi),
-                            None if softmax_scale is None else float(softmax_scale), alibi_slopes)
+                            None if softmax_scale is None else float(softmax_scale), alibi_slopes, k_scale, v_scale)
 
 
 def decoding_attn_fwd(q: torch.Tensor, k: torch.Tensor, v: Optional[torch.Tensor], cu_seq_k: torch.Tensor,
                       max_seq_k: int, dim_v: int, is_alibi: bool, *, softmax_scale: Optional[float] = None,
-                      alibi_slopes: Optional[torch.Tensor] = None) -> torch.Tensor:
+                      alibi_slopes: Optional[torch.Tensor] = None, k_scale: Optional[torch.Tensor] = None,
+                      v_scale: Optional[torch.Tensor] = None) -> torch.Tensor:
     """
     Arguments:
         q: [total_q, head_q, dim], torch.float16 / torch.bfloat16; one query token per sequence.
@@ -61,19 +63,22 @@ def decoding_attn_fwd(q: torch.Tensor, k: torch.Tensor, v: Optional[torch.Tensor
         is_alibi: whether to add the ALiBi bias slope_h * (j - (len - 1)).
         softmax_scale (keyword only): defaults to 1/sqrt(dim) as in the reference.
         alibi_slopes (keyword only): float32 [head_q] on the GPU; defaults to 2^(-8(h+1)/head_q).
+        k_scale, v_scale (keyword only): k and v may be torch.float8_e4m3fn (an FP8 K/V cache; q stays 16-bit);
+            these are then float32 [head_k] GPU tensors of de-quantisation factors (default 1): K = k_scale * k.
     Return:
         o: [total_q, head_q, dim_v], same dtype as q.
     """
     q, k, v = [maybe_contiguous(x) for x in (q, k, v)]
     return fwd(q, k, v, None, cu_seq_k, max_seq_k, dim_v, is_alibi, softmax_scale=softmax_scale,
-               alibi_slopes=alibi_slopes)
+               alibi_slopes=alibi_slopes, k_scale=k_scale, v_scale=v_scale)
 
 
 def decoding_attn_paged_fwd(q: torch.Tensor, k_pages: torch.Tensor, v_pages: Optional[torch.Tensor],
                             block_table: torch.Tensor, seq_lens: torch.Tensor, max_seq_k: int, dim_v: int,
                             is_alibi: bool, *, softmax_scale: Optional[float] = None,
                             alibi_slopes: Optional[torch.Tensor] = None, total_k: int = 0,
-                            out: Optional[torch.Tensor] = None) -> torch.Tensor:
+                            out: Optional[torch.Tensor] = None, k_scale: Optional[torch.Tensor] = None,
+                            v_scale: Optional[torch.Tensor] = None) -> torch.Tensor:
     """
     The same attention over a paged K/V cache (no counterpart in the reference; the layouts are those of the
     libraries its benchmark compares against, reference benchmarks/python/benchmark_decoding_attn.py:129-151,182-187).
@@ -87,10 +92,11 @@ def decoding_attn_paged_fwd(q: torch.Tensor, k_pages: torch.Tensor, v_pages: Opt
         max_seq_k: upper bound of seq_lens (a host integer: nothing here synchronises with the device).
         page_size (from k_pages.shape[1]) must be a power of two.
         total_k (keyword only): sum of seq_lens if the host knows it; only a hint for sizing sequence splits.
+        k_scale, v_scale (keyword only): as for decoding_attn_fwd, when the pools are torch.float8_e4m3fn.
     Return:
         o: [batch, head_q, dim_v], same dtype as q.
     """
     q = maybe_contiguous(q)
     return _extension().fwd_paged(q, k_pages, v_pages, out, block_table, seq_lens, int(max_seq_k), int(dim_v),
                                   bool(is_alibi), None if softmax_scale is None else float(softmax_scale),
-                                  alibi_slopes, int(total_k))
+                                  alibi_slopes, int(total_k), k_scale, v_scale)

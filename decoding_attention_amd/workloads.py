@@ -105,12 +105,12 @@ class PagedKV:
                        self.block_table.to(device), self.seq_lens.to(device), self.page_size)
 
 
-def to_pages(w: Workload, page_size: int, *, seed=0, combined=False, spare_pages=3) -> PagedKV:
+def to_pages(w: Workload, page_size: int, *, seed=0, combined=False, spare_pages=3, poison=True) -> PagedKV:
     """Scatter the packed K/V of `w` into page pools with shuffled page ids.
 
     Unused pages, the unused tail of each sequence's last page and unused block-table entries are poisoned (NaN
     rows, page id -1 replaced by an out-of-sequence valid id) so that a kernel that reads past a sequence's end
-    shows up in the output.  combined=True builds one [pages, 2, page_size, head_k, dim] pool (K and V interleaved
+    shows up in the output (poison=False fills with zeros instead, for integer-typed byte views).  combined=True builds one [pages, 2, page_size, head_k, dim] pool (K and V interleaved
     per page, dim == dim_v) and returns its two halves as views.
     """
     g = torch.Generator(device="cpu").manual_seed(seed)
@@ -119,7 +119,7 @@ def to_pages(w: Workload, page_size: int, *, seed=0, combined=False, spare_pages
     max_blocks = max(1, max(blocks))
     n_pages = sum(blocks) + spare_pages
     order = torch.randperm(n_pages, generator=g).tolist()
-    nan = float("nan")
+    nan = float("nan") if poison else 0
     if combined:
         assert w.v is not None and w.dim == w.dim_v
         pool = torch.full((n_pages, 2, page_size, w.head_k, w.dim), nan, dtype=w.k.dtype)

@@ -96,6 +96,37 @@ size_t da_workspace_bytes_paged(size_t max_seq_k, size_t batch, size_t head_q, s
                                 size_t dim_v, size_t total_k, size_t page_size);
 
 /*
+ * The same attention over an FP8 K/V cache (the reference lists K/V quantisation as future work, README.md:154-156;
+ * it has no such path).  q and o stay fp16 / bf16 (is_bf16); k8 and v8 hold OCP FP8 e4m3 values, one byte per
+ * element, in the layouts of the 16-bit entry points (packed [total_k, head_k, dim] with cu_seq_k, or page pools
+ * with a block table; strides are in elements).
+ *
+ *   k_scale, v_scale   device, float [head_k], or NULL for 1: K = k_scale[hk] * fp8 value, V likewise.  FP8
+ *                      values convert exactly to fp16 and bf16, so the matrix arithmetic is that of the 16-bit
+ *                      path; k_scale is folded into the softmax scale and v_scale into the final normalisation,
+ *                      both in fp32.
+ * v8 == NULL means V is the first dim_v columns of each K row.  Head dims (64,64), (128,128), (256,256) run on
+ * the grouped MFMA kernel when a KV head serves 3 or more query heads; everything else, (96,96) and (576,512)
+ * included, runs on the VALU sweep.  Workspace size from da_workspace_bytes_fp8kv (page_size 0 = packed layout).
+ */
+int da_decoding_attn_fp8kv(const void *q, const void *k8, const void *v8, void *o, const int32_t *cu_seq_k,
+                           size_t max_seq_k, size_t batch, size_t head_q, size_t head_k, size_t dim, size_t dim_v,
+                           int is_alibi, int is_bf16, float softmax_scale, const float *alibi_slopes,
+                           const float *k_scale, const float *v_scale, size_t total_k, void *workspace,
+                           size_t workspace_bytes, void *hip_stream);
+
+int da_decoding_attn_paged_fp8kv(const void *q, const void *k_pages, const void *v_pages, void *o,
+                                 const int32_t *block_table, const int32_t *seq_lens, size_t max_seq_k, size_t batch,
+                                 size_t head_q, size_t head_k, size_t dim, size_t dim_v, size_t page_size,
+                                 size_t max_blocks_per_seq, size_t k_page_stride, size_t v_page_stride, int is_alibi,
+                                 int is_bf16, float softmax_scale, const float *alibi_slopes, const float *k_scale,
+                                 const float *v_scale, size_t total_k, void *workspace, size_t workspace_bytes,
+                                 void *hip_stream);
+
+size_t da_workspace_bytes_fp8kv(size_t max_seq_k, size_t batch, size_t head_q, size_t head_k, size_t dim,
+                                size_t dim_v, size_t total_k, size_t page_size);
+
+/*
  * Launch plan the library would use for this shape, for tests and benchmarks:
  *   kernel_kind 1 = VALU sweep, 2 = latent (MLA) MFMA sweep, 3 = grouped-head MFMA sweep; nsplit = sequence splits;
  *   chunk = tokens per split; heads_per_group = query heads one work-group serves; total_k as for
