@@ -44,7 +44,7 @@ int env_int(const char* name, int dflt) {
 struct Tunables {
     int target_wgs, mfma_target_wgs, max_chunk, min_chunk, ragged_chunk, force_kind, group_min_ratio, wave_per_head;
     Tunables() {
-        target_wgs = env_int("DA_TARGET_WGS", 1024);
+        target_wgs = env_int("DA_TARGET_WGS", 512);
         mfma_target_wgs = env_int("DA_MFMA_TARGET_WGS", 256);
         max_chunk = env_int("DA_MAX_CHUNK", 1024);
         min_chunk = env_int("DA_MIN_CHUNK", 512);
