@@ -42,12 +42,14 @@ int env_int(const char* name, int dflt) {
 // Tunables, read once.  DA_TARGET_WGS: work-groups a launch should reach before the sequence
 // stops being split further; DA_MAX_CHUNK / DA_MIN_CHUNK: bounds on tokens per split.
 struct Tunables {
-    int target_wgs, mfma_target_wgs, max_chunk, min_chunk, ragged_chunk, force_kind, group_min_ratio, wave_per_head;
+    int target_wgs, mfma_target_wgs, max_chunk, min_chunk, ragged_chunk, force_kind, group_min_ratio, wave_per_head,
+        mla_heads;
     Tunables() {
         target_wgs = env_int("DA_TARGET_WGS", 512);
         mfma_target_wgs = env_int("DA_MFMA_TARGET_WGS", 256);
         max_chunk = env_int("DA_MAX_CHUNK", 1024);
         min_chunk = env_int("DA_MIN_CHUNK", 512);
+        mla_heads = env_int("DA_MLA_HEADS", 0);  // query heads per work-group of the latent kernel (32/64/128), 0 = by shape
         ragged_chunk = env_int("DA_RAGGED_CHUNK", 256);  // tokens per split when the lengths are known to be ragged
         force_kind = env_int("DA_FORCE_KIND", 0);
         wave_per_head = env_int("DA_WAVE_PER_HEAD", 1);
@@ -107,6 +109,12 @@ Plan make_plan(size_t max_seq_k, size_t batch, size_t head_q, size_t head_k, siz
     if (mfma) {
         pl.kind = kKindMfma;
         pl.rt = da::mla_heads_per_group(ratio);
+        // few sequences and short ones cannot fill the chip even at the finest split: then two work-groups of 64
+        // heads per (sequence, split) beat one of 128 (measured: batch 1, seq 4096: 35 -> 31 us)
+        if (pl.rt == 128 && (long long)batch * (long long)(max_seq_k / 256) <= 128) pl.rt = 64;
+        if ((tun().mla_heads == 32 || tun().mla_heads == 64 || tun().mla_heads == 128) && tun().mla_heads <= 128 &&
+            tun().mla_heads >= 32)
+            pl.rt = std::min(tun().mla_heads, da::mla_heads_per_group(ratio));
         trip = da::mla_rows_per_trip();
         target_wgs = tun().mfma_target_wgs;  // one 4-wave work-group fills a CU
     } else if (dim <= 256 && ratio >= tun().group_min_ratio && !force_sweep && (!kv_fp8 || dim % 64 == 0)) {
