@@ -53,7 +53,7 @@ struct Tunables {
         ragged_chunk = env_int("DA_RAGGED_CHUNK", 256);  // tokens per split when the lengths are known to be ragged
         force_kind = env_int("DA_FORCE_KIND", 0);
         wave_per_head = env_int("DA_WAVE_PER_HEAD", 1);
-        group_min_ratio = env_int("DA_GROUP_MIN_RATIO", 3);  // smallest head group that takes the grouped MFMA sweep
+        group_min_ratio = env_int("DA_GROUP_MIN_RATIO", 2);  // smallest head group that takes the grouped MFMA sweep
     }
 };
 const Tunables& tun() {
@@ -117,7 +117,14 @@ Plan make_plan(size_t max_seq_k, size_t batch, size_t head_q, size_t head_k, siz
             pl.rt = std::min(tun().mla_heads, da::mla_heads_per_group(ratio));
         trip = da::mla_rows_per_trip();
         target_wgs = tun().mfma_target_wgs;  // one 4-wave work-group fills a CU
-    } else if (dim <= 256 && ratio >= tun().group_min_ratio && !force_sweep && (!kv_fp8 || dim % 64 == 0)) {
+    } else if (dim <= 256 && !force_sweep && (!kv_fp8 || dim % 64 == 0) &&
+               (ratio >= tun().group_min_ratio ||
+                (tun().group_min_ratio > 1 && max_seq_k >= 1024 &&
+                 (long long)batch * (long long)head_k * (long long)max_seq_k >= (1ll << 21)))) {
+        // Two or more query heads per KV head, or a single one over long sequences of a large batch: the MFMA sweep streams K/V
+        // a few percent faster than the VALU sweep even though most of its matrix columns are idle (measured:
+        // ratio 2, 2048 tokens: 201 -> 185 us; ratio 1, batch 64 x 2048 tokens: 375 -> 364 us; at 128 tokens or batch 1 the VALU
+        // sweep wins).
         pl.kind = kKindGroup;
         pl.rt = ratio > 16 ? 32 : 16;
         pl.wave_per_head = head_k % 4 == 0 && tun().wave_per_head;
