@@ -173,6 +173,28 @@ def cpu_baseline(torch, w, budget_s=20.0):
     }
 
 
+def stream_read_GBps(torch, nbytes=1 << 30, reps=20):
+    """Bandwidth of the library's plain streaming-read kernel over a fresh buffer: what HBM gives a kernel that
+    only reads (the practical ceiling for the bandwidth-bound attention kernels on this GPU)."""
+    from decoding_attention_amd import _lib
+
+    lib = _lib.load()
+    buf = torch.empty(nbytes, dtype=torch.uint8, device="cuda:0").fill_(1)
+    stream = torch.cuda.current_stream().cuda_stream
+    for _ in range(3):
+        assert lib.da_probe_stream_read(buf.data_ptr(), nbytes, None, stream) == 0
+    torch.cuda.synchronize()
+    start = torch.cuda.Event(enable_timing=True)
+    end = torch.cuda.Event(enable_timing=True)
+    start.record()
+    for _ in range(reps):
+        lib.da_probe_stream_read(buf.data_ptr(), nbytes, None, stream)
+    end.record()
+    torch.cuda.synchronize()
+    ms = start.elapsed_time(end) / reps
+    return lib.da_probe_stream_read_bytes(nbytes) / (ms * 1e-3) / 1e9
+
+
 def run_default(args):
     import torch
 
@@ -201,6 +223,7 @@ def run_default(args):
     mla = None
     if not args.no_mla:
         mla = measure(torch, wl.config_mla(64, 4096), max(5, args.steps // 2), max(2, args.warmup // 2))
+    stream_gbps = stream_read_GBps(torch)
     cpu = None if args.no_cpu else cpu_baseline(torch, gqa_w, args.cpu_budget)
 
     line = {
@@ -224,7 +247,9 @@ def run_default(args):
         "pct_hbm_peak": 100.0 * gqa["hbm_frac_of_peak"],
         "roofline": {"bound": "hbm", "achieved": gqa["hbm_GBps"], "peak": HBM_PEAK_GBPS, "unit": "GB/s",
                      "frac": gqa["hbm_frac_of_peak"], "traffic": MEASURED_TRAFFIC_BYTES["gqa"],
-                     "kernel": "gqa_mfma_kernel + reduce_kernel of one call (whole-call time)"},
+                     "kernel": "gqa_mfma_kernel + reduce_kernel of one call (whole-call time)",
+                     # measured in this run: a kernel that only streams 1 GiB from HBM, and this call against it
+                     "stream_read_GBps": stream_gbps, "frac_of_stream_read": gqa["hbm_GBps"] / stream_gbps},
         "cpu_baseline": cpu,
     }
     if mla is not None:

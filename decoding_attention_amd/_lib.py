@@ -20,6 +20,8 @@ EXPORTED_SYMBOLS = (
     "da_decoding_attn_paged_fp8kv",
     "da_workspace_bytes_fp8kv",
     "da_plan",
+    "da_probe_stream_read",
+    "da_probe_stream_read_bytes",
     "da_supported_head_dims",
     "da_last_error",
     "da_version",
@@ -68,6 +70,10 @@ def load():
                                                  cf, vp, vp, vp, sz, vp, sz, vp]
     lib.da_workspace_bytes_fp8kv.restype = sz
     lib.da_workspace_bytes_fp8kv.argtypes = [sz, sz, sz, sz, sz, sz, sz, sz]
+    lib.da_probe_stream_read.restype = ci
+    lib.da_probe_stream_read.argtypes = [vp, sz, vp, vp]
+    lib.da_probe_stream_read_bytes.restype = sz
+    lib.da_probe_stream_read_bytes.argtypes = [sz]
     ip = ctypes.POINTER(ci)
     lib.da_plan.restype = ci
     lib.da_plan.argtypes = [sz, sz, sz, sz, sz, sz, ci, sz, ip, ip, ip, ip]

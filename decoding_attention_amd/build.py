@@ -23,6 +23,7 @@ SOURCES = [
     "da_gqa_mfma.hip",
     "da_sweep_kv8.hip",
     "da_gqa_mfma_kv8.hip",
+    "da_probe.hip",
 ]
 
 # packed-fp32 VALU forms are switched off on purpose: only scalar fp32 arithmetic is emitted.
