@@ -21,6 +21,7 @@ EXPORTED_SYMBOLS = (
     "da_workspace_bytes_fp8kv",
     "da_plan",
     "da_probe_stream_read",
+    "da_probe_sweep_only",
     "da_probe_stream_read_bytes",
     "da_supported_head_dims",
     "da_last_error",
@@ -72,6 +73,8 @@ def load():
     lib.da_workspace_bytes_fp8kv.argtypes = [sz, sz, sz, sz, sz, sz, sz, sz]
     lib.da_probe_stream_read.restype = ci
     lib.da_probe_stream_read.argtypes = [vp, sz, vp, vp]
+    lib.da_probe_sweep_only.restype = ci
+    lib.da_probe_sweep_only.argtypes = [vp, vp, vp, vp, vp, sz, sz, sz, sz, sz, sz, ci, ci, sz, vp, sz, vp]
     lib.da_probe_stream_read_bytes.restype = sz
     lib.da_probe_stream_read_bytes.argtypes = [sz]
     ip = ctypes.POINTER(ci)

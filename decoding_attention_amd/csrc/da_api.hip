@@ -262,6 +262,7 @@ struct Paging {
 
 // Element format of K/V: 16-bit like Q, or FP8 (e4m3) with per-KV-head de-quantisation factors (null = 1).
 struct KvFormat {
+    bool sweep_only = false;  // measurement: leave the split partials in the workspace, do not merge them
     bool fp8 = false;
     const float* k_scale = nullptr;
     const float* v_scale = nullptr;
@@ -369,7 +370,7 @@ int run_attention(const void* q, const void* k, const void* v, void* o, const in
     }
     if (e != hipSuccess) return fail(DA_ERR_HIP, "sweep kernel launch: %s", hipGetErrorString(e));
 
-    if (pl.nsplit > 1) {
+    if (pl.nsplit > 1 && !kf.sweep_only) {
         da::ReduceParams rp;
         rp.o = o;
         rp.cu_seq_k = cu_seq_k;
@@ -426,6 +427,15 @@ int da_decoding_attn_ex(const void* q, const void* k, const void* v, void* o, co
                         void* workspace, size_t workspace_bytes, void* hip_stream) {
     return run_attention(q, k, v, o, cu_seq_k, Paging{}, KvFormat{}, max_seq_k, batch, head_q, head_k, dim, dim_v, is_alibi,
                          is_bf16, softmax_scale, alibi_slopes, total_k, workspace, workspace_bytes, hip_stream);
+}
+
+int da_probe_sweep_only(const void* q, const void* k, const void* v, void* o, const int32_t* cu_seq_k, size_t max_seq_k,
+                        size_t batch, size_t head_q, size_t head_k, size_t dim, size_t dim_v, int is_alibi, int is_bf16,
+                        size_t total_k, void* workspace, size_t workspace_bytes, void* hip_stream) {
+    KvFormat kf;
+    kf.sweep_only = true;
+    return run_attention(q, k, v, o, cu_seq_k, Paging{}, kf, max_seq_k, batch, head_q, head_k, dim, dim_v, is_alibi,
+                         is_bf16, 0.0f, nullptr, total_k, workspace, workspace_bytes, hip_stream);
 }
 
 int da_decoding_attn_paged(const void* q, const void* k_pages, const void* v_pages, void* o,
