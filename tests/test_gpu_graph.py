@@ -1,0 +1,67 @@
+"""The op under HIP graph capture: the call only enqueues kernels (no allocation of its own when the caller brings
+the workspace, no memset, no host synchronisation), so it can be captured once and replayed.
+
+Each replay is checked against the eager result for the inputs of that moment, with eager work and synchronisation
+between the replays.
+"""
+import pytest
+import torch
+
+from decoding_attention_amd import decoding_attn_fwd, decoding_attn_paged_fwd
+from decoding_attention_amd import workloads as wl
+
+pytestmark = pytest.mark.gpu
+
+DEV = "cuda:0"
+
+
+def _replay_matches_eager(run, tensors_to_perturb, out_of):
+    """Capture run() once; then, several times: change the inputs in place, replay, compare with an eager call."""
+    s = torch.cuda.Stream()
+    s.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(s):
+        for _ in range(2):  # warm-up outside the capture (lazy initialisation, allocator state)
+            run()
+    torch.cuda.current_stream().wait_stream(s)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        captured = run()
+    torch.cuda.synchronize()
+    g = torch.Generator(device="cpu").manual_seed(1)
+    for step in range(4):
+        for t in tensors_to_perturb:
+            t.copy_(torch.randn(t.shape, generator=g).to(t.dtype))
+        graph.replay()
+        torch.cuda.synchronize()
+        got = out_of(captured).clone()
+        want = out_of(run())  # eager, same inputs
+        torch.cuda.synchronize()
+        assert torch.equal(got.view(torch.int16), want.view(torch.int16)), f"replay {step}"
+
+
+@pytest.mark.parametrize("shape", ["gqa_split", "mha_unsplit", "mla"])
+def test_packed_call_replays_from_a_graph(shape):
+    if shape == "gqa_split":
+        w = wl.make_workload(8, 32, 8, 128, 128, 2048, torch.bfloat16, seed=4, varlen=True)
+    elif shape == "mha_unsplit":
+        w = wl.make_workload(64, 8, 8, 128, 128, 128, torch.float16, seed=4)
+    else:
+        w = wl.config_mla(4, 700, seed=4)
+    wd = w.to(DEV)
+
+    def run():
+        return decoding_attn_fwd(wd.q, wd.k, wd.v, wd.cu_seq_k, w.max_seq_k, w.dim_v, w.is_alibi)
+
+    _replay_matches_eager(run, [wd.q, wd.k] + ([] if wd.v is None else [wd.v]), lambda o: o)
+
+
+def test_paged_call_replays_from_a_graph():
+    w = wl.make_workload(8, 32, 8, 128, 128, 1500, torch.float16, seed=6, varlen=True)
+    pk = wl.to_pages(w, 64, seed=6, poison=False).to(DEV)
+    q = w.q.to(DEV)
+
+    def run():
+        return decoding_attn_paged_fwd(q, pk.k_pages, pk.v_pages, pk.block_table, pk.seq_lens, w.max_seq_k, 128, False)
+
+    _replay_matches_eager(run, [q, pk.k_pages, pk.v_pages], lambda o: o)
