@@ -1,0 +1,49 @@
+"""K/V buffers beyond 4 GiB: byte offsets past 2^32 in every kernel's addressing.
+
+The inputs are drawn on the GPU (drawing 4 G elements on the host would dominate the test); the sequences that are
+checked are copied back and go through the CPU oracle.
+"""
+import pytest
+import torch
+
+from decoding_attention_amd import _lib, decoding_attn_fwd
+from decoding_attention_amd import workloads as wl
+from tests.gpu_util import check_against_oracle
+
+pytestmark = pytest.mark.gpu
+
+DEV = "cuda:0"
+
+
+def _check_rows(q, k, v, cu, o, rows, dim_v, name):
+    cu_l = cu.tolist()
+    ks = [k[cu_l[b]:cu_l[b + 1]].cpu() for b in rows]
+    vs = None if v is None else [v[cu_l[b]:cu_l[b + 1]].cpu() for b in rows]
+    lens = torch.tensor([x.shape[0] for x in ks], dtype=torch.int32)
+    w = wl.Workload(name, q[rows].cpu(), torch.cat(ks), None if vs is None else torch.cat(vs), wl.get_cu_seq(lens),
+                    int(lens.max()), dim_v, False, lens.tolist())
+    check_against_oracle(w, o[rows].cpu())
+
+
+@pytest.mark.parametrize("kind", ["gqa", "mha", "mla"])
+def test_offsets_beyond_4_gib(kind):
+    g = torch.Generator(device=DEV).manual_seed(5)
+    if kind == "gqa":      # grouped MFMA kernel: 2 x 5.4 GB
+        batch, hq, hk, d, dv, sk, dtype = 320, 32, 8, 128, 128, 8192, torch.bfloat16
+    elif kind == "mha":    # VALU sweep (short sequences): 2 x 5.4 GB
+        batch, hq, hk, d, dv, sk, dtype = 10240, 32, 32, 128, 128, 64, torch.float16
+    else:                  # latent MFMA kernel: 4.8 GB
+        batch, hq, hk, d, dv, sk, dtype = 512, 128, 1, 576, 512, 8192, torch.float16
+    total = batch * sk
+    assert total * hk * d * 2 > (1 << 32)
+    q = torch.randn(batch, hq, d, generator=g, device=DEV, dtype=dtype)
+    k = torch.randn(total, hk, d, generator=g, device=DEV, dtype=dtype)
+    v = None if kind == "mla" else torch.randn(total, hk, dv, generator=g, device=DEV, dtype=dtype)
+    cu = torch.arange(batch + 1, dtype=torch.int32) * sk
+    assert _lib.plan(sk, batch, hq, hk, d, dv)["kind"] == {"gqa": 3, "mha": 1, "mla": 2}[kind]
+    o = decoding_attn_fwd(q, k, v, cu.to(DEV), sk, dv, False)
+    torch.cuda.synchronize()
+    assert torch.isfinite(o.float()).all()
+    # first, last, and the sequences on either side of the 4 GiB byte offset
+    edge = (1 << 32) // (sk * hk * d * 2)
+    _check_rows(q, k, v, cu, o, [0, edge - 1, edge, edge + 1, batch - 1], dv, "large_" + kind)

@@ -81,6 +81,24 @@ def test_plan_total_k_hint_only_shortens_splits_of_ragged_batches():
     assert ws == batch * 32 * ragged["nsplit"] * (128 + 2) * 4
 
 
+def test_workspace_sizes_of_the_paged_and_fp8_variants():
+    lib = _lib.load()
+    shape = (4096, 64, 32, 8, 128, 128)
+    packed = lib.da_workspace_bytes(*shape, 0)
+    # pages of a multiple of 32 tokens take the packed layout's kernels and plan
+    assert lib.da_workspace_bytes_paged(*shape, 0, 64) == packed
+    assert lib.da_workspace_bytes_paged(*shape, 0, 256) == packed
+    # smaller pages run the VALU sweep (4 query heads per work-group): its own split plan, still a whole number
+    # of (row, split) partials of dim_v + 2 floats
+    small = lib.da_workspace_bytes_paged(*shape, 0, 16)
+    assert small > 0 and small % (64 * 32 * (128 + 2) * 4) == 0
+    assert lib.da_workspace_bytes_fp8kv(*shape, 0, 0) == packed          # same kernel kind, same plan
+    # the latent form has no FP8 MFMA kernel: the VALU sweep's plan, covering both the aliased and the distinct V
+    mla = (4096, 16, 128, 1, 576, 512)
+    assert lib.da_workspace_bytes_fp8kv(*mla, 0, 0) > 0
+    assert lib.da_workspace_bytes_fp8kv(128, 4, 6, 4, 64, 64, 0, 0) == 0   # head_q not a multiple of head_k
+
+
 def test_plan_rejects_bad_shapes():
     with pytest.raises(RuntimeError):
         _lib.plan(128, 1, 6, 4, 64, 64)
