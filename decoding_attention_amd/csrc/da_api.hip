@@ -43,12 +43,13 @@ int env_int(const char* name, int dflt) {
 // stops being split further; DA_MAX_CHUNK / DA_MIN_CHUNK: bounds on tokens per split.
 struct Tunables {
     int target_wgs, mfma_target_wgs, max_chunk, min_chunk, ragged_chunk, force_kind, group_min_ratio, wave_per_head,
-        mla_heads;
+        mla_heads, gqa_heads;
     Tunables() {
         target_wgs = env_int("DA_TARGET_WGS", 512);
         mfma_target_wgs = env_int("DA_MFMA_TARGET_WGS", 256);
         max_chunk = env_int("DA_MAX_CHUNK", 1024);
         min_chunk = env_int("DA_MIN_CHUNK", 512);
+        gqa_heads = env_int("DA_GQA_HEADS", 0);  // query heads per work-group and KV head of the grouped kernel (16/32), 0 = by shape
         mla_heads = env_int("DA_MLA_HEADS", 0);  // query heads per work-group of the latent kernel (32/64/128), 0 = by shape
         ragged_chunk = env_int("DA_RAGGED_CHUNK", 256);  // tokens per split when the lengths are known to be ragged
         force_kind = env_int("DA_FORCE_KIND", 0);
@@ -119,14 +120,16 @@ Plan make_plan(size_t max_seq_k, size_t batch, size_t head_q, size_t head_k, siz
         target_wgs = tun().mfma_target_wgs;  // one 4-wave work-group fills a CU
     } else if (dim <= 256 && !force_sweep && (!kv_fp8 || dim % 64 == 0) &&
                (ratio >= tun().group_min_ratio ||
-                (tun().group_min_ratio > 1 && max_seq_k >= 1024 &&
+                (tun().group_min_ratio > 1 && (max_seq_k >= 1024 || dim <= 96) &&
                  (long long)batch * (long long)head_k * (long long)max_seq_k >= (1ll << 21)))) {
         // Two or more query heads per KV head, or a single one over long sequences of a large batch: the MFMA sweep streams K/V
         // a few percent faster than the VALU sweep even though most of its matrix columns are idle (measured:
-        // ratio 2, 2048 tokens: 201 -> 185 us; ratio 1, batch 64 x 2048 tokens: 375 -> 364 us; at 128 tokens or batch 1 the VALU
-        // sweep wins).
+        // ratio 2, 2048 tokens: 201 -> 185 us; ratio 1, batch 64 x 2048 tokens: 375 -> 364 us; at batch 1 the VALU sweep wins, and
+        // for short sequences it is the steadier one at d = 128 and 256 but the slower one at d = 64 and 96:
+        // d 96, 256 x 512 tokens: 366 -> 275 us).
         pl.kind = kKindGroup;
         pl.rt = ratio > 16 ? 32 : 16;
+        if (tun().gqa_heads == 16 || tun().gqa_heads == 32) pl.rt = tun().gqa_heads;
         pl.wave_per_head = head_k % 4 == 0 && tun().wave_per_head;
         trip = pl.wave_per_head ? da::kGqaTile : 4 * da::kGqaTile;
     } else {

@@ -59,6 +59,21 @@ struct Elem<bf16_tag> {
 
 __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
 
+// Maximum of a value with that of the lane 16 (32) positions away, lane ^ 16 (lane ^ 32), through the row and
+// half-wave swap instructions: plain vector ALU work, no trip through the LDS crossbar as a shuffle makes.
+__device__ __forceinline__ float max_xor16(float x) {
+    const auto r = __builtin_amdgcn_permlane16_swap(__builtin_bit_cast(unsigned, x), __builtin_bit_cast(unsigned, x),
+                                                    false, false);
+    const unsigned r0 = r[0], r1 = r[1];  // (element copies first: a bit cast straight from r[1] reads r[0])
+    return fmaxf(__builtin_bit_cast(float, r0), __builtin_bit_cast(float, r1));
+}
+__device__ __forceinline__ float max_xor32(float x) {
+    const auto r = __builtin_amdgcn_permlane32_swap(__builtin_bit_cast(unsigned, x), __builtin_bit_cast(unsigned, x),
+                                                    false, false);
+    const unsigned r0 = r[0], r1 = r[1];  // (element copies first: a bit cast straight from r[1] reads r[0])
+    return fmaxf(__builtin_bit_cast(float, r0), __builtin_bit_cast(float, r1));
+}
+
 // Eight FP8 (OCP e4m3) values -> eight 16-bit elements of the compute type.  Both conversions are exact (e4m3
 // has 3 mantissa bits and |x| <= 448), so an FP8 K/V cache feeds the same arithmetic as a 16-bit one.
 template <typename Tag>

@@ -66,10 +66,13 @@ template <int DV>
 constexpr int gqa_v_pitch() { return DV * 2 + 32; }  // LDS row pitch of the V tile: conflict-free transposed reads
 
 template <int DV>
+constexpr int gqa_merge_pitch() { return DV + 4; }  // floats per row of the merge area: conflict-free row writes
+
+template <int DV>
 constexpr size_t gqa_lds_bytes(int nt) {
-    // V tiles of the four waves, reused for the final merge ([4][heads][DV] floats + (m, l))
+    // V tiles of the four waves, reused for the final merge ([4][heads][pitch] floats + (m, l))
     const size_t vt = 4 * (size_t)kGqaTile * gqa_v_pitch<DV>();
-    const size_t mg = 4 * (size_t)(16 * nt) * (DV + 2) * sizeof(float);
+    const size_t mg = 4 * (size_t)(16 * nt) * (gqa_merge_pitch<DV>() + 2) * sizeof(float);
     return vt > mg ? vt : mg;
 }
 
@@ -257,10 +260,10 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(MINW))) voi
         // online softmax; token of s[mt][nt][r]: tok0 + mt*16 + g*4 + r, head nt*16 + n
         vec8 pf[NT];
         const bool tail = tok0 + kGqaTile > c1;
+        float x[NT][8], mx[NT];
 #pragma unroll
         for (int nt = 0; nt < NT; ++nt) {
-            float x[8];
-            float mx = -INFINITY;
+            mx[nt] = -INFINITY;
             if (p.is_alibi || tail) {
 #pragma unroll
                 for (int mt = 0; mt < 2; ++mt)
@@ -269,35 +272,46 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(MINW))) voi
                         const int tok = tok0 + mt * 16 + g * 4 + r;
                         float v = s[mt][nt][r] * sl + slope[nt] * (float)(tok - (len - 1));
                         if (tok >= c1) v = -INFINITY;
-                        x[mt * 4 + r] = v;
-                        mx = fmaxf(mx, v);
+                        x[nt][mt * 4 + r] = v;
+                        mx[nt] = fmaxf(mx[nt], v);
                     }
             } else {
 #pragma unroll
                 for (int mt = 0; mt < 2; ++mt)
 #pragma unroll
                     for (int r = 0; r < 4; ++r) {
-                        x[mt * 4 + r] = s[mt][nt][r] * sl;
-                        mx = fmaxf(mx, x[mt * 4 + r]);
+                        x[nt][mt * 4 + r] = s[mt][nt][r] * sl;
+                        mx[nt] = fmaxf(mx[nt], x[nt][mt * 4 + r]);
                     }
             }
-            mx = fmaxf(mx, __shfl_xor(mx, 16));
-            mx = fmaxf(mx, __shfl_xor(mx, 32));
-            const bool up = mx > m[nt] + kLazy;
-            if (__any(up)) {
-                const float mn = up ? mx : m[nt];
+        }
+        // the four 16-lane groups hold different tokens of the same heads
+        bool up[NT], any_up = false;
+#pragma unroll
+        for (int nt = 0; nt < NT; ++nt) {
+            mx[nt] = max_xor32(max_xor16(mx[nt]));
+            up[nt] = mx[nt] > m[nt] + kLazy;
+            any_up |= up[nt];
+        }
+        if (__any(any_up)) {
+#pragma unroll
+            for (int nt = 0; nt < NT; ++nt) {
+                const float mn = up[nt] ? mx[nt] : m[nt];
                 const float alpha = fast_exp2(m[nt] - mn);
                 m[nt] = mn;
                 l[nt] *= alpha;
 #pragma unroll
                 for (int ct = 0; ct < CT; ++ct) acc[nt][ct] *= alpha;
             }
+        }
+#pragma unroll
+        for (int nt = 0; nt < NT; ++nt) {
 #pragma unroll
             for (int j = 0; j < 8; ++j) {
-                x[j] = fast_exp2(x[j] - m[nt]);
-                l[nt] += x[j];
+                x[nt][j] = fast_exp2(x[nt][j] - m[nt]);
+                l[nt] += x[nt][j];
             }
-            pf[nt] = MM::pack8(x);  // k index j <-> token g*4+j (j<4), 16+g*4+(j-4) (j>=4)
+            pf[nt] = MM::pack8(x[nt]);  // k index j <-> token g*4+j (j<4), 16+g*4+(j-4) (j>=4)
         }
 
         // O^T += V^T . P^T
@@ -359,42 +373,54 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(MINW))) voi
         return;
     }
 
-    // merge the four waves through LDS (the V tiles are dead by now)
+    // merge the four waves through LDS (the V tiles are dead by now).  Rows are padded by four floats so that the
+    // sixteen heads a 16-lane group writes (one row each, same columns) fall into different banks.
     constexpr int MW = 4;
+    constexpr int AP = gqa_merge_pitch<DV>();
     __syncthreads();
-    float* const lds_acc = reinterpret_cast<float*>(smem);                 // [MW][HG][DV]
-    float* const lds_ml = lds_acc + MW * HG * DV;                          // [MW][HG][2]
+    float* const lds_acc = reinterpret_cast<float*>(smem);                 // [MW][HG][AP]
+    float* const lds_ml = lds_acc + MW * HG * AP;                          // [MW][HG][2]
 #pragma unroll
     for (int nt = 0; nt < NT; ++nt) {
         const int hh = nt * 16 + n;
 #pragma unroll
         for (int ct = 0; ct < CT; ++ct)
-            *reinterpret_cast<f32x4*>(lds_acc + ((size_t)wave * HG + hh) * DV + ct * 16 + g * 4) = acc[nt][ct];
-        if (g == 0) {
-            lds_ml[(wave * HG + hh) * 2 + 0] = m[nt];
-            lds_ml[(wave * HG + hh) * 2 + 1] = l[nt];
-        }
+            *reinterpret_cast<f32x4*>(lds_acc + (wave * HG + hh) * AP + ct * 16 + g * 4) = acc[nt][ct];
+        if (g == 0) *reinterpret_cast<float2*>(lds_ml + (wave * HG + hh) * 2) = make_float2(m[nt], l[nt]);
     }
     __syncthreads();
 
-    for (int idx = threadIdx.x; idx < nh * DV; idx += blockDim.x) {
-        const int r = idx / DV, col = idx % DV;
-        float mm = lds_ml[(0 * HG + r) * 2];
+    // one thread per (head, four columns): the weights of a head are computed once per thread, and a wave's
+    // lanes cover two whole rows, so the weight reads are broadcasts and the rows are read 16 bytes per lane
+    constexpr int C4 = DV / 4;
+    for (int idx = threadIdx.x; idx < nh * C4; idx += blockDim.x) {
+        const int r = idx / C4, col = (idx % C4) * 4;
+        float2 ml[MW];
 #pragma unroll
-        for (int w = 1; w < MW; ++w) mm = fmaxf(mm, lds_ml[(w * HG + r) * 2]);
-        float num = 0.0f, den = 0.0f;
+        for (int w = 0; w < MW; ++w) ml[w] = *reinterpret_cast<const float2*>(lds_ml + (w * HG + r) * 2);
+        float mm = ml[0].x;
+#pragma unroll
+        for (int w = 1; w < MW; ++w) mm = fmaxf(mm, ml[w].x);
+        f32x4 num = {0.0f, 0.0f, 0.0f, 0.0f};
+        float den = 0.0f;
 #pragma unroll
         for (int w = 0; w < MW; ++w) {
-            const float wt = fast_exp2(lds_ml[(w * HG + r) * 2] - mm);
-            num += wt * lds_acc[((size_t)w * HG + r) * DV + col];
-            den += wt * lds_ml[(w * HG + r) * 2 + 1];
+            const float wt = fast_exp2(ml[w].x - mm);
+            num += *reinterpret_cast<const f32x4*>(lds_acc + (w * HG + r) * AP + col) * wt;
+            den += wt * ml[w].y;
         }
         const int h = h_base + r;
         if (p.nsplit == 1) {
-            o16[((size_t)b * p.head_q + h) * DV + col] = EL::from_f32(num * vs / den);
+            const float inv = vs / den;
+            ushort4 w16;
+            w16.x = EL::from_f32(num[0] * inv);
+            w16.y = EL::from_f32(num[1] * inv);
+            w16.z = EL::from_f32(num[2] * inv);
+            w16.w = EL::from_f32(num[3] * inv);
+            *reinterpret_cast<ushort4*>(o16 + ((size_t)b * p.head_q + h) * DV + col) = w16;
         } else {
             const size_t part = ((size_t)b * p.head_q + h) * p.nsplit + split;
-            p.ws_o[part * DV + col] = num * vs;
+            *reinterpret_cast<f32x4*>(p.ws_o + part * DV + col) = num * vs;
             if (col == 0) {
                 p.ws_ml[part * 2 + 0] = mm;
                 p.ws_ml[part * 2 + 1] = den;

@@ -372,7 +372,7 @@ __global__ __launch_bounds__(64 * NWV) void mfma_latent_kernel(const SweepParams
                 mx = fmaxf(mx, pv[r]);
             }
         }
-        mx = fmaxf(mx, __shfl_xor(mx, 32));
+        mx = max_xor32(mx);
         const bool up = mx > m + kLazy;
         if (__any(up)) {
             const float mn = up ? mx : m;
