@@ -43,7 +43,7 @@ int env_int(const char* name, int dflt) {
 // stops being split further; DA_MAX_CHUNK / DA_MIN_CHUNK: bounds on tokens per split.
 struct Tunables {
     int target_wgs, mfma_target_wgs, max_chunk, min_chunk, ragged_chunk, force_kind, group_min_ratio, wave_per_head,
-        mla_heads, gqa_heads;
+        mla_heads, gqa_heads, flat_wgs, flat_min_tokens;
     Tunables() {
         target_wgs = env_int("DA_TARGET_WGS", 512);
         mfma_target_wgs = env_int("DA_MFMA_TARGET_WGS", 256);
@@ -52,6 +52,9 @@ struct Tunables {
         gqa_heads = env_int("DA_GQA_HEADS", 0);  // query heads per work-group and KV head of the grouped kernel (16/32), 0 = by shape
         mla_heads = env_int("DA_MLA_HEADS", 0);  // query heads per work-group of the latent kernel (32/64/128), 0 = by shape
         ragged_chunk = env_int("DA_RAGGED_CHUNK", 256);  // tokens per split when the lengths are known to be ragged
+        // balanced grid of the grouped kernel for ragged batches: work-groups in all (0 = off), fewest tokens each
+        flat_wgs = env_int("DA_FLAT_WGS", 512);
+        flat_min_tokens = env_int("DA_FLAT_MIN_TOKENS", 256);
         force_kind = env_int("DA_FORCE_KIND", 0);
         wave_per_head = env_int("DA_WAVE_PER_HEAD", 1);
         group_min_ratio = env_int("DA_GROUP_MIN_RATIO", 2);  // smallest head group that takes the grouped MFMA sweep
@@ -75,6 +78,10 @@ struct Plan {
     int chunk = 0;
     size_t ws_bytes = 0;
     bool wave_per_head = false;  // grouped kernel: the four waves of a work-group take four KV heads
+    // Balanced grid (grouped kernel, ragged packed batch whose total length the caller gave): flat_wgs work-groups
+    // per (KV heads, head group), each over flat_tokens consecutive tokens of the concatenated sequences; nsplit
+    // is then the most partials one sequence can have, chunk == flat_tokens.
+    int flat_tokens = 0, flat_wgs = 0;
 };
 
 bool supported_dims(size_t dim, size_t dim_v) {
@@ -99,8 +106,9 @@ int rows_per_trip(size_t dim) {
 // tiles_contiguous: every aligned run of 32 tokens is contiguous in memory (always true for the packed layout; for
 // paged K/V only when a page holds a multiple of 32 tokens).  The two MFMA kernels fetch whole tiles and need it.
 // kv_fp8: K/V are FP8; the latent MFMA kernel has no FP8 form and the grouped kernel needs dim % 64 == 0.
+// packed: K/V are in the packed layout addressed through cu_seq_k (the balanced grid needs the prefix offsets).
 Plan make_plan(size_t max_seq_k, size_t batch, size_t head_q, size_t head_k, size_t dim, size_t dim_v,
-               bool v_distinct, size_t total_k, bool tiles_contiguous = true, bool kv_fp8 = false) {
+               bool v_distinct, size_t total_k, bool tiles_contiguous = true, bool kv_fp8 = false, bool packed = true) {
     Plan pl;
     const int ratio = (int)(head_q / head_k);
     int trip;
@@ -142,6 +150,23 @@ Plan make_plan(size_t max_seq_k, size_t batch, size_t head_q, size_t head_k, siz
     pl.groups = (ratio + pl.rt - 1) / pl.rt;
     const long long base = (long long)batch * (long long)(pl.wave_per_head ? head_k / 4 : head_k) * pl.groups;
     const bool ragged = total_k > 0 && (long long)total_k * 10 < (long long)batch * (long long)max_seq_k * 9;
+    if (pl.kind == kKindGroup && ragged && packed && tun().flat_wgs > 0 && total_k < ((size_t)1 << 30) &&
+        total_k >= 64 * batch) {
+        // Ragged batch of known total length: equal shares of the concatenated tokens instead of fixed splits of
+        // every sequence (64 sequences of 1..8192 tokens, 32/8 heads: see the tunables' documentation for the measured gain).
+        const long long ygrid = base / (long long)batch;
+        long long w = std::max<long long>(1, tun().flat_wgs / ygrid);
+        const long long unit = trip;  // a work-group's waves advance `trip` tokens per step together
+        long long t = ((long long)total_k + w - 1) / w;
+        t = std::max<long long>((t + unit - 1) / unit * unit, std::max<long long>(tun().flat_min_tokens, unit));
+        w = std::min<long long>(65535, ((long long)total_k + t - 1) / t);
+        pl.flat_tokens = (int)t;
+        pl.flat_wgs = (int)w;
+        pl.chunk = (int)t;
+        pl.nsplit = (int)std::min<long long>(w, ((long long)max_seq_k + t - 1) / t + 1);
+        pl.ws_bytes = (size_t)batch * head_q * pl.nsplit * (dim_v + 2) * sizeof(float);
+        return pl;
+    }
     int min_chunk = std::max(mfma ? 256 : tun().min_chunk, trip);
     if (!mfma) {
         // 512-token splits run best; go down to 256 only when that is needed to give every CU a work-group
@@ -238,8 +263,8 @@ size_t da_workspace_bytes_paged(size_t max_seq_k, size_t batch, size_t head_q, s
                                 size_t total_k, size_t page_size) {
     if (head_k == 0 || head_q % head_k != 0 || !supported_dims(dim, dim_v)) return 0;
     const bool contiguous = page_size % 32 == 0;
-    const size_t a = make_plan(max_seq_k, batch, head_q, head_k, dim, dim_v, false, total_k, contiguous).ws_bytes;
-    const size_t b = make_plan(max_seq_k, batch, head_q, head_k, dim, dim_v, true, total_k, contiguous).ws_bytes;
+    const size_t a = make_plan(max_seq_k, batch, head_q, head_k, dim, dim_v, false, total_k, contiguous, false, false).ws_bytes;
+    const size_t b = make_plan(max_seq_k, batch, head_q, head_k, dim, dim_v, true, total_k, contiguous, false, false).ws_bytes;
     return a > b ? a : b;
 }
 
@@ -247,8 +272,9 @@ size_t da_workspace_bytes_fp8kv(size_t max_seq_k, size_t batch, size_t head_q, s
                                 size_t dim_v, size_t total_k, size_t page_size) {
     if (head_k == 0 || head_q % head_k != 0 || !supported_dims(dim, dim_v)) return 0;
     const bool contiguous = page_size == 0 || page_size % 32 == 0;
-    const size_t a = make_plan(max_seq_k, batch, head_q, head_k, dim, dim_v, false, total_k, contiguous, true).ws_bytes;
-    const size_t b = make_plan(max_seq_k, batch, head_q, head_k, dim, dim_v, true, total_k, contiguous, true).ws_bytes;
+    const bool packed = page_size == 0;
+    const size_t a = make_plan(max_seq_k, batch, head_q, head_k, dim, dim_v, false, total_k, contiguous, true, packed).ws_bytes;
+    const size_t b = make_plan(max_seq_k, batch, head_q, head_k, dim, dim_v, true, total_k, contiguous, true, packed).ws_bytes;
     return a > b ? a : b;
 }
 
@@ -300,7 +326,8 @@ int run_attention(const void* q, const void* k, const void* v, void* o, const in
 
     hipStream_t stream = reinterpret_cast<hipStream_t>(hip_stream);
     const bool tiles_contiguous = !pg.table || pg.page_size % 32 == 0;
-    const Plan pl = make_plan(max_seq_k, batch, head_q, head_k, dim, dim_v, v != nullptr, total_k, tiles_contiguous, kf.fp8);
+    const Plan pl = make_plan(max_seq_k, batch, head_q, head_k, dim, dim_v, v != nullptr, total_k, tiles_contiguous, kf.fp8,
+                              pg.table == nullptr);
     if ((size_t)head_k * pl.groups > 65535)
         return fail(DA_ERR_INVALID_ARGUMENT, "head_k * groups exceeds the grid limit 65535");
 
@@ -349,9 +376,12 @@ int run_attention(const void* q, const void* k, const void* v, void* o, const in
     sp.max_blocks = (int)pg.max_blocks;
     sp.k_page = (int64_t)pg.k_page;
     sp.v_page = v ? (int64_t)pg.v_page : (int64_t)pg.k_page;
+    sp.flat_tokens = pl.flat_tokens;
+    sp.batch = (int)batch;
 
-    const dim3 grid((unsigned)pl.nsplit, (unsigned)((pl.wave_per_head ? head_k / 4 : head_k) * pl.groups),
-                    (unsigned)batch);
+    const dim3 grid((unsigned)(pl.flat_tokens ? pl.flat_wgs : pl.nsplit),
+                    (unsigned)((pl.wave_per_head ? head_k / 4 : head_k) * pl.groups),
+                    (unsigned)(pl.flat_tokens ? 1 : batch));
     hipError_t e;
     if (kf.fp8) {
         if (pl.kind == kKindGroup)
@@ -373,7 +403,7 @@ int run_attention(const void* q, const void* k, const void* v, void* o, const in
     }
     if (e != hipSuccess) return fail(DA_ERR_HIP, "sweep kernel launch: %s", hipGetErrorString(e));
 
-    if (pl.nsplit > 1 && !kf.sweep_only) {
+    if ((pl.nsplit > 1 || pl.flat_tokens) && !kf.sweep_only) {
         da::ReduceParams rp;
         rp.o = o;
         rp.cu_seq_k = cu_seq_k;
@@ -384,6 +414,8 @@ int run_attention(const void* q, const void* k, const void* v, void* o, const in
         rp.dim_v = (int)dim_v;
         rp.nsplit = pl.nsplit;
         rp.chunk = pl.chunk;
+        rp.flat_tokens = pl.flat_tokens;
+        rp.flat_wgs = pl.flat_wgs;
         e = da::launch_reduce(rp, is_bf16 != 0, (int)(batch * head_q), stream);
         if (e != hipSuccess) return fail(DA_ERR_HIP, "merge kernel launch: %s", hipGetErrorString(e));
     }

@@ -151,6 +151,10 @@ struct SweepParams {
     // The kernels fold k_scale into the softmax scale and v_scale into the final normalisation.
     const float* k_scale;
     const float* v_scale;
+    // Balanced form of the grouped-head kernel's grid (0 = off): tokens per work-group of the line of all
+    // sequences' tokens, and the number of sequences.
+    int flat_tokens;
+    int batch;
 };
 
 __device__ __forceinline__ float head_scale(const float* scales, int hk) { return scales ? scales[hk] : 1.0f; }
@@ -162,6 +166,7 @@ struct ReduceParams {
     const float* ws_o;
     const float* ws_ml;
     int head_q, dim_v, nsplit, chunk;
+    int flat_tokens, flat_wgs;  // balanced form of the sweep's grid (flat_tokens > 0): tokens per work-group, work-groups
 };
 
 // First token (row of the packed K/V buffers) and length of sequence b; paged sequences start at row 0 of their

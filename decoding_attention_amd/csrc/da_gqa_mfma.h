@@ -85,8 +85,13 @@ constexpr size_t gqa_lds_bytes(int nt) {
 // KV8: K and V hold FP8 (e4m3) elements.  Loads stay 16 bytes per lane (sixteen elements: the k indices of two
 // consecutive k-steps, so the Q fragments are gathered with the matching index order) and the elements are
 // converted exactly to the compute type on their way into the matrix instruction (K) or the LDS tile (V).
-template <typename Tag, int D, int DV, int NT, bool PREFETCH, bool WH, int MINW, bool KV8 = false>
-__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(MINW))) void gqa_mfma_kernel(const SweepParams p) {
+// One segment of work: tokens [c0, c1) of sequence b (first row `start`, `len` tokens) for the KV heads and head
+// group blockIdx.y selects.  `direct`: the segment is the whole sequence, so the result goes to o; otherwise the
+// un-normalised partial goes to workspace slot `split` of the sequence.
+template <typename Tag, int D, int DV, int NT, bool PREFETCH, bool WH, bool KV8>
+__device__ __forceinline__ void gqa_segment(const SweepParams& p, uint8_t* const smem, const int b, const int start,
+                                            const int len, const int c0, const int c1, const int split,
+                                            const bool direct) {
     using MM = Mma16<Tag>;
     using vec8 = typename MM::vec8;
     using EL = Elem<Tag>;
@@ -105,23 +110,14 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(MINW))) voi
     static_assert(D % 32 == 0 && DV % 16 == 0 && (kGqaTile * CPR) % 64 == 0, "shape");
     static_assert(!KV8 || (D % 64 == 0 && (kGqaTile * CPRL) % 64 == 0), "FP8 K/V: two k-steps per 16-byte load");
 
-    extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
-
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int n = lane & 15;
     const int g = lane >> 4;
 
-    const int split = blockIdx.x;
     const int hk = WH ? (blockIdx.y / p.groups) * 4 + wave : blockIdx.y / p.groups;
     const int grp = blockIdx.y % p.groups;
-    const int b = blockIdx.z;
     const int tw = WH ? 0 : wave;  // this wave's position among the waves that share the tokens
-
-    int start, len;
-    seq_range(p, b, start, len);
-    const int c0 = split * p.chunk;
-    const int c1 = (split == p.nsplit - 1) ? len : min(len, c0 + p.chunk);
 
     const int h_base = hk * p.ratio + grp * HG;
     const int nh = min(HG, p.ratio - grp * HG);  // live heads of this group
@@ -132,7 +128,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(MINW))) voi
         // work-group covers NR runs of nh heads, one per KV head
         constexpr int NR = WH ? 4 : 1;
         const int wg_h_first = (WH ? (blockIdx.y / p.groups) * 4 : hk) * p.ratio + grp * HG;
-        if (p.nsplit == 1) zero_rows<DV>(p, b, wg_h_first, nh, NR, p.ratio);
+        if (direct) zero_rows<DV>(p, b, wg_h_first, nh, NR, p.ratio);
         return;
     }
 
@@ -346,7 +342,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(MINW))) voi
             const int hh = nt * 16 + n;
             if (hh < nh) {
                 const int h = h_base + hh;
-                if (p.nsplit == 1) {
+                if (direct) {
                     const float inv = vs / l[nt];
                     uint16_t* orow = o16 + ((size_t)b * p.head_q + h) * DV + g * 4;
 #pragma unroll
@@ -410,7 +406,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(MINW))) voi
             den += wt * ml[w].y;
         }
         const int h = h_base + r;
-        if (p.nsplit == 1) {
+        if (direct) {
             const float inv = vs / den;
             ushort4 w16;
             w16.x = EL::from_f32(num[0] * inv);
@@ -426,6 +422,52 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(MINW))) voi
                 p.ws_ml[part * 2 + 1] = den;
             }
         }
+    }
+}
+
+// Grid, packed or paged K/V with a fixed split length: (split, KV heads x head groups, sequence).
+// Grid, balanced form (p.flat_tokens > 0, packed K/V only): (work-group i of W, KV heads x head groups, 1).  The
+// tokens of all sequences form one line of cu_seq_k[batch] tokens; work-group i takes tokens [i T, (i+1) T) of it
+// (the last one to the end), whatever sequences they belong to, one segment per sequence it touches.  Every
+// work-group then streams the same number of bytes, which a ragged batch cut into fixed splits does not give.
+// Sequence b spans work-groups first(b) = cu[b] / T ... last(b) = (cu[b+1] - 1) / T (both capped at W - 1); its
+// segment in work-group i is partial number i - first(b), and goes straight to o when first(b) == last(b).
+template <typename Tag, int D, int DV, int NT, bool PREFETCH, bool WH, int MINW, bool KV8 = false>
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(MINW))) void gqa_mfma_kernel(const SweepParams p) {
+    extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
+    if (p.flat_tokens == 0) {
+        const int split = blockIdx.x, b = blockIdx.z;
+        int start, len;
+        seq_range(p, b, start, len);
+        const int c0 = split * p.chunk;
+        const int c1 = (split == p.nsplit - 1) ? len : min(len, c0 + p.chunk);
+        gqa_segment<Tag, D, DV, NT, PREFETCH, WH, KV8>(p, smem, b, start, len, c0, c1, split, p.nsplit == 1);
+        return;
+    }
+    const int T = p.flat_tokens, W = (int)gridDim.x, i = (int)blockIdx.x;
+    const int32_t* const cu = p.cu_seq_k;
+    const int total = cu[p.batch];
+    const int r0 = (int)min((long long)i * T, (long long)total);
+    const int r1 = (i == W - 1) ? total : (int)min((long long)r0 + T, (long long)total);
+    if (r0 >= r1) return;
+    // the sequence that holds token r0: the last b with cu[b] <= r0 (empty sequences share their offset with
+    // the next one and are passed over)
+    int lo = 0, hi = p.batch;
+    while (lo + 1 < hi) {
+        const int mid = (lo + hi) >> 1;
+        if (cu[mid] <= r0)
+            lo = mid;
+        else
+            hi = mid;
+    }
+    for (int b = lo; b < p.batch; ++b) {
+        const int s = cu[b], e = cu[b + 1];
+        if (s >= r1) break;
+        if (e <= s) continue;
+        const int first = min(s / T, W - 1), last = min((e - 1) / T, W - 1);
+        gqa_segment<Tag, D, DV, NT, PREFETCH, WH, KV8>(p, smem, b, s, e - s, max(r0, s) - s, min(r1, e) - s, i - first,
+                                                       first == last);
+        if (!WH) __syncthreads();  // the merge area of this segment is the V tile area of the next
     }
 }
 

@@ -258,7 +258,17 @@ __global__ __launch_bounds__(256) void reduce_kernel(const ReduceParams p, int r
     const int b = row / p.head_q;
     const int len = p.cu_seq_k ? p.cu_seq_k[b + 1] - p.cu_seq_k[b] : p.seq_lens[b];
     int ns = 0;
-    if (len > 0) ns = min(p.nsplit, (len + p.chunk - 1) / p.chunk);
+    if (p.flat_tokens > 0) {
+        // balanced sweep grid: the sequence's partials come from the work-groups its tokens fall into; a sequence
+        // inside one work-group was written to o by the sweep itself
+        if (len > 0) {
+            const int s = p.cu_seq_k[b];
+            ns = min((s + len - 1) / p.flat_tokens, p.flat_wgs - 1) - min(s / p.flat_tokens, p.flat_wgs - 1) + 1;
+            if (ns == 1) return;
+        }
+    } else if (len > 0) {
+        ns = min(p.nsplit, (len + p.chunk - 1) / p.chunk);
+    }
     const size_t part0 = (size_t)row * p.nsplit;
     const float2* const ml = reinterpret_cast<const float2*>(p.ws_ml) + part0;
     const float4* const src = reinterpret_cast<const float4*>(p.ws_o + part0 * p.dim_v) + c4;

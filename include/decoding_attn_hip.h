@@ -50,8 +50,10 @@ int da_decoding_attn(const void *q, const void *k, const void *v, void *o, const
  *   softmax_scale  <= 0 selects 1/sqrt(dim)
  *   alibi_slopes   device float[head_q] or NULL for the closed form; read only when is_alibi != 0
  *   total_k        number of key tokens (cu_seq_k[batch]) if the caller knows it on the host, else 0.  Only a
- *                  hint: a batch that is much shorter than batch * max_seq_k is cut into shorter sequence splits
- *                  so that it balances; results do not depend on it.  Pass the same value to da_workspace_bytes.
+ *                  hint: a batch that is much shorter than batch * max_seq_k is cut so that it balances (shorter
+ *                  sequence splits, or equal shares of the concatenated tokens across sequence boundaries);
+ *                  results are correct for any value, also one that is not the true count.  Pass the same value
+ *                  to da_workspace_bytes.
  *   workspace      device buffer of at least da_workspace_bytes(...) bytes, 16-byte aligned, or NULL to use the
  *                  library's cached one
  */

@@ -18,6 +18,27 @@ def run_hip(w, **kw):
     return o.cpu()
 
 
+def run_hip_ex(w, total_k_hint):
+    """The packed call through da_decoding_attn_ex with a caller-owned workspace and the given token-count hint
+    (the Python face always passes k.shape[0]; 0 here selects the plan of a caller who does not know it)."""
+    from decoding_attention_amd import _lib
+    lib = _lib.load()
+    dev = torch.device("cuda:0")
+    wd = w.to(dev)
+    b, hq, d = w.q.shape
+    hk = w.k.shape[1]
+    n = lib.da_workspace_bytes(w.max_seq_k, b, hq, hk, d, w.dim_v, total_k_hint)
+    ws = torch.empty(max(n, 16), dtype=torch.uint8, device=dev)
+    o = torch.full((b, hq, w.dim_v), float("nan"), dtype=w.q.dtype, device=dev)
+    rc = lib.da_decoding_attn_ex(wd.q.data_ptr(), wd.k.data_ptr(), None if wd.v is None else wd.v.data_ptr(),
+                                 o.data_ptr(), wd.cu_seq_k.data_ptr(), w.max_seq_k, b, hq, hk, d, w.dim_v,
+                                 int(w.is_alibi), int(w.q.dtype == torch.bfloat16), 0.0, None, total_k_hint,
+                                 ws.data_ptr(), n, torch.cuda.current_stream().cuda_stream)
+    assert rc == 0, _lib.last_error()
+    torch.cuda.synchronize()
+    return o.cpu()
+
+
 def run_oracle(w, **kw):
     return oracle.attn_cpu(w.q, w.k, w.v, w.cu_seq_k, w.max_seq_k, w.dim_v, w.is_alibi, nthreads=ORACLE_THREADS,
                            return_f32=True, **kw)

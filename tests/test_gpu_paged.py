@@ -1,7 +1,9 @@
 """Paged K/V entry point: the same attention with K/V scattered over page pools.
 
-With pages of a multiple of 32 tokens the paged call runs the same kernels with the same split plan as the packed
-call, so its output must equal the packed call's bit for bit; smaller pages run the VALU sweep and are checked
+With pages of a multiple of 32 tokens the paged call runs the same kernels as the packed call, and with the same
+split plan when neither is given the batch's token count (with it, the packed call of a ragged batch may cut the
+concatenated tokens into equal shares, which pages cannot follow), so its output must then equal the packed call's
+bit for bit; smaller pages run the VALU sweep and are checked
 against the CPU oracle on the gathered (packed) inputs.  Unused pool rows are NaN: reading one poisons the output.
 """
 import pytest
@@ -9,22 +11,22 @@ import torch
 
 from decoding_attention_amd import _lib, decoding_attn_fwd, decoding_attn_paged_fwd
 from decoding_attention_amd import workloads as wl
-from tests.gpu_util import check_against_oracle
+from tests.gpu_util import TOL, check_against_oracle, run_hip_ex
 
 pytestmark = pytest.mark.gpu
 
 DEV = "cuda:0"
 
 
-def _run_both(w, page_size, combined=False, **kw):
+def _run_both(w, page_size, combined=False, hint=0):
+    """Packed and paged call on the same values, both with the token-count hint `hint` (0 = not given)."""
     pk = wl.to_pages(w, page_size, seed=3, combined=combined).to(DEV)
     wd = w.to(DEV)
-    total = int(w.k.shape[0])
-    dense = decoding_attn_fwd(wd.q, wd.k, wd.v, wd.cu_seq_k, w.max_seq_k, w.dim_v, w.is_alibi, **kw)
+    dense = run_hip_ex(w, hint)
     paged = decoding_attn_paged_fwd(wd.q, pk.k_pages, pk.v_pages, pk.block_table, pk.seq_lens, w.max_seq_k, w.dim_v,
-                                    w.is_alibi, total_k=total, **kw)
+                                    w.is_alibi, total_k=hint)
     torch.cuda.synchronize()
-    return dense.cpu(), paged.cpu()
+    return dense, paged.cpu()
 
 
 SHAPES = {
@@ -53,6 +55,16 @@ def test_tile_sized_pages_match_the_packed_call_bit_for_bit(name, page_size):
     dense, paged = _run_both(w, page_size)
     assert torch.isfinite(paged.float()).all()
     assert torch.equal(dense.view(torch.int16), paged.view(torch.int16))
+
+
+@pytest.mark.parametrize("name", ["gqa", "mqa", "mla"])
+def test_with_the_token_count_hint(name):
+    """Both calls are given the batch's token count: each may choose another split plan for the ragged batch, so
+    the outputs agree within the tolerance (and the paged one with the oracle)."""
+    w = _workload(name)
+    dense, paged = _run_both(w, 64, hint=int(w.k.shape[0]))
+    assert (dense.float() - paged.float()).abs().max().item() <= TOL[w.q.dtype]
+    check_against_oracle(w, paged)
 
 
 @pytest.mark.parametrize("page_size", [1, 4, 16])

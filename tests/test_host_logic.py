@@ -68,17 +68,26 @@ def test_plan_is_consistent(d, dv, batch, sk):
     assert ws >= need if d == 576 else ws == need
 
 
-def test_plan_total_k_hint_only_shortens_splits_of_ragged_batches():
-    """The token-count hint changes the split size of a ragged batch only, and never the kernel kind."""
+def test_plan_total_k_hint_only_changes_the_splits_of_ragged_batches():
+    """The token-count hint changes how a ragged batch is cut, and never the kernel kind."""
     sk, batch = 8192, 64
     base = _lib.plan(sk, batch, 32, 8, 128, 128)
     full = _lib.plan(sk, batch, 32, 8, 128, 128, total_k=batch * sk)
     ragged = _lib.plan(sk, batch, 32, 8, 128, 128, total_k=batch * sk // 2)
     assert full == base
-    assert ragged["kind"] == base["kind"] and ragged["chunk"] < base["chunk"]
-    assert ragged["nsplit"] * ragged["chunk"] >= sk
+    # grouped kernel: equal shares of the concatenated tokens, 512 work-groups over the 2 groups of 4 KV heads
+    assert ragged["kind"] == base["kind"] == 3
+    assert ragged["chunk"] == batch * sk // 2 // 256
+    # a sequence of max_seq_k tokens can straddle one more share than its length fills
+    assert ragged["nsplit"] == sk // ragged["chunk"] + 1
     ws = _lib.load().da_workspace_bytes(sk, batch, 32, 8, 128, 128, batch * sk // 2)
     assert ws == batch * 32 * ragged["nsplit"] * (128 + 2) * 4
+    # VALU sweep (one query head per KV head, short sequences): shorter fixed splits
+    sk, batch = 2048, 16
+    base = _lib.plan(sk, batch, 32, 32, 256, 256)
+    ragged = _lib.plan(sk, batch, 32, 32, 256, 256, total_k=batch * sk // 2)
+    assert ragged["kind"] == base["kind"] == 1 and ragged["chunk"] < base["chunk"]
+    assert ragged["nsplit"] * ragged["chunk"] >= sk
 
 
 def test_workspace_sizes_of_the_paged_and_fp8_variants():
