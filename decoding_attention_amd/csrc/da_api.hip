@@ -43,7 +43,7 @@ int env_int(const char* name, int dflt) {
 // stops being split further; DA_MAX_CHUNK / DA_MIN_CHUNK: bounds on tokens per split.
 struct Tunables {
     int target_wgs, mfma_target_wgs, max_chunk, min_chunk, ragged_chunk, force_kind, group_min_ratio, wave_per_head,
-        mla_heads, gqa_heads, flat_wgs, flat_min_tokens;
+        mla_heads, gqa_heads, flat_wgs, flat_min_tokens, nsplit, mfma_small_wgs;
     Tunables() {
         target_wgs = env_int("DA_TARGET_WGS", 512);
         mfma_target_wgs = env_int("DA_MFMA_TARGET_WGS", 256);
@@ -55,6 +55,8 @@ struct Tunables {
         // balanced grid of the grouped kernel for ragged batches: work-groups in all (0 = off), fewest tokens each
         flat_wgs = env_int("DA_FLAT_WGS", 512);
         flat_min_tokens = env_int("DA_FLAT_MIN_TOKENS", 256);
+        mfma_small_wgs = env_int("DA_MFMA_SMALL_WGS", 256);  // latent kernel: below this many 256-token splits, split finer
+        nsplit = env_int("DA_NSPLIT", 0);  // sequence splits, 0 = by shape (experiments)
         force_kind = env_int("DA_FORCE_KIND", 0);
         wave_per_head = env_int("DA_WAVE_PER_HEAD", 1);
         group_min_ratio = env_int("DA_GROUP_MIN_RATIO", 2);  // smallest head group that takes the grouped MFMA sweep
@@ -168,9 +170,17 @@ Plan make_plan(size_t max_seq_k, size_t batch, size_t head_q, size_t head_k, siz
         return pl;
     }
     int min_chunk = std::max(mfma ? 256 : tun().min_chunk, trip);
-    if (!mfma) {
-        // 512-token splits run best; go down to 256 only when that is needed to give every CU a work-group
-        if (base * std::max<long long>(1, (long long)max_seq_k / min_chunk) < 256) min_chunk = std::max(std::min(min_chunk, 256), trip);
+    const long long wgs_at_min = base * std::max<long long>(1, (long long)max_seq_k / min_chunk);
+    if (mfma) {
+        // too few work-groups for the chip even so: 128-token splits, as long as that keeps the merge at 32
+        // partials or fewer (measured: batch 1 x 512 tokens 26.8 -> 20.5 us, batch 16 x 512 33.1 -> 29.4 us,
+        // batch 4 x 2048 32.9 -> 28.3 us; batch 1 x 8192 with 64 partials loses, 36.0 -> 38.5 us)
+        if (wgs_at_min < tun().mfma_small_wgs && max_seq_k <= 32 * 128) min_chunk = std::max(std::min(min_chunk, 128), trip);
+    } else {
+        // 512-token splits run best; go down to 256 only when that is needed to give every CU a work-group (the
+        // VALU sweep: two, measured batch 4 x 1024 tokens 21.4 -> 18.6 us; the grouped kernel loses there)
+        const long long fill = pl.kind == kKindSweep ? 2 * 256 : 256;
+        if (wgs_at_min < fill) min_chunk = std::max(std::min(min_chunk, 256), trip);
         if (ragged) min_chunk = std::max(std::min(min_chunk, tun().ragged_chunk), trip);
     }
     long long want = base > 0 ? (target_wgs + base - 1) / base : 1;
@@ -181,6 +191,7 @@ Plan make_plan(size_t max_seq_k, size_t batch, size_t head_q, size_t head_k, siz
     long long by_cap = mfma ? 1 : ((long long)max_seq_k + max_chunk - 1) / max_chunk;
     long long ns = std::max(std::min(want, by_len), std::min(by_cap, by_len));
     ns = std::max<long long>(1, std::min<long long>(ns, kMaxSplits));
+    if (tun().nsplit > 0) ns = std::min<long long>(tun().nsplit, kMaxSplits);
     long long chunk = ((long long)max_seq_k + ns - 1) / ns;
     chunk = (chunk + trip - 1) / trip * trip;
     if (chunk <= 0) chunk = trip;
