@@ -43,7 +43,7 @@ int env_int(const char* name, int dflt) {
 // stops being split further; DA_MAX_CHUNK / DA_MIN_CHUNK: bounds on tokens per split.
 struct Tunables {
     int target_wgs, mfma_target_wgs, max_chunk, min_chunk, ragged_chunk, force_kind, group_min_ratio, wave_per_head,
-        mla_heads, gqa_heads, flat_wgs, flat_min_tokens, nsplit, mfma_small_wgs;
+        mla_heads, gqa_heads, flat_wgs, flat_min_tokens, flat_paged_min_mb, nsplit, mfma_small_wgs;
     Tunables() {
         target_wgs = env_int("DA_TARGET_WGS", 512);
         mfma_target_wgs = env_int("DA_MFMA_TARGET_WGS", 256);
@@ -55,6 +55,7 @@ struct Tunables {
         // balanced grid of the grouped kernel for ragged batches: work-groups in all (0 = off), fewest tokens each
         flat_wgs = env_int("DA_FLAT_WGS", 512);
         flat_min_tokens = env_int("DA_FLAT_MIN_TOKENS", 256);
+        flat_paged_min_mb = env_int("DA_FLAT_PAGED_MIN_MB", 512);  // paged K/V takes the balanced grid from this many MB of K/V
         mfma_small_wgs = env_int("DA_MFMA_SMALL_WGS", 256);  // latent kernel: below this many 256-token splits, split finer
         nsplit = env_int("DA_NSPLIT", 0);  // sequence splits, 0 = by shape (experiments)
         force_kind = env_int("DA_FORCE_KIND", 0);
@@ -84,6 +85,11 @@ struct Plan {
     // per (KV heads, head group), each over flat_tokens consecutive tokens of the concatenated sequences; nsplit
     // is then the most partials one sequence can have, chunk == flat_tokens.
     int flat_tokens = 0, flat_wgs = 0;
+    // paged K/V: the line is measured in units of flat_unit = 32 tokens, every sequence rounded up to whole units
+    // (shares then start on tile boundaries), and its positions are computed on the device by a small kernel in
+    // front of the sweep, into flat_cu_bytes at the end of the workspace
+    int flat_unit = 1;
+    size_t flat_cu_bytes = 0;
 };
 
 bool supported_dims(size_t dim, size_t dim_v) {
@@ -152,21 +158,30 @@ Plan make_plan(size_t max_seq_k, size_t batch, size_t head_q, size_t head_k, siz
     pl.groups = (ratio + pl.rt - 1) / pl.rt;
     const long long base = (long long)batch * (long long)(pl.wave_per_head ? head_k / 4 : head_k) * pl.groups;
     const bool ragged = total_k > 0 && (long long)total_k * 10 < (long long)batch * (long long)max_seq_k * 9;
-    if (pl.kind == kKindGroup && ragged && packed && tun().flat_wgs > 0 && total_k < ((size_t)1 << 30) &&
-        total_k >= 64 * batch) {
-        // Ragged batch of known total length: equal shares of the concatenated tokens instead of fixed splits of
-        // every sequence (64 sequences of 1..8192 tokens, 32/8 heads: see the tunables' documentation for the measured gain).
+    // Ragged batch of known total length on the grouped kernel: equal shares of the concatenated tokens instead of
+    // fixed splits of every sequence.  Paged K/V pays one more (tiny) kernel for the sequences' positions, so it
+    // takes this form only when the sweep is long enough to win that back.
+    const double kv_bytes = (double)total_k * (double)head_k * (double)(dim + dim_v) * (kv_fp8 ? 1.0 : 2.0);
+    if (pl.kind == kKindGroup && ragged && tun().flat_wgs > 0 && total_k < ((size_t)1 << 30) && total_k >= 64 * batch &&
+        (packed || kv_bytes >= (double)tun().flat_paged_min_mb * 1e6)) {
         const long long ygrid = base / (long long)batch;
         long long w = std::max<long long>(1, tun().flat_wgs / ygrid);
-        const long long unit = trip;  // a work-group's waves advance `trip` tokens per step together
-        long long t = ((long long)total_k + w - 1) / w;
-        t = std::max<long long>((t + unit - 1) / unit * unit, std::max<long long>(tun().flat_min_tokens, unit));
-        w = std::min<long long>(65535, ((long long)total_k + t - 1) / t);
+        const long long unit = packed ? 1 : da::kGqaTile;
+        const long long line = packed ? (long long)total_k : (long long)total_k / unit + (long long)batch;
+        const long long step = std::max<long long>(1, trip / unit);  // a work-group's waves advance `trip` tokens together
+        long long t = (line + w - 1) / w;
+        t = std::max<long long>((t + step - 1) / step * step, std::max<long long>(tun().flat_min_tokens / unit, step));
+        w = std::min<long long>(65535, (line + t - 1) / t);
         pl.flat_tokens = (int)t;
         pl.flat_wgs = (int)w;
-        pl.chunk = (int)t;
-        pl.nsplit = (int)std::min<long long>(w, ((long long)max_seq_k + t - 1) / t + 1);
+        pl.flat_unit = (int)unit;
+        pl.chunk = (int)(t * unit);
+        pl.nsplit = (int)std::min<long long>(w, (((long long)max_seq_k + unit - 1) / unit + t - 1) / t + 1);
         pl.ws_bytes = (size_t)batch * head_q * pl.nsplit * (dim_v + 2) * sizeof(float);
+        if (!packed) {
+            pl.flat_cu_bytes = ((batch + 1) * sizeof(int32_t) + 15) & ~(size_t)15;
+            pl.ws_bytes += pl.flat_cu_bytes;
+        }
         return pl;
     }
     int min_chunk = std::max(mfma ? 256 : tun().min_chunk, trip);
@@ -388,7 +403,16 @@ int run_attention(const void* q, const void* k, const void* v, void* o, const in
     sp.k_page = (int64_t)pg.k_page;
     sp.v_page = v ? (int64_t)pg.v_page : (int64_t)pg.k_page;
     sp.flat_tokens = pl.flat_tokens;
+    sp.flat_unit = pl.flat_unit;
+    sp.flat_cu = cu_seq_k;
     sp.batch = (int)batch;
+    if (pl.flat_cu_bytes > 0) {
+        // paged: positions of the sequences on the balanced grid's line, computed in front of the sweep
+        int32_t* const flat_cu = reinterpret_cast<int32_t*>(static_cast<uint8_t*>(ws) + (pl.ws_bytes - pl.flat_cu_bytes));
+        const hipError_t pe = da::launch_flat_prefix(pg.seq_lens, (int)batch, 5, flat_cu, stream);
+        if (pe != hipSuccess) return fail(DA_ERR_HIP, "prefix kernel launch: %s", hipGetErrorString(pe));
+        sp.flat_cu = flat_cu;
+    }
 
     const dim3 grid((unsigned)(pl.flat_tokens ? pl.flat_wgs : pl.nsplit),
                     (unsigned)((pl.wave_per_head ? head_k / 4 : head_k) * pl.groups),
@@ -427,6 +451,7 @@ int run_attention(const void* q, const void* k, const void* v, void* o, const in
         rp.chunk = pl.chunk;
         rp.flat_tokens = pl.flat_tokens;
         rp.flat_wgs = pl.flat_wgs;
+        rp.flat_cu = sp.flat_cu;
         e = da::launch_reduce(rp, is_bf16 != 0, (int)(batch * head_q), stream);
         if (e != hipSuccess) return fail(DA_ERR_HIP, "merge kernel launch: %s", hipGetErrorString(e));
     }

@@ -151,9 +151,14 @@ struct SweepParams {
     // The kernels fold k_scale into the softmax scale and v_scale into the final normalisation.
     const float* k_scale;
     const float* v_scale;
-    // Balanced form of the grouped-head kernel's grid (0 = off): tokens per work-group of the line of all
-    // sequences' tokens, and the number of sequences.
+    // Balanced form of the grouped-head kernel's grid (flat_tokens == 0: off).  The sequences lie end to end on
+    // one line measured in units of flat_unit tokens (1 for packed K/V, where the line is cu_seq_k itself; 32 for
+    // paged K/V, where every sequence is rounded up to whole units so that shares start on tile boundaries);
+    // flat_cu[b] is the position of sequence b on the line ([batch + 1] entries), flat_tokens the units per
+    // work-group.
     int flat_tokens;
+    int flat_unit;
+    const int32_t* flat_cu;
     int batch;
 };
 
@@ -166,7 +171,10 @@ struct ReduceParams {
     const float* ws_o;
     const float* ws_ml;
     int head_q, dim_v, nsplit, chunk;
-    int flat_tokens, flat_wgs;  // balanced form of the sweep's grid (flat_tokens > 0): tokens per work-group, work-groups
+    // balanced form of the sweep's grid (flat_tokens > 0): units per work-group, work-groups, the sequences'
+    // positions on the line (see SweepParams)
+    int flat_tokens, flat_wgs;
+    const int32_t* flat_cu;
 };
 
 // First token (row of the packed K/V buffers) and length of sequence b; paged sequences start at row 0 of their

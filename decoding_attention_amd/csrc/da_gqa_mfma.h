@@ -426,12 +426,13 @@ __device__ __forceinline__ void gqa_segment(const SweepParams& p, uint8_t* const
 }
 
 // Grid, packed or paged K/V with a fixed split length: (split, KV heads x head groups, sequence).
-// Grid, balanced form (p.flat_tokens > 0, packed K/V only): (work-group i of W, KV heads x head groups, 1).  The
-// tokens of all sequences form one line of cu_seq_k[batch] tokens; work-group i takes tokens [i T, (i+1) T) of it
-// (the last one to the end), whatever sequences they belong to, one segment per sequence it touches.  Every
-// work-group then streams the same number of bytes, which a ragged batch cut into fixed splits does not give.
-// Sequence b spans work-groups first(b) = cu[b] / T ... last(b) = (cu[b+1] - 1) / T (both capped at W - 1); its
-// segment in work-group i is partial number i - first(b), and goes straight to o when first(b) == last(b).
+// Grid, balanced form (p.flat_tokens > 0): (work-group i of W, KV heads x head groups, 1).  The tokens of all
+// sequences form one line (positions p.flat_cu, in units of p.flat_unit tokens); work-group i takes positions
+// [i T, (i+1) T) of it (the last one to the end), whatever sequences they belong to, one segment per sequence it
+// touches.  Every work-group then streams the same number of bytes, which a ragged batch cut into fixed splits
+// does not give.  Sequence b spans work-groups first(b) = cu[b] / T ... last(b) = (cu[b+1] - 1) / T (both capped
+// at W - 1); its segment in work-group i is partial number i - first(b), and goes straight to o when
+// first(b) == last(b).
 template <typename Tag, int D, int DV, int NT, bool PREFETCH, bool WH, int MINW, bool KV8 = false>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(MINW))) void gqa_mfma_kernel(const SweepParams p) {
     extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
@@ -444,13 +445,13 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(MINW))) voi
         gqa_segment<Tag, D, DV, NT, PREFETCH, WH, KV8>(p, smem, b, start, len, c0, c1, split, p.nsplit == 1);
         return;
     }
-    const int T = p.flat_tokens, W = (int)gridDim.x, i = (int)blockIdx.x;
-    const int32_t* const cu = p.cu_seq_k;
+    const int T = p.flat_tokens, W = (int)gridDim.x, i = (int)blockIdx.x, unit = p.flat_unit;
+    const int32_t* const cu = p.flat_cu;
     const int total = cu[p.batch];
     const int r0 = (int)min((long long)i * T, (long long)total);
     const int r1 = (i == W - 1) ? total : (int)min((long long)r0 + T, (long long)total);
     if (r0 >= r1) return;
-    // the sequence that holds token r0: the last b with cu[b] <= r0 (empty sequences share their offset with
+    // the sequence that holds position r0: the last b with cu[b] <= r0 (empty sequences share their position with
     // the next one and are passed over)
     int lo = 0, hi = p.batch;
     while (lo + 1 < hi) {
@@ -464,9 +465,11 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(MINW))) voi
         const int s = cu[b], e = cu[b + 1];
         if (s >= r1) break;
         if (e <= s) continue;
+        int start, len;
+        seq_range(p, b, start, len);
         const int first = min(s / T, W - 1), last = min((e - 1) / T, W - 1);
-        gqa_segment<Tag, D, DV, NT, PREFETCH, WH, KV8>(p, smem, b, s, e - s, max(r0, s) - s, min(r1, e) - s, i - first,
-                                                       first == last);
+        const int c0 = (max(r0, s) - s) * unit, c1 = min((min(r1, e) - s) * unit, len);
+        gqa_segment<Tag, D, DV, NT, PREFETCH, WH, KV8>(p, smem, b, start, len, c0, c1, i - first, first == last);
         if (!WH) __syncthreads();  // the merge area of this segment is the V tile area of the next
     }
 }

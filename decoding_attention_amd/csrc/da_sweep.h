@@ -262,8 +262,8 @@ __global__ __launch_bounds__(256) void reduce_kernel(const ReduceParams p, int r
         // balanced sweep grid: the sequence's partials come from the work-groups its tokens fall into; a sequence
         // inside one work-group was written to o by the sweep itself
         if (len > 0) {
-            const int s = p.cu_seq_k[b];
-            ns = min((s + len - 1) / p.flat_tokens, p.flat_wgs - 1) - min(s / p.flat_tokens, p.flat_wgs - 1) + 1;
+            const int s = p.flat_cu[b], e = p.flat_cu[b + 1];
+            ns = min((e - 1) / p.flat_tokens, p.flat_wgs - 1) - min(s / p.flat_tokens, p.flat_wgs - 1) + 1;
             if (ns == 1) return;
         }
     } else if (len > 0) {

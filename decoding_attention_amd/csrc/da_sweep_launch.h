@@ -49,5 +49,7 @@ hipError_t launch_sweep_d576(const SweepParams& p, bool is_bf16, int rt, dim3 gr
 // the VALU sweep over an FP8 (e4m3) K/V cache, any supported (dim, dim_v)
 hipError_t launch_sweep_kv8(const SweepParams& p, bool is_bf16, int dim, int rt, dim3 grid, hipStream_t stream);
 hipError_t launch_reduce(const ReduceParams& p, bool is_bf16, int blocks, hipStream_t stream);
+// out[0 .. batch] = running sum of ceil(seq_lens / 2^shift) (positions of paged sequences on the balanced grid's line)
+hipError_t launch_flat_prefix(const int32_t* seq_lens, int batch, int shift, int32_t* out, hipStream_t stream);
 
 }  // namespace da

@@ -3,12 +3,16 @@ every work-group takes an equal share of the concatenated tokens, across sequenc
 match the oracle exactly as the fixed-split grid's do, whatever the lengths are: empty sequences anywhere, many
 short sequences inside one share, one sequence over many shares, and a hint that is too small or too large.
 """
+import os
+import subprocess
+import sys
+
 import pytest
 import torch
 
-from decoding_attention_amd import _lib
+from decoding_attention_amd import _lib, decoding_attn_paged_fwd
 from decoding_attention_amd import workloads as wl
-from tests.gpu_util import TOL, check_against_oracle, run_hip_ex
+from tests.gpu_util import TOL, check_against_oracle, run_hip_ex, sub_workload
 
 pytestmark = pytest.mark.gpu
 
@@ -85,3 +89,35 @@ def test_same_result_as_fixed_splits_up_to_summation_order():
     a = _run_ex(w, total).float()
     b = _run_ex(w, 0).float()  # no hint: fixed splits of every sequence
     assert (a - b).abs().max().item() <= TOL[torch.bfloat16]
+
+
+def test_paged_small_cases_in_a_process_with_the_size_threshold_off():
+    """Paged K/V takes the balanced grid only from 512 MB of K/V (it costs one more small kernel); the edge cases
+    are small, so they run in a process of their own that loads the library with that threshold at zero."""
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    env = dict(os.environ, DA_FLAT_PAGED_MIN_MB="0")
+    r = subprocess.run([sys.executable, os.path.join(root, "tests", "paged_balanced_cases.py")], env=env, cwd=root,
+                       capture_output=True, text=True, timeout=600)
+    assert r.returncode == 0 and "all ok" in r.stdout, r.stdout[-2000:] + r.stderr[-4000:]
+
+
+def test_paged_large_ragged_batch_takes_the_balanced_grid():
+    """A ragged paged batch above the size threshold (0.6 GB of K/V): balanced plan, spot-checked against the oracle."""
+    g = torch.Generator().manual_seed(21)
+    lens = torch.randint(1, 16385, (18,), generator=g).tolist()
+    lens[0], lens[5] = 16384, 0
+    w = _workload(lens, 32, 8, 128, torch.bfloat16, seed=22)
+    total, b = int(w.k.shape[0]), len(lens)
+    assert total * 8 * 256 * 2 >= 512e6
+    lib = _lib.load()
+    flat = lib.da_workspace_bytes_paged(w.max_seq_k, b, 32, 8, 128, 128, total, 64)
+    assert (flat - ((b + 1) * 4 + 15) // 16 * 16) % (b * 32 * (128 + 2) * 4) == 0  # partials, then the positions
+    pk = wl.to_pages(w, 64, seed=3).to(DEV)
+    wd = w.to(DEV)
+    o = decoding_attn_paged_fwd(wd.q, pk.k_pages, pk.v_pages, pk.block_table, pk.seq_lens, w.max_seq_k, w.dim_v,
+                                False, total_k=total).cpu()
+    assert torch.isfinite(o.float()).all()
+    assert torch.count_nonzero(o[5]) == 0
+    rows = [0, 1, 7, 17]
+    sub = sub_workload(w, rows)
+    check_against_oracle(sub, o[rows])
