@@ -81,7 +81,7 @@ struct Plan {
     int chunk = 0;
     size_t ws_bytes = 0;
     bool wave_per_head = false;  // grouped kernel: the four waves of a work-group take four KV heads
-    // Balanced grid (grouped kernel, ragged packed batch whose total length the caller gave): flat_wgs work-groups
+    // Balanced grid (grouped kernel, ragged batch whose total length the caller gave): flat_wgs work-groups
     // per (KV heads, head group), each over flat_tokens consecutive tokens of the concatenated sequences; nsplit
     // is then the most partials one sequence can have, chunk == flat_tokens.
     int flat_tokens = 0, flat_wgs = 0;

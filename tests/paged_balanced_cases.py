@@ -32,8 +32,8 @@ def run_case(name, w, page_size, hint):
     hk = w.k.shape[1]
     lib = _lib.load()
     # the paged plan is the balanced one: its workspace holds one more share than max_seq_k fills, plus the positions
-    fixed = lib.da_workspace_bytes_paged(w.max_seq_k, b, hq, hk, d, d, 0, page_size)
-    flat = lib.da_workspace_bytes_paged(w.max_seq_k, b, hq, hk, d, d, hint, page_size)
+    fixed = lib.da_workspace_bytes_paged(w.max_seq_k, b, hq, hk, d, w.dim_v, 0, page_size)
+    flat = lib.da_workspace_bytes_paged(w.max_seq_k, b, hq, hk, d, w.dim_v, hint, page_size)
     assert flat != fixed and flat % 16 == 0, (name, fixed, flat)
     pk = wl.to_pages(w, page_size, seed=3).to(DEV)
     wd = w.to(DEV)

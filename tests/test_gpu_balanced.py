@@ -37,7 +37,7 @@ def _is_balanced(w, hint):
     """The planner chose equal token shares: its split length is the share, not a divisor of max_seq_k."""
     b, hq, d = w.q.shape
     hk = w.k.shape[1]
-    with_hint = _lib.plan(w.max_seq_k, b, hq, hk, d, d, True, hint)
+    with_hint = _lib.plan(w.max_seq_k, b, hq, hk, d, w.dim_v, True, hint)
     return with_hint["kind"] == 3 and with_hint["nsplit"] * with_hint["chunk"] >= w.max_seq_k + with_hint["chunk"]
 
 
