@@ -247,14 +247,27 @@ __global__ __launch_bounds__(256) void sweep_kernel(const SweepParams p) {
 
 // Second pass: merge the per-split partials in split order.  One thread per (sequence, query head, group of four
 // output columns); the partials of four splits are fetched together so that their latencies overlap.
-template <typename Tag>
+// SG > 1 (many splits of few rows: one long sequence): SG lanes share one (row, four columns), lane j of them
+// taking splits j, j + SG, ...; a wave covers 64 / SG column groups of one row, and the SG partial sums meet through
+// lane exchanges.  The order of summation then differs from SG = 1, not the result's accuracy.
+template <typename Tag, int SG>
 __global__ __launch_bounds__(256) void reduce_kernel(const ReduceParams p, int rows) {
     using EL = Elem<Tag>;
     const int nc4 = p.dim_v >> 2;
-    const int gid = blockIdx.x * 256 + threadIdx.x;
-    const int row = gid / nc4;  // (sequence, head) index
-    const int c4 = gid - row * nc4;
-    if (row >= rows) return;
+    int row, c4, sgi = 0;
+    if constexpr (SG == 1) {
+        const int gid = blockIdx.x * 256 + threadIdx.x;
+        row = gid / nc4;  // (sequence, head) index
+        c4 = gid - row * nc4;
+    } else {
+        constexpr int CW = 64 / SG;  // column groups per wave
+        const int wave_id = blockIdx.x * 4 + (threadIdx.x >> 6), lane = threadIdx.x & 63;
+        const int waves_per_row = nc4 / CW;
+        row = wave_id / waves_per_row;
+        c4 = (wave_id - row * waves_per_row) * CW + (lane % CW);
+        sgi = lane / CW;
+    }
+    if (row >= rows) return;  // (whole waves leave together when SG > 1)
     const int b = row / p.head_q;
     const int len = p.cu_seq_k ? p.cu_seq_k[b + 1] - p.cu_seq_k[b] : p.seq_lens[b];
     int ns = 0;
@@ -276,24 +289,35 @@ __global__ __launch_bounds__(256) void reduce_kernel(const ReduceParams p, int r
     for (int s = 0; s < ns; ++s) mm = fmaxf(mm, ml[s].x);
     float4 num = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
     float den = 0.0f;
-    for (int s0 = 0; s0 < ns; s0 += 4) {
+    for (int s0 = sgi; s0 < ns; s0 += 4 * SG) {
         float2 e[4];
         float4 x[4];
 #pragma unroll
         for (int u = 0; u < 4; ++u) {
-            const int s = min(s0 + u, ns - 1);
+            const int s = min(s0 + u * SG, ns - 1);
             e[u] = ml[s];
             x[u] = src[(size_t)s * nc4];
         }
 #pragma unroll
         for (int u = 0; u < 4; ++u) {
-            const float w = (s0 + u < ns) ? fast_exp2(e[u].x - mm) : 0.0f;
+            const float w = (s0 + u * SG < ns) ? fast_exp2(e[u].x - mm) : 0.0f;
             den += w * e[u].y;
             num.x += w * x[u].x;
             num.y += w * x[u].y;
             num.z += w * x[u].z;
             num.w += w * x[u].w;
         }
+    }
+    if constexpr (SG > 1) {
+#pragma unroll
+        for (int d = 64 / SG; d < 64; d <<= 1) {
+            den += __shfl_xor(den, d);
+            num.x += __shfl_xor(num.x, d);
+            num.y += __shfl_xor(num.y, d);
+            num.z += __shfl_xor(num.z, d);
+            num.w += __shfl_xor(num.w, d);
+        }
+        if (sgi != 0) return;
     }
     const float inv = ns > 0 ? 1.0f / den : 0.0f;  // an empty sequence yields a zero row
     ushort4 r;

@@ -5,14 +5,28 @@ namespace da {
 hipError_t launch_sweep_d576(const SweepParams& p, bool is_bf16, int rt, dim3 grid, hipStream_t stream) {
     return launch_sweep_dim<576, 512, 2>(p, is_bf16, rt, grid, stream);
 }
+template <typename Tag, int SG>
+static void launch_reduce_sg(const ReduceParams& p, int blocks, hipStream_t stream) {
+    const long long nc4 = p.dim_v / 4;
+    // SG = 1: one thread per (row, four columns); SG > 1: one wave per (row, 64 / SG column groups), four waves a block
+    const long long units = SG == 1 ? (long long)blocks * nc4 : (long long)blocks * (nc4 / (64 / SG)) * 64;
+    const dim3 grid((unsigned)((units + 255) / 256));
+    hipLaunchKernelGGL((reduce_kernel<Tag, SG>), grid, dim3(256), 0, stream, p, blocks);
+}
+
 hipError_t launch_reduce(const ReduceParams& p, bool is_bf16, int blocks, hipStream_t stream) {
-    // `blocks` counts (sequence, head) rows; one thread per four output columns
+    // `blocks` counts (sequence, head) rows.  Many splits of few rows (one long sequence): several lanes share the
+    // splits of one output element, so that the merge is not one long chain of dependent loads per thread.
     const long long threads = (long long)blocks * (p.dim_v / 4);
-    const dim3 grid((unsigned)((threads + 255) / 256));
-    if (is_bf16)
-        hipLaunchKernelGGL((reduce_kernel<bf16_tag>), grid, dim3(256), 0, stream, p, blocks);
-    else
-        hipLaunchKernelGGL((reduce_kernel<f16_tag>), grid, dim3(256), 0, stream, p, blocks);
+    int sg = 1;
+    while (sg < 8 && p.nsplit >= 8 * sg && threads * sg < (1ll << 18)) sg *= 2;
+    while (sg > 1 && (p.dim_v / 4) % (64 / sg) != 0) sg /= 2;
+    switch (sg) {
+        case 8: is_bf16 ? launch_reduce_sg<bf16_tag, 8>(p, blocks, stream) : launch_reduce_sg<f16_tag, 8>(p, blocks, stream); break;
+        case 4: is_bf16 ? launch_reduce_sg<bf16_tag, 4>(p, blocks, stream) : launch_reduce_sg<f16_tag, 4>(p, blocks, stream); break;
+        case 2: is_bf16 ? launch_reduce_sg<bf16_tag, 2>(p, blocks, stream) : launch_reduce_sg<f16_tag, 2>(p, blocks, stream); break;
+        default: is_bf16 ? launch_reduce_sg<bf16_tag, 1>(p, blocks, stream) : launch_reduce_sg<f16_tag, 1>(p, blocks, stream); break;
+    }
     return hipGetLastError();
 }
 namespace {
