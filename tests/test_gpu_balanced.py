@@ -91,6 +91,33 @@ def test_same_result_as_fixed_splits_up_to_summation_order():
     assert (a - b).abs().max().item() <= TOL[torch.bfloat16]
 
 
+@pytest.mark.parametrize("seed", range(8))
+def test_random_ragged_batches(seed):
+    """Random batch size, head grouping and lengths (zeros included, one long sequence so that the batch counts as
+    ragged); every row against the oracle for small batches, a sample of rows for large ones."""
+    g = torch.Generator().manual_seed(1000 + seed)
+    batch = int(torch.randint(2, 700, (1,), generator=g))
+    hq, hk = [(32, 8), (16, 16), (32, 1), (24, 4), (32, 2), (16, 4), (64, 8), (12, 12)][seed]
+    dim, dtype = [(128, torch.float16), (64, torch.bfloat16), (128, torch.bfloat16), (96, torch.float16)][seed % 4]
+    hi = int(torch.randint(80, 400, (1,), generator=g))
+    lens = torch.randint(0, hi, (batch,), generator=g)
+    lens[torch.rand(batch, generator=g) < 0.1] = 0
+    lens[int(torch.randint(0, batch, (1,), generator=g))] = max(10 * hi, 3000)
+    if int(lens.sum()) < 64 * batch:
+        lens += 64
+    w = _workload(lens.tolist(), hq, hk, dim, dtype, seed=2000 + seed, is_alibi=bool(seed & 1))
+    total = int(w.k.shape[0])
+    if not _is_balanced(w, total):
+        pytest.skip("the planner kept fixed splits for this shape (VALU sweep)")
+    o = _run_ex(w, total)
+    assert torch.isfinite(o.float()).all()
+    rows = list(range(batch)) if batch <= 64 else sorted(set(torch.randint(0, batch, (48,), generator=g).tolist()) |
+                                                         {0, batch - 1, int(lens.argmax())})
+    check_against_oracle(sub_workload(w, rows), o[rows])
+    empty = [b for b in range(batch) if w.lengths[b] == 0]
+    assert all(torch.count_nonzero(o[b]) == 0 for b in empty)
+
+
 def test_paged_small_cases_in_a_process_with_the_size_threshold_off():
     """Paged K/V takes the balanced grid only from 512 MB of K/V (it costs one more small kernel); the edge cases
     are small, so they run in a process of their own that loads the library with that threshold at zero."""
