@@ -452,14 +452,16 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(MINW))) voi
     const int r1 = (i == W - 1) ? total : (int)min((long long)r0 + T, (long long)total);
     if (r0 >= r1) return;
     // the sequence that holds position r0: the last b with cu[b] <= r0 (empty sequences share their position with
-    // the next one and are passed over)
-    int lo = 0, hi = p.batch;
-    while (lo + 1 < hi) {
-        const int mid = (lo + hi) >> 1;
-        if (cu[mid] <= r0)
-            lo = mid;
-        else
-            hi = mid;
+    // the next one and are passed over).  A 64-way search: the wave's lanes probe 64 evenly spaced entries at once,
+    // so 64 sequences take one round of loads where a binary search takes six dependent ones.
+    int lo = 0;
+    for (int n = p.batch; n > 1;) {  // invariant: cu[lo] <= r0, and the answer lies in [lo, lo + n)
+        const int stride = (n + 63) >> 6;
+        const int idx = lo + (int)(threadIdx.x & 63) * stride;
+        const bool below = idx < lo + n && cu[idx] <= r0;
+        const int k = __popcll(__ballot(below)) - 1;  // probes are sorted: the lanes that hold are a prefix, lane 0 among them
+        lo += k * stride;
+        n = min(stride, n - k * stride);
     }
     for (int b = lo; b < p.batch; ++b) {
         const int s = cu[b], e = cu[b + 1];
