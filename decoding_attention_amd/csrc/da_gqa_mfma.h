@@ -98,7 +98,6 @@ __device__ __forceinline__ void gqa_segment(const SweepParams& p, uint8_t* const
     constexpr int KS = D / 32;      // k-steps of Q K^T
     constexpr int CT = DV / 16;     // 16-column tiles of the output
     constexpr int CPR = DV / 8;     // 16-byte chunks per V row
-    constexpr int NVI = kGqaTile * CPR / 64;  // V load instructions per tile
     constexpr int VP = gqa_v_pitch<DV>();
     constexpr int NW = WH ? 1 : 4;  // wavefronts that share the tokens of one KV head
     constexpr int HG = 16 * NT;     // query heads per KV head and work-group

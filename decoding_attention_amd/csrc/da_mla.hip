@@ -295,8 +295,6 @@ __global__ __launch_bounds__(64 * NWV) void mfma_latent_kernel(const SweepParams
     //   (base_v ^ (64 c | 32 hi)) + 16 KiB s2 + 8 KiB hi
     const uint32_t base_v = smem_off + (half * 4 + ((lane & 15) >> 2)) * ROW_A + 64 * ((lane & 15) >> 2) +
                             16 * ((2 * ((lane >> 4) & 1) + ((lane >> 1) & 1)) ^ half) + 8 * (lane & 1);
-    typedef __attribute__((address_space(3))) const uint4* lds_u4;
-    typedef __attribute__((address_space(3))) s16x4* lds_s4;
     typedef short s16x8 __attribute__((__vector_size__(8 * sizeof(short))));
 
     const float bias0 = slope * (float)(half * 4 - (len - 1));  // ALiBi: slope * (token - (len - 1)), split in lane and tile parts
