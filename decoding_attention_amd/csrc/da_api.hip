@@ -113,7 +113,7 @@ int rows_per_trip(size_t dim) {
 // shorter splits so that the work-groups, whose number is sized for max_seq_k, balance.
 // tiles_contiguous: every aligned run of 32 tokens is contiguous in memory (always true for the packed layout; for
 // paged K/V only when a page holds a multiple of 32 tokens).  The two MFMA kernels fetch whole tiles and need it.
-// kv_fp8: K/V are FP8; the latent MFMA kernel has no FP8 form and the grouped kernel needs dim % 64 == 0.
+// kv_fp8: K/V are FP8; the grouped kernel then needs dim % 64 == 0.
 // packed: K/V are in the packed layout addressed through cu_seq_k (the balanced grid needs the prefix offsets).
 Plan make_plan(size_t max_seq_k, size_t batch, size_t head_q, size_t head_k, size_t dim, size_t dim_v,
                bool v_distinct, size_t total_k, bool tiles_contiguous = true, bool kv_fp8 = false, bool packed = true) {
@@ -122,7 +122,7 @@ Plan make_plan(size_t max_seq_k, size_t batch, size_t head_q, size_t head_k, siz
     int trip;
     int target_wgs = tun().target_wgs;
     const bool force_sweep = tun().force_kind == kKindSweep || !tiles_contiguous;
-    const bool mfma = !v_distinct && !kv_fp8 && da::mla_supported(dim, dim_v, ratio) && !force_sweep;
+    const bool mfma = !v_distinct && da::mla_supported(dim, dim_v, ratio) && !force_sweep;
     if (mfma) {
         pl.kind = kKindMfma;
         pl.rt = da::mla_heads_per_group(ratio);
@@ -419,7 +419,9 @@ int run_attention(const void* q, const void* k, const void* v, void* o, const in
                     (unsigned)(pl.flat_tokens ? 1 : batch));
     hipError_t e;
     if (kf.fp8) {
-        if (pl.kind == kKindGroup)
+        if (pl.kind == kKindMfma)
+            e = da::launch_mla_kv8(sp, is_bf16 != 0, pl.rt, grid, stream);
+        else if (pl.kind == kKindGroup)
             e = da::launch_gqa_mfma_kv8(sp, is_bf16 != 0, (int)dim, pl.rt, pl.wave_per_head, grid, stream);
         else
             e = da::launch_sweep_kv8(sp, is_bf16 != 0, (int)dim, pl.rt, grid, stream);

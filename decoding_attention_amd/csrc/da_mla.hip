@@ -26,6 +26,11 @@
 // -- which makes both read patterns (16 rows x one chunk for K, 4 rows x 64 bytes for V^T) conflict-free, and
 // because XOR commutes with the per-step chunk offsets every read address is one per-lane base XOR a constant.
 //
+// FP8 K cache (KV8): the tile's bytes (32 rows x 576 FP8 elements, 18 KiB) are staged in LDS by the same
+// direct-to-LDS loads, three stages deep, and the work-group converts each staged tile into the 16-bit tile layout
+// above (exact: e4m3 -> fp16/bf16) one tile ahead of its use, two 16-bit buffers deep; everything downstream of the
+// tile is the 16-bit kernel.  The per-head scales fold into the softmax scale and the final normalisation.
+//
 // Mathematics as in the reference kernel (csrc/kernel/decoding_attn/decoding_fwd_kernel.h:50-235
 // with the latent aliasing of csrc/ops/decoding_attn.cpp:30-37); the structure is unrelated.
 #include "da_mla.h"
@@ -142,7 +147,7 @@ __device__ __forceinline__ void wait_vmcnt() {
     asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory");
 }
 
-template <typename Tag, int D, int DV, int NWV>
+template <typename Tag, int D, int DV, int NWV, bool KV8>
 __global__ __launch_bounds__(64 * NWV) void mfma_latent_kernel(const SweepParams p) {
     using MM = Mma<Tag>;
     using vec8 = typename MM::vec8;
@@ -157,6 +162,13 @@ __global__ __launch_bounds__(64 * NWV) void mfma_latent_kernel(const SweepParams
     constexpr int NLW = NLA + NLB;                       // load instructions per tile per wave
     constexpr int KS = D / 16;                           // k-steps of Q K^T
     constexpr int CT = DV / 32;                          // 32-column tiles of the output
+    // FP8 K cache: stages of the tile's raw bytes, filled 1 KiB per load instruction
+    constexpr int NTB = KV8 ? 2 : kNBuf;                 // 16-bit tile buffers
+    constexpr int STG_REAL = kTile * D / 1024;           // load instructions that cover a staged tile (18)
+    constexpr int NLW8 = (STG_REAL + NWV - 1) / NWV;     // per wave (the surplus ones repeat the last KiB)
+    constexpr int STG = NLW8 * NWV * 1024;               // bytes per stage
+    constexpr int STG0 = NTB * BUF;                      // stages start behind the 16-bit buffers
+    static_assert((kTile * D) % 1024 == 0, "staged tile");
     static_assert(D % 16 == 0 && DV % 32 == 0 && DV <= D, "shape");
 
     extern __shared__ __attribute__((aligned(1024))) uint8_t smem[];  // max(kNBuf, NWV) * BUF
@@ -247,8 +259,11 @@ __global__ __launch_bounds__(64 * NWV) void mfma_latent_kernel(const SweepParams
         for (int r = 0; r < 16; ++r) acc[c][r] = 0.0f;
     float m = kNegBig, l = 0.0f;
 
-    const uint8_t* const kbytes = reinterpret_cast<const uint8_t*>(p.k) + (size_t)hk * D * 2;
-    const size_t k_row_bytes = (size_t)p.k_row * 2;
+    constexpr int KB = KV8 ? 1 : 2;  // bytes per K element in memory
+    const uint8_t* const kbytes = reinterpret_cast<const uint8_t*>(p.k) + (size_t)hk * D * KB;
+    const size_t k_row_bytes = (size_t)p.k_row * KB;
+    const float sl = p.scale_log2 * head_scale(p.k_scale, hk);  // score scale, log2 units
+    const float vs = head_scale(p.v_scale, hk);
 
     // Stage the tile that starts at token tok0 into buffer `buf`.  Rows past the end of the split re-read the
     // last valid row (they are masked later).  Every wave always issues exactly NLW loads, so the hand-placed
@@ -256,8 +271,20 @@ __global__ __launch_bounds__(64 * NWV) void mfma_latent_kernel(const SweepParams
     // `row0` is the tile's first row as row_ref() gives it (a tile never straddles pages of paged K/V: pages hold
     // a multiple of kTile tokens and tiles start at multiples of kTile).
     auto issue_tile = [&](int tok0, int64_t row0, int buf) {
-        const uint8_t* const base = kbytes + row0 * 2;
+        const uint8_t* const base = kbytes + row0 * KB;
         const int last = c1 - 1 - tok0;
+        if constexpr (KV8) {
+            // stage `buf`: the tile's bytes in row order, lane l of load j bringing bytes [1024 j + 16 l, +16)
+#pragma unroll
+            for (int q = 0; q < NLW8; ++q) {
+                const int j = min(wave + NWV * q, STG_REAL - 1);  // wave-uniform; surplus loads repeat the last KiB
+                const uint32_t off = (uint32_t)j * 1024u + lane16;
+                const uint32_t row = off / (uint32_t)D, within = off - row * (uint32_t)D;
+                lds_dma16(base, (uint32_t)min((int)row, last) * (uint32_t)k_row_bytes + within,
+                          smem_off + (uint32_t)(STG0 + buf * STG + (wave + NWV * q) * 1024));
+            }
+            return;
+        }
 #pragma unroll
         for (int q = 0; q < NLA; ++q) {
             const int row = wave + NWV * q;  // wave-uniform
@@ -274,11 +301,51 @@ __global__ __launch_bounds__(64 * NWV) void mfma_latent_kernel(const SweepParams
         }
     };
 
+    // FP8: convert stage `stg` into 16-bit tile buffer `tb` (swizzled layout).  Eight threads share a row: thread
+    // (row, j) converts the row's 8-element chunks j, j + 8, ..., j + 64, so its swizzles are constants and each
+    // chunk costs one address XOR.
+    constexpr int RPP = 8 * NWV;  // rows per pass
+    const int cv_j = (int)threadIdx.x & 7, cv_r = (int)threadIdx.x >> 3;
+    auto convert_stage = [&](int stg, int tb) {
+        typedef unsigned int u32x2 __attribute__((ext_vector_type(2)));
+        typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
+        typedef const __attribute__((address_space(3))) u32x2* lds_src;
+        typedef __attribute__((address_space(3))) u32x4* lds_dst;
+#pragma unroll
+        for (int ps = 0; ps < kTile / RPP; ++ps) {
+            const int r = cv_r + ps * RPP;
+            const uint32_t src = smem_off + (uint32_t)(STG0 + stg * STG + r * D + cv_j * 8);
+            const uint32_t dst_a = smem_off + (uint32_t)(tb * BUF + r * ROW_A + ((cv_j ^ swz_a(r)) * 16));
+            const uint32_t dst_b = smem_off + (uint32_t)(tb * BUF + OFF_B + r * ROW_B + ((cv_j ^ swz_b(r)) * 16));
+#pragma unroll
+            for (int i = 0; i < D / 64; ++i) {
+                const u32x2 rv = *reinterpret_cast<lds_src>((uintptr_t)(src + i * 64));
+                const uint4 cv = fp8x8_to_16<Tag>(make_uint2(rv.x, rv.y));
+                // chunk j + 8 i of the value columns sits at (j + 8 i) ^ swizzle = (j ^ swizzle) ^ 8 i
+                const uint32_t dst = i < DV / 64 ? (dst_a ^ (uint32_t)(i * 128)) : dst_b;
+                *reinterpret_cast<lds_dst>((uintptr_t)dst) = u32x4{cv.x, cv.y, cv.z, cv.w};
+            }
+        }
+    };
+
     const int ntiles = (c1 - c0 + kTile - 1) / kTile;
     issue_tile(c0, row_ref(p, b, start, c0).k, 0);
     if (ntiles > 1) issue_tile(c0 + kTile, row_ref(p, b, start, c0 + kTile).k, 1);
+    if constexpr (KV8) {
+        // three stages in flight; the first tile is converted here, tile t + 1 at the top of trip t
+        if (ntiles > 2) issue_tile(c0 + 2 * kTile, row_ref(p, b, start, c0 + 2 * kTile).k, 2);
+        if (ntiles > 2)
+            wait_vmcnt<2 * NLW8>();
+        else if (ntiles > 1)
+            wait_vmcnt<NLW8>();
+        else
+            wait_vmcnt<0>();
+        __syncthreads();
+        convert_stage(0, 0);
+    }
     // page of the tile after those, fetched one trip ahead of its use (a scalar load for paged K/V)
-    int page_ahead = ntiles > 2 ? page_of(p, b, c0 + 2 * kTile) : 0;
+    constexpr int AHEAD = KV8 ? 3 : 2;  // tiles in flight behind the one being read
+    int page_ahead = ntiles > AHEAD ? page_of(p, b, c0 + AHEAD * kTile) : 0;
     // Make the compiler settle its own wait for the Q loads here, before the loop.  It cannot see the
     // direct-to-LDS loads, so a wait for Q placed inside the loop would count down to vmcnt(0) on every trip
     // and drain the tiles in flight.
@@ -298,9 +365,25 @@ __global__ __launch_bounds__(64 * NWV) void mfma_latent_kernel(const SweepParams
     typedef short s16x8 __attribute__((__vector_size__(8 * sizeof(short))));
 
     const float bias0 = slope * (float)(half * 4 - (len - 1));  // ALiBi: slope * (token - (len - 1)), split in lane and tile parts
-    int buf = 0;       // buffer that holds tile t
-    int buf_next = 2;  // buffer that receives tile t + 2
+    int buf = 0;       // 16-bit buffer that holds tile t
+    int buf_next = KV8 ? 0 : 2;  // buffer (FP8: stage) that receives tile t + AHEAD
+    int stg_conv = 1;  // FP8: stage that holds tile t + 1
     for (int t = 0; t < ntiles; ++t) {
+        if constexpr (KV8) {
+            // stage of tile t+1 landed (tile t+2 may still be in flight); after the barrier every wave's share of it
+            // is in LDS, every wave has converted its share of tile t, and every wave is done with tile t-1
+            if (t + 2 < ntiles)
+                wait_vmcnt<NLW8>();
+            else
+                wait_vmcnt<0>();
+            __syncthreads();
+            if (t + 1 < ntiles) convert_stage(stg_conv, buf ^ 1);
+            stg_conv = (stg_conv == 2) ? 0 : stg_conv + 1;
+            // (the stage that held tile t was converted before the barrier: free for tile t+3)
+            if (t + 3 < ntiles)
+                issue_tile(c0 + (t + 3) * kTile, row_in_page(p, start, c0 + (t + 3) * kTile, page_ahead).k, buf_next);
+            if (t + 4 < ntiles) page_ahead = page_of(p, b, c0 + (t + 4) * kTile);
+        } else {
         if (t + 1 < ntiles)
             wait_vmcnt<NLW>();  // tile t landed; tile t+1 may still be in flight
         else
@@ -309,6 +392,7 @@ __global__ __launch_bounds__(64 * NWV) void mfma_latent_kernel(const SweepParams
         if (t + 2 < ntiles)
             issue_tile(c0 + (t + 2) * kTile, row_in_page(p, start, c0 + (t + 2) * kTile, page_ahead).k, buf_next);
         if (t + 3 < ntiles) page_ahead = page_of(p, b, c0 + (t + 3) * kTile);
+        }
 
         const int tok0 = c0 + t * kTile;
         // tile base addresses, made opaque so that the constant offsets below stay in the instructions'
@@ -319,8 +403,8 @@ __global__ __launch_bounds__(64 * NWV) void mfma_latent_kernel(const SweepParams
         for (int j = 0; j < 8; ++j) kaddr[j] = ta ^ (32 * j);
 #pragma unroll
         for (int j = 0; j < 4; ++j) kaddr_b[j] = tb ^ (32 * j);
-        buf = (buf == kNBuf - 1) ? 0 : buf + 1;
-        buf_next = (buf_next == kNBuf - 1) ? 0 : buf_next + 1;
+        buf = (buf == NTB - 1) ? 0 : buf + 1;
+        buf_next = (buf_next == kNBuf - 1) ? 0 : buf_next + 1;  // (three 16-bit buffers, or three FP8 stages)
 
         // S^T = K_tile . Q^T : rows = tokens, columns = heads.  K fragments are read kKPD steps ahead.
         f32x16 s;
@@ -359,14 +443,14 @@ __global__ __launch_bounds__(64 * NWV) void mfma_latent_kernel(const SweepParams
 #pragma unroll
             for (int r = 0; r < 16; ++r) {
                 const int off = (r >> 2) * 8 + (r & 3);
-                const float x = s[r] * p.scale_log2 + (b0 + slope * (float)off);
+                const float x = s[r] * sl + (b0 + slope * (float)off);
                 pv[r] = (tok0 + half * 4 + off) < c1 ? x : -INFINITY;
                 mx = fmaxf(mx, pv[r]);
             }
         } else {
 #pragma unroll
             for (int r = 0; r < 16; ++r) {
-                pv[r] = s[r] * p.scale_log2;
+                pv[r] = s[r] * sl;
                 mx = fmaxf(mx, pv[r]);
             }
         }
@@ -427,7 +511,7 @@ __global__ __launch_bounds__(64 * NWV) void mfma_latent_kernel(const SweepParams
     if (n < nh) {
         const int h = h_base + n;
         if (p.nsplit == 1) {
-            const float inv = 1.0f / l_tot;
+            const float inv = vs / l_tot;
             uint16_t* orow = o16 + ((size_t)b * p.head_q + h) * DV;
 #pragma unroll
             for (int c = 0; c < CT; ++c)
@@ -449,7 +533,8 @@ __global__ __launch_bounds__(64 * NWV) void mfma_latent_kernel(const SweepParams
 #pragma unroll
                 for (int r4 = 0; r4 < 4; ++r4) {
                     const int col = c * 32 + r4 * 8 + half * 4;
-                    float4 w = make_float4(acc[c][r4 * 4 + 0], acc[c][r4 * 4 + 1], acc[c][r4 * 4 + 2], acc[c][r4 * 4 + 3]);
+                    float4 w = make_float4(acc[c][r4 * 4 + 0] * vs, acc[c][r4 * 4 + 1] * vs, acc[c][r4 * 4 + 2] * vs,
+                                           acc[c][r4 * 4 + 3] * vs);
                     *reinterpret_cast<float4*>(wrow + col) = w;
                 }
             if (half == 0) {
@@ -460,33 +545,38 @@ __global__ __launch_bounds__(64 * NWV) void mfma_latent_kernel(const SweepParams
     }
 }
 
-// kNBuf tile buffers; the prologue stages each wave's Q block in a buffer of its own.
-template <int D, int NWV>
+// kNBuf tile buffers (FP8: two of them and three stages of raw bytes); the prologue stages each wave's Q block in a
+// buffer of its own.
+template <int D, int NWV, bool KV8>
 constexpr size_t lds_bytes() {
-    return (size_t)(kNBuf > NWV ? kNBuf : NWV) * kTile * D * 2;
+    constexpr size_t buf = (size_t)kTile * D * 2;
+    constexpr size_t stg = (size_t)((kTile * D / 1024 + NWV - 1) / NWV) * NWV * 1024;
+    constexpr size_t tiles = KV8 ? 2 * buf + 3 * stg : (size_t)kNBuf * buf;
+    constexpr size_t qstage = (size_t)NWV * buf;
+    return tiles > qstage ? tiles : qstage;
 }
 
-template <typename Tag, int D, int DV, int NWV>
+template <typename Tag, int D, int DV, int NWV, bool KV8>
 hipError_t launch_one(const SweepParams& p, dim3 grid, hipStream_t stream) {
     static std::once_flag once;
     static hipError_t attr_err = hipSuccess;
-    auto kern = mfma_latent_kernel<Tag, D, DV, NWV>;
+    auto kern = mfma_latent_kernel<Tag, D, DV, NWV, KV8>;
     std::call_once(once, [&] {
         attr_err = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
-                                       (int)lds_bytes<D, NWV>());
+                                       (int)lds_bytes<D, NWV, KV8>());
     });
     if (attr_err != hipSuccess) return attr_err;
-    constexpr size_t lds = lds_bytes<D, NWV>();
+    constexpr size_t lds = lds_bytes<D, NWV, KV8>();
     hipLaunchKernelGGL(kern, grid, dim3(64 * NWV), lds, stream, p);
     return hipGetLastError();
 }
 
-template <typename Tag>
+template <typename Tag, bool KV8>
 hipError_t launch_tag(const SweepParams& p, int rt, dim3 grid, hipStream_t stream) {
     switch (rt) {
-        case 32: return launch_one<Tag, 576, 512, 1>(p, grid, stream);
-        case 64: return launch_one<Tag, 576, 512, 2>(p, grid, stream);
-        case 128: return launch_one<Tag, 576, 512, 4>(p, grid, stream);
+        case 32: return launch_one<Tag, 576, 512, 1, KV8>(p, grid, stream);
+        case 64: return launch_one<Tag, 576, 512, 2, KV8>(p, grid, stream);
+        case 128: return launch_one<Tag, 576, 512, 4, KV8>(p, grid, stream);
         default: return hipErrorInvalidValue;
     }
 }
@@ -500,7 +590,11 @@ int mla_heads_per_group(int ratio) { return ratio <= 32 ? 32 : (ratio <= 64 ? 64
 int mla_rows_per_trip() { return kTile; }
 
 hipError_t launch_mla(const SweepParams& p, bool is_bf16, int rt, dim3 grid, hipStream_t stream) {
-    return is_bf16 ? launch_tag<bf16_tag>(p, rt, grid, stream) : launch_tag<f16_tag>(p, rt, grid, stream);
+    return is_bf16 ? launch_tag<bf16_tag, false>(p, rt, grid, stream) : launch_tag<f16_tag, false>(p, rt, grid, stream);
+}
+
+hipError_t launch_mla_kv8(const SweepParams& p, bool is_bf16, int rt, dim3 grid, hipStream_t stream) {
+    return is_bf16 ? launch_tag<bf16_tag, true>(p, rt, grid, stream) : launch_tag<f16_tag, true>(p, rt, grid, stream);
 }
 
 }  // namespace da

@@ -97,11 +97,43 @@ def test_alibi_and_softmax_scale_with_fp8_kv():
     assert (o.float() - torch.from_numpy(ref).float()).abs().max().item() <= TOL[torch.float16]
 
 
-def test_latent_form_with_fp8_cache_runs_on_the_valu_sweep():
-    """(576, 512) with V = K[..., :512]: no FP8 MFMA kernel, served by the VALU sweep (one scale for K and V)."""
-    w, k8, _, ks, _ = _case(2, 16, 1, 576, 512, 300, torch.float16, latent=True)
-    o = decoding_attn_fwd(w.q.to(DEV), k8.to(DEV), None, w.cu_seq_k.to(DEV), w.max_seq_k, 512, False,
+@pytest.mark.parametrize("batch,head_q,seq_k,dtype,is_alibi", [
+    (2, 16, 300, torch.float16, False),     # one wave of 32 heads, half of them idle
+    (3, 64, 700, torch.bfloat16, False),    # two waves
+    (5, 128, 1500, torch.float16, False),   # four waves, several splits
+    (4, 128, 900, torch.bfloat16, True),
+    (1, 128, 5000, torch.float16, False),   # one long sequence: many short splits
+    (7, 32, 97, torch.float16, True),       # shorter than four tiles
+])
+def test_latent_form_with_fp8_cache(batch, head_q, seq_k, dtype, is_alibi):
+    """(576, 512) with V = K[..., :512]: the latent MFMA kernel over FP8 tiles converted in LDS (one scale for K
+    and V, as they are one buffer)."""
+    w, k8, _, ks, _ = _case(batch, head_q, 1, 576, 512, seq_k, dtype, latent=True, is_alibi=is_alibi, seed=seq_k)
+    assert _lib.plan(w.max_seq_k, batch, head_q, 1, 576, 512)["kind"] == 2
+    o = decoding_attn_fwd(w.q.to(DEV), k8.to(DEV), None, w.cu_seq_k.to(DEV), w.max_seq_k, 512, is_alibi,
                           k_scale=ks.to(DEV), v_scale=ks.to(DEV)).cpu()
+    ref = torch.from_numpy(_reference(w, k8, None, ks, ks)).float()
+    assert (o.float() - ref).abs().max().item() <= TOL[dtype]
+
+
+def test_latent_fp8_unit_scales_equal_the_16_bit_call_bit_for_bit():
+    """FP8 values convert exactly and the tiles are converted before any arithmetic: with unit scales the FP8 call
+    is the 16-bit call on the same values, same kernel, same order of operations."""
+    w, k8, _, ks, _ = _case(4, 128, 1, 576, 512, 1200, torch.float16, latent=True, unit=True, seed=9)
+    k16 = k8.to(torch.float16).to(DEV)
+    args = (w.cu_seq_k.to(DEV), w.max_seq_k, 512, False)
+    o8 = decoding_attn_fwd(w.q.to(DEV), k8.to(DEV), None, *args, k_scale=ks.to(DEV), v_scale=ks.to(DEV))
+    o16 = decoding_attn_fwd(w.q.to(DEV), k16, None, *args)
+    assert torch.equal(o8.view(torch.int16), o16.view(torch.int16))
+
+
+@pytest.mark.parametrize("page_size", [32, 64])
+def test_latent_paged_fp8(page_size):
+    w, k8, _, ks, _ = _case(5, 128, 1, 576, 512, 1100, torch.float16, latent=True, seed=21)
+    w8 = wl.Workload(w.name, w.q, k8.view(torch.uint8), None, w.cu_seq_k, w.max_seq_k, w.dim_v, w.is_alibi, w.lengths)
+    pk = wl.to_pages(w8, page_size, seed=2, poison=False).to(DEV)
+    o = decoding_attn_paged_fwd(w.q.to(DEV), pk.k_pages.view(FP8), None, pk.block_table, pk.seq_lens, w.max_seq_k,
+                                512, False, k_scale=ks.to(DEV), v_scale=ks.to(DEV)).cpu()
     ref = torch.from_numpy(_reference(w, k8, None, ks, ks)).float()
     assert (o.float() - ref).abs().max().item() <= TOL[torch.float16]
 
