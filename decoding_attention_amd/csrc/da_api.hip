@@ -107,22 +107,28 @@ int rows_per_trip(size_t dim) {
     }
 }
 
+// Paged K/V: the grouped-head kernel fetches whole 32-token tiles, so pages must hold a multiple of 32 tokens; the
+// latent kernel fetches row by row, two runs of 16 tokens per tile, and takes 16-token pages too (its FP8 form
+// stages whole tiles: 32 again).
+bool pages_fit_tiles(size_t page_size, bool latent, bool kv_fp8) { return page_size % (latent && !kv_fp8 ? 16 : 32) == 0; }
+
 // v_distinct: V is its own buffer (the MFMA kernel reads V out of the K tile, so it needs the aliased form).
 // total_k: sum of the key lengths if the caller knows it (0 = unknown).  The planner never reads cu_seq_k (that
 // would need a device synchronisation); when total_k shows that the batch is ragged it cuts the sequences into
 // shorter splits so that the work-groups, whose number is sized for max_seq_k, balance.
-// tiles_contiguous: every aligned run of 32 tokens is contiguous in memory (always true for the packed layout; for
-// paged K/V only when a page holds a multiple of 32 tokens).  The two MFMA kernels fetch whole tiles and need it.
+// page_size: 0 for the packed layout, else tokens per page of paged K/V; pages that do not fit the MFMA kernels'
+// tiles (pages_fit_tiles) run on the VALU sweep, which resolves every row on its own.
 // kv_fp8: K/V are FP8; the grouped kernel then needs dim % 64 == 0.
-// packed: K/V are in the packed layout addressed through cu_seq_k (the balanced grid needs the prefix offsets).
 Plan make_plan(size_t max_seq_k, size_t batch, size_t head_q, size_t head_k, size_t dim, size_t dim_v,
-               bool v_distinct, size_t total_k, bool tiles_contiguous = true, bool kv_fp8 = false, bool packed = true) {
+               bool v_distinct, size_t total_k, size_t page_size = 0, bool kv_fp8 = false) {
+    const bool packed = page_size == 0;
     Plan pl;
     const int ratio = (int)(head_q / head_k);
     int trip;
     int target_wgs = tun().target_wgs;
-    const bool force_sweep = tun().force_kind == kKindSweep || !tiles_contiguous;
-    const bool mfma = !v_distinct && da::mla_supported(dim, dim_v, ratio) && !force_sweep;
+    const bool latent = !v_distinct && da::mla_supported(dim, dim_v, ratio);
+    const bool force_sweep = tun().force_kind == kKindSweep || (page_size != 0 && !pages_fit_tiles(page_size, latent, kv_fp8));
+    const bool mfma = latent && !force_sweep;
     if (mfma) {
         pl.kind = kKindMfma;
         pl.rt = da::mla_heads_per_group(ratio);
@@ -288,19 +294,16 @@ size_t da_workspace_bytes(size_t max_seq_k, size_t batch, size_t head_q, size_t 
 size_t da_workspace_bytes_paged(size_t max_seq_k, size_t batch, size_t head_q, size_t head_k, size_t dim, size_t dim_v,
                                 size_t total_k, size_t page_size) {
     if (head_k == 0 || head_q % head_k != 0 || !supported_dims(dim, dim_v)) return 0;
-    const bool contiguous = page_size % 32 == 0;
-    const size_t a = make_plan(max_seq_k, batch, head_q, head_k, dim, dim_v, false, total_k, contiguous, false, false).ws_bytes;
-    const size_t b = make_plan(max_seq_k, batch, head_q, head_k, dim, dim_v, true, total_k, contiguous, false, false).ws_bytes;
+    const size_t a = make_plan(max_seq_k, batch, head_q, head_k, dim, dim_v, false, total_k, page_size, false).ws_bytes;
+    const size_t b = make_plan(max_seq_k, batch, head_q, head_k, dim, dim_v, true, total_k, page_size, false).ws_bytes;
     return a > b ? a : b;
 }
 
 size_t da_workspace_bytes_fp8kv(size_t max_seq_k, size_t batch, size_t head_q, size_t head_k, size_t dim,
                                 size_t dim_v, size_t total_k, size_t page_size) {
     if (head_k == 0 || head_q % head_k != 0 || !supported_dims(dim, dim_v)) return 0;
-    const bool contiguous = page_size == 0 || page_size % 32 == 0;
-    const bool packed = page_size == 0;
-    const size_t a = make_plan(max_seq_k, batch, head_q, head_k, dim, dim_v, false, total_k, contiguous, true, packed).ws_bytes;
-    const size_t b = make_plan(max_seq_k, batch, head_q, head_k, dim, dim_v, true, total_k, contiguous, true, packed).ws_bytes;
+    const size_t a = make_plan(max_seq_k, batch, head_q, head_k, dim, dim_v, false, total_k, page_size, true).ws_bytes;
+    const size_t b = make_plan(max_seq_k, batch, head_q, head_k, dim, dim_v, true, total_k, page_size, true).ws_bytes;
     return a > b ? a : b;
 }
 
@@ -351,9 +354,8 @@ int run_attention(const void* q, const void* k, const void* v, void* o, const in
     if (batch == 0) return DA_OK;
 
     hipStream_t stream = reinterpret_cast<hipStream_t>(hip_stream);
-    const bool tiles_contiguous = !pg.table || pg.page_size % 32 == 0;
-    const Plan pl = make_plan(max_seq_k, batch, head_q, head_k, dim, dim_v, v != nullptr, total_k, tiles_contiguous, kf.fp8,
-                              pg.table == nullptr);
+    const Plan pl = make_plan(max_seq_k, batch, head_q, head_k, dim, dim_v, v != nullptr, total_k,
+                              pg.table ? pg.page_size : 0, kf.fp8);
     if ((size_t)head_k * pl.groups > 65535)
         return fail(DA_ERR_INVALID_ARGUMENT, "head_k * groups exceeds the grid limit 65535");
 

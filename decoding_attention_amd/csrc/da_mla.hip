@@ -268,10 +268,13 @@ __global__ __launch_bounds__(64 * NWV) void mfma_latent_kernel(const SweepParams
     // Stage the tile that starts at token tok0 into buffer `buf`.  Rows past the end of the split re-read the
     // last valid row (they are masked later).  Every wave always issues exactly NLW loads, so the hand-placed
     // vmcnt waits count the same on every wave.
-    // `row0` is the tile's first row as row_ref() gives it (a tile never straddles pages of paged K/V: pages hold
-    // a multiple of kTile tokens and tiles start at multiples of kTile).
-    auto issue_tile = [&](int tok0, int64_t row0, int buf) {
+    // `row0` and `row1` are the rows of the tile's tokens 0 and 16 as row_ref() gives them: a tile is fetched as two
+    // runs of 16 tokens, each inside one page (pages of paged K/V hold a multiple of 16 tokens and tiles start at
+    // multiples of kTile; for the packed layout and larger pages the second run follows the first).  A row past the
+    // end re-reads the last valid row, in whichever run that is.
+    auto issue_tile = [&](int tok0, int64_t row0, int64_t row1, int buf) {
         const uint8_t* const base = kbytes + row0 * KB;
+        const uint8_t* const base1 = kbytes + row1 * KB;
         const int last = c1 - 1 - tok0;
         if constexpr (KV8) {
             // stage `buf`: the tile's bytes in row order, lane l of load j bringing bytes [1024 j + 16 l, +16)
@@ -288,15 +291,18 @@ __global__ __launch_bounds__(64 * NWV) void mfma_latent_kernel(const SweepParams
 #pragma unroll
         for (int q = 0; q < NLA; ++q) {
             const int row = wave + NWV * q;  // wave-uniform
-            lds_dma16(base, (uint32_t)min(row, last) * (uint32_t)k_row_bytes + (lane16 ^ (uint32_t)(swz_a(row) * 16)),
+            const int rc = min(row, last), run = rc >> 4;
+            lds_dma16(run ? base1 : base,
+                      (uint32_t)(rc - run * 16) * (uint32_t)k_row_bytes + (lane16 ^ (uint32_t)(swz_a(row) * 16)),
                       smem_off + (uint32_t)(buf * BUF + row * ROW_A));
         }
 #pragma unroll
         for (int q = 0; q < NLB; ++q) {
             const int j = wave + NWV * q;
             const int row = j * 8 + rb;
-            lds_dma16(base, (uint32_t)min(row, last) * (uint32_t)k_row_bytes +
-                                (uint32_t)(DV * 2 + (((lane & 7) ^ swz_b(row)) * 16)),
+            const int run = min(j >> 1, last >> 4);  // the eight rows of a load lie in one run, clamped or not
+            lds_dma16(run ? base1 : base, (uint32_t)(min(row, last) - run * 16) * (uint32_t)k_row_bytes +
+                                              (uint32_t)(DV * 2 + (((lane & 7) ^ swz_b(row)) * 16)),
                       smem_off + (uint32_t)(buf * BUF + OFF_B + j * 1024));
         }
     };
@@ -329,11 +335,25 @@ __global__ __launch_bounds__(64 * NWV) void mfma_latent_kernel(const SweepParams
     };
 
     const int ntiles = (c1 - c0 + kTile - 1) / kTile;
-    issue_tile(c0, row_ref(p, b, start, c0).k, 0);
-    if (ntiles > 1) issue_tile(c0 + kTile, row_ref(p, b, start, c0 + kTile).k, 1);
+    // rows of tokens tok and tok + 16 (the second only looked up when the tile has it: the block table ends with
+    // the sequence's last page)
+    auto second_run = [&](int tok, int64_t first) {
+        return tok + 16 < c1 ? row_ref(p, b, start, tok + 16).k : first;
+    };
+    {
+        const int64_t r0 = row_ref(p, b, start, c0).k;
+        issue_tile(c0, r0, second_run(c0, r0), 0);
+    }
+    if (ntiles > 1) {
+        const int64_t r0 = row_ref(p, b, start, c0 + kTile).k;
+        issue_tile(c0 + kTile, r0, second_run(c0 + kTile, r0), 1);
+    }
     if constexpr (KV8) {
         // three stages in flight; the first tile is converted here, tile t + 1 at the top of trip t
-        if (ntiles > 2) issue_tile(c0 + 2 * kTile, row_ref(p, b, start, c0 + 2 * kTile).k, 2);
+        if (ntiles > 2) {
+            const int64_t r0 = row_ref(p, b, start, c0 + 2 * kTile).k;
+            issue_tile(c0 + 2 * kTile, r0, r0, 2);  // (FP8 stages whole tiles: pages hold a multiple of kTile)
+        }
         if (ntiles > 2)
             wait_vmcnt<2 * NLW8>();
         else if (ntiles > 1)
@@ -346,6 +366,7 @@ __global__ __launch_bounds__(64 * NWV) void mfma_latent_kernel(const SweepParams
     // page of the tile after those, fetched one trip ahead of its use (a scalar load for paged K/V)
     constexpr int AHEAD = KV8 ? 3 : 2;  // tiles in flight behind the one being read
     int page_ahead = ntiles > AHEAD ? page_of(p, b, c0 + AHEAD * kTile) : 0;
+    int page_ahead1 = ntiles > AHEAD && c0 + AHEAD * kTile + 16 < c1 ? page_of(p, b, c0 + AHEAD * kTile + 16) : 0;
     // Make the compiler settle its own wait for the Q loads here, before the loop.  It cannot see the
     // direct-to-LDS loads, so a wait for Q placed inside the loop would count down to vmcnt(0) on every trip
     // and drain the tiles in flight.
@@ -380,8 +401,10 @@ __global__ __launch_bounds__(64 * NWV) void mfma_latent_kernel(const SweepParams
             if (t + 1 < ntiles) convert_stage(stg_conv, buf ^ 1);
             stg_conv = (stg_conv == 2) ? 0 : stg_conv + 1;
             // (the stage that held tile t was converted before the barrier: free for tile t+3)
-            if (t + 3 < ntiles)
-                issue_tile(c0 + (t + 3) * kTile, row_in_page(p, start, c0 + (t + 3) * kTile, page_ahead).k, buf_next);
+            if (t + 3 < ntiles) {
+                const int64_t r0 = row_in_page(p, start, c0 + (t + 3) * kTile, page_ahead).k;
+                issue_tile(c0 + (t + 3) * kTile, r0, r0, buf_next);
+            }
             if (t + 4 < ntiles) page_ahead = page_of(p, b, c0 + (t + 4) * kTile);
         } else {
         if (t + 1 < ntiles)
@@ -389,9 +412,16 @@ __global__ __launch_bounds__(64 * NWV) void mfma_latent_kernel(const SweepParams
         else
             wait_vmcnt<0>();
         __syncthreads();  // every wave's share of tile t is in LDS, and every wave is done with tile t-1
-        if (t + 2 < ntiles)
-            issue_tile(c0 + (t + 2) * kTile, row_in_page(p, start, c0 + (t + 2) * kTile, page_ahead).k, buf_next);
-        if (t + 3 < ntiles) page_ahead = page_of(p, b, c0 + (t + 3) * kTile);
+        if (t + 2 < ntiles) {
+            const int tk = c0 + (t + 2) * kTile;
+            const int64_t r0 = row_in_page(p, start, tk, page_ahead).k;
+            issue_tile(tk, r0, tk + 16 < c1 ? row_in_page(p, start, tk + 16, page_ahead1).k : r0, buf_next);
+        }
+        if (t + 3 < ntiles) {
+            const int tk = c0 + (t + 3) * kTile;
+            page_ahead = page_of(p, b, tk);
+            if (tk + 16 < c1) page_ahead1 = page_of(p, b, tk + 16);
+        }
         }
 
         const int tok0 = c0 + t * kTile;

@@ -67,6 +67,19 @@ def test_with_the_token_count_hint(name):
     check_against_oracle(w, paged)
 
 
+@pytest.mark.parametrize("name", ["mla", "mla_h16"])
+def test_latent_kernel_takes_16_token_pages(name):
+    """The latent kernel fetches a tile as two runs of 16 tokens, so 16-token pages (a common cache block size) stay
+    on it: same kernel and plan as the packed call, same bits."""
+    w = _workload(name)
+    dense, paged = _run_both(w, 16)
+    assert torch.isfinite(paged.float()).all()
+    assert torch.equal(dense.view(torch.int16), paged.view(torch.int16))
+    lib = _lib.load()
+    shape = (w.max_seq_k, w.batch, w.head_q, 1, 576, 512)
+    assert lib.da_workspace_bytes_paged(*shape, 0, 16) == lib.da_workspace_bytes_paged(*shape, 0, 64)
+
+
 @pytest.mark.parametrize("page_size", [1, 4, 16])
 @pytest.mark.parametrize("name", ["mha", "gqa", "mqa", "mla_h16"])
 def test_small_pages_match_the_oracle(name, page_size):
