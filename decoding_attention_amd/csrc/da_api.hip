@@ -107,10 +107,9 @@ int rows_per_trip(size_t dim) {
     }
 }
 
-// Paged K/V: the grouped-head kernel fetches whole 32-token tiles, so pages must hold a multiple of 32 tokens; the
-// latent kernel fetches row by row, two runs of 16 tokens per tile, and takes 16-token pages too (its FP8 form
-// stages whole tiles: 32 again).
-bool pages_fit_tiles(size_t page_size, bool latent, bool kv_fp8) { return page_size % (latent && !kv_fp8 ? 16 : 32) == 0; }
+// Paged K/V: the MFMA kernels fetch a tile as two runs of 16 tokens, each from one page, so pages must hold a
+// multiple of 16 tokens; only the latent kernel's FP8 form stages whole 32-token tiles and needs a multiple of 32.
+bool pages_fit_tiles(size_t page_size, bool latent, bool kv_fp8) { return page_size % (latent && kv_fp8 ? 32 : 16) == 0; }
 
 // v_distinct: V is its own buffer (the MFMA kernel reads V out of the K tile, so it needs the aliased form).
 // total_k: sum of the key lengths if the caller knows it (0 = unknown).  The planner never reads cu_seq_k (that

@@ -88,7 +88,8 @@ constexpr size_t gqa_lds_bytes(int nt) {
 // One segment of work: tokens [c0, c1) of sequence b (first row `start`, `len` tokens) for the KV heads and head
 // group blockIdx.y selects.  `direct`: the segment is the whole sequence, so the result goes to o; otherwise the
 // un-normalised partial goes to workspace slot `split` of the sequence.
-template <typename Tag, int D, int DV, int NT, bool PREFETCH, bool WH, bool KV8>
+// HP (16-token pages of paged K/V): a tile is fetched as two runs of 16 tokens, each from one page.
+template <typename Tag, int D, int DV, int NT, bool PREFETCH, bool WH, bool KV8, bool HP>
 __device__ __forceinline__ void gqa_segment(const SweepParams& p, uint8_t* const smem, const int b, const int start,
                                             const int len, const int c0, const int c1, const int split,
                                             const bool direct) {
@@ -158,8 +159,8 @@ __device__ __forceinline__ void gqa_segment(const SweepParams& p, uint8_t* const
     }
 
     // wave-uniform byte bases (scalar registers) and 32-bit per-lane byte offsets
-    // (a tile of kGqaTile tokens is contiguous: it starts at a multiple of kGqaTile within the sequence, and pages
-    // of paged K/V hold a multiple of kGqaTile tokens, so one row_ref per tile locates it)
+    // (a tile of kGqaTile tokens starts at a multiple of kGqaTile within the sequence; pages of paged K/V hold a
+    // multiple of kGqaTile tokens, so one row_ref per tile locates it, or, with HP, 16 tokens: one per half)
     const uint8_t* const kbytes = reinterpret_cast<const uint8_t*>(p.k) + (size_t)hk * D * KB;
     const uint8_t* const vbytes = reinterpret_cast<const uint8_t*>(p.v) + (size_t)hk * p.v_head * KB;
     const uint32_t k_row_b = (uint32_t)p.k_row * KB, v_row_b = (uint32_t)p.v_row * KB;
@@ -182,24 +183,39 @@ __device__ __forceinline__ void gqa_segment(const SweepParams& p, uint8_t* const
     };
     TileRegs tr;
 
+    // Rows past the end re-read the last valid row (in whichever run of 16 that is, with 16-token pages) and are
+    // masked.  The choice between the two runs is wave-uniform: an M-tile of K is one run, and a V load instruction
+    // covers a power-of-two number of rows inside one run, except for d = 96 (12 chunks per row), which chooses
+    // per lane.
     auto load_k = [&](int tok0, TileRegs& r) __attribute__((always_inline)) {
-        const uint8_t* const base = kbytes + row_ref(p, b, start, tok0).k * KB;
-        const int last = c1 - 1 - tok0;  // rows past the end re-read the last row and are masked
+        const int last = c1 - 1 - tok0;
+        const uint8_t* const base0 = kbytes + row_ref(p, b, start, tok0).k * KB;
+        const uint8_t* base1 = base0;
+        if constexpr (HP)
+            if (last >= 16) base1 = kbytes + row_ref(p, b, start, tok0 + 16).k * KB;
 #pragma unroll
         for (int mt = 0; mt < 2; ++mt) {
-            const uint32_t off = (uint32_t)min(mt * 16 + n, last) * k_row_b + g * 16;
+            const bool second = HP && mt == 1 && last >= 16;
+            const uint8_t* const base = second ? base1 : base0;
+            const uint32_t off = (uint32_t)(min(mt * 16 + n, last) - (second ? 16 : 0)) * k_row_b + g * 16;
 #pragma unroll
             for (int ks = 0; ks < KSR; ++ks) r.k[mt][ks] = *reinterpret_cast<const uint4*>(base + off + ks * 64);
         }
     };
     auto load_v = [&](int tok0, TileRegs& r) __attribute__((always_inline)) {
-        const uint8_t* const base = vbytes + row_ref(p, b, start, tok0).v * KB;
         const int last = c1 - 1 - tok0;
+        const uint8_t* const base0 = vbytes + row_ref(p, b, start, tok0).v * KB;
+        const uint8_t* base1 = base0;
+        if constexpr (HP)
+            if (last >= 16) base1 = vbytes + row_ref(p, b, start, tok0 + 16).v * KB;
+        constexpr bool kUniform = 64 % CPRL == 0 && 16 % (64 / CPRL) == 0;
 #pragma unroll
         for (int i = 0; i < NVR; ++i) {
             const int slot = i * 64 + lane;
             const int row = slot / CPRL, ch = slot % CPRL;
-            const uint32_t off = (uint32_t)min(row, last) * v_row_b + ch * 16;
+            const bool second = HP && (kUniform ? i * (64 / CPRL) >= 16 : row >= 16) && last >= 16;
+            const uint8_t* const base = second ? base1 : base0;
+            const uint32_t off = (uint32_t)(min(row, last) - (second ? 16 : 0)) * v_row_b + ch * 16;
             r.v[i] = *reinterpret_cast<const uint4*>(base + off);
         }
     };
@@ -432,7 +448,7 @@ __device__ __forceinline__ void gqa_segment(const SweepParams& p, uint8_t* const
 // does not give.  Sequence b spans work-groups first(b) = cu[b] / T ... last(b) = (cu[b+1] - 1) / T (both capped
 // at W - 1); its segment in work-group i is partial number i - first(b), and goes straight to o when
 // first(b) == last(b).
-template <typename Tag, int D, int DV, int NT, bool PREFETCH, bool WH, int MINW, bool KV8 = false>
+template <typename Tag, int D, int DV, int NT, bool PREFETCH, bool WH, int MINW, bool KV8 = false, bool HP = false>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(MINW))) void gqa_mfma_kernel(const SweepParams p) {
     extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
     if (p.flat_tokens == 0) {
@@ -441,7 +457,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(MINW))) voi
         seq_range(p, b, start, len);
         const int c0 = split * p.chunk;
         const int c1 = (split == p.nsplit - 1) ? len : min(len, c0 + p.chunk);
-        gqa_segment<Tag, D, DV, NT, PREFETCH, WH, KV8>(p, smem, b, start, len, c0, c1, split, p.nsplit == 1);
+        gqa_segment<Tag, D, DV, NT, PREFETCH, WH, KV8, HP>(p, smem, b, start, len, c0, c1, split, p.nsplit == 1);
         return;
     }
     const int T = p.flat_tokens, W = (int)gridDim.x, i = (int)blockIdx.x, unit = p.flat_unit;
@@ -470,7 +486,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(MINW))) voi
         seq_range(p, b, start, len);
         const int first = min(s / T, W - 1), last = min((e - 1) / T, W - 1);
         const int c0 = (max(r0, s) - s) * unit, c1 = min((min(r1, e) - s) * unit, len);
-        gqa_segment<Tag, D, DV, NT, PREFETCH, WH, KV8>(p, smem, b, start, len, c0, c1, i - first, first == last);
+        gqa_segment<Tag, D, DV, NT, PREFETCH, WH, KV8, HP>(p, smem, b, start, len, c0, c1, i - first, first == last);
         if (!WH) __syncthreads();  // the merge area of this segment is the V tile area of the next
     }
 }
