@@ -278,12 +278,16 @@ __global__ __launch_bounds__(64 * NWV) void mfma_latent_kernel(const SweepParams
         const int last = c1 - 1 - tok0;
         if constexpr (KV8) {
             // stage `buf`: the tile's bytes in row order, lane l of load j bringing bytes [1024 j + 16 l, +16)
+            static_assert(16 * D % 1024 == 0, "the two runs of a staged tile meet on a load boundary");
 #pragma unroll
             for (int q = 0; q < NLW8; ++q) {
                 const int j = min(wave + NWV * q, STG_REAL - 1);  // wave-uniform; surplus loads repeat the last KiB
                 const uint32_t off = (uint32_t)j * 1024u + lane16;
                 const uint32_t row = off / (uint32_t)D, within = off - row * (uint32_t)D;
-                lds_dma16(base, (uint32_t)min((int)row, last) * (uint32_t)k_row_bytes + within,
+                // rows 0..15 fill loads 0..8 exactly, rows 16..31 loads 9..17: the run is wave-uniform
+                const int run = min(j >= 16 * D / 1024 ? 1 : 0, last >> 4);
+                lds_dma16(run ? base1 : base,
+                          (uint32_t)(min((int)row, last) - run * 16) * (uint32_t)k_row_bytes + within,
                           smem_off + (uint32_t)(STG0 + buf * STG + (wave + NWV * q) * 1024));
             }
             return;
@@ -352,7 +356,7 @@ __global__ __launch_bounds__(64 * NWV) void mfma_latent_kernel(const SweepParams
         // three stages in flight; the first tile is converted here, tile t + 1 at the top of trip t
         if (ntiles > 2) {
             const int64_t r0 = row_ref(p, b, start, c0 + 2 * kTile).k;
-            issue_tile(c0 + 2 * kTile, r0, r0, 2);  // (FP8 stages whole tiles: pages hold a multiple of kTile)
+            issue_tile(c0 + 2 * kTile, r0, second_run(c0 + 2 * kTile, r0), 2);
         }
         if (ntiles > 2)
             wait_vmcnt<2 * NLW8>();
@@ -402,10 +406,15 @@ __global__ __launch_bounds__(64 * NWV) void mfma_latent_kernel(const SweepParams
             stg_conv = (stg_conv == 2) ? 0 : stg_conv + 1;
             // (the stage that held tile t was converted before the barrier: free for tile t+3)
             if (t + 3 < ntiles) {
-                const int64_t r0 = row_in_page(p, start, c0 + (t + 3) * kTile, page_ahead).k;
-                issue_tile(c0 + (t + 3) * kTile, r0, r0, buf_next);
+                const int tk = c0 + (t + 3) * kTile;
+                const int64_t r0 = row_in_page(p, start, tk, page_ahead).k;
+                issue_tile(tk, r0, tk + 16 < c1 ? row_in_page(p, start, tk + 16, page_ahead1).k : r0, buf_next);
             }
-            if (t + 4 < ntiles) page_ahead = page_of(p, b, c0 + (t + 4) * kTile);
+            if (t + 4 < ntiles) {
+                const int tk = c0 + (t + 4) * kTile;
+                page_ahead = page_of(p, b, tk);
+                if (tk + 16 < c1) page_ahead1 = page_of(p, b, tk + 16);
+            }
         } else {
         if (t + 1 < ntiles)
             wait_vmcnt<NLW>();  // tile t landed; tile t+1 may still be in flight
