@@ -65,3 +65,26 @@ def test_paged_call_replays_from_a_graph():
         return decoding_attn_paged_fwd(q, pk.k_pages, pk.v_pages, pk.block_table, pk.seq_lens, w.max_seq_k, 128, False)
 
     _replay_matches_eager(run, [q, pk.k_pages, pk.v_pages], lambda o: o)
+
+
+def test_fp8_latent_and_16_token_pages_replay_from_a_graph():
+    """The FP8 form of the latent kernel (tiles converted in LDS) and the 16-token-page form of the grouped kernel."""
+    w = wl.config_mla(3, 900, seed=8)
+    q = w.q.to(DEV)
+    k8 = (w.k.float() / 0.02).to(torch.float8_e4m3fn).to(DEV)
+    ks = torch.full((1,), 0.02, device=DEV)
+    cu = w.cu_seq_k.to(DEV)
+
+    def run_latent():
+        return decoding_attn_fwd(q, k8, None, cu, w.max_seq_k, 512, False, k_scale=ks, v_scale=ks)
+
+    _replay_matches_eager(run_latent, [q], lambda o: o)
+
+    w2 = wl.make_workload(6, 32, 1, 128, 128, 1100, torch.bfloat16, seed=9, varlen=True)
+    pk = wl.to_pages(w2, 16, seed=9, poison=False).to(DEV)
+    q2 = w2.q.to(DEV)
+
+    def run_paged():
+        return decoding_attn_paged_fwd(q2, pk.k_pages, pk.v_pages, pk.block_table, pk.seq_lens, w2.max_seq_k, 128, False)
+
+    _replay_matches_eager(run_paged, [q2, pk.k_pages, pk.v_pages], lambda o: o)
