@@ -74,6 +74,19 @@ __device__ __forceinline__ float max_xor32(float x) {
     return fmaxf(__builtin_bit_cast(float, r0), __builtin_bit_cast(float, r1));
 }
 
+// A probability as the second matrix product will see it.  bf16 keeps 8 significant bits, so the rounded
+// probabilities of a row no longer sum to the fp32 denominator; with the denominator summed from the rounded values
+// the weights sum to one again, and the rounding errors enter as w (v - o) instead of w v -- what matters when few
+// tokens carry the weight (steep ALiBi slopes, short sequences).  fp16's 11 bits are below the output rounding
+// either way and are left alone.
+template <typename Tag>
+__device__ __forceinline__ float as_second_operand(float p) {
+    if constexpr (std::is_same<Tag, bf16_tag>::value)
+        return (float)(__bf16)p;
+    else
+        return p;
+}
+
 // Eight FP8 (OCP e4m3) values -> eight 16-bit elements of the compute type.  Both conversions are exact (e4m3
 // has 3 mantissa bits and |x| <= 448), so an FP8 K/V cache feeds the same arithmetic as a 16-bit one.
 template <typename Tag>

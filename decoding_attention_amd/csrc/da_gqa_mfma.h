@@ -319,7 +319,7 @@ __device__ __forceinline__ void gqa_segment(const SweepParams& p, uint8_t* const
         for (int nt = 0; nt < NT; ++nt) {
 #pragma unroll
             for (int j = 0; j < 8; ++j) {
-                x[nt][j] = fast_exp2(x[nt][j] - m[nt]);
+                x[nt][j] = as_second_operand<Tag>(fast_exp2(x[nt][j] - m[nt]));
                 l[nt] += x[nt][j];
             }
             pf[nt] = MM::pack8(x[nt]);  // k index j <-> token g*4+j (j<4), 16+g*4+(j-4) (j>=4)

@@ -511,7 +511,7 @@ __global__ __launch_bounds__(64 * NWV) void mfma_latent_kernel(const SweepParams
         }
 #pragma unroll
         for (int r = 0; r < 16; ++r) {
-            pv[r] = fast_exp2(pv[r] - m);
+            pv[r] = as_second_operand<Tag>(fast_exp2(pv[r] - m));
             l += pv[r];
         }
         vec8 pf[2];
