@@ -1,0 +1,103 @@
+"""Randomised differential test: every path of the library (packed with and without the token-count hint, paged with
+pages of 1..128 tokens, FP8 caches, the latent form, ALiBi, ragged and empty sequences) against float64 attention on
+a sample of rows.  Shapes, layouts and options are drawn from a fixed seed, so a failure names its case.
+
+The tolerance is the acceptance bar scaled by the magnitude of the result: a bf16 output of magnitude 2..4 is only
+representable to 0.0078, so the absolute bar of 1e-2 is widened in proportion when |o| > 1.
+"""
+import random
+
+import pytest
+import torch
+
+from decoding_attention_amd import decoding_attn_fwd, decoding_attn_paged_fwd
+from decoding_attention_amd import workloads as wl
+from oracle import oracle
+from tests.gpu_util import TOL, run_hip_ex, sub_workload
+
+pytestmark = pytest.mark.gpu
+
+DEV = "cuda:0"
+FP8 = torch.float8_e4m3fn
+HEADS = [(32, 8), (32, 32), (32, 1), (8, 2), (28, 4), (16, 16), (64, 8), (12, 4), (40, 8), (4, 1), (6, 3), (64, 2)]
+CASES_PER_CHUNK = 12
+
+
+def _one_case(rng, seed, case):
+    latent = rng.random() < 0.3
+    dtype = rng.choice([torch.float16, torch.bfloat16])
+    if latent:
+        hq, hk, d, dv = rng.choice([16, 32, 64, 128, 96, 8]), 1, 576, 512
+    else:
+        hq, hk = rng.choice(HEADS)
+        d = dv = rng.choice([64, 96, 128, 256])
+    batch = rng.choice([1, 2, 3, 5, 8, 17, 40, 90])
+    maxlen = rng.choice([5, 33, 100, 300, 777, 1500, 3000, 6000])
+    if batch * maxlen * hk * d > 1.5e8:
+        maxlen = max(5, int(1.5e8 / (batch * hk * d)))
+    g = torch.Generator().manual_seed(seed * 100003 + case)
+    mode = rng.choice(["fixed", "ragged", "ragged0"])
+    if mode == "fixed":
+        lens = torch.full((batch,), maxlen, dtype=torch.int32)
+    else:
+        lens = torch.randint(1, maxlen + 1, (batch,), generator=g, dtype=torch.int32)
+        if mode == "ragged0" and batch > 1:
+            lens[torch.rand(batch, generator=g) < 0.2] = 0
+        if int(lens.max()) == 0:
+            lens[0] = maxlen
+    alibi = rng.random() < 0.3
+    total = int(lens.sum())
+    q = torch.randn(batch, hq, d, generator=g).to(dtype)
+    k = torch.randn(total, hk, d, generator=g).to(dtype)
+    v = None if latent else torch.randn(total, hk, dv, generator=g).to(dtype)
+    fp8 = rng.random() < 0.35
+    layout = rng.choice(["packed", "packed_nohint", "paged"])
+    page = rng.choice([1, 8, 16, 32, 64, 128])
+    desc = (f"seed {seed} case {case}: latent={latent} {hq}/{hk} d{d} {dtype} b{batch} max{maxlen} {mode} "
+            f"alibi={alibi} fp8={fp8} {layout} page={page} total={total}")
+    kw, k8, v8 = {}, None, None
+    k_true, v_true = k.float(), None if v is None else v.float()
+    if fp8:
+        ks = 0.015 + 0.015 * torch.rand(hk, generator=g)
+        vs = ks if latent else 0.015 + 0.015 * torch.rand(hk, generator=g)
+        k8 = (k.float() / ks.view(1, -1, 1)).to(FP8)
+        k_true = k8.float() * ks.view(1, -1, 1)
+        if v is not None:
+            v8 = (v.float() / vs.view(1, -1, 1)).to(FP8)
+            v_true = v8.float() * vs.view(1, -1, 1)
+        kw = dict(k_scale=ks.to(DEV), v_scale=vs.to(DEV))
+    cu = wl.get_cu_seq(lens)
+    max_seq_k = int(lens.max())
+    if layout == "paged":
+        src = wl.Workload("p", q, k8.view(torch.uint8) if fp8 else k,
+                          None if v is None else (v8.view(torch.uint8) if fp8 else v), cu, max_seq_k, dv, alibi,
+                          lens.tolist())
+        pk = wl.to_pages(src, page, seed=case, poison=not fp8).to(DEV)
+        kp = pk.k_pages.view(FP8) if fp8 else pk.k_pages
+        vp = None if pk.v_pages is None else (pk.v_pages.view(FP8) if fp8 else pk.v_pages)
+        o = decoding_attn_paged_fwd(q.to(DEV), kp, vp, pk.block_table, pk.seq_lens, max_seq_k, dv, alibi,
+                                    total_k=rng.choice([0, total]), **kw)
+    elif layout == "packed_nohint" and not fp8:
+        o = run_hip_ex(wl.Workload("x", q, k, v, cu, max_seq_k, dv, alibi, lens.tolist()), 0)
+    else:
+        o = decoding_attn_fwd(q.to(DEV), (k8 if fp8 else k).to(DEV),
+                              None if v is None else (v8 if fp8 else v).to(DEV), cu.to(DEV), max_seq_k, dv, alibi, **kw)
+    torch.cuda.synchronize()
+    o = o.cpu()
+    assert torch.isfinite(o.float()).all(), desc
+    rows = list(range(batch)) if batch <= 8 else sorted(set(rng.sample(range(batch), 8)) | {int(lens.argmax())})
+    sub = sub_workload(wl.Workload("o", q.float(), k_true, v_true, cu, max_seq_k, dv, alibi, lens.tolist()), rows)
+    ref = torch.from_numpy(oracle.attn_f64(sub.q, sub.k, sub.v, sub.cu_seq_k, dv, alibi)).float()
+    err = (o[rows].float() - ref).abs().max().item()
+    assert err <= TOL[dtype] * max(1.0, ref.abs().max().item()), f"{desc}: max-abs {err:.3e}"
+    for b in range(batch):
+        if int(lens[b]) == 0:
+            assert torch.count_nonzero(o[b]) == 0, desc
+
+
+@pytest.mark.parametrize("chunk", range(8))
+def test_random_cases(chunk):
+    seed = 7
+    rng = random.Random(seed * 1000 + chunk)
+    for i in range(CASES_PER_CHUNK):
+        _one_case(rng, seed, chunk * CASES_PER_CHUNK + i)
