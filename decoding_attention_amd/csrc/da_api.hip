@@ -108,8 +108,8 @@ int rows_per_trip(size_t dim) {
 }
 
 // Paged K/V: the MFMA kernels fetch a tile as two runs of 16 tokens, each from one page, so pages must hold a
-// multiple of 16 tokens.
-bool pages_fit_tiles(size_t page_size) { return page_size % 16 == 0; }
+// multiple of 16 tokens; the latent kernel's 16-bit form also has a per-row lookup variant for smaller pages.
+bool pages_fit_tiles(size_t page_size, bool latent_16bit) { return page_size % 16 == 0 || latent_16bit; }
 
 // v_distinct: V is its own buffer (the MFMA kernel reads V out of the K tile, so it needs the aliased form).
 // total_k: sum of the key lengths if the caller knows it (0 = unknown).  The planner never reads cu_seq_k (that
@@ -126,7 +126,7 @@ Plan make_plan(size_t max_seq_k, size_t batch, size_t head_q, size_t head_k, siz
     int trip;
     int target_wgs = tun().target_wgs;
     const bool latent = !v_distinct && da::mla_supported(dim, dim_v, ratio);
-    const bool force_sweep = tun().force_kind == kKindSweep || (page_size != 0 && !pages_fit_tiles(page_size));
+    const bool force_sweep = tun().force_kind == kKindSweep || (page_size != 0 && !pages_fit_tiles(page_size, latent && !kv_fp8));
     const bool mfma = latent && !force_sweep;
     if (mfma) {
         pl.kind = kKindMfma;

@@ -106,6 +106,12 @@ __device__ __forceinline__ void lds_dma16(const void* gbase, uint32_t lane_off, 
                  : "memory");
 }
 
+// The same with a full per-lane address (rows of different pages in one load).
+__device__ __forceinline__ void lds_dma16_v(const void* lane_addr, uint32_t lds_off) {
+    const uint32_t off = __builtin_amdgcn_readfirstlane(lds_off);
+    asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off" ::"v"(lane_addr), "s"(off) : "memory");
+}
+
 // x *= alpha for an MFMA accumulator element that lives in an accumulation register.  Written as
 // assembly on the AGPR so that the (rare) rescale path does not pull the 256 accumulators of a
 // wave into ordinary VGPRs around the whole loop.
@@ -147,8 +153,10 @@ __device__ __forceinline__ void wait_vmcnt() {
     asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory");
 }
 
-template <typename Tag, int D, int DV, int NWV, bool KV8>
+// PG: paged K/V with pages of fewer than 16 tokens (down to 1): every row of a tile has its own page lookup.
+template <typename Tag, int D, int DV, int NWV, bool KV8, bool PG = false>
 __global__ __launch_bounds__(64 * NWV) void mfma_latent_kernel(const SweepParams p) {
+    static_assert(!(KV8 && PG), "the FP8 form stages runs of 16 tokens");
     using MM = Mma<Tag>;
     using vec8 = typename MM::vec8;
     using EL = Elem<Tag>;
@@ -311,6 +319,46 @@ __global__ __launch_bounds__(64 * NWV) void mfma_latent_kernel(const SweepParams
         }
     };
 
+    // PG: the wave's kTile / NWV rows are consecutive here (rows wave * NLA + q), the same rows for both regions, so
+    // one set of page lookups (scalar loads, fetched a trip ahead like the page of a whole tile otherwise) serves
+    // both; the second region's load covers eight rows, so its lanes pick their row's address out of the set.
+    struct RowPages {
+        int pg[NLA];
+    };
+    auto lookup_rows = [&](int tok0) {
+        RowPages r;
+        const int last = c1 - 1 - tok0;
+#pragma unroll
+        for (int q = 0; q < NLA; ++q) r.pg[q] = page_of(p, b, tok0 + min(wave * NLA + q, last));
+        return r;
+    };
+    auto issue_tile_pg = [&](int tok0, const RowPages& rp, int buf) {
+        const int last = c1 - 1 - tok0;
+        const int mask = (1 << p.page_shift) - 1;
+        int64_t rowoff[NLA];  // byte offsets of the wave's rows
+#pragma unroll
+        for (int q = 0; q < NLA; ++q) {
+            const int tok = tok0 + min(wave * NLA + q, last);
+            rowoff[q] = ((int64_t)rp.pg[q] * p.k_page + (int64_t)(tok & mask) * p.k_row) * KB;
+        }
+#pragma unroll
+        for (int q = 0; q < NLA; ++q) {
+            const int row = wave * NLA + q;
+            lds_dma16(kbytes + rowoff[q], lane16 ^ (uint32_t)(swz_a(row) * 16),
+                      smem_off + (uint32_t)(buf * BUF + row * ROW_A));
+        }
+#pragma unroll
+        for (int q = 0; q < NLB; ++q) {
+            const int j = wave * NLB + q;
+            const int row = j * 8 + rb;
+            int64_t mine = rowoff[8 * q];
+#pragma unroll
+            for (int i = 1; i < 8; ++i) mine = rb == i ? rowoff[8 * q + i] : mine;
+            lds_dma16_v(kbytes + mine + (DV * 2 + (((lane & 7) ^ swz_b(row)) * 16)),
+                        smem_off + (uint32_t)(buf * BUF + OFF_B + j * 1024));
+        }
+    };
+
     // FP8: convert stage `stg` into 16-bit tile buffer `tb` (swizzled layout).  Eight threads share a row: thread
     // (row, j) converts the row's 8-element chunks j, j + 8, ..., j + 64, so its swizzles are constants and each
     // chunk costs one address XOR.
@@ -344,13 +392,18 @@ __global__ __launch_bounds__(64 * NWV) void mfma_latent_kernel(const SweepParams
     auto second_run = [&](int tok, int64_t first) {
         return tok + 16 < c1 ? row_ref(p, b, start, tok + 16).k : first;
     };
-    {
+    RowPages rows_ahead{};
+    if constexpr (PG) {
+        issue_tile_pg(c0, lookup_rows(c0), 0);
+        if (ntiles > 1) issue_tile_pg(c0 + kTile, lookup_rows(c0 + kTile), 1);
+        if (ntiles > 2) rows_ahead = lookup_rows(c0 + 2 * kTile);
+    } else {
         const int64_t r0 = row_ref(p, b, start, c0).k;
         issue_tile(c0, r0, second_run(c0, r0), 0);
-    }
-    if (ntiles > 1) {
-        const int64_t r0 = row_ref(p, b, start, c0 + kTile).k;
-        issue_tile(c0 + kTile, r0, second_run(c0 + kTile, r0), 1);
+        if (ntiles > 1) {
+            const int64_t r1 = row_ref(p, b, start, c0 + kTile).k;
+            issue_tile(c0 + kTile, r1, second_run(c0 + kTile, r1), 1);
+        }
     }
     if constexpr (KV8) {
         // three stages in flight; the first tile is converted here, tile t + 1 at the top of trip t
@@ -369,8 +422,8 @@ __global__ __launch_bounds__(64 * NWV) void mfma_latent_kernel(const SweepParams
     }
     // page of the tile after those, fetched one trip ahead of its use (a scalar load for paged K/V)
     constexpr int AHEAD = KV8 ? 3 : 2;  // tiles in flight behind the one being read
-    int page_ahead = ntiles > AHEAD ? page_of(p, b, c0 + AHEAD * kTile) : 0;
-    int page_ahead1 = ntiles > AHEAD && c0 + AHEAD * kTile + 16 < c1 ? page_of(p, b, c0 + AHEAD * kTile + 16) : 0;
+    int page_ahead = !PG && ntiles > AHEAD ? page_of(p, b, c0 + AHEAD * kTile) : 0;
+    int page_ahead1 = !PG && ntiles > AHEAD && c0 + AHEAD * kTile + 16 < c1 ? page_of(p, b, c0 + AHEAD * kTile + 16) : 0;
     // Make the compiler settle its own wait for the Q loads here, before the loop.  It cannot see the
     // direct-to-LDS loads, so a wait for Q placed inside the loop would count down to vmcnt(0) on every trip
     // and drain the tiles in flight.
@@ -421,6 +474,10 @@ __global__ __launch_bounds__(64 * NWV) void mfma_latent_kernel(const SweepParams
         else
             wait_vmcnt<0>();
         __syncthreads();  // every wave's share of tile t is in LDS, and every wave is done with tile t-1
+        if constexpr (PG) {
+            if (t + 2 < ntiles) issue_tile_pg(c0 + (t + 2) * kTile, rows_ahead, buf_next);
+            if (t + 3 < ntiles) rows_ahead = lookup_rows(c0 + (t + 3) * kTile);
+        } else {
         if (t + 2 < ntiles) {
             const int tk = c0 + (t + 2) * kTile;
             const int64_t r0 = row_in_page(p, start, tk, page_ahead).k;
@@ -430,6 +487,7 @@ __global__ __launch_bounds__(64 * NWV) void mfma_latent_kernel(const SweepParams
             const int tk = c0 + (t + 3) * kTile;
             page_ahead = page_of(p, b, tk);
             if (tk + 16 < c1) page_ahead1 = page_of(p, b, tk + 16);
+        }
         }
         }
 
@@ -595,11 +653,11 @@ constexpr size_t lds_bytes() {
     return tiles > qstage ? tiles : qstage;
 }
 
-template <typename Tag, int D, int DV, int NWV, bool KV8>
-hipError_t launch_one(const SweepParams& p, dim3 grid, hipStream_t stream) {
+template <typename Tag, int D, int DV, int NWV, bool KV8, bool PG>
+hipError_t launch_form(const SweepParams& p, dim3 grid, hipStream_t stream) {
     static std::once_flag once;
     static hipError_t attr_err = hipSuccess;
-    auto kern = mfma_latent_kernel<Tag, D, DV, NWV, KV8>;
+    auto kern = mfma_latent_kernel<Tag, D, DV, NWV, KV8, PG>;
     std::call_once(once, [&] {
         attr_err = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
                                        (int)lds_bytes<D, NWV, KV8>());
@@ -608,6 +666,13 @@ hipError_t launch_one(const SweepParams& p, dim3 grid, hipStream_t stream) {
     constexpr size_t lds = lds_bytes<D, NWV, KV8>();
     hipLaunchKernelGGL(kern, grid, dim3(64 * NWV), lds, stream, p);
     return hipGetLastError();
+}
+
+template <typename Tag, int D, int DV, int NWV, bool KV8>
+hipError_t launch_one(const SweepParams& p, dim3 grid, hipStream_t stream) {
+    if constexpr (!KV8)
+        if (p.block_table != nullptr && p.page_shift < 4) return launch_form<Tag, D, DV, NWV, false, true>(p, grid, stream);
+    return launch_form<Tag, D, DV, NWV, KV8, false>(p, grid, stream);
 }
 
 template <typename Tag, bool KV8>

@@ -67,6 +67,17 @@ def test_with_the_token_count_hint(name):
     check_against_oracle(w, paged)
 
 
+@pytest.mark.parametrize("page_size", [1, 2, 4, 8])
+@pytest.mark.parametrize("name", ["mla", "mla_h16"])
+def test_latent_kernel_takes_small_pages_with_a_lookup_per_row(name, page_size):
+    """Pages under 16 tokens (token-level paging included): the latent kernel's per-row lookup form; same arithmetic
+    as the packed call, same bits."""
+    w = _workload(name)
+    dense, paged = _run_both(w, page_size)
+    assert torch.isfinite(paged.float()).all()
+    assert torch.equal(dense.view(torch.int16), paged.view(torch.int16))
+
+
 @pytest.mark.parametrize("name", ["mla", "mla_h16"])
 def test_latent_kernel_takes_16_token_pages(name):
     """The latent kernel fetches a tile as two runs of 16 tokens, so 16-token pages (a common cache block size) stay
