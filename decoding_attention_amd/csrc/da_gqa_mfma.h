@@ -88,8 +88,10 @@ constexpr size_t gqa_lds_bytes(int nt) {
 // One segment of work: tokens [c0, c1) of sequence b (first row `start`, `len` tokens) for the KV heads and head
 // group blockIdx.y selects.  `direct`: the segment is the whole sequence, so the result goes to o; otherwise the
 // un-normalised partial goes to workspace slot `split` of the sequence.
-// HP (16-token pages of paged K/V): a tile is fetched as two runs of 16 tokens, each from one page.
-template <typename Tag, int D, int DV, int NT, bool PREFETCH, bool WH, bool KV8, bool HP>
+// PGM: how paged K/V is addressed.  0: one page lookup per tile (pages hold a multiple of 32 tokens; also the packed
+// layout); 1: 16-token pages, a tile is fetched as two runs of 16 tokens, each from one page; 2: smaller pages, every
+// lane looks up the page of the row it loads.
+template <typename Tag, int D, int DV, int NT, bool PREFETCH, bool WH, bool KV8, int PGM>
 __device__ __forceinline__ void gqa_segment(const SweepParams& p, uint8_t* const smem, const int b, const int start,
                                             const int len, const int c0, const int c1, const int split,
                                             const bool direct) {
@@ -187,8 +189,24 @@ __device__ __forceinline__ void gqa_segment(const SweepParams& p, uint8_t* const
     // masked.  The choice between the two runs is wave-uniform: an M-tile of K is one run, and a V load instruction
     // covers a power-of-two number of rows inside one run, except for d = 96 (12 chunks per row), which chooses
     // per lane.
+    constexpr bool HP = PGM == 1;
+    // per-lane address of row `row` of the tile at tok0 (PGM == 2): its page from the block table, then the row in it
+    auto lane_row = [&](int tok0, int row, const uint8_t* bytes, int64_t page_stride, uint32_t row_bytes) {
+        const int tok = tok0 + row;
+        const int page = p.block_table[(int64_t)b * p.max_blocks + (tok >> p.page_shift)];
+        return bytes + ((int64_t)page * page_stride * KB + (int64_t)(tok & ((1 << p.page_shift) - 1)) * row_bytes);
+    };
     auto load_k = [&](int tok0, TileRegs& r) __attribute__((always_inline)) {
         const int last = c1 - 1 - tok0;
+        if constexpr (PGM == 2) {
+#pragma unroll
+            for (int mt = 0; mt < 2; ++mt) {
+                const uint8_t* const row = lane_row(tok0, min(mt * 16 + n, last), kbytes, p.k_page, k_row_b) + g * 16;
+#pragma unroll
+                for (int ks = 0; ks < KSR; ++ks) r.k[mt][ks] = *reinterpret_cast<const uint4*>(row + ks * 64);
+            }
+            return;
+        }
         const uint8_t* const base0 = kbytes + row_ref(p, b, start, tok0).k * KB;
         const uint8_t* base1 = base0;
         if constexpr (HP)
@@ -204,6 +222,15 @@ __device__ __forceinline__ void gqa_segment(const SweepParams& p, uint8_t* const
     };
     auto load_v = [&](int tok0, TileRegs& r) __attribute__((always_inline)) {
         const int last = c1 - 1 - tok0;
+        if constexpr (PGM == 2) {
+#pragma unroll
+            for (int i = 0; i < NVR; ++i) {
+                const int slot = i * 64 + lane;
+                const int row = slot / CPRL, ch = slot % CPRL;
+                r.v[i] = *reinterpret_cast<const uint4*>(lane_row(tok0, min(row, last), vbytes, p.v_page, v_row_b) + ch * 16);
+            }
+            return;
+        }
         const uint8_t* const base0 = vbytes + row_ref(p, b, start, tok0).v * KB;
         const uint8_t* base1 = base0;
         if constexpr (HP)
@@ -448,7 +475,7 @@ __device__ __forceinline__ void gqa_segment(const SweepParams& p, uint8_t* const
 // does not give.  Sequence b spans work-groups first(b) = cu[b] / T ... last(b) = (cu[b+1] - 1) / T (both capped
 // at W - 1); its segment in work-group i is partial number i - first(b), and goes straight to o when
 // first(b) == last(b).
-template <typename Tag, int D, int DV, int NT, bool PREFETCH, bool WH, int MINW, bool KV8 = false, bool HP = false>
+template <typename Tag, int D, int DV, int NT, bool PREFETCH, bool WH, int MINW, bool KV8 = false, int PGM = 0>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(MINW))) void gqa_mfma_kernel(const SweepParams p) {
     extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
     if (p.flat_tokens == 0) {
@@ -457,7 +484,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(MINW))) voi
         seq_range(p, b, start, len);
         const int c0 = split * p.chunk;
         const int c1 = (split == p.nsplit - 1) ? len : min(len, c0 + p.chunk);
-        gqa_segment<Tag, D, DV, NT, PREFETCH, WH, KV8, HP>(p, smem, b, start, len, c0, c1, split, p.nsplit == 1);
+        gqa_segment<Tag, D, DV, NT, PREFETCH, WH, KV8, PGM>(p, smem, b, start, len, c0, c1, split, p.nsplit == 1);
         return;
     }
     const int T = p.flat_tokens, W = (int)gridDim.x, i = (int)blockIdx.x, unit = p.flat_unit;
@@ -486,7 +513,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(MINW))) voi
         seq_range(p, b, start, len);
         const int first = min(s / T, W - 1), last = min((e - 1) / T, W - 1);
         const int c0 = (max(r0, s) - s) * unit, c1 = min((min(r1, e) - s) * unit, len);
-        gqa_segment<Tag, D, DV, NT, PREFETCH, WH, KV8, HP>(p, smem, b, start, len, c0, c1, i - first, first == last);
+        gqa_segment<Tag, D, DV, NT, PREFETCH, WH, KV8, PGM>(p, smem, b, start, len, c0, c1, i - first, first == last);
         if (!WH) __syncthreads();  // the merge area of this segment is the V tile area of the next
     }
 }

@@ -9,11 +9,11 @@ namespace da {
 
 namespace gqa_launch {
 
-template <typename Tag, int D, int NT, bool WH, bool KV8, bool HP>
+template <typename Tag, int D, int NT, bool WH, bool KV8, int PGM>
 hipError_t launch_form(const SweepParams& p, dim3 grid, hipStream_t stream) {
     constexpr bool kPrefetch = D <= 128;
     constexpr int kMinWaves = (D <= 128 && (NT == 1 || D <= 64)) ? 2 : 1;
-    auto kern = gqa_mfma_kernel<Tag, D, D, NT, kPrefetch, WH, kMinWaves, KV8, HP>;
+    auto kern = gqa_mfma_kernel<Tag, D, D, NT, kPrefetch, WH, kMinWaves, KV8, PGM>;
     const size_t lds = gqa_lds_bytes<D>(NT);
     static std::once_flag once;
     static hipError_t attr_err = hipSuccess;
@@ -27,12 +27,13 @@ hipError_t launch_form(const SweepParams& p, dim3 grid, hipStream_t stream) {
     return hipGetLastError();
 }
 
-// 16-token pages of paged K/V take the form that fetches a tile as two runs (its own instantiation: the second
-// set of base addresses costs registers the other layouts should not pay for)
+// 16-token pages of paged K/V take the form that fetches a tile as two runs, smaller pages the form with a lookup
+// per row (instantiations of their own: the extra addresses cost registers the other layouts should not pay for)
 template <typename Tag, int D, int NT, bool WH, bool KV8>
 hipError_t launch_one(const SweepParams& p, dim3 grid, hipStream_t stream) {
-    return p.block_table != nullptr && p.page_shift == 4 ? launch_form<Tag, D, NT, WH, KV8, true>(p, grid, stream)
-                                                         : launch_form<Tag, D, NT, WH, KV8, false>(p, grid, stream);
+    if (p.block_table != nullptr && p.page_shift < 4) return launch_form<Tag, D, NT, WH, KV8, 2>(p, grid, stream);
+    if (p.block_table != nullptr && p.page_shift == 4) return launch_form<Tag, D, NT, WH, KV8, 1>(p, grid, stream);
+    return launch_form<Tag, D, NT, WH, KV8, 0>(p, grid, stream);
 }
 
 template <typename Tag, int D, bool KV8>

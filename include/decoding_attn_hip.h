@@ -83,8 +83,9 @@ size_t da_workspace_bytes(size_t max_seq_k, size_t batch, size_t head_q, size_t 
  *   block_table    device, int32 [batch, max_blocks_per_seq]: page ids of each sequence in token order; entries
  *                  past ceil(seq_lens[b] / page_size) are not read
  *   seq_lens       device, int32 [batch]: key tokens of each sequence (0 gives zero output rows)
- *   page_size      tokens per page, a power of two.  Multiples of 16 run on the same kernels as the packed layout;
- *                  smaller pages are served by the VALU sweep with one table lookup per row.
+ *   page_size      tokens per page, a power of two (1 included).  All sizes run on the same kernels as the packed
+ *                  layout: whole tiles from pages of 32 tokens and more, two runs per tile from 16-token pages,
+ *                  a table lookup per row below that.
  * The remaining arguments are those of da_decoding_attn_ex; workspace size from da_workspace_bytes_paged.
  */
 int da_decoding_attn_paged(const void *q, const void *k_pages, const void *v_pages, void *o,
@@ -109,7 +110,7 @@ size_t da_workspace_bytes_paged(size_t max_seq_k, size_t batch, size_t head_q, s
  *                      both in fp32.
  * v8 == NULL means V is the first dim_v columns of each K row.  Head dims (64,64), (128,128), (256,256) run on
  * the grouped MFMA kernel and (576,512) with v8 == NULL on the latent MFMA kernel, as the 16-bit forms do; (96,96)
- * and pages under 16 tokens run on the VALU sweep.  Workspace size from da_workspace_bytes_fp8kv (page_size 0 =
+ * and (576,512) with pages under 16 tokens run on the VALU sweep.  Workspace size from da_workspace_bytes_fp8kv (page_size 0 =
  * packed layout).
  */
 int da_decoding_attn_fp8kv(const void *q, const void *k8, const void *v8, void *o, const int32_t *cu_seq_k,

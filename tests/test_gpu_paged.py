@@ -1,10 +1,10 @@
 """Paged K/V entry point: the same attention with K/V scattered over page pools.
 
-With pages of a multiple of 16 tokens the paged call runs the same kernels as the packed call, and with the same
-split plan when neither is given the batch's token count (with it, the packed call of a ragged batch may cut the
-concatenated tokens into equal shares, which pages cannot follow), so its output must then equal the packed call's
-bit for bit; smaller pages run the VALU sweep and are checked
-against the CPU oracle on the gathered (packed) inputs.  Unused pool rows are NaN: reading one poisons the output.
+Whatever the page size, the paged call runs the same kernels as the packed call, and with the same split plan when
+neither is given the batch's token count (with it, a ragged batch may be cut into equal shares of the concatenated
+tokens, differently for the two layouts), so its output must then equal the packed call's bit for bit; the cases are
+also checked against the CPU oracle on the gathered (packed) inputs.  Unused pool rows are NaN: reading one poisons
+the output.
 """
 import pytest
 import torch
@@ -48,7 +48,7 @@ def _workload(name, **over):
                             name="paged_" + name, **args)
 
 
-@pytest.mark.parametrize("page_size", [16, 32, 64, 256])
+@pytest.mark.parametrize("page_size", [1, 4, 16, 32, 64, 256])
 @pytest.mark.parametrize("name", list(SHAPES))
 def test_tile_sized_pages_match_the_packed_call_bit_for_bit(name, page_size):
     w = _workload(name)
