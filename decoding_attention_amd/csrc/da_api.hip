@@ -107,17 +107,12 @@ int rows_per_trip(size_t dim) {
     }
 }
 
-// Paged K/V: the MFMA kernels fetch a tile whole (pages of a multiple of 32 tokens), as two runs of 16 tokens, or row
-// by row with a page lookup each (smaller pages); only the latent kernel's FP8 form, which stages runs of 16 rows,
-// has no row-by-row variant.
-bool pages_fit_tiles(size_t page_size, bool latent_fp8) { return page_size % 16 == 0 || !latent_fp8; }
-
 // v_distinct: V is its own buffer (the MFMA kernel reads V out of the K tile, so it needs the aliased form).
 // total_k: sum of the key lengths if the caller knows it (0 = unknown).  The planner never reads cu_seq_k (that
 // would need a device synchronisation); when total_k shows that the batch is ragged it cuts the sequences into
 // shorter splits so that the work-groups, whose number is sized for max_seq_k, balance.
-// page_size: 0 for the packed layout, else tokens per page of paged K/V (see pages_fit_tiles; what does not fit
-// runs on the VALU sweep, which resolves every row on its own).
+// page_size: 0 for the packed layout, else tokens per page of paged K/V (any power of two: the MFMA kernels fetch a
+// tile whole from pages of 32 tokens and more, as two runs from 16-token pages, row by row below that).
 // kv_fp8: K/V are FP8; the grouped kernel then needs dim % 64 == 0.
 Plan make_plan(size_t max_seq_k, size_t batch, size_t head_q, size_t head_k, size_t dim, size_t dim_v,
                bool v_distinct, size_t total_k, size_t page_size = 0, bool kv_fp8 = false) {
@@ -127,7 +122,7 @@ Plan make_plan(size_t max_seq_k, size_t batch, size_t head_q, size_t head_k, siz
     int trip;
     int target_wgs = tun().target_wgs;
     const bool latent = !v_distinct && da::mla_supported(dim, dim_v, ratio);
-    const bool force_sweep = tun().force_kind == kKindSweep || (page_size != 0 && !pages_fit_tiles(page_size, latent && kv_fp8));
+    const bool force_sweep = tun().force_kind == kKindSweep;
     const bool mfma = latent && !force_sweep;
     if (mfma) {
         pl.kind = kKindMfma;

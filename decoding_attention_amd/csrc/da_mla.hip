@@ -156,7 +156,7 @@ __device__ __forceinline__ void wait_vmcnt() {
 // PG: paged K/V with pages of fewer than 16 tokens (down to 1): every row of a tile has its own page lookup.
 template <typename Tag, int D, int DV, int NWV, bool KV8, bool PG = false>
 __global__ __launch_bounds__(64 * NWV) void mfma_latent_kernel(const SweepParams p) {
-    static_assert(!(KV8 && PG), "the FP8 form stages runs of 16 tokens");
+    // (FP8 with PG: the stage is filled a row per load, 36 of the 64 lanes active, instead of 1 KiB per load)
     using MM = Mma<Tag>;
     using vec8 = typename MM::vec8;
     using EL = Elem<Tag>;
@@ -173,8 +173,9 @@ __global__ __launch_bounds__(64 * NWV) void mfma_latent_kernel(const SweepParams
     // FP8 K cache: stages of the tile's raw bytes, filled 1 KiB per load instruction
     constexpr int NTB = KV8 ? 2 : kNBuf;                 // 16-bit tile buffers
     constexpr int STG_REAL = kTile * D / 1024;           // load instructions that cover a staged tile (18)
-    constexpr int NLW8 = (STG_REAL + NWV - 1) / NWV;     // per wave (the surplus ones repeat the last KiB)
-    constexpr int STG = NLW8 * NWV * 1024;               // bytes per stage
+    constexpr int NLW8 = PG ? kTile / NWV : (STG_REAL + NWV - 1) / NWV;  // per wave (the surplus ones repeat the last
+                                                                         // KiB); PG: a row per load
+    constexpr int STG = ((STG_REAL + NWV - 1) / NWV) * NWV * 1024;  // bytes per stage
     constexpr int STG0 = NTB * BUF;                      // stages start behind the 16-bit buffers
     static_assert((kTile * D) % 1024 == 0, "staged tile");
     static_assert(D % 16 == 0 && DV % 32 == 0 && DV <= D, "shape");
@@ -341,6 +342,15 @@ __global__ __launch_bounds__(64 * NWV) void mfma_latent_kernel(const SweepParams
             const int tok = tok0 + min(wave * NLA + q, last);
             rowoff[q] = ((int64_t)rp.pg[q] * p.k_page + (int64_t)(tok & mask) * p.k_row) * KB;
         }
+        if constexpr (KV8) {
+            // stage `buf`: row r of the tile at r * D bytes; one row (D bytes, D / 16 lanes) per load
+#pragma unroll
+            for (int q = 0; q < NLA; ++q) {
+                const int row = wave * NLA + q;
+                if (lane < D / 16) lds_dma16(kbytes + rowoff[q], lane16, smem_off + (uint32_t)(STG0 + buf * STG + row * D));
+            }
+            return;
+        }
 #pragma unroll
         for (int q = 0; q < NLA; ++q) {
             const int row = wave * NLA + q;
@@ -408,11 +418,16 @@ __global__ __launch_bounds__(64 * NWV) void mfma_latent_kernel(const SweepParams
     if constexpr (KV8) {
         // three stages in flight; the first tile is converted here, tile t + 1 at the top of trip t
         if (ntiles > 2) {
-            const int64_t r0 = row_ref(p, b, start, c0 + 2 * kTile).k;
-            issue_tile(c0 + 2 * kTile, r0, second_run(c0 + 2 * kTile, r0), 2);
+            if constexpr (PG) {
+                issue_tile_pg(c0 + 2 * kTile, rows_ahead, 2);
+                if (ntiles > 3) rows_ahead = lookup_rows(c0 + 3 * kTile);
+            } else {
+                const int64_t r0 = row_ref(p, b, start, c0 + 2 * kTile).k;
+                issue_tile(c0 + 2 * kTile, r0, second_run(c0 + 2 * kTile, r0), 2);
+            }
         }
         if (ntiles > 2)
-            wait_vmcnt<2 * NLW8>();
+            wait_vmcnt<(2 * NLW8 < 63 ? 2 * NLW8 : 63)>();  // (the counter has six bits; waiting for fewer is safe)
         else if (ntiles > 1)
             wait_vmcnt<NLW8>();
         else
@@ -458,6 +473,10 @@ __global__ __launch_bounds__(64 * NWV) void mfma_latent_kernel(const SweepParams
             if (t + 1 < ntiles) convert_stage(stg_conv, buf ^ 1);
             stg_conv = (stg_conv == 2) ? 0 : stg_conv + 1;
             // (the stage that held tile t was converted before the barrier: free for tile t+3)
+            if constexpr (PG) {
+                if (t + 3 < ntiles) issue_tile_pg(c0 + (t + 3) * kTile, rows_ahead, buf_next);
+                if (t + 4 < ntiles) rows_ahead = lookup_rows(c0 + (t + 4) * kTile);
+            } else {
             if (t + 3 < ntiles) {
                 const int tk = c0 + (t + 3) * kTile;
                 const int64_t r0 = row_in_page(p, start, tk, page_ahead).k;
@@ -467,6 +486,7 @@ __global__ __launch_bounds__(64 * NWV) void mfma_latent_kernel(const SweepParams
                 const int tk = c0 + (t + 4) * kTile;
                 page_ahead = page_of(p, b, tk);
                 if (tk + 16 < c1) page_ahead1 = page_of(p, b, tk + 16);
+            }
             }
         } else {
         if (t + 1 < ntiles)
@@ -670,8 +690,7 @@ hipError_t launch_form(const SweepParams& p, dim3 grid, hipStream_t stream) {
 
 template <typename Tag, int D, int DV, int NWV, bool KV8>
 hipError_t launch_one(const SweepParams& p, dim3 grid, hipStream_t stream) {
-    if constexpr (!KV8)
-        if (p.block_table != nullptr && p.page_shift < 4) return launch_form<Tag, D, DV, NWV, false, true>(p, grid, stream);
+    if (p.block_table != nullptr && p.page_shift < 4) return launch_form<Tag, D, DV, NWV, KV8, true>(p, grid, stream);
     return launch_form<Tag, D, DV, NWV, KV8, false>(p, grid, stream);
 }
 

@@ -127,7 +127,7 @@ def test_latent_fp8_unit_scales_equal_the_16_bit_call_bit_for_bit():
     assert torch.equal(o8.view(torch.int16), o16.view(torch.int16))
 
 
-@pytest.mark.parametrize("page_size", [16, 32, 64])
+@pytest.mark.parametrize("page_size", [1, 4, 16, 32, 64])
 def test_latent_paged_fp8(page_size):
     w, k8, _, ks, _ = _case(5, 128, 1, 576, 512, 1100, torch.float16, latent=True, seed=21)
     w8 = wl.Workload(w.name, w.q, k8.view(torch.uint8), None, w.cu_seq_k, w.max_seq_k, w.dim_v, w.is_alibi, w.lengths)
@@ -138,7 +138,7 @@ def test_latent_paged_fp8(page_size):
     assert (o.float() - ref).abs().max().item() <= TOL[torch.float16]
 
 
-@pytest.mark.parametrize("page_size", [16, 64])
+@pytest.mark.parametrize("page_size", [1, 8, 16, 64])
 def test_paged_fp8_kv(page_size):
     w, k8, v8, ks, vs = _case(6, 32, 8, 128, 128, 1100, torch.bfloat16)
     w8 = wl.Workload(w.name, w.q, k8.view(torch.uint8), v8.view(torch.uint8), w.cu_seq_k, w.max_seq_k, w.dim_v,
