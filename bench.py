@@ -91,7 +91,7 @@ def measure(torch, w, steps, warmup, page_size=0, kv_fp8=False):
         if kv_fp8:  # K/V as FP8 (e4m3) with per-head scales; q and o stay 16-bit
             ks = torch.full((w.head_k,), 0.02, device=dev)
             k8 = (c.k.float() / 0.02).to(torch.float8_e4m3fn)
-            v8 = (c.v.float() / 0.02).to(torch.float8_e4m3fn)
+            v8 = None if c.v is None else (c.v.float() / 0.02).to(torch.float8_e4m3fn)  # (latent form: V is in K)
 
             def call_fp8():
                 outs[:] = [decoding_attn_fwd(c.q, k8, v8, c.cu_seq_k, c.max_seq_k, c.dim_v, c.is_alibi, k_scale=ks,
@@ -332,16 +332,16 @@ def run_sweep(args):
     if args.sweep in ("gqa", "all"):
         shapes += [("gqa-varlen", wl.config_gqa_varlen()), ("gqa-fixed", wl.config_gqa_fixed()),
                    ("mqa-alibi", wl.config_mqa_alibi())]
-    if args.sweep == "paged":  # the two benchmark shapes over shuffled 64-token pages, beside the packed layout
-        for w in (wl.config_gqa_fixed(), wl.config_mla(64, 4096)):
-            shapes += [("packed", w), ("paged-64", w)]
-    if args.sweep == "fp8":  # 16-bit against FP8 K/V on the bandwidth-bound shapes
+    if args.sweep == "paged":  # the benchmark shapes over shuffled pages of 64, 16 and 1 tokens, beside the packed layout
+        for w in (wl.config_gqa_fixed(), wl.config_gqa_varlen(), wl.config_mqa_alibi(), wl.config_mla(64, 4096)):
+            shapes += [("packed", w), ("paged-64", w), ("paged-16", w), ("paged-1", w)]
+    if args.sweep == "fp8":  # 16-bit against FP8 K/V on the bandwidth-bound shapes and the latent form
         for w in (wl.config_gqa_fixed(), wl.config_mha_sweep(512, 128), wl.config_mha_sweep(1, 8192),
-                  wl.config_mqa_alibi()):
+                  wl.config_mqa_alibi(), wl.config_mla(64, 4096), wl.config_mla(16, 4096)):
             shapes += [("kv16", w), ("kv-fp8", w)]
     results = []
     for tag, w in shapes:
-        r = measure(torch, w, args.steps, args.warmup, page_size=64 if tag == "paged-64" else 0,
+        r = measure(torch, w, args.steps, args.warmup, page_size=int(tag[6:]) if tag.startswith("paged-") else 0,
                     kv_fp8=tag == "kv-fp8")
         ms = r["us_per_call"] / 1e3
         sk = w.max_seq_k
