@@ -79,7 +79,7 @@ def _device_copies(torch, w, dev, min_total_bytes=768 << 20):
     return copies
 
 
-def measure(torch, w, steps, warmup, page_size=0, kv_fp8=False):
+def measure(torch, w, steps, warmup, page_size=0, kv_fp8=False, kv_int8=False):
     from decoding_attention_amd import _lib, decoding_attn_fwd
     from decoding_attention_amd import workloads as wl
 
@@ -88,10 +88,16 @@ def measure(torch, w, steps, warmup, page_size=0, kv_fp8=False):
     outs = []
 
     def make(c):
-        if kv_fp8:  # K/V as FP8 (e4m3) with per-head scales; q and o stay 16-bit
-            ks = torch.full((w.head_k,), 0.02, device=dev)
-            k8 = (c.k.float() / 0.02).to(torch.float8_e4m3fn)
-            v8 = None if c.v is None else (c.v.float() / 0.02).to(torch.float8_e4m3fn)  # (latent form: V is in K)
+        if kv_fp8 or kv_int8:  # K/V as FP8 (e4m3) or int8 with per-head scales; q and o stay 16-bit
+            def quantise(x, step):
+                if kv_int8:
+                    return torch.round(x.float() / step).clamp(-128, 127).to(torch.int8)
+                return (x.float() / step).to(torch.float8_e4m3fn)
+
+            step = 4.0 / 127 if kv_int8 else 0.02
+            ks = torch.full((w.head_k,), step, device=dev)
+            k8 = quantise(c.k, step)
+            v8 = None if c.v is None else quantise(c.v, step)  # (latent form: V is in K)
 
             def call_fp8():
                 outs[:] = [decoding_attn_fwd(c.q, k8, v8, c.cu_seq_k, c.max_seq_k, c.dim_v, c.is_alibi, k_scale=ks,
@@ -116,7 +122,7 @@ def measure(torch, w, steps, warmup, page_size=0, kv_fp8=False):
     mean_ms, min_ms = _time_calls(torch, fns, steps, warmup)
     assert torch.isfinite(outs[0].float()).all()
     nbytes = wl.workload_bytes(w)
-    if kv_fp8:  # one byte per K/V element
+    if kv_fp8 or kv_int8:  # one byte per K/V element
         nbytes = wl.algorithmic_bytes(w.batch, w.head_q, w.head_k, w.dim, w.dim_v, int(w.k.shape[0]), w.v is not None,
                                       elem_bytes=2) - int(w.k.numel() + (w.v.numel() if w.v is not None else 0))
     flops = wl.workload_flops(w)
@@ -335,14 +341,14 @@ def run_sweep(args):
     if args.sweep == "paged":  # the benchmark shapes over shuffled pages of 64, 16 and 1 tokens, beside the packed layout
         for w in (wl.config_gqa_fixed(), wl.config_gqa_varlen(), wl.config_mqa_alibi(), wl.config_mla(64, 4096)):
             shapes += [("packed", w), ("paged-64", w), ("paged-16", w), ("paged-1", w)]
-    if args.sweep == "fp8":  # 16-bit against FP8 K/V on the bandwidth-bound shapes and the latent form
+    if args.sweep == "fp8":  # 16-bit against FP8 and int8 K/V on the bandwidth-bound shapes and the latent form
         for w in (wl.config_gqa_fixed(), wl.config_mha_sweep(512, 128), wl.config_mha_sweep(1, 8192),
                   wl.config_mqa_alibi(), wl.config_mla(64, 4096), wl.config_mla(16, 4096)):
-            shapes += [("kv16", w), ("kv-fp8", w)]
+            shapes += [("kv16", w), ("kv-fp8", w), ("kv-int8", w)]
     results = []
     for tag, w in shapes:
         r = measure(torch, w, args.steps, args.warmup, page_size=int(tag[6:]) if tag.startswith("paged-") else 0,
-                    kv_fp8=tag == "kv-fp8")
+                    kv_fp8=tag == "kv-fp8", kv_int8=tag == "kv-int8")
         ms = r["us_per_call"] / 1e3
         sk = w.max_seq_k
         ref_bytes = wl.reference_formula_bytes(w.batch, w.head_q, w.head_k, w.dim, w.dim_v, sk)
@@ -373,7 +379,7 @@ def main():
                     "traffic figure for scaling profiler byte counters)")
     ap.add_argument("--cpu-budget", type=float, default=15.0, help="seconds of single-thread CPU work to sample")
     ap.add_argument("--sweep", choices=["mha", "mla", "gqa", "all", "paged", "fp8"], help="print the reference's sweeps instead "
-                    "(paged / fp8: benchmark shapes over a paged or an FP8 K/V cache)")
+                    "(paged / fp8: benchmark shapes over a paged or an 8-bit, FP8 and int8, K/V cache)")
     ap.add_argument("--json-out", help="with --sweep: also write the results as JSON")
     args = ap.parse_args()
     if args.gpus != 1:

@@ -19,6 +19,9 @@ EXPORTED_SYMBOLS = (
     "da_decoding_attn_fp8kv",
     "da_decoding_attn_paged_fp8kv",
     "da_workspace_bytes_fp8kv",
+    "da_decoding_attn_int8kv",
+    "da_decoding_attn_paged_int8kv",
+    "da_workspace_bytes_int8kv",
     "da_plan",
     "da_probe_stream_read",
     "da_probe_sweep_only",
@@ -71,6 +74,13 @@ def load():
                                                  cf, vp, vp, vp, sz, vp, sz, vp]
     lib.da_workspace_bytes_fp8kv.restype = sz
     lib.da_workspace_bytes_fp8kv.argtypes = [sz, sz, sz, sz, sz, sz, sz, sz]
+    # the int8 entry points take the FP8 ones' arguments
+    lib.da_decoding_attn_int8kv.restype = ci
+    lib.da_decoding_attn_int8kv.argtypes = lib.da_decoding_attn_fp8kv.argtypes
+    lib.da_decoding_attn_paged_int8kv.restype = ci
+    lib.da_decoding_attn_paged_int8kv.argtypes = lib.da_decoding_attn_paged_fp8kv.argtypes
+    lib.da_workspace_bytes_int8kv.restype = sz
+    lib.da_workspace_bytes_int8kv.argtypes = lib.da_workspace_bytes_fp8kv.argtypes
     lib.da_probe_stream_read.restype = ci
     lib.da_probe_stream_read.argtypes = [vp, sz, vp, vp]
     lib.da_probe_sweep_only.restype = ci

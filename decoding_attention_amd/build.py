@@ -23,6 +23,7 @@ SOURCES = [
     "da_gqa_mfma.hip",
     "da_sweep_kv8.hip",
     "da_gqa_mfma_kv8.hip",
+    "da_gqa_mfma_i8.hip",
     "da_probe.hip",
 ]
 

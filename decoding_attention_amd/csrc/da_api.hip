@@ -113,9 +113,9 @@ int rows_per_trip(size_t dim) {
 // shorter splits so that the work-groups, whose number is sized for max_seq_k, balance.
 // page_size: 0 for the packed layout, else tokens per page of paged K/V (any power of two: the MFMA kernels fetch a
 // tile whole from pages of 32 tokens and more, as two runs from 16-token pages, row by row below that).
-// kv_fp8: K/V are FP8; the grouped kernel then needs dim % 64 == 0.
+// kv_8bit: K/V are FP8 or int8; the grouped kernel then needs dim % 64 == 0.
 Plan make_plan(size_t max_seq_k, size_t batch, size_t head_q, size_t head_k, size_t dim, size_t dim_v,
-               bool v_distinct, size_t total_k, size_t page_size = 0, bool kv_fp8 = false) {
+               bool v_distinct, size_t total_k, size_t page_size = 0, bool kv_8bit = false) {
     const bool packed = page_size == 0;
     Plan pl;
     const int ratio = (int)(head_q / head_k);
@@ -135,7 +135,7 @@ Plan make_plan(size_t max_seq_k, size_t batch, size_t head_q, size_t head_k, siz
             pl.rt = std::min(tun().mla_heads, da::mla_heads_per_group(ratio));
         trip = da::mla_rows_per_trip();
         target_wgs = tun().mfma_target_wgs;  // one 4-wave work-group fills a CU
-    } else if (dim <= 256 && !force_sweep && (!kv_fp8 || dim % 64 == 0) &&
+    } else if (dim <= 256 && !force_sweep && (!kv_8bit || dim % 64 == 0) &&
                (ratio >= tun().group_min_ratio ||
                 (tun().group_min_ratio > 1 && (max_seq_k >= 1024 || dim <= 96) &&
                  (long long)batch * (long long)head_k * (long long)max_seq_k >= (1ll << 21)))) {
@@ -162,7 +162,7 @@ Plan make_plan(size_t max_seq_k, size_t batch, size_t head_q, size_t head_k, siz
     // Ragged batch of known total length on the grouped kernel: equal shares of the concatenated tokens instead of
     // fixed splits of every sequence.  Paged K/V pays one more (tiny) kernel for the sequences' positions, so it
     // takes this form only when the sweep is long enough to win that back.
-    const double kv_bytes = (double)total_k * (double)head_k * (double)(dim + dim_v) * (kv_fp8 ? 1.0 : 2.0);
+    const double kv_bytes = (double)total_k * (double)head_k * (double)(dim + dim_v) * (kv_8bit ? 1.0 : 2.0);
     if (pl.kind == kKindGroup && ragged && tun().flat_wgs > 0 && total_k < ((size_t)1 << 30) && total_k >= 64 * batch &&
         (packed || kv_bytes >= (double)tun().flat_paged_min_mb * 1e6)) {
         const long long ygrid = base / (long long)batch;
@@ -302,6 +302,11 @@ size_t da_workspace_bytes_fp8kv(size_t max_seq_k, size_t batch, size_t head_q, s
     return a > b ? a : b;
 }
 
+size_t da_workspace_bytes_int8kv(size_t max_seq_k, size_t batch, size_t head_q, size_t head_k, size_t dim,
+                                 size_t dim_v, size_t total_k, size_t page_size) {
+    return da_workspace_bytes_fp8kv(max_seq_k, batch, head_q, head_k, dim, dim_v, total_k, page_size);  // same plans
+}
+
 }  // extern "C"
 
 namespace {
@@ -313,13 +318,22 @@ struct Paging {
     size_t page_size = 0, max_blocks = 0, k_page = 0, v_page = 0;
 };
 
-// Element format of K/V: 16-bit like Q, or FP8 (e4m3) with per-KV-head de-quantisation factors (null = 1).
+// Element format of K/V: 16-bit like Q (fmt 0), or 8-bit (da::kKvFp8, da::kKvInt8) with per-KV-head de-quantisation
+// factors (null = 1).
 struct KvFormat {
     bool sweep_only = false;  // measurement: leave the split partials in the workspace, do not merge them
-    bool fp8 = false;
+    int fmt = 0;
     const float* k_scale = nullptr;
     const float* v_scale = nullptr;
 };
+
+KvFormat kv8_format(int fmt, const float* k_scale, const float* v_scale) {
+    KvFormat kf;
+    kf.fmt = fmt;
+    kf.k_scale = k_scale;
+    kf.v_scale = v_scale;
+    return kf;
+}
 
 int run_attention(const void* q, const void* k, const void* v, void* o, const int32_t* cu_seq_k, const Paging& pg,
                   const KvFormat& kf, size_t max_seq_k, size_t batch, size_t head_q, size_t head_k, size_t dim, size_t dim_v,
@@ -350,7 +364,7 @@ int run_attention(const void* q, const void* k, const void* v, void* o, const in
 
     hipStream_t stream = reinterpret_cast<hipStream_t>(hip_stream);
     const Plan pl = make_plan(max_seq_k, batch, head_q, head_k, dim, dim_v, v != nullptr, total_k,
-                              pg.table ? pg.page_size : 0, kf.fp8);
+                              pg.table ? pg.page_size : 0, kf.fmt != 0);
     if ((size_t)head_k * pl.groups > 65535)
         return fail(DA_ERR_INVALID_ARGUMENT, "head_k * groups exceeds the grid limit 65535");
 
@@ -415,13 +429,15 @@ int run_attention(const void* q, const void* k, const void* v, void* o, const in
                     (unsigned)((pl.wave_per_head ? head_k / 4 : head_k) * pl.groups),
                     (unsigned)(pl.flat_tokens ? 1 : batch));
     hipError_t e;
-    if (kf.fp8) {
+    if (kf.fmt != 0) {
         if (pl.kind == kKindMfma)
-            e = da::launch_mla_kv8(sp, is_bf16 != 0, pl.rt, grid, stream);
+            e = da::launch_mla_kv8(sp, kf.fmt, is_bf16 != 0, pl.rt, grid, stream);
+        else if (pl.kind == kKindGroup && kf.fmt == da::kKvInt8)
+            e = da::launch_gqa_mfma_i8(sp, is_bf16 != 0, (int)dim, pl.rt, pl.wave_per_head, grid, stream);
         else if (pl.kind == kKindGroup)
             e = da::launch_gqa_mfma_kv8(sp, is_bf16 != 0, (int)dim, pl.rt, pl.wave_per_head, grid, stream);
         else
-            e = da::launch_sweep_kv8(sp, is_bf16 != 0, (int)dim, pl.rt, grid, stream);
+            e = da::launch_sweep_kv8(sp, kf.fmt, is_bf16 != 0, (int)dim, pl.rt, grid, stream);
     } else if (pl.kind == kKindMfma) {
         e = da::launch_mla(sp, is_bf16 != 0, pl.rt, grid, stream);
     } else if (pl.kind == kKindGroup) {
@@ -528,12 +544,19 @@ int da_decoding_attn_fp8kv(const void* q, const void* k8, const void* v8, void* 
                            int is_alibi, int is_bf16, float softmax_scale, const float* alibi_slopes,
                            const float* k_scale, const float* v_scale, size_t total_k, void* workspace,
                            size_t workspace_bytes, void* hip_stream) {
-    KvFormat kf;
-    kf.fp8 = true;
-    kf.k_scale = k_scale;
-    kf.v_scale = v_scale;
-    return run_attention(q, k8, v8, o, cu_seq_k, Paging{}, kf, max_seq_k, batch, head_q, head_k, dim, dim_v, is_alibi,
-                         is_bf16, softmax_scale, alibi_slopes, total_k, workspace, workspace_bytes, hip_stream);
+    return run_attention(q, k8, v8, o, cu_seq_k, Paging{}, kv8_format(da::kKvFp8, k_scale, v_scale), max_seq_k, batch,
+                         head_q, head_k, dim, dim_v, is_alibi, is_bf16, softmax_scale, alibi_slopes, total_k,
+                         workspace, workspace_bytes, hip_stream);
+}
+
+int da_decoding_attn_int8kv(const void* q, const void* k8, const void* v8, void* o, const int32_t* cu_seq_k,
+                            size_t max_seq_k, size_t batch, size_t head_q, size_t head_k, size_t dim, size_t dim_v,
+                            int is_alibi, int is_bf16, float softmax_scale, const float* alibi_slopes,
+                            const float* k_scale, const float* v_scale, size_t total_k, void* workspace,
+                            size_t workspace_bytes, void* hip_stream) {
+    return run_attention(q, k8, v8, o, cu_seq_k, Paging{}, kv8_format(da::kKvInt8, k_scale, v_scale), max_seq_k, batch,
+                         head_q, head_k, dim, dim_v, is_alibi, is_bf16, softmax_scale, alibi_slopes, total_k,
+                         workspace, workspace_bytes, hip_stream);
 }
 
 int da_decoding_attn_paged_fp8kv(const void* q, const void* k_pages, const void* v_pages, void* o,
@@ -547,13 +570,25 @@ int da_decoding_attn_paged_fp8kv(const void* q, const void* k_pages, const void*
     const int rc = check_paging(block_table, seq_lens, max_seq_k, head_k, dim, dim_v, page_size, max_blocks_per_seq,
                                 k_page_stride, v_page_stride, v_pages != nullptr, &pg);
     if (rc != DA_OK) return rc;
-    KvFormat kf;
-    kf.fp8 = true;
-    kf.k_scale = k_scale;
-    kf.v_scale = v_scale;
-    return run_attention(q, k_pages, v_pages, o, nullptr, pg, kf, max_seq_k, batch, head_q, head_k, dim, dim_v,
-                         is_alibi, is_bf16, softmax_scale, alibi_slopes, total_k, workspace, workspace_bytes,
-                         hip_stream);
+    return run_attention(q, k_pages, v_pages, o, nullptr, pg, kv8_format(da::kKvFp8, k_scale, v_scale), max_seq_k,
+                         batch, head_q, head_k, dim, dim_v, is_alibi, is_bf16, softmax_scale, alibi_slopes, total_k,
+                         workspace, workspace_bytes, hip_stream);
+}
+
+int da_decoding_attn_paged_int8kv(const void* q, const void* k_pages, const void* v_pages, void* o,
+                                  const int32_t* block_table, const int32_t* seq_lens, size_t max_seq_k, size_t batch,
+                                  size_t head_q, size_t head_k, size_t dim, size_t dim_v, size_t page_size,
+                                  size_t max_blocks_per_seq, size_t k_page_stride, size_t v_page_stride, int is_alibi,
+                                  int is_bf16, float softmax_scale, const float* alibi_slopes, const float* k_scale,
+                                  const float* v_scale, size_t total_k, void* workspace, size_t workspace_bytes,
+                                  void* hip_stream) {
+    Paging pg;
+    const int rc = check_paging(block_table, seq_lens, max_seq_k, head_k, dim, dim_v, page_size, max_blocks_per_seq,
+                                k_page_stride, v_page_stride, v_pages != nullptr, &pg);
+    if (rc != DA_OK) return rc;
+    return run_attention(q, k_pages, v_pages, o, nullptr, pg, kv8_format(da::kKvInt8, k_scale, v_scale), max_seq_k,
+                         batch, head_q, head_k, dim, dim_v, is_alibi, is_bf16, softmax_scale, alibi_slopes, total_k,
+                         workspace, workspace_bytes, hip_stream);
 }
 
 int da_decoding_attn(const void* q, const void* k, const void* v, void* o, const int32_t* cu_seq_k, size_t max_seq_k,

@@ -87,6 +87,10 @@ __device__ __forceinline__ float as_second_operand(float p) {
         return p;
 }
 
+// Formats of an 8-bit K/V cache (template argument KV8 of the kernels; 0 = 16-bit K/V).
+constexpr int kKvFp8 = 1;   // OCP e4m3
+constexpr int kKvInt8 = 2;  // two's-complement integers
+
 // Eight FP8 (OCP e4m3) values -> eight 16-bit elements of the compute type.  Both conversions are exact (e4m3
 // has 3 mantissa bits and |x| <= 448), so an FP8 K/V cache feeds the same arithmetic as a 16-bit one.
 template <typename Tag>
@@ -104,6 +108,47 @@ __device__ __forceinline__ uint4 fp8x8_to_16(uint2 w) {
         r.w = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8((int)w.y, 1.0f, true));
     }
     return r;
+}
+
+// Four int8 values -> four 16-bit elements of the compute type, exactly (|x| <= 128 fits the 8 significant bits
+// of bf16).  The bytes are biased to 0..255 and planted in the mantissa of a constant whose unit in the last place
+// is one, and the constant and the bias are subtracted again: for fp16 two elements at a time (0x6400 | u is
+// 1024 + u), for bf16 through fp32 (0x4B000000 | u is 2^23 + u), whose upper half is the bf16 value.
+// v_perm_b32 picks result bytes from {first operand, second operand}: selector 0..3 = bytes of the second,
+// 4..7 = bytes of the first, 0x0c = zero.
+template <typename Tag>
+__device__ __forceinline__ uint2 int8x4_to_16(uint32_t w) {
+    const uint32_t u = w ^ 0x80808080u;
+    uint2 r;
+    if constexpr (std::is_same<Tag, f16_tag>::value) {
+        typedef _Float16 half2_t __attribute__((ext_vector_type(2)));
+        const half2_t bias = {(_Float16)-1152.0f, (_Float16)-1152.0f};
+        const uint32_t lo = __builtin_amdgcn_perm(0x64646464u, u, 0x04010400u);  // {0x64, u1, 0x64, u0}
+        const uint32_t hi = __builtin_amdgcn_perm(0x64646464u, u, 0x04030402u);  // {0x64, u3, 0x64, u2}
+        r.x = __builtin_bit_cast(uint32_t, __builtin_bit_cast(half2_t, lo) + bias);
+        r.y = __builtin_bit_cast(uint32_t, __builtin_bit_cast(half2_t, hi) + bias);
+    } else {
+        constexpr float kBias = 8388608.0f + 128.0f;
+        const float f0 = __builtin_bit_cast(float, __builtin_amdgcn_perm(0x4B000000u, u, 0x070c0c00u)) - kBias;
+        const float f1 = __builtin_bit_cast(float, __builtin_amdgcn_perm(0x4B000000u, u, 0x070c0c01u)) - kBias;
+        const float f2 = __builtin_bit_cast(float, __builtin_amdgcn_perm(0x4B000000u, u, 0x070c0c02u)) - kBias;
+        const float f3 = __builtin_bit_cast(float, __builtin_amdgcn_perm(0x4B000000u, u, 0x070c0c03u)) - kBias;
+        r.x = __builtin_amdgcn_perm(__builtin_bit_cast(uint32_t, f1), __builtin_bit_cast(uint32_t, f0), 0x07060302u);
+        r.y = __builtin_amdgcn_perm(__builtin_bit_cast(uint32_t, f3), __builtin_bit_cast(uint32_t, f2), 0x07060302u);
+    }
+    return r;
+}
+
+// Eight elements of an 8-bit K/V cache of format FMT -> eight 16-bit elements of the compute type.
+template <typename Tag, int FMT>
+__device__ __forceinline__ uint4 kv8x8_to_16(uint2 w) {
+    static_assert(FMT == kKvFp8 || FMT == kKvInt8, "8-bit K/V format");
+    if constexpr (FMT == kKvFp8) {
+        return fp8x8_to_16<Tag>(w);
+    } else {
+        const uint2 a = int8x4_to_16<Tag>(w.x), b = int8x4_to_16<Tag>(w.y);
+        return make_uint4(a.x, a.y, b.x, b.y);
+    }
 }
 
 // f(integral_constant<int, B>), ..., f(integral_constant<int, E-1>): a loop whose index is a constant

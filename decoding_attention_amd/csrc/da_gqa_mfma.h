@@ -82,7 +82,7 @@ constexpr size_t gqa_lds_bytes(int nt) {
 // Otherwise (head_k not a multiple of 4) the wavefronts split the tokens of one KV head and merge at the end.
 // MINW: wavefronts per SIMD the register allocation must leave room for (2 caps the kernel at 256 registers
 // and keeps the accumulators in ordinary VGPRs, so the rescale needs no accumulation-register copies).
-// KV8: K and V hold FP8 (e4m3) elements.  Loads stay 16 bytes per lane (sixteen elements: the k indices of two
+// KV8: K and V hold 8-bit elements (1 = FP8 e4m3, 2 = int8; 0 = 16-bit K/V).  Loads stay 16 bytes per lane (sixteen elements: the k indices of two
 // consecutive k-steps, so the Q fragments are gathered with the matching index order) and the elements are
 // converted exactly to the compute type on their way into the matrix instruction (K) or the LDS tile (V).
 // One segment of work: tokens [c0, c1) of sequence b (first row `start`, `len` tokens) for the KV heads and head
@@ -91,7 +91,7 @@ constexpr size_t gqa_lds_bytes(int nt) {
 // PGM: how paged K/V is addressed.  0: one page lookup per tile (pages hold a multiple of 32 tokens; also the packed
 // layout); 1: 16-token pages, a tile is fetched as two runs of 16 tokens, each from one page; 2: smaller pages, every
 // lane looks up the page of the row it loads.
-template <typename Tag, int D, int DV, int NT, bool PREFETCH, bool WH, bool KV8, int PGM>
+template <typename Tag, int D, int DV, int NT, bool PREFETCH, bool WH, int KV8, int PGM>
 __device__ __forceinline__ void gqa_segment(const SweepParams& p, uint8_t* const smem, const int b, const int start,
                                             const int len, const int c0, const int c1, const int split,
                                             const bool direct) {
@@ -110,7 +110,7 @@ __device__ __forceinline__ void gqa_segment(const SweepParams& p, uint8_t* const
     constexpr int CPRL = KV8 ? DV / 16 : CPR;       // 16-byte chunks per V row as loaded
     constexpr int NVR = kGqaTile * CPRL / 64;       // V registers (16 bytes) per tile
     static_assert(D % 32 == 0 && DV % 16 == 0 && (kGqaTile * CPR) % 64 == 0, "shape");
-    static_assert(!KV8 || (D % 64 == 0 && (kGqaTile * CPRL) % 64 == 0), "FP8 K/V: two k-steps per 16-byte load");
+    static_assert(!KV8 || (D % 64 == 0 && (kGqaTile * CPRL) % 64 == 0), "8-bit K/V: two k-steps per 16-byte load");
 
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
@@ -263,10 +263,11 @@ __device__ __forceinline__ void gqa_segment(const SweepParams& p, uint8_t* const
         for (int i = 0; i < NVR; ++i) {
             const int slot = i * 64 + lane;
             const int row = slot / CPRL, ch = slot % CPRL;
-            if constexpr (KV8) {  // sixteen FP8 elements become 32 bytes of the 16-bit tile
-                *reinterpret_cast<uint4*>(vt + row * VP + ch * 32) = fp8x8_to_16<Tag>(make_uint2(tr.v[i].x, tr.v[i].y));
+            if constexpr (KV8) {  // sixteen 8-bit elements become 32 bytes of the 16-bit tile
+                *reinterpret_cast<uint4*>(vt + row * VP + ch * 32) =
+                    kv8x8_to_16<Tag, KV8>(make_uint2(tr.v[i].x, tr.v[i].y));
                 *reinterpret_cast<uint4*>(vt + row * VP + ch * 32 + 16) =
-                    fp8x8_to_16<Tag>(make_uint2(tr.v[i].z, tr.v[i].w));
+                    kv8x8_to_16<Tag, KV8>(make_uint2(tr.v[i].z, tr.v[i].w));
             } else {
                 *reinterpret_cast<uint4*>(vt + row * VP + ch * 16) = tr.v[i];
             }
@@ -285,7 +286,7 @@ __device__ __forceinline__ void gqa_segment(const SweepParams& p, uint8_t* const
                     uint4 kfrag;
                     if constexpr (KV8) {
                         const uint4 w = tr.k[mt][ks >> 1];
-                        kfrag = fp8x8_to_16<Tag>((ks & 1) ? make_uint2(w.z, w.w) : make_uint2(w.x, w.y));
+                        kfrag = kv8x8_to_16<Tag, KV8>((ks & 1) ? make_uint2(w.z, w.w) : make_uint2(w.x, w.y));
                     } else {
                         kfrag = tr.k[mt][ks];
                     }
@@ -475,7 +476,7 @@ __device__ __forceinline__ void gqa_segment(const SweepParams& p, uint8_t* const
 // does not give.  Sequence b spans work-groups first(b) = cu[b] / T ... last(b) = (cu[b+1] - 1) / T (both capped
 // at W - 1); its segment in work-group i is partial number i - first(b), and goes straight to o when
 // first(b) == last(b).
-template <typename Tag, int D, int DV, int NT, bool PREFETCH, bool WH, int MINW, bool KV8 = false, int PGM = 0>
+template <typename Tag, int D, int DV, int NT, bool PREFETCH, bool WH, int MINW, int KV8 = 0, int PGM = 0>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(MINW))) void gqa_mfma_kernel(const SweepParams p) {
     extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
     if (p.flat_tokens == 0) {
@@ -524,5 +525,8 @@ hipError_t launch_gqa_mfma(const SweepParams& p, bool is_bf16, int dim, int head
 // the same with FP8 (e4m3) K and V; dim must be a multiple of 64
 hipError_t launch_gqa_mfma_kv8(const SweepParams& p, bool is_bf16, int dim, int heads_per_group, bool wave_per_head,
                                dim3 grid, hipStream_t stream);
+// the same with int8 K and V; dim must be a multiple of 64
+hipError_t launch_gqa_mfma_i8(const SweepParams& p, bool is_bf16, int dim, int heads_per_group, bool wave_per_head,
+                              dim3 grid, hipStream_t stream);
 
 }  // namespace da

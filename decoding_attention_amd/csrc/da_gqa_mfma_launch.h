@@ -1,5 +1,6 @@
 // Launch helpers of the grouped-head MFMA sweep, shared by the translation units that instantiate it (16-bit
-// K/V in da_gqa_mfma.hip, FP8 K/V in da_gqa_mfma_kv8.hip; two units so that the two sets compile in parallel).
+// K/V in da_gqa_mfma.hip, FP8 in da_gqa_mfma_kv8.hip, int8 in da_gqa_mfma_i8.hip; separate units so that the sets
+// compile in parallel).
 #pragma once
 #include "da_gqa_mfma.h"
 
@@ -9,7 +10,7 @@ namespace da {
 
 namespace gqa_launch {
 
-template <typename Tag, int D, int NT, bool WH, bool KV8, int PGM>
+template <typename Tag, int D, int NT, bool WH, int KV8, int PGM>
 hipError_t launch_form(const SweepParams& p, dim3 grid, hipStream_t stream) {
     constexpr bool kPrefetch = D <= 128;
     constexpr int kMinWaves = (D <= 128 && (NT == 1 || D <= 64)) ? 2 : 1;
@@ -29,14 +30,14 @@ hipError_t launch_form(const SweepParams& p, dim3 grid, hipStream_t stream) {
 
 // 16-token pages of paged K/V take the form that fetches a tile as two runs, smaller pages the form with a lookup
 // per row (instantiations of their own: the extra addresses cost registers the other layouts should not pay for)
-template <typename Tag, int D, int NT, bool WH, bool KV8>
+template <typename Tag, int D, int NT, bool WH, int KV8>
 hipError_t launch_one(const SweepParams& p, dim3 grid, hipStream_t stream) {
     if (p.block_table != nullptr && p.page_shift < 4) return launch_form<Tag, D, NT, WH, KV8, 2>(p, grid, stream);
     if (p.block_table != nullptr && p.page_shift == 4) return launch_form<Tag, D, NT, WH, KV8, 1>(p, grid, stream);
     return launch_form<Tag, D, NT, WH, KV8, 0>(p, grid, stream);
 }
 
-template <typename Tag, int D, bool KV8>
+template <typename Tag, int D, int KV8>
 hipError_t launch_dim(const SweepParams& p, int heads_per_group, bool wh, dim3 grid, hipStream_t stream) {
     if (heads_per_group == 16)
         return wh ? launch_one<Tag, D, 1, true, KV8>(p, grid, stream) : launch_one<Tag, D, 1, false, KV8>(p, grid, stream);
@@ -45,13 +46,13 @@ hipError_t launch_dim(const SweepParams& p, int heads_per_group, bool wh, dim3 g
     return hipErrorInvalidValue;
 }
 
-template <typename Tag, bool KV8>
+template <typename Tag, int KV8>
 hipError_t launch_tag(const SweepParams& p, int dim, int heads_per_group, bool wh, dim3 grid, hipStream_t stream) {
     switch (dim) {
         case 64: return launch_dim<Tag, 64, KV8>(p, heads_per_group, wh, grid, stream);
         case 96:
-            if constexpr (!KV8) return launch_dim<Tag, 96, false>(p, heads_per_group, wh, grid, stream);
-            return hipErrorInvalidValue;  // FP8 loads pair up k-steps: head dims that are multiples of 64 only
+            if constexpr (!KV8) return launch_dim<Tag, 96, 0>(p, heads_per_group, wh, grid, stream);
+            return hipErrorInvalidValue;  // 8-bit loads pair up k-steps: head dims that are multiples of 64 only
         case 128: return launch_dim<Tag, 128, KV8>(p, heads_per_group, wh, grid, stream);
         case 256: return launch_dim<Tag, 256, KV8>(p, heads_per_group, wh, grid, stream);
         default: return hipErrorInvalidValue;

@@ -26,9 +26,9 @@
 // -- which makes both read patterns (16 rows x one chunk for K, 4 rows x 64 bytes for V^T) conflict-free, and
 // because XOR commutes with the per-step chunk offsets every read address is one per-lane base XOR a constant.
 //
-// FP8 K cache (KV8): the tile's bytes (32 rows x 576 FP8 elements, 18 KiB) are staged in LDS by the same
-// direct-to-LDS loads, three stages deep, and the work-group converts each staged tile into the 16-bit tile layout
-// above (exact: e4m3 -> fp16/bf16) one tile ahead of its use, two 16-bit buffers deep; everything downstream of the
+// 8-bit K cache (KV8: FP8 e4m3 or int8): the tile's bytes (32 rows x 576 elements, 18 KiB) are staged in LDS by the
+// same direct-to-LDS loads, three stages deep, and the work-group converts each staged tile into the 16-bit tile
+// layout above (exact: e4m3 or int8 -> fp16/bf16) one tile ahead of its use, two 16-bit buffers deep; everything downstream of the
 // tile is the 16-bit kernel.  The per-head scales fold into the softmax scale and the final normalisation.
 //
 // Mathematics as in the reference kernel (csrc/kernel/decoding_attn/decoding_fwd_kernel.h:50-235
@@ -154,7 +154,7 @@ __device__ __forceinline__ void wait_vmcnt() {
 }
 
 // PG: paged K/V with pages of fewer than 16 tokens (down to 1): every row of a tile has its own page lookup.
-template <typename Tag, int D, int DV, int NWV, bool KV8, bool PG = false>
+template <typename Tag, int D, int DV, int NWV, int KV8, bool PG = false>
 __global__ __launch_bounds__(64 * NWV) void mfma_latent_kernel(const SweepParams p) {
     // (FP8 with PG: the stage is filled a row per load, 36 of the 64 lanes active, instead of 1 KiB per load)
     using MM = Mma<Tag>;
@@ -388,7 +388,8 @@ __global__ __launch_bounds__(64 * NWV) void mfma_latent_kernel(const SweepParams
 #pragma unroll
             for (int i = 0; i < D / 64; ++i) {
                 const u32x2 rv = *reinterpret_cast<lds_src>((uintptr_t)(src + i * 64));
-                const uint4 cv = fp8x8_to_16<Tag>(make_uint2(rv.x, rv.y));
+                // (this lambda is compiled, and never called, for 16-bit K as well)
+                const uint4 cv = kv8x8_to_16<Tag, KV8 ? KV8 : kKvFp8>(make_uint2(rv.x, rv.y));
                 // chunk j + 8 i of the value columns sits at (j + 8 i) ^ swizzle = (j ^ swizzle) ^ 8 i
                 const uint32_t dst = i < DV / 64 ? (dst_a ^ (uint32_t)(i * 128)) : dst_b;
                 *reinterpret_cast<lds_dst>((uintptr_t)dst) = u32x4{cv.x, cv.y, cv.z, cv.w};
@@ -664,7 +665,7 @@ __global__ __launch_bounds__(64 * NWV) void mfma_latent_kernel(const SweepParams
 
 // kNBuf tile buffers (FP8: two of them and three stages of raw bytes); the prologue stages each wave's Q block in a
 // buffer of its own.
-template <int D, int NWV, bool KV8>
+template <int D, int NWV, int KV8>
 constexpr size_t lds_bytes() {
     constexpr size_t buf = (size_t)kTile * D * 2;
     constexpr size_t stg = (size_t)((kTile * D / 1024 + NWV - 1) / NWV) * NWV * 1024;
@@ -673,7 +674,7 @@ constexpr size_t lds_bytes() {
     return tiles > qstage ? tiles : qstage;
 }
 
-template <typename Tag, int D, int DV, int NWV, bool KV8, bool PG>
+template <typename Tag, int D, int DV, int NWV, int KV8, bool PG>
 hipError_t launch_form(const SweepParams& p, dim3 grid, hipStream_t stream) {
     static std::once_flag once;
     static hipError_t attr_err = hipSuccess;
@@ -688,13 +689,13 @@ hipError_t launch_form(const SweepParams& p, dim3 grid, hipStream_t stream) {
     return hipGetLastError();
 }
 
-template <typename Tag, int D, int DV, int NWV, bool KV8>
+template <typename Tag, int D, int DV, int NWV, int KV8>
 hipError_t launch_one(const SweepParams& p, dim3 grid, hipStream_t stream) {
     if (p.block_table != nullptr && p.page_shift < 4) return launch_form<Tag, D, DV, NWV, KV8, true>(p, grid, stream);
     return launch_form<Tag, D, DV, NWV, KV8, false>(p, grid, stream);
 }
 
-template <typename Tag, bool KV8>
+template <typename Tag, int KV8>
 hipError_t launch_tag(const SweepParams& p, int rt, dim3 grid, hipStream_t stream) {
     switch (rt) {
         case 32: return launch_one<Tag, 576, 512, 1, KV8>(p, grid, stream);
@@ -713,11 +714,14 @@ int mla_heads_per_group(int ratio) { return ratio <= 32 ? 32 : (ratio <= 64 ? 64
 int mla_rows_per_trip() { return kTile; }
 
 hipError_t launch_mla(const SweepParams& p, bool is_bf16, int rt, dim3 grid, hipStream_t stream) {
-    return is_bf16 ? launch_tag<bf16_tag, false>(p, rt, grid, stream) : launch_tag<f16_tag, false>(p, rt, grid, stream);
+    return is_bf16 ? launch_tag<bf16_tag, 0>(p, rt, grid, stream) : launch_tag<f16_tag, 0>(p, rt, grid, stream);
 }
 
-hipError_t launch_mla_kv8(const SweepParams& p, bool is_bf16, int rt, dim3 grid, hipStream_t stream) {
-    return is_bf16 ? launch_tag<bf16_tag, true>(p, rt, grid, stream) : launch_tag<f16_tag, true>(p, rt, grid, stream);
+hipError_t launch_mla_kv8(const SweepParams& p, int fmt, bool is_bf16, int rt, dim3 grid, hipStream_t stream) {
+    if (fmt == kKvInt8)
+        return is_bf16 ? launch_tag<bf16_tag, kKvInt8>(p, rt, grid, stream)
+                       : launch_tag<f16_tag, kKvInt8>(p, rt, grid, stream);
+    return is_bf16 ? launch_tag<bf16_tag, kKvFp8>(p, rt, grid, stream) : launch_tag<f16_tag, kKvFp8>(p, rt, grid, stream);
 }
 
 }  // namespace da

@@ -24,8 +24,9 @@
 
 namespace da {
 
-// KV8: K and V hold FP8 (e4m3) elements, converted exactly to the compute type as they are loaded.
-template <typename Tag, int D, int DV, int G, int RT, int U, bool KV8 = false>
+// KV8: K and V hold 8-bit elements (1 = FP8 e4m3, 2 = int8), converted exactly to the compute type as they are
+// loaded; 0 = 16-bit K/V.
+template <typename Tag, int D, int DV, int G, int RT, int U, int KV8 = 0>
 __global__ __launch_bounds__(256) void sweep_kernel(const SweepParams p) {
     static_assert(D % (8 * G) == 0 && DV % (8 * G) == 0, "row must split into 16-byte chunks over G lanes");
     constexpr int CPL = D / 8 / G;    // K chunks per lane
@@ -93,7 +94,7 @@ __global__ __launch_bounds__(256) void sweep_kernel(const SweepParams p) {
     const float vs = head_scale(p.v_scale, hk);
     auto load8 = [](const uint8_t* ptr) __attribute__((always_inline)) {  // eight elements as 16-bit pairs
         if constexpr (KV8)
-            return fp8x8_to_16<Tag>(*reinterpret_cast<const uint2*>(ptr));
+            return kv8x8_to_16<Tag, KV8>(*reinterpret_cast<const uint2*>(ptr));
         else
             return *reinterpret_cast<const uint4*>(ptr);
     };

@@ -13,14 +13,14 @@ template <> struct SweepTile<128> { static constexpr int G = 8,  U = 4; };
 template <> struct SweepTile<256> { static constexpr int G = 16, U = 4; };
 template <> struct SweepTile<576> { static constexpr int G = 8,  U = 1; };
 
-template <typename Tag, int D, int DV, int RT, bool KV8 = false>
+template <typename Tag, int D, int DV, int RT, int KV8 = 0>
 inline hipError_t launch_sweep_rt(const SweepParams& p, dim3 grid, hipStream_t stream) {
     constexpr int G = SweepTile<D>::G, U = SweepTile<D>::U;
     hipLaunchKernelGGL((sweep_kernel<Tag, D, DV, G, RT, U, KV8>), grid, dim3(256), 0, stream, p);
     return hipGetLastError();
 }
 
-template <int D, int DV, int MAXRT, bool KV8 = false>
+template <int D, int DV, int MAXRT, int KV8 = 0>
 inline hipError_t launch_sweep_dim(const SweepParams& p, bool is_bf16, int rt, dim3 grid, hipStream_t stream) {
     if (is_bf16) {
         if (rt == 1) return launch_sweep_rt<bf16_tag, D, DV, 1, KV8>(p, grid, stream);
@@ -47,7 +47,9 @@ hipError_t launch_sweep_d128(const SweepParams& p, bool is_bf16, int rt, dim3 gr
 hipError_t launch_sweep_d256(const SweepParams& p, bool is_bf16, int rt, dim3 grid, hipStream_t stream);
 hipError_t launch_sweep_d576(const SweepParams& p, bool is_bf16, int rt, dim3 grid, hipStream_t stream);
 // the VALU sweep over an FP8 (e4m3) K/V cache, any supported (dim, dim_v)
-hipError_t launch_sweep_kv8(const SweepParams& p, bool is_bf16, int dim, int rt, dim3 grid, hipStream_t stream);
+// 8-bit K/V of format fmt (kKvFp8 or kKvInt8)
+hipError_t launch_sweep_kv8(const SweepParams& p, int fmt, bool is_bf16, int dim, int rt, dim3 grid,
+                            hipStream_t stream);
 hipError_t launch_reduce(const ReduceParams& p, bool is_bf16, int blocks, hipStream_t stream);
 // out[0 .. batch] = running sum of ceil(seq_lens / 2^shift) (positions of paged sequences on the balanced grid's line)
 hipError_t launch_flat_prefix(const int32_t* seq_lens, int batch, int shift, int32_t* out, hipStream_t stream);

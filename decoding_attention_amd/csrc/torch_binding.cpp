@@ -22,17 +22,20 @@ namespace {
     TORCH_CHECK(x.sizes() == torch::IntArrayRef({__VA_ARGS__}), #x " must have shape (" #__VA_ARGS__ ")")
 #define DA_CHECK_CONTIGUOUS(x) TORCH_CHECK(x.is_contiguous(), #x " must be contiguous")
 
-// K/V element format: the 16-bit type of q, or FP8 (e4m3) with optional per-KV-head de-quantisation factors.
-bool is_fp8_kv(const at::Tensor &q, const at::Tensor &k) {
-    if (k.dtype() == torch::kFloat8_e4m3fn) return true;
-    TORCH_CHECK(k.dtype() == q.dtype(), "query and key must have the same dtype (or the key cache is float8_e4m3fn)");
-    return false;
+// K/V element format: the 16-bit type of q (0), or FP8 e4m3 (1) or int8 (2) with optional per-KV-head
+// de-quantisation factors.
+int kv8_format(const at::Tensor &q, const at::Tensor &k) {
+    if (k.dtype() == torch::kFloat8_e4m3fn) return 1;
+    if (k.dtype() == torch::kInt8) return 2;
+    TORCH_CHECK(k.dtype() == q.dtype(),
+                "query and key must have the same dtype (or the key cache is float8_e4m3fn or int8)");
+    return 0;
 }
 
 const float *scale_ptr(const std::optional<at::Tensor> &t, const at::Tensor &q, int64_t head_k, const char *name,
-                       bool fp8) {
+                       int kv8) {
     if (!t.has_value()) return nullptr;
-    TORCH_CHECK(fp8, name, " applies to a float8_e4m3fn K/V cache only");
+    TORCH_CHECK(kv8 != 0, name, " applies to a float8_e4m3fn or int8 K/V cache only");
     const at::Tensor &s = t.value();
     TORCH_CHECK(s.dtype() == torch::kFloat32 && s.is_cuda() && s.device() == q.device() && s.is_contiguous() &&
                     s.numel() == head_k,
@@ -49,7 +52,7 @@ at::Tensor dmha_fwd(const at::Tensor &q, const at::Tensor &k, const std::optiona
     TORCH_CHECK(q_dtype == torch::kFloat16 || q_dtype == torch::kBFloat16,
                 "Decoding-Attention only support FP16 and BF16 data type");
     const bool is_bf16 = q_dtype == torch::kBFloat16;
-    const bool fp8 = is_fp8_kv(q, k);
+    const int kv8 = kv8_format(q, k);  // 0: 16-bit K/V
     const auto kv_dtype = k.dtype();
     TORCH_CHECK(cu_seq_k.dtype() == torch::kInt32, "cu_seq_k must have dtype int32");
 
@@ -123,12 +126,12 @@ at::Tensor dmha_fwd(const at::Tensor &q, const at::Tensor &k, const std::optiona
     c10::hip::HIPGuardMasqueradingAsCUDA guard(q.device());
     hipStream_t stream = c10::hip::getCurrentHIPStreamMasqueradingAsCUDA(q.device().index()).stream();
 
-    const float *k_scale_ptr = scale_ptr(k_scale, q, head_k, "k_scale", fp8);
-    const float *v_scale_ptr = scale_ptr(v_scale, q, head_k, "v_scale", fp8);
+    const float *k_scale_ptr = scale_ptr(k_scale, q, head_k, "k_scale", kv8);
+    const float *v_scale_ptr = scale_ptr(v_scale, q, head_k, "v_scale", kv8);
 
     // k.size(0) is the sum of the key lengths: a free host-side hint for sizing the sequence splits
     const size_t ws_bytes =
-        fp8 ? da_workspace_bytes_fp8kv((size_t)max_seq_k, (size_t)batch, (size_t)head_q, (size_t)head_k, (size_t)dim,
+        kv8 ? da_workspace_bytes_fp8kv((size_t)max_seq_k, (size_t)batch, (size_t)head_q, (size_t)head_k, (size_t)dim,
                                        (size_t)dim_v, (size_t)total_k, 0)
             : da_workspace_bytes((size_t)max_seq_k, (size_t)batch, (size_t)head_q, (size_t)head_k, (size_t)dim,
                                  (size_t)dim_v, (size_t)total_k);
@@ -136,12 +139,12 @@ at::Tensor dmha_fwd(const at::Tensor &q, const at::Tensor &k, const std::optiona
     if (ws_bytes > 0) ws = torch::empty({(int64_t)ws_bytes}, q.options().dtype(torch::kUInt8));
 
     const float scale = softmax_scale.has_value() ? (float)softmax_scale.value() : 0.0f;
+    const auto kv8_entry = kv8 == 2 ? da_decoding_attn_int8kv : da_decoding_attn_fp8kv;
     const int rc =
-        fp8 ? da_decoding_attn_fp8kv(q.data_ptr(), k.data_ptr(), v_ptr, o.data_ptr(), cu_seq_k.data_ptr<int32_t>(),
-                                     (size_t)max_seq_k, (size_t)batch, (size_t)head_q, (size_t)head_k, (size_t)dim,
-                                     (size_t)dim_v, is_alibi ? 1 : 0, is_bf16 ? 1 : 0, scale, slopes_ptr, k_scale_ptr,
-                                     v_scale_ptr, (size_t)total_k, ws_bytes > 0 ? ws.data_ptr() : nullptr, ws_bytes,
-                                     (void *)stream)
+        kv8 ? kv8_entry(q.data_ptr(), k.data_ptr(), v_ptr, o.data_ptr(), cu_seq_k.data_ptr<int32_t>(),
+                        (size_t)max_seq_k, (size_t)batch, (size_t)head_q, (size_t)head_k, (size_t)dim, (size_t)dim_v,
+                        is_alibi ? 1 : 0, is_bf16 ? 1 : 0, scale, slopes_ptr, k_scale_ptr, v_scale_ptr,
+                        (size_t)total_k, ws_bytes > 0 ? ws.data_ptr() : nullptr, ws_bytes, (void *)stream)
             : da_decoding_attn_ex(q.data_ptr(), k.data_ptr(), v_ptr, o.data_ptr(), cu_seq_k.data_ptr<int32_t>(),
                                   (size_t)max_seq_k, (size_t)batch, (size_t)head_q, (size_t)head_k, (size_t)dim,
                                   (size_t)dim_v, is_alibi ? 1 : 0, is_bf16 ? 1 : 0, scale, slopes_ptr,
@@ -163,7 +166,7 @@ at::Tensor dmha_fwd_paged(const at::Tensor &q, const at::Tensor &k_pages, const 
     TORCH_CHECK(q_dtype == torch::kFloat16 || q_dtype == torch::kBFloat16,
                 "Decoding-Attention only support FP16 and BF16 data type");
     const bool is_bf16 = q_dtype == torch::kBFloat16;
-    const bool fp8 = is_fp8_kv(q, k_pages);
+    const int kv8 = kv8_format(q, k_pages);  // 0: 16-bit K/V
     const auto kv_dtype = k_pages.dtype();
     TORCH_CHECK(block_table.dtype() == torch::kInt32, "block_table must have dtype int32");
     TORCH_CHECK(seq_lens.dtype() == torch::kInt32, "seq_lens must have dtype int32");
@@ -235,11 +238,11 @@ at::Tensor dmha_fwd_paged(const at::Tensor &q, const at::Tensor &k_pages, const 
     c10::hip::HIPGuardMasqueradingAsCUDA guard(q.device());
     hipStream_t stream = c10::hip::getCurrentHIPStreamMasqueradingAsCUDA(q.device().index()).stream();
 
-    const float *k_scale_ptr = scale_ptr(k_scale, q, head_k, "k_scale", fp8);
-    const float *v_scale_ptr = scale_ptr(v_scale, q, head_k, "v_scale", fp8);
+    const float *k_scale_ptr = scale_ptr(k_scale, q, head_k, "k_scale", kv8);
+    const float *v_scale_ptr = scale_ptr(v_scale, q, head_k, "v_scale", kv8);
     const size_t hint = total_k > 0 ? (size_t)total_k : 0;
     const size_t ws_bytes =
-        fp8 ? da_workspace_bytes_fp8kv((size_t)max_seq_k, (size_t)batch, (size_t)head_q, (size_t)head_k, (size_t)dim,
+        kv8 ? da_workspace_bytes_fp8kv((size_t)max_seq_k, (size_t)batch, (size_t)head_q, (size_t)head_k, (size_t)dim,
                                        (size_t)dim_v, hint, (size_t)page_size)
             : da_workspace_bytes_paged((size_t)max_seq_k, (size_t)batch, (size_t)head_q, (size_t)head_k, (size_t)dim,
                                        (size_t)dim_v, hint, (size_t)page_size);
@@ -247,8 +250,9 @@ at::Tensor dmha_fwd_paged(const at::Tensor &q, const at::Tensor &k_pages, const 
     if (ws_bytes > 0) ws = torch::empty({(int64_t)ws_bytes}, q.options().dtype(torch::kUInt8));
 
     const float scale = softmax_scale.has_value() ? (float)softmax_scale.value() : 0.0f;
+    const auto kv8_entry = kv8 == 2 ? da_decoding_attn_paged_int8kv : da_decoding_attn_paged_fp8kv;
     const int rc =
-        fp8 ? da_decoding_attn_paged_fp8kv(
+        kv8 ? kv8_entry(
                   q.data_ptr(), k_pages.data_ptr(), v_ptr, o.data_ptr(), block_table.data_ptr<int32_t>(),
                   seq_lens.data_ptr<int32_t>(), (size_t)max_seq_k, (size_t)batch, (size_t)head_q, (size_t)head_k,
                   (size_t)dim, (size_t)dim_v, (size_t)page_size, (size_t)block_table.size(1),

@@ -63,8 +63,9 @@ def decoding_attn_fwd(q: torch.Tensor, k: torch.Tensor, v: Optional[torch.Tensor
         is_alibi: whether to add the ALiBi bias slope_h * (j - (len - 1)).
         softmax_scale (keyword only): defaults to 1/sqrt(dim) as in the reference.
         alibi_slopes (keyword only): float32 [head_q] on the GPU; defaults to 2^(-8(h+1)/head_q).
-        k_scale, v_scale (keyword only): k and v may be torch.float8_e4m3fn (an FP8 K/V cache; q stays 16-bit);
-            these are then float32 [head_k] GPU tensors of de-quantisation factors (default 1): K = k_scale * k.
+        k_scale, v_scale (keyword only): k and v may be torch.float8_e4m3fn or torch.int8 (an 8-bit K/V cache; q
+            stays 16-bit); these are then float32 [head_k] GPU tensors of de-quantisation factors (default 1):
+            K = k_scale * k.
     Return:
         o: [total_q, head_q, dim_v], same dtype as q.
     """
@@ -92,7 +93,7 @@ def decoding_attn_paged_fwd(q: torch.Tensor, k_pages: torch.Tensor, v_pages: Opt
         max_seq_k: upper bound of seq_lens (a host integer: nothing here synchronises with the device).
         page_size (from k_pages.shape[1]) must be a power of two.
         total_k (keyword only): sum of seq_lens if the host knows it; only a hint for sizing sequence splits.
-        k_scale, v_scale (keyword only): as for decoding_attn_fwd, when the pools are torch.float8_e4m3fn.
+        k_scale, v_scale (keyword only): as for decoding_attn_fwd, when the pools are torch.float8_e4m3fn or torch.int8.
     Return:
         o: [batch, head_q, dim_v], same dtype as q.
     """

@@ -130,6 +130,30 @@ size_t da_workspace_bytes_fp8kv(size_t max_seq_k, size_t batch, size_t head_q, s
                                 size_t dim_v, size_t total_k, size_t page_size);
 
 /*
+ * The same attention over an int8 K/V cache (the second format of the reference's quantisation to-do,
+ * README.md:154-156; it has no such path).  k8 and v8 hold two's-complement int8 values, symmetric quantisation
+ * with one factor per KV head: K = k_scale[hk] * int8 value, V likewise (NULL for 1).  Layouts, arguments and
+ * kernels are those of the FP8 entry points above; int8 values convert exactly to fp16 and bf16 too, so with unit
+ * scales the result equals the 16-bit call's on the widened values bit for bit.
+ */
+int da_decoding_attn_int8kv(const void *q, const void *k8, const void *v8, void *o, const int32_t *cu_seq_k,
+                            size_t max_seq_k, size_t batch, size_t head_q, size_t head_k, size_t dim, size_t dim_v,
+                            int is_alibi, int is_bf16, float softmax_scale, const float *alibi_slopes,
+                            const float *k_scale, const float *v_scale, size_t total_k, void *workspace,
+                            size_t workspace_bytes, void *hip_stream);
+
+int da_decoding_attn_paged_int8kv(const void *q, const void *k_pages, const void *v_pages, void *o,
+                                  const int32_t *block_table, const int32_t *seq_lens, size_t max_seq_k,
+                                  size_t batch, size_t head_q, size_t head_k, size_t dim, size_t dim_v,
+                                  size_t page_size, size_t max_blocks_per_seq, size_t k_page_stride,
+                                  size_t v_page_stride, int is_alibi, int is_bf16, float softmax_scale,
+                                  const float *alibi_slopes, const float *k_scale, const float *v_scale,
+                                  size_t total_k, void *workspace, size_t workspace_bytes, void *hip_stream);
+
+size_t da_workspace_bytes_int8kv(size_t max_seq_k, size_t batch, size_t head_q, size_t head_k, size_t dim,
+                                 size_t dim_v, size_t total_k, size_t page_size);
+
+/*
  * Launch plan the library would use for this shape, for tests and benchmarks:
  *   kernel_kind 1 = VALU sweep, 2 = latent (MLA) MFMA sweep, 3 = grouped-head MFMA sweep; nsplit = sequence splits;
  *   chunk = tokens per split; heads_per_group = query heads one work-group serves; total_k as for

@@ -1,6 +1,6 @@
 """Randomised differential test: every path of the library (packed with and without the token-count hint, paged with
-pages of 1..128 tokens, FP8 caches, the latent form, ALiBi, ragged and empty sequences) against float64 attention on
-a sample of rows.  Shapes, layouts and options are drawn from a fixed seed, so a failure names its case.
+pages of 1..128 tokens, FP8 and int8 caches, the latent form, ALiBi, ragged and empty sequences) against float64
+attention on a sample of rows.  Shapes, layouts and options are drawn from a fixed seed, so a failure names its case.
 
 The tolerance is the acceptance bar scaled by the magnitude of the result: a bf16 output of magnitude 2..4 is only
 representable to 0.0078, so the absolute bar of 1e-2 is widened in proportion when |o| > 1.
@@ -53,17 +53,23 @@ def _one_case(rng, seed, case):
     fp8 = rng.random() < 0.35
     layout = rng.choice(["packed", "packed_nohint", "paged"])
     page = rng.choice([1, 8, 16, 32, 64, 128])
+    int8 = fp8 and rng.random() < 0.4  # the 8-bit cache holds int8 instead of FP8
+    kv8_dtype = torch.int8 if int8 else FP8
     desc = (f"seed {seed} case {case}: latent={latent} {hq}/{hk} d{d} {dtype} b{batch} max{maxlen} {mode} "
-            f"alibi={alibi} fp8={fp8} {layout} page={page} total={total}")
+            f"alibi={alibi} fp8={fp8} int8={int8} {layout} page={page} total={total}")
     kw, k8, v8 = {}, None, None
     k_true, v_true = k.float(), None if v is None else v.float()
     if fp8:
+        def quantise(x, scale):
+            y = x.float() / scale.view(1, -1, 1)
+            return torch.round(y).clamp(-128, 127).to(torch.int8) if int8 else y.to(FP8)
+
         ks = 0.015 + 0.015 * torch.rand(hk, generator=g)
         vs = ks if latent else 0.015 + 0.015 * torch.rand(hk, generator=g)
-        k8 = (k.float() / ks.view(1, -1, 1)).to(FP8)
+        k8 = quantise(k, ks)
         k_true = k8.float() * ks.view(1, -1, 1)
         if v is not None:
-            v8 = (v.float() / vs.view(1, -1, 1)).to(FP8)
+            v8 = quantise(v, vs)
             v_true = v8.float() * vs.view(1, -1, 1)
         kw = dict(k_scale=ks.to(DEV), v_scale=vs.to(DEV))
     cu = wl.get_cu_seq(lens)
@@ -73,8 +79,8 @@ def _one_case(rng, seed, case):
                           None if v is None else (v8.view(torch.uint8) if fp8 else v), cu, max_seq_k, dv, alibi,
                           lens.tolist())
         pk = wl.to_pages(src, page, seed=case, poison=not fp8).to(DEV)
-        kp = pk.k_pages.view(FP8) if fp8 else pk.k_pages
-        vp = None if pk.v_pages is None else (pk.v_pages.view(FP8) if fp8 else pk.v_pages)
+        kp = pk.k_pages.view(kv8_dtype) if fp8 else pk.k_pages
+        vp = None if pk.v_pages is None else (pk.v_pages.view(kv8_dtype) if fp8 else pk.v_pages)
         o = decoding_attn_paged_fwd(q.to(DEV), kp, vp, pk.block_table, pk.seq_lens, max_seq_k, dv, alibi,
                                     total_k=rng.choice([0, total]), **kw)
     elif layout == "packed_nohint" and not fp8:

@@ -98,10 +98,11 @@ def test_workspace_sizes_of_the_paged_and_fp8_variants():
     for page in (1, 8, 16, 64, 256):
         assert lib.da_workspace_bytes_paged(*shape, 0, page) == packed
     assert lib.da_workspace_bytes_fp8kv(*shape, 0, 0) == packed          # same kernel kind, same plan
-    # the latent form has no FP8 MFMA kernel: the VALU sweep's plan, covering both the aliased and the distinct V
+    # the latent form: the larger of the MFMA kernel's plan (V inside K) and the VALU sweep's (a distinct V buffer)
     mla = (4096, 16, 128, 1, 576, 512)
     assert lib.da_workspace_bytes_fp8kv(*mla, 0, 0) > 0
     assert lib.da_workspace_bytes_fp8kv(128, 4, 6, 4, 64, 64, 0, 0) == 0   # head_q not a multiple of head_k
+    assert lib.da_workspace_bytes_int8kv(*shape, 0, 0) == packed and lib.da_workspace_bytes_int8kv(*mla, 0, 0) > 0
 
 
 def test_plan_rejects_bad_shapes():
