@@ -112,6 +112,15 @@ def test_head_group_shapes(hq, hk, dtype):
     check_against_oracle(w, run_hip(w))
 
 
+@pytest.mark.parametrize("dim", [64, 128, 256])
+@pytest.mark.parametrize("hq,hk", [(33, 1), (40, 1), (64, 1), (128, 1), (80, 2), (144, 4)])
+def test_more_than_32_query_heads_per_kv_head(hq, hk, dim):
+    """Groups beyond the 32 heads one work-group serves: several work-groups per KV head, the last partly idle."""
+    dtype = torch.bfloat16 if (hq + dim) % 3 == 0 else torch.float16
+    w = wl.make_workload(3, hq, hk, dim, dim, 700, dtype, seed=hq + dim, varlen=True, is_alibi=hq == 40)
+    check_against_oracle(w, run_hip(w))
+
+
 @pytest.mark.parametrize("dim", [64, 96, 128, 256])
 def test_ragged_lengths_with_empty_and_single(dim):
     lens = torch.tensor([0, 1, 2, 63, 64, 65, 127, 129, 0, 700, 1, 0], dtype=torch.int32)
