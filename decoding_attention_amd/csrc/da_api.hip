@@ -43,7 +43,7 @@ int env_int(const char* name, int dflt) {
 // stops being split further; DA_MAX_CHUNK / DA_MIN_CHUNK: bounds on tokens per split.
 struct Tunables {
     int target_wgs, mfma_target_wgs, max_chunk, min_chunk, ragged_chunk, force_kind, group_min_ratio, wave_per_head,
-        mla_heads, gqa_heads, flat_wgs, flat_min_tokens, flat_paged_min_mb, nsplit, mfma_small_wgs;
+        mla_heads, gqa_heads, flat_wgs, flat_min_tokens, flat_paged_min_mb, nsplit, mfma_small_wgs, group_small_wgs, group_small_chunk;
     Tunables() {
         target_wgs = env_int("DA_TARGET_WGS", 512);
         mfma_target_wgs = env_int("DA_MFMA_TARGET_WGS", 256);
@@ -57,6 +57,8 @@ struct Tunables {
         flat_min_tokens = env_int("DA_FLAT_MIN_TOKENS", 256);
         flat_paged_min_mb = env_int("DA_FLAT_PAGED_MIN_MB", 512);  // paged K/V takes the balanced grid from this many MB of K/V
         mfma_small_wgs = env_int("DA_MFMA_SMALL_WGS", 256);  // latent kernel: below this many 256-token splits, split finer
+        group_small_wgs = env_int("DA_GROUP_SMALL_WGS", 256);  // grouped kernel: likewise
+        group_small_chunk = env_int("DA_GROUP_SMALL_CHUNK", 64);
         nsplit = env_int("DA_NSPLIT", 0);  // sequence splits, 0 = by shape (experiments)
         force_kind = env_int("DA_FORCE_KIND", 0);
         wave_per_head = env_int("DA_WAVE_PER_HEAD", 1);
@@ -197,6 +199,18 @@ Plan make_plan(size_t max_seq_k, size_t batch, size_t head_q, size_t head_k, siz
         // VALU sweep: two, measured batch 4 x 1024 tokens 21.4 -> 18.6 us; the grouped kernel loses there)
         const long long fill = pl.kind == kKindSweep ? 2 * 256 : 256;
         if (wgs_at_min < fill) min_chunk = std::max(std::min(min_chunk, 256), trip);
+        // One wave per KV head on a chip that even 256-token splits leave half empty: a work-group's time is then
+        // mostly the latency of its few serial tiles, so split down to 64 tokens, just far enough to give every CU
+        // a work-group and with at most 32 partials to merge (measured, 32/8 heads d 128: batch 1 x 4096 tokens
+        // 20.1 -> 15.7 us, batch 4 x 1024 18.9 -> 13.4, batch 16 x 1024 21.1 -> 18.2; 16/8 heads d 256: batch 1 x
+        // 2048 29.1 -> 15.5).  Below 512 tokens at d < 128 the second launch costs more than the split saves, and
+        // where four waves share one KV head's tokens the finer split changes nothing.
+        if (pl.kind == kKindGroup && pl.wave_per_head && (max_seq_k >= 512 || dim >= 128) &&
+            base * std::max<long long>(1, (long long)max_seq_k / 256) < tun().group_small_wgs) {
+            const int by_partials = (int)(((long long)max_seq_k + 31) / 32 + trip - 1) / trip * trip;
+            min_chunk = std::max(std::min(min_chunk, std::max(tun().group_small_chunk, by_partials)), trip);
+            target_wgs = tun().group_small_wgs;
+        }
         if (ragged) min_chunk = std::max(std::min(min_chunk, tun().ragged_chunk), trip);
     }
     long long want = base > 0 ? (target_wgs + base - 1) / base : 1;
