@@ -233,6 +233,8 @@ struct ReduceParams {
     // positions on the line (see SweepParams)
     int flat_tokens, flat_wgs;
     const int32_t* flat_cu;
+    // the workspace is small (cache-resident): request the first partials before the sequence's length is known
+    int early;
 };
 
 // First token (row of the packed K/V buffers) and length of sequence b; paged sequences start at row 0 of their

@@ -247,7 +247,8 @@ __global__ __launch_bounds__(256) void sweep_kernel(const SweepParams p) {
 }
 
 // Second pass: merge the per-split partials in split order.  One thread per (sequence, query head, group of four
-// output columns); the partials of four splits are fetched together so that their latencies overlap.
+// output columns); the partials of four splits are fetched together so that their latencies overlap, and the maxima
+// are folded in on the way (running maximum, as in the sweeps), so there is no pass over them in front.
 // SG > 1 (many splits of few rows: one long sequence): SG lanes share one (row, four columns), lane j of them
 // taking splits j, j + SG, ...; a wave covers 64 / SG column groups of one row, and the SG partial sums meet through
 // lane exchanges.  The order of summation then differs from SG = 1, not the result's accuracy.
@@ -269,6 +270,24 @@ __global__ __launch_bounds__(256) void reduce_kernel(const ReduceParams p, int r
         sgi = lane / CW;
     }
     if (row >= rows) return;  // (whole waves leave together when SG > 1)
+    const size_t part0 = (size_t)row * p.nsplit;
+    const float2* const ml = reinterpret_cast<const float2*>(p.ws_ml) + part0;
+    const float4* const src = reinterpret_cast<const float4*>(p.ws_o + part0 * p.dim_v) + c4;
+    // This lane's next four partials: slots s0, s0 + SG, ... (clamped to `last`; the caller masks the rest).
+    float2 e[4];
+    float4 x[4];
+    auto fetch = [&](int s0, int last) {
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+            const int s = min(s0 + u * SG, last);
+            e[u] = ml[s];
+            x[u] = src[(size_t)s * nc4];
+        }
+    };
+    // A small workspace (p.early): the first four are requested before the sequence's length is known, so that
+    // their trip to memory overlaps the one for the length; slots past the sequence's last split hold stale data
+    // and are masked below.
+    if (p.early) fetch(sgi, p.nsplit - 1);
     const int b = row / p.head_q;
     const int len = p.cu_seq_k ? p.cu_seq_k[b + 1] - p.cu_seq_k[b] : p.seq_lens[b];
     int ns = 0;
@@ -276,38 +295,52 @@ __global__ __launch_bounds__(256) void reduce_kernel(const ReduceParams p, int r
         // balanced sweep grid: the sequence's partials come from the work-groups its tokens fall into; a sequence
         // inside one work-group was written to o by the sweep itself
         if (len > 0) {
-            const int s = p.flat_cu[b], e = p.flat_cu[b + 1];
-            ns = min((e - 1) / p.flat_tokens, p.flat_wgs - 1) - min(s / p.flat_tokens, p.flat_wgs - 1) + 1;
+            const int lo = p.flat_cu[b], hi = p.flat_cu[b + 1];
+            ns = min((hi - 1) / p.flat_tokens, p.flat_wgs - 1) - min(lo / p.flat_tokens, p.flat_wgs - 1) + 1;
             if (ns == 1) return;
         }
     } else if (len > 0) {
         ns = min(p.nsplit, (len + p.chunk - 1) / p.chunk);
     }
-    const size_t part0 = (size_t)row * p.nsplit;
-    const float2* const ml = reinterpret_cast<const float2*>(p.ws_ml) + part0;
-    const float4* const src = reinterpret_cast<const float4*>(p.ws_o + part0 * p.dim_v) + c4;
+    // One pass with a running maximum (the sum is rescaled when a later partial raises it).
     float mm = kNegBig;
-    for (int s = 0; s < ns; ++s) mm = fmaxf(mm, ml[s].x);
     float4 num = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
     float den = 0.0f;
     for (int s0 = sgi; s0 < ns; s0 += 4 * SG) {
-        float2 e[4];
-        float4 x[4];
+        if (!p.early || s0 != sgi) fetch(s0, ns - 1);
+        float m_new = mm;
+#pragma unroll
+        for (int u = 0; u < 4; ++u)
+            if (s0 + u * SG < ns) m_new = fmaxf(m_new, e[u].x);
+        const float keep = fast_exp2(mm - m_new);  // 0 on the first round
+        mm = m_new;
+        den *= keep;
+        num.x *= keep;
+        num.y *= keep;
+        num.z *= keep;
+        num.w *= keep;
 #pragma unroll
         for (int u = 0; u < 4; ++u) {
-            const int s = min(s0 + u * SG, ns - 1);
-            e[u] = ml[s];
-            x[u] = src[(size_t)s * nc4];
+            const bool valid = s0 + u * SG < ns;
+            const float w = valid ? fast_exp2(e[u].x - mm) : 0.0f;
+            den += valid ? w * e[u].y : 0.0f;
+            num.x += valid ? w * x[u].x : 0.0f;
+            num.y += valid ? w * x[u].y : 0.0f;
+            num.z += valid ? w * x[u].z : 0.0f;
+            num.w += valid ? w * x[u].w : 0.0f;
         }
+    }
+    if constexpr (SG > 1) {
+        // the SG lanes of an element bring their sums to a common maximum first
+        float m_all = mm;
 #pragma unroll
-        for (int u = 0; u < 4; ++u) {
-            const float w = (s0 + u * SG < ns) ? fast_exp2(e[u].x - mm) : 0.0f;
-            den += w * e[u].y;
-            num.x += w * x[u].x;
-            num.y += w * x[u].y;
-            num.z += w * x[u].z;
-            num.w += w * x[u].w;
-        }
+        for (int d = 64 / SG; d < 64; d <<= 1) m_all = fmaxf(m_all, __shfl_xor(m_all, d));
+        const float keep = fast_exp2(mm - m_all);
+        den *= keep;
+        num.x *= keep;
+        num.y *= keep;
+        num.z *= keep;
+        num.w *= keep;
     }
     if constexpr (SG > 1) {
 #pragma unroll
