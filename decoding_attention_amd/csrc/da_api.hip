@@ -199,6 +199,11 @@ Plan make_plan(size_t max_seq_k, size_t batch, size_t head_q, size_t head_k, siz
         // VALU sweep: two, measured batch 4 x 1024 tokens 21.4 -> 18.6 us; the grouped kernel loses there)
         const long long fill = pl.kind == kKindSweep ? 2 * 256 : 256;
         if (wgs_at_min < fill) min_chunk = std::max(std::min(min_chunk, 256), trip);
+        // the VALU sweep at d = 256 (long rows, long tiles): 128-token splits while the chip is not full
+        // (measured, MHA batch 1 x 512 tokens 17.2 -> 13.2 us, batch 2 x 1024 19.7 -> 18.0; no gain at d <= 128)
+        if (pl.kind == kKindSweep && dim >= 256 && max_seq_k >= 512 &&
+            base * std::max<long long>(1, (long long)max_seq_k / 256) < fill)
+            min_chunk = std::max(std::min(min_chunk, 128), trip);
         // One wave per KV head on a chip that even 256-token splits leave half empty: a work-group's time is then
         // mostly the latency of its few serial tiles, so split down to 64 tokens, just far enough to give every CU
         // a work-group and with at most 32 partials to merge (measured, 32/8 heads d 128: batch 1 x 4096 tokens
