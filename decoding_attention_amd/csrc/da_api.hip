@@ -137,6 +137,9 @@ Plan make_plan(size_t max_seq_k, size_t batch, size_t head_q, size_t head_k, siz
             pl.rt = std::min(tun().mla_heads, da::mla_heads_per_group(ratio));
         trip = da::mla_rows_per_trip();
         target_wgs = tun().mfma_target_wgs;  // one 4-wave work-group fills a CU
+        // work-groups of one or two waves over 16-bit K take two tile buffers instead of three when there are more
+        // of them than CUs, and then run two to a CU
+        if (pl.rt <= 64 && !kv_8bit) target_wgs *= 2;
     } else if (dim <= 256 && !force_sweep && (!kv_8bit || dim % 64 == 0) &&
                (ratio >= tun().group_min_ratio ||
                 (tun().group_min_ratio > 1 && (max_seq_k >= 1024 || dim <= 96) &&

@@ -6,6 +6,9 @@ namespace da {
 bool mla_supported(size_t dim, size_t dim_v, int ratio);
 int mla_heads_per_group(int ratio);
 int mla_rows_per_trip();
+// work-groups of one or two waves run two to a CU (two tile buffers instead of three) when the grid has more
+// work-groups than this (DA_MLA_TWO_PER_CU_FROM, default 256)
+int mla_two_per_cu_from();
 hipError_t launch_mla(const SweepParams& p, bool is_bf16, int rt, dim3 grid, hipStream_t stream);
 // the same over an 8-bit K cache of format fmt (kKvFp8 or kKvInt8)
 hipError_t launch_mla_kv8(const SweepParams& p, int fmt, bool is_bf16, int rt, dim3 grid, hipStream_t stream);

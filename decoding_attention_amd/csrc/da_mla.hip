@@ -35,6 +35,7 @@
 // with the latent aliasing of csrc/ops/decoding_attn.cpp:30-37); the structure is unrelated.
 #include "da_mla.h"
 
+#include <cstdlib>
 #include <mutex>
 
 namespace da {
@@ -154,7 +155,9 @@ __device__ __forceinline__ void wait_vmcnt() {
 }
 
 // PG: paged K/V with pages of fewer than 16 tokens (down to 1): every row of a tile has its own page lookup.
-template <typename Tag, int D, int DV, int NWV, int KV8, bool PG = false>
+// NB: tile buffers of the 16-bit form.  Three keep two tiles in flight behind the one being read; two (one in
+// flight) halve the LDS footprint, so that two work-groups of one or two waves share a CU.
+template <typename Tag, int D, int DV, int NWV, int KV8, bool PG = false, int NB = kNBuf>
 __global__ __launch_bounds__(64 * NWV) void mfma_latent_kernel(const SweepParams p) {
     // (FP8 with PG: the stage is filled a row per load, 36 of the 64 lanes active, instead of 1 KiB per load)
     using MM = Mma<Tag>;
@@ -171,7 +174,8 @@ __global__ __launch_bounds__(64 * NWV) void mfma_latent_kernel(const SweepParams
     constexpr int KS = D / 16;                           // k-steps of Q K^T
     constexpr int CT = DV / 32;                          // 32-column tiles of the output
     // FP8 K cache: stages of the tile's raw bytes, filled 1 KiB per load instruction
-    constexpr int NTB = KV8 ? 2 : kNBuf;                 // 16-bit tile buffers
+    static_assert(NB == kNBuf || (NB == 2 && !KV8), "buffer count");
+    constexpr int NTB = KV8 ? 2 : NB;                    // 16-bit tile buffers
     constexpr int STG_REAL = kTile * D / 1024;           // load instructions that cover a staged tile (18)
     constexpr int NLW8 = PG ? kTile / NWV : (STG_REAL + NWV - 1) / NWV;  // per wave (the surplus ones repeat the last
                                                                          // KiB); PG: a row per load
@@ -180,7 +184,7 @@ __global__ __launch_bounds__(64 * NWV) void mfma_latent_kernel(const SweepParams
     static_assert((kTile * D) % 1024 == 0, "staged tile");
     static_assert(D % 16 == 0 && DV % 32 == 0 && DV <= D, "shape");
 
-    extern __shared__ __attribute__((aligned(1024))) uint8_t smem[];  // max(kNBuf, NWV) * BUF
+    extern __shared__ __attribute__((aligned(1024))) uint8_t smem[];  // lds_bytes<D, NWV, KV8, NB>()
     const uint32_t smem_off = (uint32_t)(uintptr_t)smem;
 
     const int lane = threadIdx.x & 63;
@@ -403,15 +407,16 @@ __global__ __launch_bounds__(64 * NWV) void mfma_latent_kernel(const SweepParams
     auto second_run = [&](int tok, int64_t first) {
         return tok + 16 < c1 ? row_ref(p, b, start, tok + 16).k : first;
     };
+    constexpr int AHEAD = KV8 ? 3 : NB - 1;  // tiles in flight behind the one being read
     RowPages rows_ahead{};
     if constexpr (PG) {
         issue_tile_pg(c0, lookup_rows(c0), 0);
-        if (ntiles > 1) issue_tile_pg(c0 + kTile, lookup_rows(c0 + kTile), 1);
-        if (ntiles > 2) rows_ahead = lookup_rows(c0 + 2 * kTile);
+        if (NB > 2 && ntiles > 1) issue_tile_pg(c0 + kTile, lookup_rows(c0 + kTile), 1);
+        if (ntiles > NB - 1) rows_ahead = lookup_rows(c0 + (NB - 1) * kTile);
     } else {
         const int64_t r0 = row_ref(p, b, start, c0).k;
         issue_tile(c0, r0, second_run(c0, r0), 0);
-        if (ntiles > 1) {
+        if (NB > 2 && ntiles > 1) {
             const int64_t r1 = row_ref(p, b, start, c0 + kTile).k;
             issue_tile(c0 + kTile, r1, second_run(c0 + kTile, r1), 1);
         }
@@ -437,7 +442,6 @@ __global__ __launch_bounds__(64 * NWV) void mfma_latent_kernel(const SweepParams
         convert_stage(0, 0);
     }
     // page of the tile after those, fetched one trip ahead of its use (a scalar load for paged K/V)
-    constexpr int AHEAD = KV8 ? 3 : 2;  // tiles in flight behind the one being read
     int page_ahead = !PG && ntiles > AHEAD ? page_of(p, b, c0 + AHEAD * kTile) : 0;
     int page_ahead1 = !PG && ntiles > AHEAD && c0 + AHEAD * kTile + 16 < c1 ? page_of(p, b, c0 + AHEAD * kTile + 16) : 0;
     // Make the compiler settle its own wait for the Q loads here, before the loop.  It cannot see the
@@ -460,7 +464,7 @@ __global__ __launch_bounds__(64 * NWV) void mfma_latent_kernel(const SweepParams
 
     const float bias0 = slope * (float)(half * 4 - (len - 1));  // ALiBi: slope * (token - (len - 1)), split in lane and tile parts
     int buf = 0;       // 16-bit buffer that holds tile t
-    int buf_next = KV8 ? 0 : 2;  // buffer (FP8: stage) that receives tile t + AHEAD
+    int buf_next = KV8 ? 0 : NB - 1;  // buffer (FP8: stage) that receives tile t + AHEAD
     int stg_conv = 1;  // FP8: stage that holds tile t + 1
     for (int t = 0; t < ntiles; ++t) {
         if constexpr (KV8) {
@@ -490,22 +494,22 @@ __global__ __launch_bounds__(64 * NWV) void mfma_latent_kernel(const SweepParams
             }
             }
         } else {
-        if (t + 1 < ntiles)
+        if (AHEAD > 1 && t + 1 < ntiles)
             wait_vmcnt<NLW>();  // tile t landed; tile t+1 may still be in flight
         else
             wait_vmcnt<0>();
         __syncthreads();  // every wave's share of tile t is in LDS, and every wave is done with tile t-1
         if constexpr (PG) {
-            if (t + 2 < ntiles) issue_tile_pg(c0 + (t + 2) * kTile, rows_ahead, buf_next);
-            if (t + 3 < ntiles) rows_ahead = lookup_rows(c0 + (t + 3) * kTile);
+            if (t + AHEAD < ntiles) issue_tile_pg(c0 + (t + AHEAD) * kTile, rows_ahead, buf_next);
+            if (t + AHEAD + 1 < ntiles) rows_ahead = lookup_rows(c0 + (t + AHEAD + 1) * kTile);
         } else {
-        if (t + 2 < ntiles) {
-            const int tk = c0 + (t + 2) * kTile;
+        if (t + AHEAD < ntiles) {
+            const int tk = c0 + (t + AHEAD) * kTile;
             const int64_t r0 = row_in_page(p, start, tk, page_ahead).k;
             issue_tile(tk, r0, tk + 16 < c1 ? row_in_page(p, start, tk + 16, page_ahead1).k : r0, buf_next);
         }
-        if (t + 3 < ntiles) {
-            const int tk = c0 + (t + 3) * kTile;
+        if (t + AHEAD + 1 < ntiles) {
+            const int tk = c0 + (t + AHEAD + 1) * kTile;
             page_ahead = page_of(p, b, tk);
             if (tk + 16 < c1) page_ahead1 = page_of(p, b, tk + 16);
         }
@@ -522,7 +526,7 @@ __global__ __launch_bounds__(64 * NWV) void mfma_latent_kernel(const SweepParams
 #pragma unroll
         for (int j = 0; j < 4; ++j) kaddr_b[j] = tb ^ (32 * j);
         buf = (buf == NTB - 1) ? 0 : buf + 1;
-        buf_next = (buf_next == kNBuf - 1) ? 0 : buf_next + 1;  // (three 16-bit buffers, or three FP8 stages)
+        buf_next = (buf_next == (KV8 ? kNBuf : NB) - 1) ? 0 : buf_next + 1;  // (NB 16-bit buffers, or three FP8 stages)
 
         // S^T = K_tile . Q^T : rows = tokens, columns = heads.  K fragments are read kKPD steps ahead.
         f32x16 s;
@@ -665,34 +669,42 @@ __global__ __launch_bounds__(64 * NWV) void mfma_latent_kernel(const SweepParams
 
 // kNBuf tile buffers (FP8: two of them and three stages of raw bytes); the prologue stages each wave's Q block in a
 // buffer of its own.
-template <int D, int NWV, int KV8>
+template <int D, int NWV, int KV8, int NB>
 constexpr size_t lds_bytes() {
     constexpr size_t buf = (size_t)kTile * D * 2;
     constexpr size_t stg = (size_t)((kTile * D / 1024 + NWV - 1) / NWV) * NWV * 1024;
-    constexpr size_t tiles = KV8 ? 2 * buf + 3 * stg : (size_t)kNBuf * buf;
+    constexpr size_t tiles = KV8 ? 2 * buf + 3 * stg : (size_t)NB * buf;
     constexpr size_t qstage = (size_t)NWV * buf;
     return tiles > qstage ? tiles : qstage;
 }
 
-template <typename Tag, int D, int DV, int NWV, int KV8, bool PG>
+template <typename Tag, int D, int DV, int NWV, int KV8, bool PG, int NB>
 hipError_t launch_form(const SweepParams& p, dim3 grid, hipStream_t stream) {
     static std::once_flag once;
     static hipError_t attr_err = hipSuccess;
-    auto kern = mfma_latent_kernel<Tag, D, DV, NWV, KV8, PG>;
+    auto kern = mfma_latent_kernel<Tag, D, DV, NWV, KV8, PG, NB>;
     std::call_once(once, [&] {
         attr_err = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
-                                       (int)lds_bytes<D, NWV, KV8>());
+                                       (int)lds_bytes<D, NWV, KV8, NB>());
     });
     if (attr_err != hipSuccess) return attr_err;
-    constexpr size_t lds = lds_bytes<D, NWV, KV8>();
+    constexpr size_t lds = lds_bytes<D, NWV, KV8, NB>();
     hipLaunchKernelGGL(kern, grid, dim3(64 * NWV), lds, stream, p);
     return hipGetLastError();
 }
 
 template <typename Tag, int D, int DV, int NWV, int KV8>
 hipError_t launch_one(const SweepParams& p, dim3 grid, hipStream_t stream) {
-    if (p.block_table != nullptr && p.page_shift < 4) return launch_form<Tag, D, DV, NWV, KV8, true>(p, grid, stream);
-    return launch_form<Tag, D, DV, NWV, KV8, false>(p, grid, stream);
+    const bool pg = p.block_table != nullptr && p.page_shift < 4;
+    if constexpr (NWV <= 2 && KV8 == 0) {
+        // more work-groups than CUs: the two-buffer form, two work-groups to a CU
+        if ((long long)grid.x * grid.y * grid.z > mla_two_per_cu_from()) {
+            if (pg) return launch_form<Tag, D, DV, NWV, KV8, true, 2>(p, grid, stream);
+            return launch_form<Tag, D, DV, NWV, KV8, false, 2>(p, grid, stream);
+        }
+    }
+    if (pg) return launch_form<Tag, D, DV, NWV, KV8, true, kNBuf>(p, grid, stream);
+    return launch_form<Tag, D, DV, NWV, KV8, false, kNBuf>(p, grid, stream);
 }
 
 template <typename Tag, int KV8>
@@ -706,6 +718,14 @@ hipError_t launch_tag(const SweepParams& p, int rt, dim3 grid, hipStream_t strea
 }
 
 }  // namespace
+
+int mla_two_per_cu_from() {
+    static const int v = [] {
+        const char* s = getenv("DA_MLA_TWO_PER_CU_FROM");
+        return s && *s ? atoi(s) : 256;
+    }();
+    return v;
+}
 
 bool mla_supported(size_t dim, size_t dim_v, int ratio) { return dim == 576 && dim_v == 512 && ratio >= 1; }
 
