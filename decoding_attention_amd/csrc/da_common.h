@@ -1,6 +1,8 @@
 // Shared device helpers and launch parameter blocks for the gfx950 decoding-attention kernels.
 #pragma once
 #include <hip/hip_runtime.h>
+
+#include <atomic>
 #include <stdint.h>
 
 #include <type_traits>
@@ -289,6 +291,19 @@ __device__ __forceinline__ float alibi_slope_log2(const float* slopes, int h, in
     // closed form 2^(-8(h+1)/head_q); a slope array overrides it
     float s = slopes ? slopes[h] : fast_exp2(-8.0f * (float)(h + 1) / (float)head_q);
     return s * kLog2e;
+}
+
+// Raise a kernel's dynamic LDS limit once per device (the attribute belongs to the function on the current
+// device, and one process may drive several).  `done` is the caller's per-kernel bit mask of devices served.
+inline hipError_t ensure_lds_limit(const void* kernel, size_t lds_bytes, std::atomic<uint64_t>& done) {
+    int dev = 0;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return e;
+    const uint64_t bit = 1ull << (dev & 63);
+    if (done.load(std::memory_order_acquire) & bit) return hipSuccess;
+    e = hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes);
+    if (e == hipSuccess) done.fetch_or(bit, std::memory_order_release);  // (a failure is retried by the next call)
+    return e;
 }
 
 }  // namespace da

@@ -4,7 +4,6 @@
 #pragma once
 #include "da_gqa_mfma.h"
 
-#include <mutex>
 
 namespace da {
 
@@ -16,14 +15,11 @@ hipError_t launch_form(const SweepParams& p, dim3 grid, hipStream_t stream) {
     constexpr int kMinWaves = (D <= 128 && (NT == 1 || D <= 64)) ? 2 : 1;
     auto kern = gqa_mfma_kernel<Tag, D, D, NT, kPrefetch, WH, kMinWaves, KV8, PGM>;
     const size_t lds = gqa_lds_bytes<D>(NT);
-    static std::once_flag once;
-    static hipError_t attr_err = hipSuccess;
-    std::call_once(once, [&] {
-        if (lds > 48 * 1024)
-            attr_err = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
-                                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
-    });
-    if (attr_err != hipSuccess) return attr_err;
+    if (lds > 48 * 1024) {
+        static std::atomic<uint64_t> devices_done{0};
+        const hipError_t attr_err = ensure_lds_limit(reinterpret_cast<const void*>(kern), lds, devices_done);
+        if (attr_err != hipSuccess) return attr_err;
+    }
     hipLaunchKernelGGL(kern, grid, dim3(256), lds, stream, p);
     return hipGetLastError();
 }

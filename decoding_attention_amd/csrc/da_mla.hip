@@ -36,7 +36,6 @@
 #include "da_mla.h"
 
 #include <cstdlib>
-#include <mutex>
 
 namespace da {
 
@@ -680,13 +679,10 @@ constexpr size_t lds_bytes() {
 
 template <typename Tag, int D, int DV, int NWV, int KV8, bool PG, int NB>
 hipError_t launch_form(const SweepParams& p, dim3 grid, hipStream_t stream) {
-    static std::once_flag once;
-    static hipError_t attr_err = hipSuccess;
     auto kern = mfma_latent_kernel<Tag, D, DV, NWV, KV8, PG, NB>;
-    std::call_once(once, [&] {
-        attr_err = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
-                                       (int)lds_bytes<D, NWV, KV8, NB>());
-    });
+    static std::atomic<uint64_t> devices_done{0};
+    const hipError_t attr_err =
+        ensure_lds_limit(reinterpret_cast<const void*>(kern), lds_bytes<D, NWV, KV8, NB>(), devices_done);
     if (attr_err != hipSuccess) return attr_err;
     constexpr size_t lds = lds_bytes<D, NWV, KV8, NB>();
     hipLaunchKernelGGL(kern, grid, dim3(64 * NWV), lds, stream, p);
