@@ -43,7 +43,8 @@ int env_int(const char* name, int dflt) {
 // stops being split further; DA_MAX_CHUNK / DA_MIN_CHUNK: bounds on tokens per split.
 struct Tunables {
     int target_wgs, mfma_target_wgs, max_chunk, min_chunk, ragged_chunk, force_kind, group_min_ratio, wave_per_head,
-        mla_heads, gqa_heads, flat_wgs, flat_min_tokens, flat_paged_min_mb, nsplit, mfma_small_wgs, group_small_wgs, group_small_chunk;
+        mla_heads, gqa_heads, flat_wgs, flat_min_tokens, flat_paged_min_mb, nsplit, mfma_small_wgs, group_small_wgs,
+        group_small_chunk, mla_group_heads;
     Tunables() {
         target_wgs = env_int("DA_TARGET_WGS", 512);
         mfma_target_wgs = env_int("DA_MFMA_TARGET_WGS", 256);
@@ -57,6 +58,8 @@ struct Tunables {
         flat_min_tokens = env_int("DA_FLAT_MIN_TOKENS", 256);
         flat_paged_min_mb = env_int("DA_FLAT_PAGED_MIN_MB", 512);  // paged K/V takes the balanced grid from this many MB of K/V
         mfma_small_wgs = env_int("DA_MFMA_SMALL_WGS", 256);  // latent kernel: below this many 256-token splits, split finer
+        // latent form: up to this many query heads take the grouped kernel (0 = never)
+        mla_group_heads = env_int("DA_MLA_GROUP_HEADS", 16);
         group_small_wgs = env_int("DA_GROUP_SMALL_WGS", 256);  // grouped kernel: likewise
         group_small_chunk = env_int("DA_GROUP_SMALL_CHUNK", 64);
         nsplit = env_int("DA_NSPLIT", 0);  // sequence splits, 0 = by shape (experiments)
@@ -123,10 +126,24 @@ Plan make_plan(size_t max_seq_k, size_t batch, size_t head_q, size_t head_k, siz
     const int ratio = (int)(head_q / head_k);
     int trip;
     int target_wgs = tun().target_wgs;
+    int max_chunk_scale = 1;
     const bool latent = !v_distinct && da::mla_supported(dim, dim_v, ratio);
     const bool force_sweep = tun().force_kind == kKindSweep;
-    const bool mfma = latent && !force_sweep;
-    if (mfma) {
+    // the latent form with up to 16 query heads (a tensor-parallel shard) runs on the grouped kernel, which keeps more
+    // bytes in flight per CU than the latent kernel's one-wave form can (its tiles need LDS landing space)
+    const bool latent_group = latent && !force_sweep && ratio <= tun().mla_group_heads;
+    const bool mfma = latent && !force_sweep && !latent_group;
+    if (latent_group) {
+        pl.kind = kKindGroup;
+        pl.rt = 16;
+        pl.wave_per_head = false;
+        trip = 4 * da::kGqaTile;
+        // one work-group (its four V tiles take 132 KB of LDS) per CU, and splits up to twice the usual length
+        // (measured, 16 heads: batch 64 x 4096 tokens 73 -> 64 us with 256 work-groups instead of 512; batch 128
+        // 126 -> 118 us with 2048-token splits)
+        target_wgs = tun().mfma_target_wgs;
+        max_chunk_scale = 2;
+    } else if (mfma) {
         pl.kind = kKindMfma;
         pl.rt = da::mla_heads_per_group(ratio);
         // few sequences and short ones cannot fill the chip even at the finest split: then two work-groups of 64
@@ -135,6 +152,9 @@ Plan make_plan(size_t max_seq_k, size_t batch, size_t head_q, size_t head_k, siz
         if ((tun().mla_heads == 32 || tun().mla_heads == 64 || tun().mla_heads == 128) && tun().mla_heads <= 128 &&
             tun().mla_heads >= 32)
             pl.rt = std::min(tun().mla_heads, da::mla_heads_per_group(ratio));
+        // an 8-bit K cache is converted by the whole work-group: always four waves, those without heads of their
+        // own only load and convert (measured, FP8, 32 heads, batch 64 x 4096 tokens: 206 us with one wave)
+        if (kv_8bit) pl.rt = 128;
         trip = da::mla_rows_per_trip();
         target_wgs = tun().mfma_target_wgs;  // one 4-wave work-group fills a CU
         // work-groups of one or two waves over 16-bit K take two tile buffers instead of three when there are more
@@ -225,7 +245,7 @@ Plan make_plan(size_t max_seq_k, size_t batch, size_t head_q, size_t head_k, siz
     const long long by_len = std::max<long long>(1, (long long)max_seq_k / min_chunk);
     // sweep work-groups are also kept short (shorter still for a ragged batch); the latent MFMA kernel's partials
     // are too large (heads x dim_v floats per split) to split more than occupancy asks for
-    const int max_chunk = std::max(1, ragged ? tun().ragged_chunk : tun().max_chunk);
+    const int max_chunk = std::max(1, ragged ? tun().ragged_chunk : tun().max_chunk * max_chunk_scale);
     long long by_cap = mfma ? 1 : ((long long)max_seq_k + max_chunk - 1) / max_chunk;
     long long ns = std::max(std::min(want, by_len), std::min(by_cap, by_len));
     ns = std::max<long long>(1, std::min<long long>(ns, kMaxSplits));

@@ -20,6 +20,10 @@
 //   (ds_read_b64_tr_b16: 8 tokens of one column per lane) as the A-operand of
 //   O^T[DV x 16 heads] += V^T . P^T.
 //
+// The latent form with up to 16 query heads (D = 576, DV = 512, V the first 512 columns of each K row: a
+// tensor-parallel shard of an MLA model) runs here too: the rows are loaded once, as K, and their value columns are
+// parked in the LDS tile from the K registers.
+//
 // Mathematics as in the reference kernel (csrc/kernel/decoding_attn/decoding_fwd_kernel.h:50-235,
 // head mapping block_info.h:14-30); the reference streams K and V once per query head on CUDA
 // cores and keeps the whole score row in shared memory.
@@ -39,6 +43,15 @@ struct Mma16<f16_tag> {
     static __device__ __forceinline__ f32x4 mma(vec8 a, vec8 b, f32x4 c) {
         return __builtin_amdgcn_mfma_f32_16x16x32_f16(a, b, c, 0, 0, 0);
     }
+    // the same product with the second operand held in accumulation registers (frees ordinary ones where a kernel
+    // is short of them); issued from assembly, so the caller pads the result hazard itself (settle)
+    // (the wait states in front cover an operand that a vector instruction has just written)
+    static __device__ __forceinline__ void mma_bacc(vec8 a, const vec8& b, f32x4& c) {
+        asm volatile("s_nop 1\n\tv_mfma_f32_16x16x32_f16 %0, %1, %2, %0" : "+v"(c) : "v"(a), "a"(b));
+    }
+    static __device__ __forceinline__ void mma_bacc0(vec8 a, const vec8& b, f32x4& c) {  // c = a.b
+        asm volatile("s_nop 1\n\tv_mfma_f32_16x16x32_f16 %0, %1, %2, 0" : "=v"(c) : "v"(a), "a"(b));
+    }
     static __device__ __forceinline__ vec8 pack8(const float* x) {
         vec8 v;
 #pragma unroll
@@ -52,6 +65,12 @@ struct Mma16<bf16_tag> {
     static __device__ __forceinline__ f32x4 mma(vec8 a, vec8 b, f32x4 c) {
         return __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, c, 0, 0, 0);
     }
+    static __device__ __forceinline__ void mma_bacc(vec8 a, const vec8& b, f32x4& c) {
+        asm volatile("s_nop 1\n\tv_mfma_f32_16x16x32_bf16 %0, %1, %2, %0" : "+v"(c) : "v"(a), "a"(b));
+    }
+    static __device__ __forceinline__ void mma_bacc0(vec8 a, const vec8& b, f32x4& c) {
+        asm volatile("s_nop 1\n\tv_mfma_f32_16x16x32_bf16 %0, %1, %2, 0" : "=v"(c) : "v"(a), "a"(b));
+    }
     static __device__ __forceinline__ vec8 pack8(const float* x) {
         vec8 v;
 #pragma unroll
@@ -59,6 +78,10 @@ struct Mma16<bf16_tag> {
         return v;
     }
 };
+
+// Wait states between the last matrix instruction issued from assembly and the first ordinary read of its result
+// (the compiler cannot see into the assembly to place them).
+__device__ __forceinline__ void settle(f32x4& c) { asm volatile("s_nop 15\n\ts_nop 3" : "+v"(c)); }
 
 constexpr int kGqaTile = 32;  // tokens per wave iteration
 
@@ -108,7 +131,11 @@ __device__ __forceinline__ void gqa_segment(const SweepParams& p, uint8_t* const
     constexpr int KB = KV8 ? 1 : 2;                 // bytes per K/V element
     constexpr int KSR = KV8 ? KS / 2 : KS;          // K registers (16 bytes) per 16-token tile
     constexpr int CPRL = KV8 ? DV / 16 : CPR;       // 16-byte chunks per V row as loaded
-    constexpr int NVR = kGqaTile * CPRL / 64;       // V registers (16 bytes) per tile
+    // VK: V is the first DV columns of each K row (the latent form, D = 576 and DV = 512).  The rows are loaded once,
+    // as K, and their value columns go to the LDS tile from the K registers after the score products.
+    constexpr bool VK = D != DV;
+    constexpr int NVR = VK ? 1 : kGqaTile * CPRL / 64;  // V registers (16 bytes) per tile
+    static_assert(!VK || (DV < D && DV % 64 == 0), "value columns inside the key rows");
     static_assert(D % 32 == 0 && DV % 16 == 0 && (kGqaTile * CPR) % 64 == 0, "shape");
     static_assert(!KV8 || (D % 64 == 0 && (kGqaTile * CPRL) % 64 == 0), "8-bit K/V: two k-steps per 16-byte load");
 
@@ -249,7 +276,7 @@ __device__ __forceinline__ void gqa_segment(const SweepParams& p, uint8_t* const
 
     const int ntiles = (c1 - c0 + kGqaTile - 1) / kGqaTile;
     if (tw < ntiles) {
-        load_v(c0 + tw * kGqaTile, tr);
+        if constexpr (!VK) load_v(c0 + tw * kGqaTile, tr);
         load_k(c0 + tw * kGqaTile, tr);
     }
 
@@ -259,6 +286,7 @@ __device__ __forceinline__ void gqa_segment(const SweepParams& p, uint8_t* const
         const int tok_next = tok0 + NW * kGqaTile;
 
         // park V in LDS (row-major, padded pitch), then refill the V registers
+        if constexpr (!VK) {
 #pragma unroll
         for (int i = 0; i < NVR; ++i) {
             const int slot = i * 64 + lane;
@@ -273,6 +301,7 @@ __device__ __forceinline__ void gqa_segment(const SweepParams& p, uint8_t* const
             }
         }
         if (PREFETCH && more) load_v(tok_next, tr);
+        }
 
         // S^T = K . Q^T for the two 16-token tiles, then refill the K registers
         f32x4 s[2][NT];
@@ -290,10 +319,38 @@ __device__ __forceinline__ void gqa_segment(const SweepParams& p, uint8_t* const
                     } else {
                         kfrag = tr.k[mt][ks];
                     }
-                    c = MM::mma(__builtin_bit_cast(vec8, kfrag), qf[nt][ks], c);
+                    if constexpr (VK) {  // (Q in accumulation registers: this form needs the ordinary ones for the K tile)
+                        if (ks == 0)
+                            MM::mma_bacc0(__builtin_bit_cast(vec8, kfrag), qf[nt][ks], c);
+                        else
+                            MM::mma_bacc(__builtin_bit_cast(vec8, kfrag), qf[nt][ks], c);
+                    } else
+                        c = MM::mma(__builtin_bit_cast(vec8, kfrag), qf[nt][ks], c);
                 }
+                if constexpr (VK) settle(c);
                 s[mt][nt] = c;
             }
+        if constexpr (VK) {
+            // the value columns of the tile, from the K registers: lane (n, g) holds 16-byte chunk ks * 4 + g of row
+            // mt * 16 + n (8-bit: elements [64 j + 16 g, +16) of it in register j)
+#pragma unroll
+            for (int mt = 0; mt < 2; ++mt) {
+                uint8_t* const row = vt + (mt * 16 + n) * VP;
+                if constexpr (KV8) {
+#pragma unroll
+                    for (int j = 0; j < DV / 64; ++j) {
+                        const uint4 w = tr.k[mt][j];
+                        *reinterpret_cast<uint4*>(row + j * 128 + g * 32) = kv8x8_to_16<Tag, KV8>(make_uint2(w.x, w.y));
+                        *reinterpret_cast<uint4*>(row + j * 128 + g * 32 + 16) =
+                            kv8x8_to_16<Tag, KV8>(make_uint2(w.z, w.w));
+                    }
+                } else {
+#pragma unroll
+                    for (int ks = 0; ks < DV / 32; ++ks)
+                        *reinterpret_cast<uint4*>(row + (ks * 4 + g) * 16) = tr.k[mt][ks];
+                }
+            }
+        }
         if (PREFETCH && more) load_k(tok_next, tr);
 
         // online softmax; token of s[mt][nt][r]: tok0 + mt*16 + g*4 + r, head nt*16 + n
@@ -365,7 +422,7 @@ __device__ __forceinline__ void gqa_segment(const SweepParams& p, uint8_t* const
         }
 
         if (!PREFETCH && more) {
-            load_v(tok_next, tr);
+            if constexpr (!VK) load_v(tok_next, tr);
             load_k(tok_next, tr);
         }
     }

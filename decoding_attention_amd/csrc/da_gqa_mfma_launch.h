@@ -11,10 +11,11 @@ namespace gqa_launch {
 
 template <typename Tag, int D, int NT, bool WH, int KV8, int PGM>
 hipError_t launch_form(const SweepParams& p, dim3 grid, hipStream_t stream) {
-    constexpr bool kPrefetch = D <= 128;
+    constexpr int DV = D == 576 ? 512 : D;  // (576, 512): the latent form, V inside the K rows
+    constexpr bool kPrefetch = D <= 128 || D == 576;
     constexpr int kMinWaves = (D <= 128 && (NT == 1 || D <= 64)) ? 2 : 1;
-    auto kern = gqa_mfma_kernel<Tag, D, D, NT, kPrefetch, WH, kMinWaves, KV8, PGM>;
-    const size_t lds = gqa_lds_bytes<D>(NT);
+    auto kern = gqa_mfma_kernel<Tag, D, DV, NT, kPrefetch, WH, kMinWaves, KV8, PGM>;
+    const size_t lds = gqa_lds_bytes<DV>(NT);
     if (lds > 48 * 1024) {
         static std::atomic<uint64_t> devices_done{0};
         const hipError_t attr_err = ensure_lds_limit(reinterpret_cast<const void*>(kern), lds, devices_done);
@@ -51,6 +52,9 @@ hipError_t launch_tag(const SweepParams& p, int dim, int heads_per_group, bool w
             return hipErrorInvalidValue;  // 8-bit loads pair up k-steps: head dims that are multiples of 64 only
         case 128: return launch_dim<Tag, 128, KV8>(p, heads_per_group, wh, grid, stream);
         case 256: return launch_dim<Tag, 256, KV8>(p, heads_per_group, wh, grid, stream);
+        case 576:  // the latent form with up to 16 query heads: one KV head, its tokens shared by the four waves
+            if (heads_per_group == 16 && !wh) return launch_one<Tag, 576, 1, false, KV8>(p, grid, stream);
+            return hipErrorInvalidValue;
         default: return hipErrorInvalidValue;
     }
 }

@@ -465,6 +465,43 @@ __global__ __launch_bounds__(64 * NWV) void mfma_latent_kernel(const SweepParams
     int buf = 0;       // 16-bit buffer that holds tile t
     int buf_next = KV8 ? 0 : NB - 1;  // buffer (FP8: stage) that receives tile t + AHEAD
     int stg_conv = 1;  // FP8: stage that holds tile t + 1
+    if constexpr (KV8 != 0) {
+        // 8-bit K with fewer than 32 NWV heads: the work-group keeps all its waves for the loads and the conversion;
+        // a wave without heads of its own runs only that part of every trip (the same loads, conversions and
+        // barriers as in the loop below) and is done.
+        if (nh == 0) {
+            for (int t = 0; t < ntiles; ++t) {
+            // stage of tile t+1 landed (tile t+2 may still be in flight); after the barrier every wave's share of it
+            // is in LDS, every wave has converted its share of tile t, and every wave is done with tile t-1
+            if (t + 2 < ntiles)
+                wait_vmcnt<NLW8>();
+            else
+                wait_vmcnt<0>();
+            __syncthreads();
+            if (t + 1 < ntiles) convert_stage(stg_conv, buf ^ 1);
+            stg_conv = (stg_conv == 2) ? 0 : stg_conv + 1;
+            // (the stage that held tile t was converted before the barrier: free for tile t+3)
+            if constexpr (PG) {
+                if (t + 3 < ntiles) issue_tile_pg(c0 + (t + 3) * kTile, rows_ahead, buf_next);
+                if (t + 4 < ntiles) rows_ahead = lookup_rows(c0 + (t + 4) * kTile);
+            } else {
+            if (t + 3 < ntiles) {
+                const int tk = c0 + (t + 3) * kTile;
+                const int64_t r0 = row_in_page(p, start, tk, page_ahead).k;
+                issue_tile(tk, r0, tk + 16 < c1 ? row_in_page(p, start, tk + 16, page_ahead1).k : r0, buf_next);
+            }
+            if (t + 4 < ntiles) {
+                const int tk = c0 + (t + 4) * kTile;
+                page_ahead = page_of(p, b, tk);
+                if (tk + 16 < c1) page_ahead1 = page_of(p, b, tk + 16);
+            }
+            }
+                buf = (buf == NTB - 1) ? 0 : buf + 1;
+                buf_next = (buf_next == kNBuf - 1) ? 0 : buf_next + 1;
+            }
+            return;
+        }
+    }
     for (int t = 0; t < ntiles; ++t) {
         if constexpr (KV8) {
             // stage of tile t+1 landed (tile t+2 may still be in flight); after the barrier every wave's share of it

@@ -109,7 +109,8 @@ size_t da_workspace_bytes_paged(size_t max_seq_k, size_t batch, size_t head_q, s
  *                      path; k_scale is folded into the softmax scale and v_scale into the final normalisation,
  *                      both in fp32.
  * v8 == NULL means V is the first dim_v columns of each K row.  Head dims (64,64), (128,128), (256,256) run on
- * the grouped MFMA kernel and (576,512) with v8 == NULL on the latent MFMA kernel, as the 16-bit forms do; (96,96)
+ * the grouped MFMA kernel and (576,512) with v8 == NULL on the latent MFMA kernel (up to 16 query heads: on the
+ * grouped kernel), as the 16-bit forms do; (96,96)
  * runs on the VALU sweep.  Workspace size from da_workspace_bytes_fp8kv (page_size 0 = packed layout).
  */
 int da_decoding_attn_fp8kv(const void *q, const void *k8, const void *v8, void *o, const int32_t *cu_seq_k,
@@ -155,7 +156,8 @@ size_t da_workspace_bytes_int8kv(size_t max_seq_k, size_t batch, size_t head_q, 
 
 /*
  * Launch plan the library would use for this shape, for tests and benchmarks:
- *   kernel_kind 1 = VALU sweep, 2 = latent (MLA) MFMA sweep, 3 = grouped-head MFMA sweep; nsplit = sequence splits;
+ *   kernel_kind 1 = VALU sweep, 2 = latent (MLA) MFMA sweep, 3 = grouped-head MFMA sweep (also the latent form with
+ *   16 query heads or fewer); nsplit = sequence splits;
  *   chunk = tokens per split; heads_per_group = query heads one work-group serves; total_k as for
  *   da_decoding_attn_ex (0 = unknown).
  * Any output pointer may be NULL.  Returns DA_ERR_UNSUPPORTED for an unsupported (dim, dim_v).

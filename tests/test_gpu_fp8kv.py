@@ -109,7 +109,8 @@ def test_latent_form_with_fp8_cache(batch, head_q, seq_k, dtype, is_alibi):
     """(576, 512) with V = K[..., :512]: the latent MFMA kernel over FP8 tiles converted in LDS (one scale for K
     and V, as they are one buffer)."""
     w, k8, _, ks, _ = _case(batch, head_q, 1, 576, 512, seq_k, dtype, latent=True, is_alibi=is_alibi, seed=seq_k)
-    assert _lib.plan(w.max_seq_k, batch, head_q, 1, 576, 512)["kind"] == 2
+    # (up to 16 heads: the grouped kernel's latent form; above: the latent kernel)
+    assert _lib.plan(w.max_seq_k, batch, head_q, 1, 576, 512)["kind"] == (3 if head_q <= 16 else 2)
     o = decoding_attn_fwd(w.q.to(DEV), k8.to(DEV), None, w.cu_seq_k.to(DEV), w.max_seq_k, 512, is_alibi,
                           k_scale=ks.to(DEV), v_scale=ks.to(DEV)).cpu()
     ref = torch.from_numpy(_reference(w, k8, None, ks, ks)).float()
