@@ -232,8 +232,9 @@ Plan make_plan(size_t max_seq_k, size_t batch, size_t head_q, size_t head_k, siz
         // a work-group and with at most 32 partials to merge (measured, 32/8 heads d 128: batch 1 x 4096 tokens
         // 20.1 -> 15.7 us, batch 4 x 1024 18.9 -> 13.4, batch 16 x 1024 21.1 -> 18.2; 16/8 heads d 256: batch 1 x
         // 2048 29.1 -> 15.5).  Below 512 tokens at d < 128 the second launch costs more than the split saves, and
-        // where four waves share one KV head's tokens the finer split changes nothing.
-        if (pl.kind == kKindGroup && pl.wave_per_head && (max_seq_k >= 512 || dim >= 128) &&
+        // where four waves share one KV head's tokens the finer split changes nothing, except in the latent form
+        // (long rows: 16 heads, batch 1 x 4096 tokens 20.0 -> 17.0 us with 128-token splits, one tile per wave).
+        if (pl.kind == kKindGroup && (pl.wave_per_head || latent_group) && (max_seq_k >= 512 || dim >= 128) &&
             base * std::max<long long>(1, (long long)max_seq_k / 256) < tun().group_small_wgs) {
             const int by_partials = (int)(((long long)max_seq_k + 31) / 32 + trip - 1) / trip * trip;
             min_chunk = std::max(std::min(min_chunk, std::max(tun().group_small_chunk, by_partials)), trip);

@@ -110,8 +110,7 @@ size_t da_workspace_bytes_paged(size_t max_seq_k, size_t batch, size_t head_q, s
  *                      both in fp32.
  * v8 == NULL means V is the first dim_v columns of each K row.  Head dims (64,64), (128,128), (256,256) run on
  * the grouped MFMA kernel and (576,512) with v8 == NULL on the latent MFMA kernel (up to 16 query heads: on the
- * grouped kernel), as the 16-bit forms do; (96,96)
- * runs on the VALU sweep.  Workspace size from da_workspace_bytes_fp8kv (page_size 0 = packed layout).
+ * grouped kernel), as the 16-bit forms do; (96,96) runs on the VALU sweep.  Workspace size from da_workspace_bytes_fp8kv (page_size 0 = packed layout).
  */
 int da_decoding_attn_fp8kv(const void *q, const void *k8, const void *v8, void *o, const int32_t *cu_seq_k,
                            size_t max_seq_k, size_t batch, size_t head_q, size_t head_k, size_t dim, size_t dim_v,
