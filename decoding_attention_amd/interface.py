@@ -39,6 +39,15 @@ def maybe_contiguous(x):
     return x.contiguous() if x is not None and not x.is_contiguous() else x
 
 
+def is_leading_columns_view(v, k) -> bool:
+    """True when v is a view of k's own memory that selects the leading columns of every row, as
+    `k[..., :dim_v]` does: the values are then read out of the K rows (v = None), which is what the latent form's
+    fast kernels need, instead of from a copy."""
+    return (v is not None and v.dtype == k.dtype and v.device == k.device and v.dim() == k.dim() and
+            v.shape[:-1] == k.shape[:-1] and v.shape[-1] <= k.shape[-1] and v.stride() == k.stride() and
+            v.data_ptr() == k.data_ptr())
+
+
 def fwd(q: torch.Tensor, k: torch.Tensor, v_: Optional[torch.Tensor], o_: Optional[torch.Tensor],
         cu_seq_k: torch.Tensor, max_seq_k: int, dim_v: int, is_alibi: bool, *,
         softmax_scale: Optional[float] = None, alibi_slopes: Optional[torch.Tensor] = None,
@@ -69,6 +78,8 @@ def decoding_attn_fwd(q: torch.Tensor, k: torch.Tensor, v: Optional[torch.Tensor
     Return:
         o: [total_q, head_q, dim_v], same dtype as q.
     """
+    if is_leading_columns_view(v, k) and v.shape[-1] == dim_v:
+        v = None  # (the reference's callers pass None themselves: tests/test_decoding_attn.py:45 builds this view)
     q, k, v = [maybe_contiguous(x) for x in (q, k, v)]
     return fwd(q, k, v, None, cu_seq_k, max_seq_k, dim_v, is_alibi, softmax_scale=softmax_scale,
                alibi_slopes=alibi_slopes, k_scale=k_scale, v_scale=v_scale)
@@ -98,6 +109,8 @@ def decoding_attn_paged_fwd(q: torch.Tensor, k_pages: torch.Tensor, v_pages: Opt
         o: [batch, head_q, dim_v], same dtype as q.
     """
     q = maybe_contiguous(q)
+    if is_leading_columns_view(v_pages, k_pages) and v_pages.shape[-1] == dim_v:
+        v_pages = None
     return _extension().fwd_paged(q, k_pages, v_pages, out, block_table, seq_lens, int(max_seq_k), int(dim_v),
                                   bool(is_alibi), None if softmax_scale is None else float(softmax_scale),
                                   alibi_slopes, int(total_k), k_scale, v_scale)

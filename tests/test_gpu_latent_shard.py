@@ -83,3 +83,16 @@ def test_ragged_batch_with_token_count_takes_the_balanced_grid():
     for b, n in enumerate(lens):
         if n == 0:
             assert torch.count_nonzero(o[b]) == 0
+
+
+@pytest.mark.parametrize("head_q", [16, 128])
+def test_value_passed_as_a_view_of_the_key_rows(head_q):
+    """`v = k[..., :512]` is the aliasing the latent kernels are built on: same bits as v = None, not a copy that
+    would take the slow path for a distinct V buffer."""
+    w = _latent(3, head_q, 900, torch.float16, seed=44)
+    q, k, cu = w.q.to(DEV), w.k.to(DEV), w.cu_seq_k.to(DEV)
+    o_none = decoding_attn_fwd(q, k, None, cu, w.max_seq_k, 512, False)
+    o_view = decoding_attn_fwd(q, k, k[..., :512], cu, w.max_seq_k, 512, False)
+    assert torch.equal(o_none.view(torch.int16), o_view.view(torch.int16))
+    o_copy = decoding_attn_fwd(q, k, k[..., :512].contiguous(), cu, w.max_seq_k, 512, False)  # a distinct buffer
+    assert (o_copy.float() - o_none.float()).abs().max().item() <= 2 ** -10

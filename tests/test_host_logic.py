@@ -124,6 +124,18 @@ def test_python_face_checks_cpu_inputs():
         interface.fwd(w.q, w.k, None, None, w.cu_seq_k.long(), 8, 64, False)
 
 
+def test_value_view_of_the_key_rows_is_recognised():
+    """`k[..., :dim_v]` passed as v is the latent form's aliasing: it must not be copied into a buffer of its own."""
+    k = torch.randn(10, 1, 576).to(torch.float16)
+    assert interface.is_leading_columns_view(k[..., :512], k)
+    assert interface.is_leading_columns_view(k, k)
+    assert not interface.is_leading_columns_view(k[..., :512].contiguous(), k)
+    assert not interface.is_leading_columns_view(k[..., 64:], k)          # not the leading columns
+    assert not interface.is_leading_columns_view(k[1:, :, :512], k[1:].clone())
+    assert not interface.is_leading_columns_view(None, k)
+    assert not interface.is_leading_columns_view(k[::2, :, :512], k)       # other rows
+
+
 def test_drop_in_package_name():
     import decoding_attn
 
