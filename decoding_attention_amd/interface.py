@@ -43,9 +43,10 @@ def is_leading_columns_view(v, k) -> bool:
     """True when v is a view of k's own memory that selects the leading columns of every row, as
     `k[..., :dim_v]` does: the values are then read out of the K rows (v = None), which is what the latent form's
     fast kernels need, instead of from a copy."""
-    return (v is not None and v.dtype == k.dtype and v.device == k.device and v.dim() == k.dim() and
-            v.shape[:-1] == k.shape[:-1] and v.shape[-1] <= k.shape[-1] and v.stride() == k.stride() and
-            v.data_ptr() == k.data_ptr())
+    # (the address comparison first: it settles the ordinary case, a V buffer of its own, at once)
+    return (v is not None and v.data_ptr() == k.data_ptr() and v.dtype == k.dtype and v.device == k.device and
+            v.dim() == k.dim() and v.shape[:-1] == k.shape[:-1] and v.shape[-1] <= k.shape[-1] and
+            v.stride() == k.stride())
 
 
 def fwd(q: torch.Tensor, k: torch.Tensor, v_: Optional[torch.Tensor], o_: Optional[torch.Tensor],
