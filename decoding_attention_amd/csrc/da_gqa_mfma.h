@@ -105,9 +105,10 @@ constexpr size_t gqa_lds_bytes(int nt) {
 // Otherwise (head_k not a multiple of 4) the wavefronts split the tokens of one KV head and merge at the end.
 // MINW: wavefronts per SIMD the register allocation must leave room for (2 caps the kernel at 256 registers
 // and keeps the accumulators in ordinary VGPRs, so the rescale needs no accumulation-register copies).
-// KV8: K and V hold 8-bit elements (1 = FP8 e4m3, 2 = int8; 0 = 16-bit K/V).  Loads stay 16 bytes per lane (sixteen elements: the k indices of two
-// consecutive k-steps, so the Q fragments are gathered with the matching index order) and the elements are
-// converted exactly to the compute type on their way into the matrix instruction (K) or the LDS tile (V).
+// KV8: K and V hold 8-bit elements (1 = FP8 e4m3, 2 = int8; 0 = 16-bit K/V).  Loads stay 16 bytes per lane
+// (sixteen elements: the k indices of two consecutive k-steps, so the Q fragments are gathered with the matching
+// index order) and the elements are converted exactly to the compute type on their way into the matrix instruction
+// (K) or the LDS tile (V).
 // One segment of work: tokens [c0, c1) of sequence b (first row `start`, `len` tokens) for the KV heads and head
 // group blockIdx.y selects.  `direct`: the segment is the whole sequence, so the result goes to o; otherwise the
 // un-normalised partial goes to workspace slot `split` of the sequence.
@@ -254,7 +255,8 @@ __device__ __forceinline__ void gqa_segment(const SweepParams& p, uint8_t* const
             for (int i = 0; i < NVR; ++i) {
                 const int slot = i * 64 + lane;
                 const int row = slot / CPRL, ch = slot % CPRL;
-                r.v[i] = *reinterpret_cast<const uint4*>(lane_row(tok0, min(row, last), vbytes, p.v_page, v_row_b) + ch * 16);
+                r.v[i] = *reinterpret_cast<const uint4*>(lane_row(tok0, min(row, last), vbytes, p.v_page, v_row_b) +
+                                                         ch * 16);
             }
             return;
         }
@@ -319,7 +321,7 @@ __device__ __forceinline__ void gqa_segment(const SweepParams& p, uint8_t* const
                     } else {
                         kfrag = tr.k[mt][ks];
                     }
-                    if constexpr (VK) {  // (Q in accumulation registers: this form needs the ordinary ones for the K tile)
+                    if constexpr (VK) {  // (Q in accumulation registers: the ordinary ones hold the K tile)
                         if (ks == 0)
                             MM::mma_bacc0(__builtin_bit_cast(vec8, kfrag), qf[nt][ks], c);
                         else
@@ -559,7 +561,8 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(MINW))) voi
         const int stride = (n + 63) >> 6;
         const int idx = lo + (int)(threadIdx.x & 63) * stride;
         const bool below = idx < lo + n && cu[idx] <= r0;
-        const int k = __popcll(__ballot(below)) - 1;  // probes are sorted: the lanes that hold are a prefix, lane 0 among them
+        // probes are sorted: the lanes that hold are a prefix, lane 0 among them
+        const int k = __popcll(__ballot(below)) - 1;
         lo += k * stride;
         n = min(stride, n - k * stride);
     }
