@@ -147,8 +147,11 @@ Plan make_plan(size_t max_seq_k, size_t batch, size_t head_q, size_t head_k, siz
         pl.kind = kKindMfma;
         pl.rt = da::mla_heads_per_group(ratio);
         // few sequences and short ones cannot fill the chip even at the finest split: then two work-groups of 64
-        // heads per (sequence, split) beat one of 128 (measured: batch 1, seq 4096: 35 -> 31 us)
-        if (pl.rt == 128 && (long long)batch * (long long)(max_seq_k / 256) <= 128) pl.rt = 64;
+        // heads per (sequence, split) beat one of 128 (measured: batch 1, seq 4096: 35 -> 31 us).  The same holds for
+        // up to four long sequences (batch 1 x 65536 tokens 64.2 -> 55.7 us, batch 2 x 32768 63.7 -> 56.3, batch 4 x
+        // 16384 63.5 -> 56.8; batch 8 x 8192 and larger batches lose, 53.2 -> 57.6).
+        const long long tiles256 = (long long)batch * (long long)(max_seq_k / 256);
+        if (pl.rt == 128 && (tiles256 <= 128 || (batch <= 4 && tiles256 <= 512))) pl.rt = 64;
         if ((tun().mla_heads == 32 || tun().mla_heads == 64 || tun().mla_heads == 128) && tun().mla_heads <= 128 &&
             tun().mla_heads >= 32)
             pl.rt = std::min(tun().mla_heads, da::mla_heads_per_group(ratio));
