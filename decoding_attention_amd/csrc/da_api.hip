@@ -44,7 +44,7 @@ int env_int(const char* name, int dflt) {
 struct Tunables {
     int target_wgs, mfma_target_wgs, max_chunk, min_chunk, ragged_chunk, force_kind, group_min_ratio, wave_per_head,
         mla_heads, gqa_heads, flat_wgs, flat_min_tokens, flat_paged_min_mb, nsplit, mfma_small_wgs, group_small_wgs,
-        group_small_chunk, mla_group_heads;
+        group_small_chunk, mla_group_heads, mla_group_small;
     Tunables() {
         target_wgs = env_int("DA_TARGET_WGS", 512);
         mfma_target_wgs = env_int("DA_MFMA_TARGET_WGS", 256);
@@ -60,6 +60,8 @@ struct Tunables {
         mfma_small_wgs = env_int("DA_MFMA_SMALL_WGS", 256);  // latent kernel: below this many 256-token splits, split finer
         // latent form: up to this many query heads take the grouped kernel (0 = never)
         mla_group_heads = env_int("DA_MLA_GROUP_HEADS", 16);
+        // ... and any head count while groups x batch x max_seq_k stays within this (twice this for two groups)
+        mla_group_small = env_int("DA_MLA_GROUP_SMALL", 65536);
         group_small_wgs = env_int("DA_GROUP_SMALL_WGS", 256);  // grouped kernel: likewise
         group_small_chunk = env_int("DA_GROUP_SMALL_CHUNK", 64);
         nsplit = env_int("DA_NSPLIT", 0);  // sequence splits, 0 = by shape (experiments)
@@ -133,8 +135,16 @@ Plan make_plan(size_t max_seq_k, size_t batch, size_t head_q, size_t head_k, siz
     // bytes in flight per CU than the latent kernel's one-wave form can (its tiles need LDS landing space)
     // (an 8-bit cache: up to twice as many, as two groups that read the same rows; the latent kernel's single
     // computing wave is the slower there: FP8, 32 heads, batch 64 x 4096 tokens 96 -> 60 us)
+    // Small problems of any head count go there as well, as ceil(heads / 16) groups per sequence that read the same
+    // rows: the latent kernel's work-groups pay ~6 us to stage Q before their first tile, which a few tiles do not
+    // win back (measured, 128 heads: batch 1 x 8192 tokens 34.4 -> 24.8 us, batch 16 x 512 29.8 -> 23.4; 32 heads:
+    // batch 1 x 16384 33.4 -> 23.0; past the bound below the re-read rows cost more than the staging).
+    const long long groups16 = (ratio + 15) / 16;
+    const long long group_rows = groups16 * (long long)batch * (long long)max_seq_k;
+    const bool latent_small =
+        tun().mla_group_heads > 0 && group_rows <= (groups16 <= 2 ? 2 : 1) * (long long)tun().mla_group_small;
     const bool latent_group = latent && !force_sweep &&
-                              ratio <= (kv_8bit ? 2 * tun().mla_group_heads : tun().mla_group_heads);
+                              (ratio <= (kv_8bit ? 2 * tun().mla_group_heads : tun().mla_group_heads) || latent_small);
     const bool mfma = latent && !force_sweep && !latent_group;
     if (latent_group) {
         pl.kind = kKindGroup;

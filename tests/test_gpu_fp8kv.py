@@ -109,8 +109,6 @@ def test_latent_form_with_fp8_cache(batch, head_q, seq_k, dtype, is_alibi):
     """(576, 512) with V = K[..., :512]: the latent MFMA kernel over FP8 tiles converted in LDS (one scale for K
     and V, as they are one buffer)."""
     w, k8, _, ks, _ = _case(batch, head_q, 1, 576, 512, seq_k, dtype, latent=True, is_alibi=is_alibi, seed=seq_k)
-    # (up to 16 heads: the grouped kernel's latent form; above: the latent kernel)
-    assert _lib.plan(w.max_seq_k, batch, head_q, 1, 576, 512)["kind"] == (3 if head_q <= 16 else 2)
     o = decoding_attn_fwd(w.q.to(DEV), k8.to(DEV), None, w.cu_seq_k.to(DEV), w.max_seq_k, 512, is_alibi,
                           k_scale=ks.to(DEV), v_scale=ks.to(DEV)).cpu()
     ref = torch.from_numpy(_reference(w, k8, None, ks, ks)).float()
@@ -120,7 +118,9 @@ def test_latent_form_with_fp8_cache(batch, head_q, seq_k, dtype, is_alibi):
 def test_latent_fp8_unit_scales_equal_the_16_bit_call_bit_for_bit():
     """FP8 values convert exactly and the tiles are converted before any arithmetic: with unit scales the FP8 call
     is the 16-bit call on the same values, same kernel, same order of operations."""
-    w, k8, _, ks, _ = _case(4, 128, 1, 576, 512, 1200, torch.float16, latent=True, unit=True, seed=9)
+    # (large enough for the planner to pick the latent kernel, whose property this is)
+    w, k8, _, ks, _ = _case(6, 128, 1, 576, 512, 3000, torch.float16, latent=True, unit=True, seed=9)
+    assert _lib.plan(w.max_seq_k, 6, 128, 1, 576, 512)["kind"] == 2
     k16 = k8.to(torch.float16).to(DEV)
     args = (w.cu_seq_k.to(DEV), w.max_seq_k, 512, False)
     o8 = decoding_attn_fwd(w.q.to(DEV), k8.to(DEV), None, *args, k_scale=ks.to(DEV), v_scale=ks.to(DEV))
