@@ -159,6 +159,8 @@ size_t da_workspace_bytes_int8kv(size_t max_seq_k, size_t batch, size_t head_q, 
  *   16 query heads or fewer); nsplit = sequence splits;
  *   chunk = tokens per split; heads_per_group = query heads one work-group serves; total_k as for
  *   da_decoding_attn_ex (0 = unknown).
+ * The plan is that of the 16-bit packed call (V inside K for (576, 512)); paged and 8-bit calls may be planned
+ * differently.
  * Any output pointer may be NULL.  Returns DA_ERR_UNSUPPORTED for an unsupported (dim, dim_v).
  * Mirrors the role of the reference's per-head-dim tile choice (csrc/kernel/decoding_attn/decoding_fwd_hd*.cu).
  */
