@@ -96,3 +96,13 @@ def test_value_passed_as_a_view_of_the_key_rows(head_q):
     assert torch.equal(o_none.view(torch.int16), o_view.view(torch.int16))
     o_copy = decoding_attn_fwd(q, k, k[..., :512].contiguous(), cu, w.max_seq_k, 512, False)  # a distinct buffer
     assert (o_copy.float() - o_none.float()).abs().max().item() <= 2 ** -10
+
+
+@pytest.mark.parametrize("head_q", [20, 40, 100, 128])
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+def test_small_problems_of_any_head_count_as_groups_of_16(head_q, dtype):
+    """Small latent problems run on the grouped kernel whatever the head count, ceil(heads / 16) groups per sequence,
+    the last one partly idle when 16 does not divide the head count."""
+    w = _latent(3, head_q, 700, dtype, seed=head_q, is_alibi=head_q == 40)
+    assert _lib.plan(w.max_seq_k, 3, head_q, 1, 576, 512)["kind"] == 3
+    check_against_oracle(w, run_hip(w))
