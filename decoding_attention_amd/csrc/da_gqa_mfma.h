@@ -110,15 +110,15 @@ constexpr size_t gqa_lds_bytes(int nt) {
 // index order) and the elements are converted exactly to the compute type on their way into the matrix instruction
 // (K) or the LDS tile (V).
 // One segment of work: tokens [c0, c1) of sequence b (first row `start`, `len` tokens) for the KV heads and head
-// group blockIdx.y selects.  `direct`: the segment is the whole sequence, so the result goes to o; otherwise the
+// group `by` selects (blockIdx.y, or its renumbered stand-in).  `direct`: the segment is the whole sequence, so the result goes to o; otherwise the
 // un-normalised partial goes to workspace slot `split` of the sequence.
 // PGM: how paged K/V is addressed.  0: one page lookup per tile (pages hold a multiple of 32 tokens; also the packed
 // layout); 1: 16-token pages, a tile is fetched as two runs of 16 tokens, each from one page; 2: smaller pages, every
 // lane looks up the page of the row it loads.
 template <typename Tag, int D, int DV, int NT, bool PREFETCH, bool WH, int KV8, int PGM>
-__device__ __forceinline__ void gqa_segment(const SweepParams& p, uint8_t* const smem, const int b, const int start,
-                                            const int len, const int c0, const int c1, const int split,
-                                            const bool direct) {
+__device__ __forceinline__ void gqa_segment(const SweepParams& p, uint8_t* const smem, const int by, const int b,
+                                            const int start, const int len, const int c0, const int c1,
+                                            const int split, const bool direct) {
     using MM = Mma16<Tag>;
     using vec8 = typename MM::vec8;
     using EL = Elem<Tag>;
@@ -145,8 +145,8 @@ __device__ __forceinline__ void gqa_segment(const SweepParams& p, uint8_t* const
     const int n = lane & 15;
     const int g = lane >> 4;
 
-    const int hk = WH ? (blockIdx.y / p.groups) * 4 + wave : blockIdx.y / p.groups;
-    const int grp = blockIdx.y % p.groups;
+    const int hk = WH ? (by / p.groups) * 4 + wave : by / p.groups;
+    const int grp = by % p.groups;
     const int tw = WH ? 0 : wave;  // this wave's position among the waves that share the tokens
 
     const int h_base = hk * p.ratio + grp * HG;
@@ -157,7 +157,7 @@ __device__ __forceinline__ void gqa_segment(const SweepParams& p, uint8_t* const
         // every wave of the work-group sees the same (sequence, split), so they all leave together; the
         // work-group covers NR runs of nh heads, one per KV head
         constexpr int NR = WH ? 4 : 1;
-        const int wg_h_first = (WH ? (blockIdx.y / p.groups) * 4 : hk) * p.ratio + grp * HG;
+        const int wg_h_first = (WH ? (by / p.groups) * 4 : hk) * p.ratio + grp * HG;
         if (direct) zero_rows<DV>(p, b, wg_h_first, nh, NR, p.ratio);
         return;
     }
@@ -539,12 +539,27 @@ template <typename Tag, int D, int DV, int NT, bool PREFETCH, bool WH, int MINW,
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(MINW))) void gqa_mfma_kernel(const SweepParams p) {
     extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
     if (p.flat_tokens == 0) {
-        const int split = blockIdx.x, b = blockIdx.z;
+        int split = blockIdx.x, by = blockIdx.y, b = blockIdx.z;
+        // Several head groups per KV head read the same K/V rows.  Work-groups go to the eight XCDs round-robin by
+        // linear id, and each XCD has its own L2: renumber so that the groups of one (sequence, KV heads, split) are
+        // neighbours on one XCD, and the rows leave HBM once for all of them.
+        const int total = (int)(gridDim.x * gridDim.y * gridDim.z);
+        if (p.groups > 1 && total % (8 * p.groups) == 0) {
+            const int lin = (int)(blockIdx.x + gridDim.x * (blockIdx.y + gridDim.y * blockIdx.z));
+            const int slot = lin >> 3;
+            const int grp = slot % p.groups;
+            int rest = (slot / p.groups) * 8 + (lin & 7);  // index over (split, KV heads, sequence)
+            const int nky = (int)gridDim.y / p.groups;
+            split = rest % (int)gridDim.x;
+            rest /= (int)gridDim.x;
+            by = (rest % nky) * p.groups + grp;
+            b = rest / nky;
+        }
         int start, len;
         seq_range(p, b, start, len);
         const int c0 = split * p.chunk;
         const int c1 = (split == p.nsplit - 1) ? len : min(len, c0 + p.chunk);
-        gqa_segment<Tag, D, DV, NT, PREFETCH, WH, KV8, PGM>(p, smem, b, start, len, c0, c1, split, p.nsplit == 1);
+        gqa_segment<Tag, D, DV, NT, PREFETCH, WH, KV8, PGM>(p, smem, by, b, start, len, c0, c1, split, p.nsplit == 1);
         return;
     }
     const int T = p.flat_tokens, W = (int)gridDim.x, i = (int)blockIdx.x, unit = p.flat_unit;
@@ -574,7 +589,8 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(MINW))) voi
         seq_range(p, b, start, len);
         const int first = min(s / T, W - 1), last = min((e - 1) / T, W - 1);
         const int c0 = (max(r0, s) - s) * unit, c1 = min((min(r1, e) - s) * unit, len);
-        gqa_segment<Tag, D, DV, NT, PREFETCH, WH, KV8, PGM>(p, smem, b, start, len, c0, c1, i - first, first == last);
+        gqa_segment<Tag, D, DV, NT, PREFETCH, WH, KV8, PGM>(p, smem, (int)blockIdx.y, b, start, len, c0, c1, i - first,
+                                                            first == last);
         if (!WH) __syncthreads();  // the merge area of this segment is the V tile area of the next
     }
 }
