@@ -259,11 +259,20 @@ Plan make_plan(size_t max_seq_k, size_t batch, size_t head_q, size_t head_k, siz
         if (ragged) min_chunk = std::max(std::min(min_chunk, tun().ragged_chunk), trip);
     }
     long long want = base > 0 ? (target_wgs + base - 1) / base : 1;
+    // The latent forms hold one work-group per CU (two for the latent kernel's one- and two-wave forms over 16-bit
+    // K, for which the target is doubled): a grid a little over that capacity would run as two rounds, the second
+    // nearly empty, so round down there (measured: 48 heads, batch 64 x 256 tokens, 384 work-groups 33.6 us, 192
+    // work-groups 19.1 us; 128 heads, batch 100 x 4096 tokens, 300 work-groups 247 us, 200 work-groups 198 us; batch
+    // 40 x 8192, 280 work-groups 209 us, 240 work-groups 146 us; 16 heads, batch 150 x 4096, 300 work-groups 183 us,
+    // 150 work-groups 153 us).
+    if ((latent_group || mfma) && base > 0) want = std::max<long long>(1, target_wgs / base);
     const long long by_len = std::max<long long>(1, (long long)max_seq_k / min_chunk);
     // sweep work-groups are also kept short (shorter still for a ragged batch); the latent MFMA kernel's partials
     // are too large (heads x dim_v floats per split) to split more than occupancy asks for
     const int max_chunk = std::max(1, ragged ? tun().ragged_chunk : tun().max_chunk * max_chunk_scale);
     long long by_cap = mfma ? 1 : ((long long)max_seq_k + max_chunk - 1) / max_chunk;
+    // (one round of long splits beats two rounds with the second nearly empty)
+    if (latent_group && base <= target_wgs && base * by_cap > target_wgs) by_cap = 1;
     long long ns = std::max(std::min(want, by_len), std::min(by_cap, by_len));
     ns = std::max<long long>(1, std::min<long long>(ns, kMaxSplits));
     if (tun().nsplit > 0) ns = std::min<long long>(tun().nsplit, kMaxSplits);
