@@ -44,7 +44,7 @@ int env_int(const char* name, int dflt) {
 struct Tunables {
     int target_wgs, mfma_target_wgs, max_chunk, min_chunk, ragged_chunk, force_kind, group_min_ratio, wave_per_head,
         mla_heads, gqa_heads, flat_wgs, flat_min_tokens, flat_paged_min_mb, nsplit, mfma_small_wgs, group_small_wgs,
-        group_small_chunk, mla_group_heads, mla_group_small;
+        group_small_chunk, mla_group_heads, mla_group_small, fill_rounds;
     Tunables() {
         target_wgs = env_int("DA_TARGET_WGS", 512);
         mfma_target_wgs = env_int("DA_MFMA_TARGET_WGS", 256);
@@ -62,6 +62,7 @@ struct Tunables {
         mla_group_heads = env_int("DA_MLA_GROUP_HEADS", 16);
         // ... and any head count while groups x batch x max_seq_k stays within this (twice this for two groups)
         mla_group_small = env_int("DA_MLA_GROUP_SMALL", 65536);
+        fill_rounds = env_int("DA_FILL_ROUNDS", 1);  // grouped kernel: re-plan grids that fill their last round of CUs poorly
         group_small_wgs = env_int("DA_GROUP_SMALL_WGS", 256);  // grouped kernel: likewise
         group_small_chunk = env_int("DA_GROUP_SMALL_CHUNK", 64);
         nsplit = env_int("DA_NSPLIT", 0);  // sequence splits, 0 = by shape (experiments)
@@ -275,6 +276,33 @@ Plan make_plan(size_t max_seq_k, size_t batch, size_t head_q, size_t head_k, siz
     if (latent_group && base <= target_wgs && base * by_cap > target_wgs) by_cap = 1;
     long long ns = std::max(std::min(want, by_len), std::min(by_cap, by_len));
     ns = std::max<long long>(1, std::min<long long>(ns, kMaxSplits));
+    // The grouped kernel's grids and the 256 CUs: work-groups are handed out as CUs free up, so a grid that is not
+    // close to a multiple of the CU count ends with most of the chip idle while a few CUs finish (and up to 256
+    // work-groups run one per CU, which saturates HBM from about 200).  When the plan above fills its last round of
+    // 256 poorly, take the split count that fills it best instead (fewer splits on a tie).  Measured, 32/8 heads d
+    // 128, 4096 tokens: batch 40, 7 splits (560 work-groups) 138.6 us, 3 splits (240) 117.9; batch 48, 6 splits (576)
+    // 158.8, 5 splits (480) 142.4; batch 100, 4 splits (800) 320.5, 1 split (200) 284.8.
+    // (d >= 128: at d = 64 a work-group streams half the bytes per token and the same re-planning loses as often as
+    // it wins)
+    if (pl.kind == kKindGroup && dim >= 128 && dim <= 256 && tun().fill_rounds) {
+        auto fill = [&](long long c) {
+            const double w = (double)(base * c);
+            if (w <= 256.0) return std::min(1.0, w / 200.0);
+            return w / (std::ceil(w / 256.0) * 256.0);
+        };
+        if (fill(ns) < 0.85) {
+            long long best_ns = ns;
+            double best = fill(ns) - 0.004 * (double)ns;
+            for (long long c = 1; c <= std::min<long long>(by_len, 64); ++c) {
+                const double score = fill(c) - 0.004 * (double)c;
+                if (score > best + 1e-9) {
+                    best = score;
+                    best_ns = c;
+                }
+            }
+            ns = best_ns;
+        }
+    }
     if (tun().nsplit > 0) ns = std::min<long long>(tun().nsplit, kMaxSplits);
     long long chunk = ((long long)max_seq_k + ns - 1) / ns;
     chunk = (chunk + trip - 1) / trip * trip;
