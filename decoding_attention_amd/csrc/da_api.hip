@@ -282,13 +282,15 @@ Plan make_plan(size_t max_seq_k, size_t batch, size_t head_q, size_t head_k, siz
     // 256 poorly, take the split count that fills it best instead (fewer splits on a tie).  Measured, 32/8 heads d
     // 128, 4096 tokens: batch 40, 7 splits (560 work-groups) 138.6 us, 3 splits (240) 117.9; batch 48, 6 splits (576)
     // 158.8, 5 splits (480) 142.4; batch 100, 4 splits (800) 320.5, 1 split (200) 284.8.
-    // (d >= 128: at d = 64 a work-group streams half the bytes per token and the same re-planning loses as often as
-    // it wins)
-    if (pl.kind == kKindGroup && dim >= 128 && dim <= 256 && tun().fill_rounds) {
+    // (not at d = 96, where the re-planning loses as often as it wins)
+    if (pl.kind == kKindGroup && dim != 96 && dim <= 256 && tun().fill_rounds) {
+        // (at d = 64 a work-group streams too few bytes for one per CU to saturate HBM: rounds of two per CU there;
+        // 32/8 heads, batch 56 x 4096 tokens 100.1 -> 84.9 us, 32/4 heads, batch 150 x 4096 127.2 -> 112.3)
+        const double gran = dim >= 128 ? 256.0 : 512.0, sat = dim >= 128 ? 200.0 : 400.0;
         auto fill = [&](long long c) {
             const double w = (double)(base * c);
-            if (w <= 256.0) return std::min(1.0, w / 200.0);
-            return w / (std::ceil(w / 256.0) * 256.0);
+            if (w <= gran) return std::min(1.0, w / sat);
+            return w / (std::ceil(w / gran) * gran);
         };
         if (fill(ns) < 0.85) {
             long long best_ns = ns;
