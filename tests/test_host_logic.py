@@ -68,13 +68,14 @@ def test_plan_is_consistent(d, dv, batch, sk):
     assert ws >= need if d == 576 else ws == need
 
 
-def test_plan_total_k_hint_only_changes_the_splits_of_ragged_batches():
-    """The token-count hint changes how a ragged batch is cut, and never the kernel kind."""
+def test_plan_total_k_hint_changes_the_splits_and_never_the_kernel():
+    """The token-count hint changes how a batch is cut (a ragged one into equal shares, one known to be uniform
+    into splits that may be longer), and never the kernel kind."""
     sk, batch = 8192, 64
     base = _lib.plan(sk, batch, 32, 8, 128, 128)
     full = _lib.plan(sk, batch, 32, 8, 128, 128, total_k=batch * sk)
     ragged = _lib.plan(sk, batch, 32, 8, 128, 128, total_k=batch * sk // 2)
-    assert full == base
+    assert full["kind"] == base["kind"] and full["chunk"] >= base["chunk"] and full["nsplit"] <= base["nsplit"]
     # grouped kernel: equal shares of the concatenated tokens, 512 work-groups over the 2 groups of 4 KV heads
     assert ragged["kind"] == base["kind"] == 3
     assert ragged["chunk"] == batch * sk // 2 // 256
