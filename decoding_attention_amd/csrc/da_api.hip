@@ -44,7 +44,7 @@ int env_int(const char* name, int dflt) {
 struct Tunables {
     int target_wgs, mfma_target_wgs, max_chunk, min_chunk, ragged_chunk, force_kind, group_min_ratio, wave_per_head,
         mla_heads, gqa_heads, flat_wgs, flat_min_tokens, flat_paged_min_mb, nsplit, mfma_small_wgs, group_small_wgs,
-        group_small_chunk, mla_group_heads, mla_group_small, fill_rounds;
+        group_small_chunk, mla_group_heads, mla_group_small, fill_rounds, group_target_wgs_d128;
     Tunables() {
         target_wgs = env_int("DA_TARGET_WGS", 512);
         mfma_target_wgs = env_int("DA_MFMA_TARGET_WGS", 256);
@@ -62,6 +62,7 @@ struct Tunables {
         mla_group_heads = env_int("DA_MLA_GROUP_HEADS", 16);
         // ... and any head count while groups x batch x max_seq_k stays within this (twice this for two groups)
         mla_group_small = env_int("DA_MLA_GROUP_SMALL", 65536);
+        group_target_wgs_d128 = env_int("DA_GROUP_TARGET_WGS_D128", 256);
         fill_rounds = env_int("DA_FILL_ROUNDS", 1);  // grouped kernel: re-plan grids that fill their last round of CUs poorly
         group_small_wgs = env_int("DA_GROUP_SMALL_WGS", 256);  // grouped kernel: likewise
         group_small_chunk = env_int("DA_GROUP_SMALL_CHUNK", 64);
@@ -191,6 +192,10 @@ Plan make_plan(size_t max_seq_k, size_t batch, size_t head_q, size_t head_k, siz
         if (tun().gqa_heads == 16 || tun().gqa_heads == 32) pl.rt = tun().gqa_heads;
         pl.wave_per_head = head_k % 4 == 0 && tun().wave_per_head;
         trip = pl.wave_per_head ? da::kGqaTile : 4 * da::kGqaTile;
+        // d = 128: one work-group per CU already saturates HBM, and half as many splits halve the merge (measured,
+        // 256 against 512 work-groups: 32/8 heads, batch 64 x 4096 tokens 183.8 -> 181.8 us, batch 128 x 2048 183.6 ->
+        // 178.0; MQA 32/1, batch 64 x 4096 35.8 -> 31.5; 16/2 heads, batch 32 x 4096 30.6 -> 27.6)
+        if (dim == 128) target_wgs = tun().group_target_wgs_d128;
     } else {
         pl.kind = kKindSweep;
         const int max_rt = dim > 256 ? 2 : 4;
@@ -275,7 +280,10 @@ Plan make_plan(size_t max_seq_k, size_t batch, size_t head_q, size_t head_k, siz
     // the grouped kernel on a batch known to be uniform (token count given, not ragged) needs no cap: fewer, longer
     // splits mean a smaller merge (measured, 32/8 heads d 128: batch 256 x 4096 tokens 726 -> 703 us, batch 128 x
     // 4096 366 -> 360, batch 64 x 16384 727 -> 713); without the count the cap keeps a ragged batch balanced
-    if (pl.kind == kKindGroup && !latent_group && total_k > 0 && !ragged) by_cap = 1;
+    // (up to 2048 tokens while the grid is one work-group per CU: with nothing to balance the CUs against each other a
+    // longer split loses again, batch 32 x 16384 tokens 360 -> 377 us with 4096-token splits)
+    if (pl.kind == kKindGroup && !latent_group && total_k > 0 && !ragged)
+        by_cap = base >= 512 ? 1 : ((long long)max_seq_k + 2047) / 2048;
     // (one round of long splits beats two rounds with the second nearly empty)
     if (latent_group && base <= target_wgs && base * by_cap > target_wgs) by_cap = 1;
     long long ns = std::max(std::min(want, by_len), std::min(by_cap, by_len));
