@@ -31,7 +31,7 @@ HBM_PEAK_GBPS = 8000.0      # MI355X HBM3E, published
 MFMA_PEAK_TFLOPS = 2500.0   # MI355X dense fp16/bf16 MFMA, published
 # HBM bytes per call from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of `bench.py --only gqa|mla`, each counter
 # scaled by what it reads for a 1 GiB device copy (profiles/*_hbm_traffic.md); valid for the default launch plan.
-MEASURED_TRAFFIC_BYTES = {"gqa": 1085278208, "mla": 473240576}
+MEASURED_TRAFFIC_BYTES = {"gqa": 1079830528, "mla": 471680000}
 
 
 def _time_calls(torch, fn_list, steps, warmup):
