@@ -195,7 +195,9 @@ Plan make_plan(size_t max_seq_k, size_t batch, size_t head_q, size_t head_k, siz
         // d = 128: one work-group per CU already saturates HBM, and half as many splits halve the merge (measured,
         // 256 against 512 work-groups: 32/8 heads, batch 64 x 4096 tokens 183.8 -> 181.8 us, batch 128 x 2048 183.6 ->
         // 178.0; MQA 32/1, batch 64 x 4096 35.8 -> 31.5; 16/2 heads, batch 32 x 4096 30.6 -> 27.6)
-        if (dim == 128) target_wgs = tun().group_target_wgs_d128;
+        // (16-bit K/V in whole tiles or 16-token runs only: the 8-bit forms and the per-row page lookups keep fewer
+        // bytes in flight per work-group and need the 512; FP8, batch 64 x 4096 tokens: 96 us against 110)
+        if (dim == 128 && !kv_8bit && (packed || page_size >= 16)) target_wgs = tun().group_target_wgs_d128;
     } else {
         pl.kind = kKindSweep;
         const int max_rt = dim > 256 ? 2 : 4;
@@ -282,7 +284,7 @@ Plan make_plan(size_t max_seq_k, size_t batch, size_t head_q, size_t head_k, siz
     // 4096 366 -> 360, batch 64 x 16384 727 -> 713); without the count the cap keeps a ragged batch balanced
     // (up to 2048 tokens while the grid is one work-group per CU: with nothing to balance the CUs against each other a
     // longer split loses again, batch 32 x 16384 tokens 360 -> 377 us with 4096-token splits)
-    if (pl.kind == kKindGroup && !latent_group && total_k > 0 && !ragged)
+    if (pl.kind == kKindGroup && !latent_group && total_k > 0 && !ragged && !kv_8bit && (packed || page_size >= 16))
         by_cap = base >= 512 ? 1 : ((long long)max_seq_k + 2047) / 2048;
     // (one round of long splits beats two rounds with the second nearly empty)
     if (latent_group && base <= target_wgs && base * by_cap > target_wgs) by_cap = 1;
@@ -295,7 +297,9 @@ Plan make_plan(size_t max_seq_k, size_t batch, size_t head_q, size_t head_k, siz
     // 128, 4096 tokens: batch 40, 7 splits (560 work-groups) 138.6 us, 3 splits (240) 117.9; batch 48, 6 splits (576)
     // 158.8, 5 splits (480) 142.4; batch 100, 4 splits (800) 320.5, 1 split (200) 284.8.
     // (not at d = 96, where the re-planning loses as often as it wins)
-    if (pl.kind == kKindGroup && dim != 96 && dim <= 256 && tun().fill_rounds) {
+    // (measured on 16-bit K/V in whole tiles or 16-token runs, and applied there only)
+    const bool plain16 = !kv_8bit && (packed || page_size >= 16);
+    if (pl.kind == kKindGroup && plain16 && dim != 96 && dim <= 256 && tun().fill_rounds) {
         // (at d = 64 a work-group streams too few bytes for one per CU to saturate HBM: rounds of two per CU there;
         // 32/8 heads, batch 56 x 4096 tokens 100.1 -> 84.9 us, 32/4 heads, batch 150 x 4096 127.2 -> 112.3)
         const double gran = dim >= 128 ? 256.0 : 512.0, sat = dim >= 128 ? 200.0 : 400.0;
