@@ -298,11 +298,16 @@ Plan make_plan(size_t max_seq_k, size_t batch, size_t head_q, size_t head_k, siz
     // 158.8, 5 splits (480) 142.4; batch 100, 4 splits (800) 320.5, 1 split (200) 284.8.
     // (not at d = 96, where the re-planning loses as often as it wins)
     // (measured on 16-bit K/V in whole tiles or 16-token runs, and applied there only)
-    const bool plain16 = !kv_8bit && (packed || page_size >= 16);
-    if (pl.kind == kKindGroup && plain16 && dim != 96 && dim <= 256 && tun().fill_rounds) {
+    // (... and on 8-bit K/V at d = 128, whose rows are as short as 16-bit rows at d = 64: FP8, 32/8 heads, batch 100
+    // x 4096 tokens 184 -> 154 us, batch 72 131 -> 116, batch 40 74 -> 66)
+    const bool whole_tiles = packed || page_size >= 16;
+    const bool plain16 = !kv_8bit && whole_tiles;
+    const bool short_rows = dim < 128 || kv_8bit;
+    if (pl.kind == kKindGroup && (plain16 || (kv_8bit && dim == 128 && whole_tiles)) && dim != 96 && dim <= 256 &&
+        tun().fill_rounds) {
         // (at d = 64 a work-group streams too few bytes for one per CU to saturate HBM: rounds of two per CU there;
         // 32/8 heads, batch 56 x 4096 tokens 100.1 -> 84.9 us, 32/4 heads, batch 150 x 4096 127.2 -> 112.3)
-        const double gran = dim >= 128 ? 256.0 : 512.0, sat = dim >= 128 ? 200.0 : 400.0;
+        const double gran = short_rows ? 512.0 : 256.0, sat = short_rows ? 400.0 : 200.0;
         auto fill = [&](long long c) {
             const double w = (double)(base * c);
             if (w <= gran) return std::min(1.0, w / sat);
