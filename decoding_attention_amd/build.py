@@ -20,6 +20,7 @@ SOURCES = [
     "da_sweep_d256.hip",
     "da_sweep_d576.hip",
     "da_mla.hip",
+    "da_mla_pipe.hip",
     "da_gqa_mfma.hip",
     "da_sweep_kv8.hip",
     "da_gqa_mfma_kv8.hip",
@@ -39,14 +40,28 @@ def _hipcc():
     return os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 
 
+# Per-file flags.  da_mla_pipe.hip names most of the register file in its instruction text and confines the compiler
+# to the rest; the compiler must then never park its own values in accumulation registers.
+EXTRA_FLAGS = {
+    "da_mla_pipe.hip": ["-mllvm", "-amdgpu-spill-vgpr-to-agpr=0"],
+}
+
+
+# Sources whose generated code is verified after compiling (check_isa.py).
+ISA_CHECKED = {"da_mla_pipe.hip"}
+
+
 def _compile(src):
     obj = os.path.join(OBJ_DIR, os.path.splitext(src)[0] + ".o")
-    cmd = [_hipcc()] + HIPCC_FLAGS + ["-c", os.path.join(CSRC, src), "-o", obj]
+    cmd = [_hipcc()] + HIPCC_FLAGS + EXTRA_FLAGS.get(src, []) + ["-c", os.path.join(CSRC, src), "-o", obj]
     if os.environ.get("DA_SAVE_TEMPS"):
         cmd += ["-save-temps=obj"]
     res = subprocess.run(cmd, capture_output=True, text=True)
     if res.returncode != 0:
         raise RuntimeError(f"hipcc failed for {src}:\n{res.stdout}\n{res.stderr}")
+    if src in ISA_CHECKED:
+        from . import check_isa
+        check_isa.check_source(_hipcc(), HIPCC_FLAGS + EXTRA_FLAGS.get(src, []), os.path.join(CSRC, src))
     warn = "\n".join(ln for ln in res.stderr.splitlines() if "packed-fp32-ops" not in ln and ln.strip())
     return obj, warn
 

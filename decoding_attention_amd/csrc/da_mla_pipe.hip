@@ -1,0 +1,746 @@
+// Software-pipelined MFMA sweep for 65..128 query heads over one latent KV head (key width 576, values = the
+// first 512 key columns), 16-bit K.
+//
+// One work-group of four wavefronts serves one (sequence, 128 heads, sequence split); each wavefront owns 32
+// heads: Q as MFMA B-operands in 144 registers, the un-normalised output O^T[512 x 32] in all 256 accumulation
+// registers -- one wavefront per SIMD.  K tiles of 32 tokens stream HBM -> LDS with direct-to-LDS loads into four
+// buffers (the tile layout of da_mla_dev.h); every tile is read from LDS twice, as K rows for
+// S^T = K . Q^T and transposed for O^T += V^T . P^T.
+//
+// The matrix pipe is the resource to keep busy (2 x 68 matrix instructions of 32 clocks per tile and wavefront), and
+// a wavefront's vector-ALU, LDS and load instructions issue beside its own matrix instructions when they do not
+// depend on them.  So the tile loop is software-pipelined by one tile and written as one fixed instruction sequence:
+//
+//   trip t:   phase A   S(t+1) = K(t+1) . Q^T   36 matrix steps, between them the online softmax of S(t)
+//                                               (subtract, exp2, sum, pack: two instructions per step) and the
+//                                               nine direct-to-LDS loads of tile t+3
+//             phase B   O += V(t)^T . P(t)^T    32 matrix steps
+//
+// Registers.  Q (v112 .. v255), the output tiles (a0 .. a255), the ring of LDS fragments (v80 .. v111) and the
+// probability tile (v64 .. v79) are named
+// in the instruction text and never seen by the compiler, whose own allocation is confined to v0 .. v63 (kernel
+// attribute amdgpu_num_vgpr; the translation unit is built with VGPR-to-AGPR spilling switched off): with 400 of
+// the 512 registers pinned down for the whole loop, a register allocator that may move them is the one thing the loop
+// cannot afford.  What the compiler allocates: the score tile being accumulated, addresses and scalars.
+//
+// LDS fragments for the matrix steps run through a ring of eight register sets, requested eight steps ahead of
+// their use across the A -> B boundary; the ring drains at the end of a trip (the next trip's K tile is only known
+// to be in LDS after the trip's barrier), and the scaling and maximum of S(t+1) are computed while it refills.
+// One barrier per trip: behind it every wave's share of tile t+1 has landed and every wave is done with tile t-1,
+// whose buffer then receives tile t+3.
+//
+// Mathematics as in the reference kernel (csrc/kernel/decoding_attn/decoding_fwd_kernel.h:50-235 with the latent
+// aliasing of csrc/ops/decoding_attn.cpp:30-37); the structure is unrelated.
+#include "da_mla.h"
+#include "da_mla_dev.h"
+
+#include <cstdlib>
+
+namespace da {
+
+namespace {
+
+using namespace mla;
+
+constexpr int kPipeBufs = 4;  // LDS tile buffers
+constexpr int kRing = 8;      // LDS fragments requested ahead of the matrix step that uses them
+
+typedef short s16x8 __attribute__((__vector_size__(8 * sizeof(short))));
+
+// Registers named in the instruction text (see the header comment).
+constexpr int kScV = 64;    // the probability tile: v[64 .. 79]
+constexpr int kRingV = 80;  // ring slot s: v[80 + 4 s .. 83 + 4 s]
+constexpr int kQV = 112;    // Q fragment of k-step ks: v[112 + 4 ks .. 115 + 4 ks]
+
+// ds_read_b128 into v[R .. R+3] from (base ^ X) + OFF; the XOR goes through `tmp`
+template <int R, int X, int OFF>
+__device__ __forceinline__ void ring_read_b128(uint32_t base, uint32_t& tmp) {
+    if constexpr (X == 0) {
+        asm volatile("ds_read_b128 v[%1:%2], %0 offset:%3" ::"v"(base), "n"(R), "n"(R + 3), "n"(OFF));
+    } else {
+        asm volatile("v_xor_b32 %0, %2, %1\n\tds_read_b128 v[%3:%4], %0 offset:%5"
+                     : "=&v"(tmp)
+                     : "v"(base), "n"(X), "n"(R), "n"(R + 3), "n"(OFF));
+    }
+}
+// ds_read_b64_tr_b16 into v[R .. R+1]
+template <int R, int OFF>
+__device__ __forceinline__ void ring_read_tr16(uint32_t addr) {
+    asm volatile("ds_read_b64_tr_b16 v[%1:%2], %0 offset:%3" ::"v"(addr), "n"(R), "n"(R + 1), "n"(OFF));
+}
+template <int N>
+__device__ __forceinline__ void wait_lgkm_n() {
+    asm volatile("s_waitcnt lgkmcnt(%0)" ::"n"(N));
+}
+template <int X>
+__device__ __forceinline__ void xor_const(uint32_t& dst, uint32_t base) {
+    asm volatile("v_xor_b32 %0, %2, %1" : "=v"(dst) : "v"(base), "n"(X));
+}
+// Matrix instructions on the named registers.  S: acc (the compiler's) (+)= v[A..] . v[B..]; O: a[C..] += v[A..] . b
+template <typename Tag, int A, int B, bool FIRST>
+__device__ __forceinline__ void mma_s(f32x16& acc) {
+    if constexpr (std::is_same<Tag, bf16_tag>::value) {
+        if constexpr (FIRST)
+            asm volatile("v_mfma_f32_32x32x16_bf16 %0, v[%1:%2], v[%3:%4], 0" : "=v"(acc) : "n"(A), "n"(A + 3), "n"(B), "n"(B + 3));
+        else
+            asm volatile("v_mfma_f32_32x32x16_bf16 %0, v[%1:%2], v[%3:%4], %0" : "+v"(acc) : "n"(A), "n"(A + 3), "n"(B), "n"(B + 3));
+    } else {
+        if constexpr (FIRST)
+            asm volatile("v_mfma_f32_32x32x16_f16 %0, v[%1:%2], v[%3:%4], 0" : "=v"(acc) : "n"(A), "n"(A + 3), "n"(B), "n"(B + 3));
+        else
+            asm volatile("v_mfma_f32_32x32x16_f16 %0, v[%1:%2], v[%3:%4], %0" : "+v"(acc) : "n"(A), "n"(A + 3), "n"(B), "n"(B + 3));
+    }
+}
+// a[N] *= alpha
+template <int N>
+__device__ __forceinline__ void scale_acc_n(float alpha) {
+    float tmp;
+    asm volatile("v_accvgpr_read_b32 %0, a[%2]\n\tv_mul_f32 %0, %0, %1\n\ts_nop 0\n\tv_accvgpr_write_b32 a[%2], %0"
+                 : "=&v"(tmp)
+                 : "v"(alpha), "n"(N));
+}
+template <int N>
+__device__ __forceinline__ float read_acc_n() {
+    float x;
+    asm volatile("v_accvgpr_read_b32 %0, a[%1]" : "=v"(x) : "n"(N));
+    return x;
+}
+template <typename Tag, int A, int B, int C>
+__device__ __forceinline__ void mma_o() {
+    if constexpr (std::is_same<Tag, bf16_tag>::value)
+        asm volatile("v_mfma_f32_32x32x16_bf16 a[%0:%1], v[%2:%3], v[%4:%5], a[%0:%1]" ::"n"(C), "n"(C + 15), "n"(A), "n"(A + 3), "n"(B), "n"(B + 3));
+    else
+        asm volatile("v_mfma_f32_32x32x16_f16 a[%0:%1], v[%2:%3], v[%4:%5], a[%0:%1]" ::"n"(C), "n"(C + 15), "n"(A), "n"(A + 3), "n"(B), "n"(B + 3));
+}
+// The probability tile: v[kScV + r], r = 0 .. 15, holds score r of the tile minus the running maximum, then the
+// probability, then (r < 8) the probabilities of the pair (2 r, 2 r + 1) packed as one register of two B-operands.
+// Single vector-ALU instructions on it, each with a fixed place in the instruction sequence:
+template <int I>
+__device__ __forceinline__ void sc_set(float x) { asm volatile("v_mov_b32 v[%1], %0" ::"v"(x), "n"(kScV + I)); }
+// v[I] = s * scale + negm
+template <int I>
+__device__ __forceinline__ void sc_fma(float s, float scale, float negm) {
+    asm volatile("v_fma_f32 v[%3], %0, %1, %2" ::"v"(s), "v"(scale), "v"(negm), "n"(kScV + I));
+}
+template <int I>
+__device__ __forceinline__ void sc_exp2() { asm volatile("v_exp_f32 v[%0], v[%0]" ::"n"(kScV + I)); }
+template <int I>
+__device__ __forceinline__ void sc_acc(float& l) { asm volatile("v_add_f32 %0, %0, v[%1]" : "+v"(l) : "n"(kScV + I)); }
+__device__ __forceinline__ void v_add(float& x, float y) { asm volatile("v_add_f32 %0, %0, %1" : "+v"(x) : "v"(y)); }
+// x += s, s wave-uniform
+__device__ __forceinline__ void v_add_s(uint32_t& x, uint32_t s) { asm volatile("v_add_u32 %0, %1, %0" : "+v"(x) : "s"(s)); }
+// v[K] = the pair (v[2K], v[2K+1]) rounded to two 16-bit values (round to nearest even).  In place: register K held
+// element K, which pair K/2 <= K has consumed by now.  (bf16, s_nop: a result of the transcendental unit needs one
+// wait state before an ordinary vector instruction reads it, and there this directly follows the exp2 of v[2K+1].)
+template <typename Tag, int K>
+__device__ __forceinline__ void sc_pack() {
+    if constexpr (std::is_same<Tag, bf16_tag>::value)
+        asm volatile("s_nop 0\n\tv_cvt_pk_bf16_f32 v[%0], v[%1], v[%2]" ::"n"(kScV + K), "n"(kScV + 2 * K), "n"(kScV + 2 * K + 1));
+    else
+        asm volatile("v_cvt_pk_f16_f32 v[%0], v[%1], v[%2]" ::"n"(kScV + K), "n"(kScV + 2 * K), "n"(kScV + 2 * K + 1));
+}
+// the two 16-bit halves of register K as fp32 values (bf16: the value itself)
+template <int K>
+__device__ __forceinline__ void sc_bf16_lo(float& dst) { asm volatile("v_lshlrev_b32 %0, 16, v[%1]" : "=v"(dst) : "n"(kScV + K)); }
+template <int K>
+__device__ __forceinline__ void sc_bf16_hi(float& dst) { asm volatile("v_and_b32 %0, 0xffff0000, v[%1]" : "=v"(dst) : "n"(kScV + K)); }
+
+// PG: paged K/V with pages of fewer than 16 tokens (down to 1): every row of a tile has its own page lookup.
+template <typename Tag, bool PG>
+__global__ __launch_bounds__(256) __attribute__((amdgpu_num_vgpr(kScV))) void latent_pipe_kernel(const SweepParams p) {
+    // the register file as this kernel uses it: v0 .. v255 and a0 .. a255 (the compiler itself stays below v64)
+    asm volatile("" ::: "v255", "a255");
+    using EL = Elem<Tag>;
+    constexpr bool kBf16 = std::is_same<Tag, bf16_tag>::value;
+    constexpr int D = 576, DV = 512, NWV = 4;
+    constexpr int ROW_A = DV * 2;           // bytes per row, region A (value columns)
+    constexpr int ROW_B = (D - DV) * 2;     // bytes per row, region B (remaining key columns)
+    constexpr int OFF_B = kTile * ROW_A;    // region B starts here
+    constexpr int BUF = kTile * D * 2;      // bytes per tile buffer
+    constexpr int NLA = kTile / NWV;        // region-A load instructions per tile per wave (one row each)
+    constexpr int NLB = (kTile / 8) / NWV;  // region-B load instructions per tile per wave (eight rows each)
+    constexpr int NLW = NLA + NLB;          // load instructions per tile per wave
+    constexpr int KS = D / 16;              // k-steps of Q K^T
+    constexpr int CT = DV / 32;             // 32-column tiles of the output
+    constexpr int NV = CT * 2;              // matrix steps of O += V^T P^T
+    constexpr int NB = kPipeBufs;
+    static_assert(NLB == 1 && KS == 36 && NV == 32, "schedule below is written for (576, 512), four waves");
+
+    extern __shared__ __attribute__((aligned(1024))) uint8_t smem[];  // NB * BUF bytes
+    const uint32_t smem_off = (uint32_t)(uintptr_t)smem;
+
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int half = lane >> 5;
+    const int n = lane & 31;
+
+    // Work-groups are handed to the eight XCDs round-robin by linear id, and each XCD has its own L2.  Renumber
+    // so that the sequence splits of one (sequence, head group) run on one XCD: they read the same Q block, which
+    // then leaves HBM once instead of once per split.
+    int split = blockIdx.x, by = blockIdx.y, b = blockIdx.z;
+    {
+        const int outer_n = gridDim.y * gridDim.z;
+        if (gridDim.x > 1 && outer_n % 8 == 0) {
+            const int lin = blockIdx.x + gridDim.x * (blockIdx.y + gridDim.y * blockIdx.z);
+            const int slot = lin >> 3;
+            split = slot % (int)gridDim.x;
+            const int outer = (slot / (int)gridDim.x) * 8 + (lin & 7);
+            by = outer % (int)gridDim.y;
+            b = outer / (int)gridDim.y;
+        }
+    }
+    const int hk = by / p.groups;
+    const int grp = by % p.groups;
+
+    int start, len;
+    seq_range(p, b, start, len);
+    const int c0 = split * p.chunk;
+    const int c1 = (split == p.nsplit - 1) ? len : min(len, c0 + p.chunk);
+
+    const int wg_heads = min(32 * NWV, p.ratio - grp * 32 * NWV);  // live heads of this work-group
+    const int nh = max(0, min(32, wg_heads - wave * 32));          // live heads of this wave
+    const int h_base = hk * p.ratio + grp * 32 * NWV + wave * 32;
+    uint16_t* const o16 = reinterpret_cast<uint16_t*>(p.o);
+
+    if (c0 >= c1) {
+        if (p.nsplit == 1) zero_rows<DV>(p, b, hk * p.ratio + grp * 32 * NWV, wg_heads, 1, 0);
+        return;
+    }
+
+    // Q rows of this wave's heads as B-operands: lane (n, half) holds Q[head n][ks*16 + half*8 .. +8).  The wave's
+    // 32 x 576 block of Q is staged like a K tile (whole-row direct-to-LDS loads, same swizzle, into the wave's own
+    // buffer) and read back with the K-row read pattern, which is the same operand layout.
+    const int q_last = max(nh, 1) - 1;
+    const int hq = min(h_base + min(n, q_last), p.head_q - 1);
+    const uint32_t lane16 = lane * 16;
+    const int rb = lane >> 3;  // region B: row within the group of eight, chunk lane & 7
+    {
+        const uint8_t* const qb = reinterpret_cast<const uint8_t*>(p.q) + (size_t)b * p.head_q * (D * 2);
+        const uint32_t qbuf = smem_off + wave * BUF;
+        static_for<0, kTile>([&](auto rc) {
+            constexpr int row = decltype(rc)::value;
+            const int head = min(h_base + min(row, q_last), p.head_q - 1);  // wave-uniform
+            lds_dma16(qb, (uint32_t)head * (uint32_t)(D * 2) + (lane16 ^ (uint32_t)(swz_a(row) * 16)),
+                      qbuf + (uint32_t)(row * ROW_A));
+        });
+        static_for<0, kTile / 8>([&](auto jc) {
+            constexpr int j = decltype(jc)::value;
+            const int row = j * 8 + rb;
+            const int head = min(h_base + min(row, q_last), p.head_q - 1);
+            lds_dma16(qb, (uint32_t)head * (uint32_t)(D * 2) + (uint32_t)(DV * 2 + (((lane & 7) ^ swz_b(row)) * 16)),
+                      qbuf + (uint32_t)(OFF_B + j * 1024));
+        });
+        wait_vmcnt<0>();
+        const uint32_t qa = qbuf + n * ROW_A + ((swz_a(n) ^ half) * 16);
+        const uint32_t qbb = qbuf + OFF_B + n * ROW_B + ((swz_b(n) ^ half) * 16);
+        static_for<0, KS>([&](auto ic) {
+            constexpr int ks = decltype(ic)::value;
+            uint32_t tmp;
+            if constexpr (ks < 32)
+                ring_read_b128<kQV + 4 * ks, 32 * (ks & 7), (ks >> 3) * 256>(qa, tmp);
+            else
+                ring_read_b128<kQV + 4 * ks, 32 * (ks - 32), 0>(qbb, tmp);
+            if constexpr (ks % 12 == 11) wait_lgkm_n<0>();  // the counter of outstanding reads is 4 bits wide
+        });
+    }
+    __syncthreads();  // the tile buffers are free for K once every wave has its Q in registers
+    const float slope = p.is_alibi ? alibi_slope_log2(p.slopes, hq, p.head_q) : 0.0f;
+
+    static_for<0, CT * 16>([&](auto ic) { asm volatile("v_accvgpr_write_b32 a[%0], 0" ::"n"(decltype(ic)::value)); });
+    float m = kNegBig, l = 0.0f;
+
+    const uint8_t* const kbytes = reinterpret_cast<const uint8_t*>(p.k) + (size_t)hk * D * 2;
+    const size_t k_row_bytes = (size_t)p.k_row * 2;
+    const float sl = p.scale_log2;  // score scale, log2 units
+
+    // One direct-to-LDS load of a tile: region-A row wave + 4 q for q < NLA, then the wave's eight region-B rows.
+    // `base` / `base1`: addresses of the rows of the tile's tokens 0 and 16 (a tile is fetched as two runs of 16
+    // tokens, each inside one page; for the packed layout and larger pages the second run follows the first); `last`:
+    // last valid token of the tile, rows past it re-read that row (they are masked later).
+    auto issue_load = [&](auto qc, const uint8_t* base, const uint8_t* base1, int last, int buf) {
+        constexpr int q = decltype(qc)::value;
+        if constexpr (q < NLA) {
+            const int row = wave + NWV * q;  // wave-uniform
+            const int rc = min(row, last), run = rc >> 4;
+            // lane offset (row part in a scalar register) computed at the load, not kept in a register per q
+            uint32_t off;
+            asm volatile("v_xor_b32 %0, %1, %2\n\tv_add_u32 %0, %3, %0"
+                         : "=&v"(off)
+                         : "s"((uint32_t)(swz_a(row) * 16)), "v"(lane16), "s"((uint32_t)(rc - run * 16) * (uint32_t)k_row_bytes));
+            lds_dma16(run ? base1 : base, off, smem_off + (uint32_t)(buf * BUF + row * ROW_A));
+        } else {
+            const int j = wave;
+            const int row = j * 8 + rb;
+            const int run = min(j >> 1, last >> 4);  // the eight rows of a load lie in one run, clamped or not
+            lds_dma16(run ? base1 : base, (uint32_t)(min(row, last) - run * 16) * (uint32_t)k_row_bytes +
+                                              (uint32_t)(DV * 2 + (((lane & 7) ^ swz_b(row)) * 16)),
+                      smem_off + (uint32_t)(buf * BUF + OFF_B + j * 1024));
+        }
+    };
+    // rows of tokens tok and tok + 16 of the sequence (the second only looked up when the tile has it: the block
+    // table ends with the sequence's last page)
+    struct TileRows {
+        const uint8_t* base;
+        const uint8_t* base1;
+        int last;
+    };
+    auto tile_rows = [&](int tok0) {
+        const int64_t r0 = row_ref(p, b, start, tok0).k;
+        const int64_t r1 = tok0 + 16 < c1 ? row_ref(p, b, start, tok0 + 16).k : r0;
+        return TileRows{kbytes + r0 * 2, kbytes + r1 * 2, c1 - 1 - tok0};
+    };
+    auto issue_tile = [&](int tok0, int buf) {
+        const TileRows tr = tile_rows(tok0);
+        static_for<0, NLW>([&](auto qc) { issue_load(qc, tr.base, tr.base1, tr.last, buf); });
+    };
+
+    // PG: the wave's kTile / NWV rows are consecutive here (rows wave * NLA + q), the same rows for both regions, so
+    // one set of page lookups (scalar loads) serves both; the second region's load covers eight rows, so its lanes
+    // pick their row's address out of the set.
+    auto issue_tile_pg = [&](int tok0, int buf) {
+        const int last = c1 - 1 - tok0;
+        const int mask = (1 << p.page_shift) - 1;
+        int64_t rowoff[NLA];  // byte offsets of the wave's rows
+#pragma unroll
+        for (int q = 0; q < NLA; ++q) {
+            const int tok = tok0 + min(wave * NLA + q, last);
+            rowoff[q] = ((int64_t)page_of(p, b, tok) * p.k_page + (int64_t)(tok & mask) * p.k_row) * 2;
+        }
+#pragma unroll
+        for (int q = 0; q < NLA; ++q) {
+            const int row = wave * NLA + q;
+            lds_dma16(kbytes + rowoff[q], lane16 ^ (uint32_t)(swz_a(row) * 16),
+                      smem_off + (uint32_t)(buf * BUF + row * ROW_A));
+        }
+        {
+            const int j = wave;
+            const int row = j * 8 + rb;
+            int64_t mine = rowoff[0];
+#pragma unroll
+            for (int i = 1; i < 8; ++i) mine = rb == i ? rowoff[i] : mine;
+            lds_dma16_v(kbytes + mine + (DV * 2 + (((lane & 7) ^ swz_b(row)) * 16)),
+                        smem_off + (uint32_t)(buf * BUF + OFF_B + j * 1024));
+        }
+    };
+
+    const int ntiles = (c1 - c0 + kTile - 1) / kTile;
+    // tiles 0 .. 2 go out at once (buffers 0 .. 2); tile t + 3 follows in trip t
+#pragma unroll
+    for (int i = 0; i < NB - 1; ++i)
+        if (i < ntiles) {
+            if constexpr (PG)
+                issue_tile_pg(c0 + i * kTile, i);
+            else
+                issue_tile(c0 + i * kTile, i);
+        }
+
+    // The fast form of a tile's loads, for whole tiles (no row past the end) between the matrix steps of phase A: the
+    // row part of the address is added to the tile's base in scalar registers, the lane part is one XOR.
+    // rowoff[j] = (wave + 4 j) * pitch, j < 4: region-A rows of the first run; those of the second run (q >= 4) lie
+    // the same distances behind the second run's base.
+    uint32_t rowoff[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) rowoff[j] = (uint32_t)(wave + NWV * j) * (uint32_t)k_row_bytes;
+    // region B: the wave's eight rows 8 wave .. 8 wave + 7 lie in run wave / 2; lane part (row within the eight,
+    // swizzled chunk) kept in a register
+    const uint32_t voff_b = (uint32_t)(((wave & 1) * 8 + rb) * (int)k_row_bytes) +
+                            (uint32_t)(DV * 2 + (((lane & 7) ^ swz_b(wave * 8 + rb)) * 16));
+    const uint32_t lane16w = lane16 ^ (uint32_t)(wave << 6);  // lane16 ^ 16 * (swizzle bits from row & 3 = wave)
+    auto issue_load_fast = [&](auto qc, const uint8_t* base, const uint8_t* base1, uint32_t lds_buf) {
+        constexpr int q = decltype(qc)::value;
+        if constexpr (q < NLA) {
+            // row = wave + 4 q: swizzle = wave << 2 | (q & 3)
+            uint32_t off;
+            if constexpr ((q & 3) == 0)
+                off = lane16w;
+            else
+                asm volatile("v_xor_b32 %0, %1, %2" : "=v"(off) : "n"((q & 3) * 16), "v"(lane16w));
+            lds_dma16((q < 4 ? base : base1) + rowoff[q & 3], off,
+                      lds_buf + (uint32_t)(q * NWV * ROW_A) + (uint32_t)(wave * ROW_A));
+        } else {
+            lds_dma16((wave >> 1) ? base1 : base, voff_b, lds_buf + (uint32_t)OFF_B + (uint32_t)(wave * 1024));
+        }
+    };
+
+    // Per-lane LDS read bases (buffer 0); per-step chunk offsets are XORed in, the rest is instruction offset.
+    // K rows: lane (n, half) reads chunk 2 ks + half of row n.
+    //   ks < 32: (base_a ^ 32 (ks & 7)) + 256 (ks >> 3)        ks >= 32: base_b ^ 32 (ks - 32)
+    const uint32_t base_a = smem_off + n * ROW_A + ((swz_a(n) ^ half) * 16);
+    const uint32_t base_b = smem_off + OFF_B + n * ROW_B + ((swz_b(n) ^ half) * 16);
+    // V^T: as a source lane of the transpose read this lane addresses row half*4 + q (+16 s2, +8 for the second
+    // read), 8 bytes at chunk 4 c + 2 b1 + b0 of it, q = (lane & 15) >> 2, b1 = lane bit 4, b0 = lane bit 1:
+    //   (base_v ^ (64 c | 32 hi)) + 16 KiB s2 + 8 KiB hi
+    const uint32_t base_v = smem_off + (half * 4 + ((lane & 15) >> 2)) * ROW_A + 64 * ((lane & 15) >> 2) +
+                            16 * ((2 * ((lane >> 4) & 1) + ((lane >> 1) & 1)) ^ half) + 8 * (lane & 1);
+
+    const float bias0 = slope * (float)(half * 4 - (len - 1));  // ALiBi: slope * (token - (len - 1)), split in lane and tile parts
+
+    // ---- the fragment ring -------------------------------------------------------------------------------------
+    // Matrix steps of a trip in order: g = 0 .. 35 the k-steps of S = K Q^T (one ds_read_b128 each), g = 36 .. 67 the
+    // steps of O += V^T P^T (two transpose reads each).  The reads of step g + kRing are issued behind the matrix
+    // instruction of step g; ring slot g % kRing.
+    // Addresses of the K reads of the tile being multiplied (region A: one register per k-step % 8, moved from buffer
+    // to buffer once a trip; region B: XOR in front of the read)
+    constexpr int NKA = PG ? 1 : 8;
+    uint32_t ka[NKA];
+    uint32_t xa = 0, xb = 0;  // V^T read addresses of the current column tile
+    uint32_t xt = 0;          // scratch for K read addresses
+    f32x16 sacc;              // S(t+1), being accumulated
+    float mxr = 0.0f;         // maximum of the raw scores of the tile in sacc (over the tile's tokens, this lane's head)
+
+    // read for k-step ks of the K tile whose region-B base is tb (region A: ka[]; the PG form, short of registers for
+    // its row addresses, keeps one base, ka[0], and XORs in front of every read)
+    auto read_k = [&](auto ksc, uint32_t tb) {
+        constexpr int ks = decltype(ksc)::value;
+        if constexpr (ks < 32 && PG)
+            ring_read_b128<kRingV + 4 * (ks % kRing), 32 * (ks & 7), (ks >> 3) * 256>(ka[0], xt);
+        else if constexpr (ks < 32)
+            ring_read_b128<kRingV + 4 * (ks % kRing), 0, (ks >> 3) * 256>(ka[ks & 7], xt);
+        else
+            ring_read_b128<kRingV + 4 * (ks % kRing), 32 * (ks - 32), 0>(tb, xt);
+    };
+    // reads for step i of O += V^T P^T (column tile i / 2, token half i % 2) of the tile at tv; ring slot (KS + i) % kRing
+    auto read_v = [&](auto ic, uint32_t tv) {
+        constexpr int i = decltype(ic)::value;
+        constexpr int c = i >> 1, s2 = i & 1, slot = (KS + i) % kRing;
+        if constexpr (s2 == 0) {
+            if constexpr (c == 0)
+                asm volatile("v_mov_b32 %0, %1" : "=v"(xa) : "v"(tv));
+            else
+                xor_const<64 * c>(xa, tv);
+            xor_const<64 * c + 32>(xb, tv);
+        }
+        ring_read_tr16<kRingV + 4 * slot, s2 * 16 * ROW_A>(xa);
+        ring_read_tr16<kRingV + 4 * slot + 2, s2 * 16 * ROW_A + 8 * ROW_A>(xb);
+    };
+
+    // softmax of S(t), the part that runs between matrix steps.  sc holds the scores minus the running maximum; for
+    // each register pair (2 k, 2 k + 1): exponentiate, add to the denominator, pack.  fp16: 5 instructions a pair,
+    // bf16: 7 (the denominator is summed from the rounded values, see as_second_operand in da_common.h).
+    constexpr int SMP = kBf16 ? 7 : 5;  // instructions per pair
+    constexpr int SMN = 8 * SMP;        // in all
+    float tlo, thi;
+    auto sm_op = [&](auto jc) {
+        constexpr int j = decltype(jc)::value;
+        constexpr int k = j / SMP, o = j % SMP;
+        if constexpr (o == 0) sc_exp2<2 * k>();
+        if constexpr (o == 1) sc_exp2<2 * k + 1>();
+        if constexpr (!kBf16) {
+            if constexpr (o == 2) sc_acc<2 * k>(l);
+            if constexpr (o == 3) sc_acc<2 * k + 1>(l);
+            if constexpr (o == 4) sc_pack<Tag, k>();
+        } else {
+            if constexpr (o == 2) sc_pack<Tag, k>();
+            if constexpr (o == 3) sc_bf16_lo<k>(tlo);
+            if constexpr (o == 4) sc_bf16_hi<k>(thi);
+            if constexpr (o == 5) v_add(l, tlo);
+            if constexpr (o == 6) v_add(l, thi);
+        }
+    };
+    // maximum of the raw scores in sacc, between the matrix steps of phase B (its first instruction well behind the
+    // last matrix instruction that wrote sacc): eleven instructions
+    auto mx_op = [&](auto jc) {
+        constexpr int j = decltype(jc)::value;
+        if constexpr (j == 0) asm volatile("v_max3_f32 %0, %1, %2, %3" : "=v"(mxr) : "v"(sacc[0]), "v"(sacc[1]), "v"(sacc[2]));
+        if constexpr (j >= 1 && j <= 6)
+            asm volatile("v_max3_f32 %0, %0, %1, %2" : "+v"(mxr) : "v"(sacc[2 * j + 1]), "v"(sacc[2 * j + 2]));
+        if constexpr (j == 7) asm volatile("v_max_f32 %0, %0, %1" : "+v"(mxr) : "v"(sacc[15]));
+        if constexpr (j == 8) asm volatile("v_mov_b32 %0, %1" : "=v"(tlo) : "v"(mxr));
+        // (lanes 32 .. 63 of tlo <-> lanes 0 .. 31 of mxr: tlo = the lower half's maximum everywhere, mxr the upper's)
+        if constexpr (j == 9) asm volatile("s_nop 1\n\tv_permlane32_swap_b32 %0, %1" : "+v"(tlo), "+v"(mxr));
+        if constexpr (j == 10) asm volatile("v_max_f32 %0, %0, %1" : "+v"(mxr) : "v"(tlo));
+    };
+
+    // ---- phase A: S(t+1) = K(t+1) Q^T beside the softmax of S(t) and the loads of tile t+3 ------------------------
+    // QK: the matrix steps (else only the softmax runs: last trip); SM: the softmax (else only the matrix steps:
+    // prologue); DMA: the nine loads of a whole tile go out behind steps 1, 5, ..., 33.
+    auto phase_a = [&](auto qk_c, auto sm_c, auto dma_c, uint32_t tb, uint32_t tv, const uint8_t* base,
+                       const uint8_t* base1, uint32_t dma_lds) {
+        constexpr bool QK = decltype(qk_c)::value, SM = decltype(sm_c)::value, DMA = decltype(dma_c)::value;
+        constexpr bool VNEXT = SM;  // a trip with a softmax continues with phase B
+        if constexpr (QK) {
+            // the ring was primed by the caller with steps 0 .. kRing-1
+            static_for<0, KS>([&](auto gc) {
+                constexpr int g = decltype(gc)::value;
+                // reads outstanding behind step g's: steps g+1 .. g+kRing-1
+                constexpr int last_issued = VNEXT ? g + kRing - 1 : (g + kRing - 1 < KS ? g + kRing - 1 : KS - 1);
+                constexpr int nk = (last_issued < KS ? last_issued : KS - 1) - g;           // K reads among them
+                constexpr int nv = last_issued >= KS ? last_issued - KS + 1 : 0;            // V steps among them
+                wait_lgkm_n<nk + 2 * nv>();
+                mma_s<Tag, kRingV + 4 * (g % kRing), kQV + 4 * g, g == 0>(sacc);
+                if constexpr (g + kRing < KS)
+                    read_k(std::integral_constant<int, g + kRing>{}, tb);
+                else if constexpr (VNEXT)
+                    read_v(std::integral_constant<int, g + kRing - KS>{}, tv);
+                if constexpr (SM) {
+                    constexpr int per = (SMN + 27) / 28;  // spread over the first 28 steps (the last 8 carry two reads)
+                    static_for<(g * per < SMN ? g * per : SMN), ((g + 1) * per < SMN ? (g + 1) * per : SMN)>(sm_op);
+                }
+                if constexpr (DMA && g % 4 == 1) issue_load_fast(std::integral_constant<int, g / 4>{}, base, base1, dma_lds);
+            });
+        } else {
+            static_for<0, SMN>(sm_op);
+            // prime the ring with V steps 0 .. kRing-2 (two reads each; the counter of outstanding reads is 4 bits)
+            static_for<0, kRing - 1>([&](auto ic) { read_v(ic, tv); });
+        }
+    };
+
+    // ---- phase B: O += V(t)^T P(t)^T --------------------------------------------------------------------------------
+    // AHEAD: V steps requested ahead (kRing behind a phase A with matrix steps, kRing - 1 otherwise); MX: the maximum
+    // of the scores in sacc is taken on the way (steps 4 .. 14)
+    auto phase_b = [&](auto ahead_c, auto mx_c, uint32_t tv, uint32_t ka_delta) {
+        constexpr int AHEAD = decltype(ahead_c)::value;
+        constexpr bool MX = decltype(mx_c)::value;
+        static_for<0, NV>([&](auto ic) {
+            constexpr int i = decltype(ic)::value;
+            constexpr int slot = (KS + i) % kRing;
+            constexpr int left = NV - 1 - i;
+            wait_lgkm_n<2 * (left < AHEAD - 1 ? left : AHEAD - 1)>();
+            mma_o<Tag, kRingV + 4 * slot, kScV + 4 * (i & 1), 16 * (i >> 1)>();
+            if constexpr (i + AHEAD < NV) read_v(std::integral_constant<int, i + AHEAD>{}, tv);
+            if constexpr (MX && i >= 4 && i < 15) mx_op(std::integral_constant<int, i - 4>{});
+            // the K read addresses move on to the buffer of the tile after next
+            if constexpr (MX && i >= 16 && i < 16 + NKA)
+                v_add_s(ka[i - 16], ka_delta);
+        });
+    };
+
+    // the first kRing reads of a K tile (its region-A addresses were moved to it in the preceding phase B)
+#pragma unroll
+    for (int j = 0; j < NKA; ++j) ka[j] = base_a ^ (uint32_t)(32 * j);
+    auto prime_k = [&](uint32_t tb) { static_for<0, kRing>([&](auto gc) { read_k(gc, tb); }); };
+
+    // The part of the softmax of tile t that precedes phase A: running maximum (moved only when exceeded by kLazy;
+    // then the denominator and the output tiles are rescaled) and sc = scores - maximum in log2 units.  Whole tiles
+    // without ALiBi under a non-negative scale take the maximum of the raw scores from phase B.
+    // token of register r: tok0 + (r/4)*8 + half*4 + r%4
+    const bool gen_all = p.is_alibi || !(sl >= 0.0f);
+    auto softmax_head = [&](int t) {
+        const int tok0 = c0 + t * kTile;
+        const bool gen = gen_all || tok0 + kTile > c1;
+        float mx;
+        float xs[16];  // (general form only)
+        if (gen) {
+            mx = -INFINITY;
+            const float b0 = bias0 + slope * (float)tok0;
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                const int off = (r >> 2) * 8 + (r & 3);
+                // (fused so that no slope * off products are kept in registers across the loop)
+                const float x = __builtin_fmaf(sacc[r], sl, __builtin_fmaf(slope, (float)off, b0));
+                xs[r] = (tok0 + half * 4 + off) < c1 ? x : -INFINITY;
+                mx = fmaxf(mx, xs[r]);
+            }
+            mx = max_xor32(mx);
+        } else {
+            mx = mxr * sl;
+        }
+        const bool up = mx > m + kLazy;
+        if (__any(up)) {
+            const float mn = up ? mx : m;
+            const float alpha = fast_exp2(m - mn);
+            m = mn;
+            l *= alpha;
+            if (t > 0) {  // (the accumulators are still zero in the first trip)
+                static_for<0, CT * 16>([&](auto ic) { scale_acc_n<decltype(ic)::value>(alpha); });
+            }
+        }
+        if (gen) {
+            static_for<0, 16>([&](auto rc) { sc_set<decltype(rc)::value>(xs[decltype(rc)::value] - m); });
+        } else {
+            const float negm = -m;
+            static_for<0, 16>([&](auto rc) { sc_fma<decltype(rc)::value>(sacc[decltype(rc)::value], sl, negm); });
+        }
+    };
+
+    // ---- prologue: S(0) ---------------------------------------------------------------------------------------------
+    if (ntiles > 2)
+        wait_vmcnt<2 * NLW>();
+    else if (ntiles > 1)
+        wait_vmcnt<NLW>();
+    else
+        wait_vmcnt<0>();
+    __syncthreads();
+    {
+        prime_k(base_b);
+        phase_a(std::true_type{}, std::false_type{}, std::false_type{}, base_b, base_v, nullptr, nullptr, 0);
+#pragma unroll
+        for (int j = 0; j < NKA; ++j) ka[j] += (uint32_t)BUF;  // on to buffer 1
+        // the compiler does not see the matrix instructions inside the assembly: cover the result latency of the
+        // last one before anything reads the scores
+        asm volatile("s_nop 15\n\ts_nop 7" : "+v"(sacc));
+        float mx0 = sacc[0];
+#pragma unroll
+        for (int r = 1; r < 16; ++r) mx0 = fmaxf(mx0, sacc[r]);
+        mxr = max_xor32(mx0);
+    }
+
+#ifdef DA_PIPE_PROBE
+    const long long pr_t0 = clock64();
+    const long long pr_w0 = wall_clock64();
+#endif
+    // ---- all trips but the last ------------------------------------------------------------------------------------
+    // Tile t+3 goes out in trip t: a whole tile between the matrix steps of phase A (fast form), a partial tile (the
+    // split's last) or rows looked up one by one (PG) in one go behind the barrier.
+    const int nfull = (c1 - c0) / kTile;  // whole tiles
+    const bool packed = p.block_table == nullptr;
+    const uint8_t* kt3 = kbytes + (size_t)(start + c0 + (NB - 1) * kTile) * k_row_bytes;  // packed: first row of tile t+3
+    int t = 0;
+#ifdef DA_PIPE_PROBE
+    long long pr_top = 0, pr_a = 0, pr_b = 0, pr_x0 = 0, pr_x1 = 0, pr_x2 = 0;
+#endif
+    for (; t + 1 < ntiles; ++t) {
+#if DA_PIPE_PROBE > 1
+        const long long pr_s0 = clock64();
+#endif
+        const uint32_t cur = (uint32_t)((t & (NB - 1)) * BUF), nxt = (uint32_t)(((t + 1) & (NB - 1)) * BUF);
+        const bool fast = !PG && t + NB - 1 < nfull;
+        TileRows tr{nullptr, nullptr, 0};
+        if (fast) {
+            if (packed) {  // rows follow each other at the pitch
+                tr.base = kt3;
+                tr.base1 = kt3 + 16 * k_row_bytes;
+                kt3 += kTile * k_row_bytes;
+            } else {
+                tr = tile_rows(c0 + (t + NB - 1) * kTile);
+            }
+        }
+#if DA_PIPE_PROBE > 1
+        const long long pr_s0a = clock64();
+#endif
+        if (t + 2 < ntiles)
+            wait_vmcnt<NLW>();  // tile t+1 landed; tile t+2 may still be in flight
+        else
+            wait_vmcnt<0>();
+#if DA_PIPE_PROBE > 1
+        const long long pr_s0b = clock64();
+#endif
+        __syncthreads();  // every wave's share of tile t+1 is in LDS, and every wave is done with tile t-1
+#if DA_PIPE_PROBE > 1
+        const long long pr_s0c = clock64();
+        pr_x0 += pr_s0a - pr_s0;
+        pr_x1 += pr_s0b - pr_s0a;
+        pr_x2 += pr_s0c - pr_s0b;
+#endif
+        prime_k(base_b + nxt);
+        if (!fast && t + NB - 1 < ntiles) {
+            if constexpr (PG)
+                issue_tile_pg(c0 + (t + NB - 1) * kTile, (t + NB - 1) & (NB - 1));
+            else
+                issue_tile(c0 + (t + NB - 1) * kTile, (t + NB - 1) & (NB - 1));
+        }
+        softmax_head(t);
+#if DA_PIPE_PROBE > 1
+        const long long pr_s1 = clock64();
+        pr_top += pr_s1 - pr_s0;
+#endif
+        if (fast)
+            phase_a(std::true_type{}, std::true_type{}, std::true_type{}, base_b + nxt, base_v + cur, tr.base, tr.base1,
+                    smem_off + (uint32_t)(((t + NB - 1) & (NB - 1)) * BUF));
+        else
+            phase_a(std::true_type{}, std::true_type{}, std::false_type{}, base_b + nxt, base_v + cur, nullptr, nullptr, 0);
+#if DA_PIPE_PROBE > 1
+        const long long pr_s2 = clock64();
+        pr_a += pr_s2 - pr_s1;
+#endif
+        // (tile t+2 lies in buffer (t+2) % NB)
+        phase_b(std::integral_constant<int, kRing>{}, std::true_type{}, base_v + cur,
+                (uint32_t)(((t + 2) & (NB - 1)) * BUF) - nxt);
+#if DA_PIPE_PROBE > 1
+        pr_b += clock64() - pr_s2;
+#endif
+    }
+    // ---- the last trip: softmax and O += V^T P^T of the last tile -------------------------------------------------------
+    {
+        const uint32_t cur = (uint32_t)((t & (NB - 1)) * BUF);
+        softmax_head(t);
+        phase_a(std::false_type{}, std::true_type{}, std::false_type{}, 0, base_v + cur, nullptr, nullptr, 0);
+        phase_b(std::integral_constant<int, kRing - 1>{}, std::false_type{}, base_v + cur, 0);
+    }
+
+#ifdef DA_PIPE_PROBE
+    const long long pr_t1 = clock64();
+    const long long pr_w1 = wall_clock64();
+#endif
+    // finish: the two half-waves hold partial denominators over disjoint tokens
+    const float l_tot = l + __shfl_xor(l, 32);
+    // (the last matrix instructions' results must have landed before the accumulation registers are read)
+    asm volatile("s_nop 15\n\ts_nop 15" ::: "memory");
+    auto acc_at = [&](auto ic) { return read_acc_n<decltype(ic)::value>(); };
+    if (n < nh) {
+        const int h = h_base + n;
+        if (p.nsplit == 1) {
+            const float inv = 1.0f / l_tot;
+            uint16_t* orow = o16 + ((size_t)b * p.head_q + h) * DV;
+            static_for<0, CT * 4>([&](auto ic) {
+                constexpr int c = decltype(ic)::value / 4, r4 = decltype(ic)::value % 4;
+                const int col = c * 32 + r4 * 8 + half * 4;
+                ushort4 w;
+                w.x = EL::from_f32(acc_at(std::integral_constant<int, c * 16 + r4 * 4 + 0>{}) * inv);
+                w.y = EL::from_f32(acc_at(std::integral_constant<int, c * 16 + r4 * 4 + 1>{}) * inv);
+                w.z = EL::from_f32(acc_at(std::integral_constant<int, c * 16 + r4 * 4 + 2>{}) * inv);
+                w.w = EL::from_f32(acc_at(std::integral_constant<int, c * 16 + r4 * 4 + 3>{}) * inv);
+                *reinterpret_cast<ushort4*>(orow + col) = w;
+            });
+        } else {
+            const size_t part = ((size_t)b * p.head_q + h) * p.nsplit + split;
+            float* wrow = p.ws_o + part * DV;
+            static_for<0, CT * 4>([&](auto ic) {
+                constexpr int c = decltype(ic)::value / 4, r4 = decltype(ic)::value % 4;
+                const int col = c * 32 + r4 * 8 + half * 4;
+                float4 w = make_float4(acc_at(std::integral_constant<int, c * 16 + r4 * 4 + 0>{}),
+                                       acc_at(std::integral_constant<int, c * 16 + r4 * 4 + 1>{}),
+                                       acc_at(std::integral_constant<int, c * 16 + r4 * 4 + 2>{}),
+                                       acc_at(std::integral_constant<int, c * 16 + r4 * 4 + 3>{}));
+                *reinterpret_cast<float4*>(wrow + col) = w;
+            });
+            if (half == 0) {
+                p.ws_ml[part * 2 + 0] = m;
+                p.ws_ml[part * 2 + 1] = l_tot;
+            }
+#ifdef DA_PIPE_PROBE
+            if (lane == 0) {
+                wrow[0] = (float)(pr_t1 - pr_t0);
+                wrow[1] = (float)(pr_w1 - pr_w0);
+                wrow[2] = (float)pr_top;
+                wrow[3] = (float)pr_a;
+                wrow[4] = (float)pr_b;
+                wrow[5] = (float)ntiles;
+                wrow[6] = (float)(pr_w0 & 0xffffff);
+                wrow[7] = (float)(pr_w1 & 0xffffff);
+                wrow[8] = (float)pr_x0;
+                wrow[9] = (float)pr_x1;
+                wrow[10] = (float)pr_x2;
+            }
+#endif
+        }
+    }
+}
+
+template <typename Tag, bool PG>
+hipError_t launch_form(const SweepParams& p, dim3 grid, hipStream_t stream) {
+    auto kern = latent_pipe_kernel<Tag, PG>;
+    constexpr size_t lds = (size_t)kPipeBufs * kTile * 576 * 2;
+    static std::atomic<uint64_t> devices_done{0};
+    const hipError_t attr_err = ensure_lds_limit(reinterpret_cast<const void*>(kern), lds, devices_done);
+    if (attr_err != hipSuccess) return attr_err;
+    hipLaunchKernelGGL(kern, grid, dim3(256), lds, stream, p);
+    return hipGetLastError();
+}
+
+}  // namespace
+
+hipError_t launch_mla_pipe(const SweepParams& p_in, bool is_bf16, dim3 grid, hipStream_t stream) {
+    SweepParams p = p_in;
+#ifdef DA_PIPE_PROBE
+    {
+        const char* s = getenv("DA_PIPE_FLAGS");
+        p.flat_tokens = s ? atoi(s) : 0;
+    }
+#endif
+    const bool pg = p.block_table != nullptr && p.page_shift < 4;
+    if (is_bf16) return pg ? launch_form<bf16_tag, true>(p, grid, stream) : launch_form<bf16_tag, false>(p, grid, stream);
+    return pg ? launch_form<f16_tag, true>(p, grid, stream) : launch_form<f16_tag, false>(p, grid, stream);
+}
+
+}  // namespace da
