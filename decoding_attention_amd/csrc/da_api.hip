@@ -587,6 +587,7 @@ int run_attention(const void* q, const void* k, const void* v, void* o, const in
         rp.flat_wgs = pl.flat_wgs;
         rp.flat_cu = sp.flat_cu;
         rp.early = pl.ws_bytes <= ((size_t)8 << 20) ? 1 : 0;
+        rp.half_partials = da::mla_half_partials(pl.kind == kKindMfma, pl.rt, kf.fmt) ? 1 : 0;
         e = da::launch_reduce(rp, is_bf16 != 0, (int)(batch * head_q), stream);
         if (e != hipSuccess) return fail(DA_ERR_HIP, "merge kernel launch: %s", hipGetErrorString(e));
     }

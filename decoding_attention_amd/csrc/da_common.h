@@ -237,6 +237,10 @@ struct ReduceParams {
     const int32_t* flat_cu;
     // the workspace is small (cache-resident): request the first partials before the sequence's length is known
     int early;
+    // the partial outputs are normalised (divided by their denominators) and stored as 16-bit values of the output
+    // type, [rows, nsplit, dim_v] from the start of ws_o, instead of un-normalised fp32 (the pipelined latent kernel:
+    // its partials, 128 heads x 512 columns per split, are most of the traffic that splitting adds)
+    int half_partials;
 };
 
 // First token (row of the packed K/V buffers) and length of sequence b; paged sequences start at row 0 of their

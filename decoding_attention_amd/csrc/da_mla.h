@@ -10,6 +10,9 @@ int mla_rows_per_trip();
 // work-groups than this (DA_MLA_TWO_PER_CU_FROM, default 256)
 int mla_two_per_cu_from();
 hipError_t launch_mla(const SweepParams& p, bool is_bf16, int rt, dim3 grid, hipStream_t stream);
+// whether a latent-kernel launch (heads per work-group rt, K format kv_fmt: 0 = 16-bit) leaves its split partials as
+// normalised 16-bit values (ReduceParams::half_partials): the pipelined kernel does
+inline bool mla_half_partials(bool latent_kernel, int rt, int kv_fmt) { return latent_kernel && rt == 128 && kv_fmt == 0; }
 // the software-pipelined kernel for work-groups of 128 heads over 16-bit K (da_mla_pipe.hip); launch_mla routes to it
 hipError_t launch_mla_pipe(const SweepParams& p, bool is_bf16, dim3 grid, hipStream_t stream);
 // the same over an 8-bit K cache of format fmt (kKvFp8 or kKvInt8)

@@ -637,14 +637,11 @@ hipError_t launch_tag(const SweepParams& p, int rt, dim3 grid, hipStream_t strea
         case 32: return launch_one<Tag, 576, 512, 1, KV8>(p, grid, stream);
         case 64: return launch_one<Tag, 576, 512, 2, KV8>(p, grid, stream);
         case 128:
-            if constexpr (KV8 == 0) {
-                static const bool old_form = [] {
-                    const char* s = getenv("DA_MLA_OLD");
-                    return s && *s == '1';
-                }();
-                if (!old_form) return launch_mla_pipe(p, std::is_same<Tag, bf16_tag>::value, grid, stream);
-            }
-            return launch_one<Tag, 576, 512, 4, KV8>(p, grid, stream);
+            // 16-bit K: the software-pipelined kernel (da_mla_pipe.hip); this kernel's four-wave form serves 8-bit K
+            if constexpr (KV8 == 0)
+                return launch_mla_pipe(p, std::is_same<Tag, bf16_tag>::value, grid, stream);
+            else
+                return launch_one<Tag, 576, 512, 4, KV8>(p, grid, stream);
         default: return hipErrorInvalidValue;
     }
 }

@@ -166,6 +166,9 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_num_vgpr(kScV))) void la
     constexpr int NB = kPipeBufs;
     static_assert(NLB == 1 && KS == 36 && NV == 32, "schedule below is written for (576, 512), four waves");
 
+#ifdef DA_PIPE_PROBE
+    const long long pr_wk = wall_clock64();
+#endif
     extern __shared__ __attribute__((aligned(1024))) uint8_t smem[];  // NB * BUF bytes
     const uint32_t smem_off = (uint32_t)(uintptr_t)smem;
 
@@ -515,9 +518,12 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_num_vgpr(kScV))) void la
     // without ALiBi under a non-negative scale take the maximum of the raw scores from phase B.
     // token of register r: tok0 + (r/4)*8 + half*4 + r%4
     const bool gen_all = p.is_alibi || !(sl >= 0.0f);
-    auto softmax_head = [&](int t) {
+    // PLAIN (compile-time): the caller knows that this is a whole tile of a launch without ALiBi and with a
+    // non-negative scale
+    auto softmax_head = [&](int t, auto plain_c) {
+        constexpr bool PLAIN = decltype(plain_c)::value;
         const int tok0 = c0 + t * kTile;
-        const bool gen = gen_all || tok0 + kTile > c1;
+        const bool gen = !PLAIN && (gen_all || tok0 + kTile > c1);
         float mx;
         float xs[16];  // (general form only)
         if (gen) {
@@ -561,6 +567,9 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_num_vgpr(kScV))) void la
     else
         wait_vmcnt<0>();
     __syncthreads();
+#ifdef DA_PIPE_PROBE
+    const long long pr_wq = wall_clock64();
+#endif
     {
         prime_k(base_b);
         phase_a(std::true_type{}, std::false_type{}, std::false_type{}, base_b, base_v, nullptr, nullptr, 0);
@@ -589,6 +598,26 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_num_vgpr(kScV))) void la
 #ifdef DA_PIPE_PROBE
     long long pr_top = 0, pr_a = 0, pr_b = 0, pr_x0 = 0, pr_x1 = 0, pr_x2 = 0;
 #endif
+    // The common case on its own, with nothing left to decide per trip: packed rows, no ALiBi, a whole tile t+3.
+    if (!PG && packed && !gen_all) {
+        uint32_t cur = 0, nxt = (uint32_t)BUF, dst = (uint32_t)((NB - 1) * BUF);  // buffers of tiles t, t+1, t+3
+        for (; t + NB - 1 < nfull; ++t) {
+            wait_vmcnt<NLW>();  // tile t+1 landed; tile t+2 may still be in flight
+            __syncthreads();    // every wave's share of tile t+1 is in LDS, and every wave is done with tile t-1
+            prime_k(base_b + nxt);
+            softmax_head(t, std::true_type{});
+            phase_a(std::true_type{}, std::true_type{}, std::true_type{}, base_b + nxt, base_v + cur, kt3,
+                    kt3 + 16 * k_row_bytes, smem_off + dst);
+            kt3 += kTile * k_row_bytes;
+            const uint32_t nn = dst == (uint32_t)((NB - 1) * BUF) ? 0u : dst + (uint32_t)BUF;  // buffer after dst = that of tile t+4
+            // (tile t+2 lies in the buffer behind nxt)
+            const uint32_t nx2 = nxt == (uint32_t)((NB - 1) * BUF) ? 0u : nxt + (uint32_t)BUF;
+            phase_b(std::integral_constant<int, kRing>{}, std::true_type{}, base_v + cur, nx2 - nxt);
+            cur = nxt;
+            nxt = nx2;
+            dst = nn;
+        }
+    }
     for (; t + 1 < ntiles; ++t) {
 #if DA_PIPE_PROBE > 1
         const long long pr_s0 = clock64();
@@ -629,7 +658,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_num_vgpr(kScV))) void la
             else
                 issue_tile(c0 + (t + NB - 1) * kTile, (t + NB - 1) & (NB - 1));
         }
-        softmax_head(t);
+        softmax_head(t, std::false_type{});
 #if DA_PIPE_PROBE > 1
         const long long pr_s1 = clock64();
         pr_top += pr_s1 - pr_s0;
@@ -653,7 +682,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_num_vgpr(kScV))) void la
     // ---- the last trip: softmax and O += V^T P^T of the last tile -------------------------------------------------------
     {
         const uint32_t cur = (uint32_t)((t & (NB - 1)) * BUF);
-        softmax_head(t);
+        softmax_head(t, std::false_type{});
         phase_a(std::false_type{}, std::true_type{}, std::false_type{}, 0, base_v + cur, nullptr, nullptr, 0);
         phase_b(std::integral_constant<int, kRing - 1>{}, std::false_type{}, base_v + cur, 0);
     }
@@ -667,54 +696,85 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_num_vgpr(kScV))) void la
     // (the last matrix instructions' results must have landed before the accumulation registers are read)
     asm volatile("s_nop 15\n\ts_nop 15" ::: "memory");
     auto acc_at = [&](auto ic) { return read_acc_n<decltype(ic)::value>(); };
-    if (n < nh) {
-        const int h = h_base + n;
+    // The wave's 32 output rows (its heads) leave through LDS: a lane holds groups of four columns of its head's row,
+    // so storing from registers would scatter 8-byte pieces over 32 rows per instruction; instead the rows are
+    // written to the wave's own tile buffer (pitch 1040 bytes: lanes of one write fall on different banks) and read
+    // back a whole row (1 KiB, 16 bytes a lane) per instruction.  Normalised by the denominator, as 16-bit values:
+    // the final output, or (sequence split) the split's partial (ReduceParams::half_partials) beside the running
+    // maximum and the denominator as fp32.
+    __syncthreads();  // every wave is done with the tile buffers
+    {
+        constexpr int PITCH = DV * 2 + 16;  // (a multiple of 16: the rows are read back 16 bytes a lane)
+        static_assert(32 * PITCH <= BUF, "a wave's rows fit its tile buffer");
+        typedef __attribute__((address_space(3))) uint8_t* lds_ptr;
+        typedef unsigned int u32x2 __attribute__((ext_vector_type(2)));
+        typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
+        const lds_ptr wbuf = (lds_ptr)(uintptr_t)(smem_off + (uint32_t)(wave * BUF));
+        const float inv = 1.0f / l_tot;
+        static_for<0, CT * 4>([&](auto ic) {
+            constexpr int c = decltype(ic)::value / 4, r4 = decltype(ic)::value % 4;
+            const int col = c * 32 + r4 * 8 + half * 4;
+            u32x2 w;
+            w.x = (uint32_t)EL::from_f32(acc_at(std::integral_constant<int, c * 16 + r4 * 4 + 0>{}) * inv) |
+                  ((uint32_t)EL::from_f32(acc_at(std::integral_constant<int, c * 16 + r4 * 4 + 1>{}) * inv) << 16);
+            w.y = (uint32_t)EL::from_f32(acc_at(std::integral_constant<int, c * 16 + r4 * 4 + 2>{}) * inv) |
+                  ((uint32_t)EL::from_f32(acc_at(std::integral_constant<int, c * 16 + r4 * 4 + 3>{}) * inv) << 16);
+            *reinterpret_cast<__attribute__((address_space(3))) u32x2*>(wbuf + n * PITCH + col * 2) = w;
+        });
+        // (LDS operations of one wave complete in order: the wave reads its own rows back)
+        uint16_t* dst;
+        size_t row_elems;  // elements between consecutive heads' rows
         if (p.nsplit == 1) {
-            const float inv = 1.0f / l_tot;
-            uint16_t* orow = o16 + ((size_t)b * p.head_q + h) * DV;
-            static_for<0, CT * 4>([&](auto ic) {
-                constexpr int c = decltype(ic)::value / 4, r4 = decltype(ic)::value % 4;
-                const int col = c * 32 + r4 * 8 + half * 4;
-                ushort4 w;
-                w.x = EL::from_f32(acc_at(std::integral_constant<int, c * 16 + r4 * 4 + 0>{}) * inv);
-                w.y = EL::from_f32(acc_at(std::integral_constant<int, c * 16 + r4 * 4 + 1>{}) * inv);
-                w.z = EL::from_f32(acc_at(std::integral_constant<int, c * 16 + r4 * 4 + 2>{}) * inv);
-                w.w = EL::from_f32(acc_at(std::integral_constant<int, c * 16 + r4 * 4 + 3>{}) * inv);
-                *reinterpret_cast<ushort4*>(orow + col) = w;
-            });
+            dst = o16 + ((size_t)b * p.head_q + h_base) * DV;
+            row_elems = DV;
         } else {
-            const size_t part = ((size_t)b * p.head_q + h) * p.nsplit + split;
-            float* wrow = p.ws_o + part * DV;
-            static_for<0, CT * 4>([&](auto ic) {
-                constexpr int c = decltype(ic)::value / 4, r4 = decltype(ic)::value % 4;
-                const int col = c * 32 + r4 * 8 + half * 4;
-                float4 w = make_float4(acc_at(std::integral_constant<int, c * 16 + r4 * 4 + 0>{}),
-                                       acc_at(std::integral_constant<int, c * 16 + r4 * 4 + 1>{}),
-                                       acc_at(std::integral_constant<int, c * 16 + r4 * 4 + 2>{}),
-                                       acc_at(std::integral_constant<int, c * 16 + r4 * 4 + 3>{}));
-                *reinterpret_cast<float4*>(wrow + col) = w;
-            });
-            if (half == 0) {
-                p.ws_ml[part * 2 + 0] = m;
-                p.ws_ml[part * 2 + 1] = l_tot;
+            dst = reinterpret_cast<uint16_t*>(p.ws_o) + (((size_t)b * p.head_q + h_base) * p.nsplit + split) * DV;
+            row_elems = (size_t)p.nsplit * DV;
+        }
+        typedef const __attribute__((address_space(3))) u32x4* lds_row;
+        if (nh == 32) {
+            // eight rows read, then eight rows stored
+#pragma unroll
+            for (int r0 = 0; r0 < 32; r0 += 8) {
+                u32x4 v[8];
+#pragma unroll
+                for (int i = 0; i < 8; ++i) v[i] = *reinterpret_cast<lds_row>(wbuf + (r0 + i) * PITCH + lane * 16);
+#pragma unroll
+                for (int i = 0; i < 8; ++i) *reinterpret_cast<u32x4*>(dst + (size_t)(r0 + i) * row_elems + lane * 8) = v[i];
             }
-#ifdef DA_PIPE_PROBE
-            if (lane == 0) {
-                wrow[0] = (float)(pr_t1 - pr_t0);
-                wrow[1] = (float)(pr_w1 - pr_w0);
-                wrow[2] = (float)pr_top;
-                wrow[3] = (float)pr_a;
-                wrow[4] = (float)pr_b;
-                wrow[5] = (float)ntiles;
-                wrow[6] = (float)(pr_w0 & 0xffffff);
-                wrow[7] = (float)(pr_w1 & 0xffffff);
-                wrow[8] = (float)pr_x0;
-                wrow[9] = (float)pr_x1;
-                wrow[10] = (float)pr_x2;
+        } else {
+            for (int r = 0; r < nh; ++r) {
+                const u32x4 v = *reinterpret_cast<lds_row>(wbuf + r * PITCH + lane * 16);
+                *reinterpret_cast<u32x4*>(dst + (size_t)r * row_elems + lane * 8) = v;
             }
-#endif
+        }
+        if (p.nsplit > 1 && n < nh && half == 0) {
+            const size_t part = ((size_t)b * p.head_q + h_base + n) * p.nsplit + split;
+            p.ws_ml[part * 2 + 0] = m;
+            p.ws_ml[part * 2 + 1] = l_tot;
         }
     }
+#ifdef DA_PIPE_PROBE
+    if (p.nsplit > 1) {
+        // stamps into the unused upper half of the fp32-sized partial area, 16 floats per work-group
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        const long long pr_w2 = wall_clock64();
+        if (threadIdx.x == 0) {
+            float* pa = p.ws_o + (size_t)p.batch * p.head_q * p.nsplit * (DV / 2) + ((size_t)b * p.nsplit + split) * 16;
+            pa[0] = (float)(pr_t1 - pr_t0);
+            pa[1] = (float)(pr_w1 - pr_w0);
+            pa[2] = (float)pr_top;
+            pa[3] = (float)pr_a;
+            pa[4] = (float)pr_b;
+            pa[5] = (float)ntiles;
+            pa[6] = (float)(pr_wk & 0xffffff);
+            pa[7] = (float)(pr_w0 & 0xffffff);
+            pa[8] = (float)(pr_w1 & 0xffffff);
+            pa[9] = (float)(pr_w2 & 0xffffff);
+            pa[10] = (float)(pr_wq & 0xffffff);
+        }
+    }
+#endif
 }
 
 template <typename Tag, bool PG>

@@ -252,7 +252,9 @@ __global__ __launch_bounds__(256) void sweep_kernel(const SweepParams p) {
 // SG > 1 (many splits of few rows: one long sequence): SG lanes share one (row, four columns), lane j of them
 // taking splits j, j + SG, ...; a wave covers 64 / SG column groups of one row, and the SG partial sums meet through
 // lane exchanges.  The order of summation then differs from SG = 1, not the result's accuracy.
-template <typename Tag, int SG>
+// H16: the partial outputs are normalised 16-bit values (ReduceParams::half_partials); a partial's weight then
+// carries its denominator.
+template <typename Tag, int SG, bool H16 = false>
 __global__ __launch_bounds__(256) void reduce_kernel(const ReduceParams p, int rows) {
     using EL = Elem<Tag>;
     const int nc4 = p.dim_v >> 2;
@@ -273,6 +275,7 @@ __global__ __launch_bounds__(256) void reduce_kernel(const ReduceParams p, int r
     const size_t part0 = (size_t)row * p.nsplit;
     const float2* const ml = reinterpret_cast<const float2*>(p.ws_ml) + part0;
     const float4* const src = reinterpret_cast<const float4*>(p.ws_o + part0 * p.dim_v) + c4;
+    const uint2* const src16 = reinterpret_cast<const uint2*>(reinterpret_cast<const uint16_t*>(p.ws_o) + part0 * p.dim_v) + c4;
     // This lane's next four partials: slots s0, s0 + SG, ... (clamped to `last`; the caller masks the rest).
     float2 e[4];
     float4 x[4];
@@ -281,7 +284,12 @@ __global__ __launch_bounds__(256) void reduce_kernel(const ReduceParams p, int r
         for (int u = 0; u < 4; ++u) {
             const int s = min(s0 + u * SG, last);
             e[u] = ml[s];
-            x[u] = src[(size_t)s * nc4];
+            if constexpr (H16) {
+                const uint2 h = src16[(size_t)s * nc4];
+                x[u] = make_float4(EL::lo(h.x), EL::hi(h.x), EL::lo(h.y), EL::hi(h.y));
+            } else {
+                x[u] = src[(size_t)s * nc4];
+            }
         }
     };
     // A small workspace (p.early): the first four are requested before the sequence's length is known, so that
@@ -322,8 +330,9 @@ __global__ __launch_bounds__(256) void reduce_kernel(const ReduceParams p, int r
 #pragma unroll
         for (int u = 0; u < 4; ++u) {
             const bool valid = s0 + u * SG < ns;
-            const float w = valid ? fast_exp2(e[u].x - mm) : 0.0f;
-            den += valid ? w * e[u].y : 0.0f;
+            float w = valid ? fast_exp2(e[u].x - mm) : 0.0f;
+            if constexpr (H16) w = valid ? w * e[u].y : 0.0f;  // normalised partial: weight x denominator
+            den += valid ? (H16 ? w : w * e[u].y) : 0.0f;
             num.x += valid ? w * x[u].x : 0.0f;
             num.y += valid ? w * x[u].y : 0.0f;
             num.z += valid ? w * x[u].z : 0.0f;
@@ -360,6 +369,71 @@ __global__ __launch_bounds__(256) void reduce_kernel(const ReduceParams p, int r
     r.z = EL::from_f32(num.z * inv);
     r.w = EL::from_f32(num.w * inv);
     *reinterpret_cast<ushort4*>(reinterpret_cast<uint16_t*>(p.o) + (size_t)row * p.dim_v + c4 * 4) = r;
+}
+
+// The merge for normalised 16-bit partials (ReduceParams::half_partials) in its one-lane-per-element form: one thread
+// per (sequence, query head, eight output columns), 16-byte loads; the partials of four splits are fetched together.
+// A partial's weight is 2^(m_i - m) times its denominator l_i.
+template <typename Tag>
+__global__ __launch_bounds__(256) void reduce16_kernel(const ReduceParams p, int rows) {
+    using EL = Elem<Tag>;
+    const int nc8 = p.dim_v >> 3;
+    const int gid = blockIdx.x * 256 + threadIdx.x;
+    const int row = gid / nc8;  // (sequence, head) index
+    const int c8 = gid - row * nc8;
+    if (row >= rows) return;
+    const size_t part0 = (size_t)row * p.nsplit;
+    const float2* const ml = reinterpret_cast<const float2*>(p.ws_ml) + part0;
+    const uint4* const src = reinterpret_cast<const uint4*>(reinterpret_cast<const uint16_t*>(p.ws_o) + part0 * p.dim_v) + c8;
+    float2 e[4];
+    uint4 x[4];
+    auto fetch = [&](int s0, int last) {
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+            const int s = min(s0 + u, last);
+            e[u] = ml[s];
+            x[u] = src[(size_t)s * nc8];
+        }
+    };
+    if (p.early) fetch(0, p.nsplit - 1);
+    const int b = row / p.head_q;
+    const int len = p.cu_seq_k ? p.cu_seq_k[b + 1] - p.cu_seq_k[b] : p.seq_lens[b];
+    const int ns = len > 0 ? min(p.nsplit, (len + p.chunk - 1) / p.chunk) : 0;
+    float mm = kNegBig, den = 0.0f;
+    float num[8];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) num[j] = 0.0f;
+    for (int s0 = 0; s0 < ns; s0 += 4) {
+        if (!p.early || s0 != 0) fetch(s0, ns - 1);
+        float m_new = mm;
+#pragma unroll
+        for (int u = 0; u < 4; ++u)
+            if (s0 + u < ns) m_new = fmaxf(m_new, e[u].x);
+        const float keep = fast_exp2(mm - m_new);  // 0 on the first round
+        mm = m_new;
+        den *= keep;
+#pragma unroll
+        for (int j = 0; j < 8; ++j) num[j] *= keep;
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+            const float w = s0 + u < ns ? fast_exp2(e[u].x - mm) * e[u].y : 0.0f;
+            den += w;
+            const uint32_t h[4] = {x[u].x, x[u].y, x[u].z, x[u].w};
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                // (a slot past the sequence's last split holds stale data, possibly NaN: select, do not multiply by 0)
+                num[2 * j] += s0 + u < ns ? w * EL::lo(h[j]) : 0.0f;
+                num[2 * j + 1] += s0 + u < ns ? w * EL::hi(h[j]) : 0.0f;
+            }
+        }
+    }
+    const float inv = ns > 0 ? 1.0f / den : 0.0f;  // an empty sequence yields a zero row
+    uint4 r;
+    r.x = (uint32_t)EL::from_f32(num[0] * inv) | ((uint32_t)EL::from_f32(num[1] * inv) << 16);
+    r.y = (uint32_t)EL::from_f32(num[2] * inv) | ((uint32_t)EL::from_f32(num[3] * inv) << 16);
+    r.z = (uint32_t)EL::from_f32(num[4] * inv) | ((uint32_t)EL::from_f32(num[5] * inv) << 16);
+    r.w = (uint32_t)EL::from_f32(num[6] * inv) | ((uint32_t)EL::from_f32(num[7] * inv) << 16);
+    *reinterpret_cast<uint4*>(reinterpret_cast<uint16_t*>(p.o) + (size_t)row * p.dim_v + c8 * 8) = r;
 }
 
 }  // namespace da

@@ -11,7 +11,10 @@ static void launch_reduce_sg(const ReduceParams& p, int blocks, hipStream_t stre
     // SG = 1: one thread per (row, four columns); SG > 1: one wave per (row, 64 / SG column groups), four waves a block
     const long long units = SG == 1 ? (long long)blocks * nc4 : (long long)blocks * (nc4 / (64 / SG)) * 64;
     const dim3 grid((unsigned)((units + 255) / 256));
-    hipLaunchKernelGGL((reduce_kernel<Tag, SG>), grid, dim3(256), 0, stream, p, blocks);
+    if (p.half_partials)
+        hipLaunchKernelGGL((reduce_kernel<Tag, SG, true>), grid, dim3(256), 0, stream, p, blocks);
+    else
+        hipLaunchKernelGGL((reduce_kernel<Tag, SG, false>), grid, dim3(256), 0, stream, p, blocks);
 }
 
 hipError_t launch_reduce(const ReduceParams& p, bool is_bf16, int blocks, hipStream_t stream) {
@@ -21,6 +24,16 @@ hipError_t launch_reduce(const ReduceParams& p, bool is_bf16, int blocks, hipStr
     int sg = 1;
     while (sg < 8 && p.nsplit >= 8 * sg && threads * sg < (1ll << 18)) sg *= 2;
     while (sg > 1 && (p.dim_v / 4) % (64 / sg) != 0) sg /= 2;
+    // normalised 16-bit partials, one lane per element: eight columns a thread (the balanced grid never has them)
+    if (p.half_partials && sg == 1 && p.flat_tokens == 0 && p.dim_v % 8 == 0) {
+        const long long units = (long long)blocks * (p.dim_v / 8);
+        const dim3 grid((unsigned)((units + 255) / 256));
+        if (is_bf16)
+            hipLaunchKernelGGL((reduce16_kernel<bf16_tag>), grid, dim3(256), 0, stream, p, blocks);
+        else
+            hipLaunchKernelGGL((reduce16_kernel<f16_tag>), grid, dim3(256), 0, stream, p, blocks);
+        return hipGetLastError();
+    }
     switch (sg) {
         case 8: is_bf16 ? launch_reduce_sg<bf16_tag, 8>(p, blocks, stream) : launch_reduce_sg<f16_tag, 8>(p, blocks, stream); break;
         case 4: is_bf16 ? launch_reduce_sg<bf16_tag, 4>(p, blocks, stream) : launch_reduce_sg<f16_tag, 4>(p, blocks, stream); break;
