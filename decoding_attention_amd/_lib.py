@@ -14,6 +14,8 @@ EXPORTED_SYMBOLS = (
     "da_decoding_attn",
     "da_decoding_attn_ex",
     "da_workspace_bytes",
+    "da_decoding_attn_noalloc",
+    "da_noalloc_workspace_limit",
     "da_decoding_attn_paged",
     "da_workspace_bytes_paged",
     "da_decoding_attn_fp8kv",
@@ -61,6 +63,10 @@ def load():
     lib.da_decoding_attn_ex.argtypes = [vp, vp, vp, vp, vp, sz, sz, sz, sz, sz, sz, ci, ci, cf, vp, sz, vp, sz, vp]
     lib.da_workspace_bytes.restype = sz
     lib.da_workspace_bytes.argtypes = [sz, sz, sz, sz, sz, sz, sz]
+    lib.da_decoding_attn_noalloc.restype = ci
+    lib.da_decoding_attn_noalloc.argtypes = [vp, vp, vp, vp, vp, sz, sz, sz, sz, sz, sz, ci, ci, cf, vp, sz, vp]
+    lib.da_noalloc_workspace_limit.restype = sz
+    lib.da_noalloc_workspace_limit.argtypes = []
     lib.da_decoding_attn_paged.restype = ci
     lib.da_decoding_attn_paged.argtypes = [vp, vp, vp, vp, vp, vp, sz, sz, sz, sz, sz, sz, sz, sz, sz, sz, ci, ci, cf,
                                            vp, sz, vp, sz, vp]

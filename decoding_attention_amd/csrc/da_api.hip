@@ -374,6 +374,39 @@ bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) ==
 
 }  // namespace
 
+// Workspace of da_decoding_attn_noalloc: a device array that exists on every GPU the library is loaded on, from
+// load to process end.  The largest workspace any plan asks for is 256 work-groups x 128 heads x 514 floats =
+// 67.4 MB (the latent kernel's split partials), except for the balanced grid on pathologically ragged batches.
+constexpr size_t kScratchBytes = (size_t)80 << 20;
+static __device__ __align__(256) unsigned char scratch[kScratchBytes];
+
+namespace {
+
+// Device address of `scratch` on the current device (each GPU holds its own copy at its own address), looked up on
+// the first call per device.  The array's name itself is only a host-side handle.
+constexpr int kMaxDevices = 64;
+std::mutex g_scratch_mutex;
+void* g_scratch_ptr[kMaxDevices] = {};
+
+int scratch_on_current_device(void** out) {
+    int dev = 0;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return fail(DA_ERR_HIP, "hipGetDevice: %s", hipGetErrorString(e));
+    if (dev < 0 || dev >= kMaxDevices) return fail(DA_ERR_HIP, "device index %d out of range", dev);
+    std::lock_guard<std::mutex> lock(g_scratch_mutex);
+    if (g_scratch_ptr[dev] == nullptr) {
+        void* ptr = nullptr;
+        e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));
+        if (e != hipSuccess || ptr == nullptr)
+            return fail(DA_ERR_HIP, "hipGetSymbolAddress(scratch): %s", hipGetErrorString(e));
+        g_scratch_ptr[dev] = ptr;
+    }
+    *out = g_scratch_ptr[dev];
+    return DA_OK;
+}
+
+}  // namespace
+
 extern "C" {
 
 const char* da_last_error(void) { return g_last_error.c_str(); }
@@ -710,6 +743,29 @@ int da_decoding_attn_paged_int8kv(const void* q, const void* k_pages, const void
     return run_attention(q, k_pages, v_pages, o, nullptr, pg, kv8_format(da::kKvInt8, k_scale, v_scale), max_seq_k,
                          batch, head_q, head_k, dim, dim_v, is_alibi, is_bf16, softmax_scale, alibi_slopes, total_k,
                          workspace, workspace_bytes, hip_stream);
+}
+
+size_t da_noalloc_workspace_limit(void) { return kScratchBytes; }
+
+int da_decoding_attn_noalloc(const void* q, const void* k, const void* v, void* o, const int32_t* cu_seq_k,
+                             size_t max_seq_k, size_t batch, size_t head_q, size_t head_k, size_t dim, size_t dim_v,
+                             int is_alibi, int is_bf16, float softmax_scale, const float* alibi_slopes, size_t total_k,
+                             void* hip_stream) {
+    // the split partials go to the static device array; a plan that needs more than it holds is refused here, with
+    // the numbers, before anything is enqueued (the remaining argument checks are run_attention's)
+    if (head_k != 0 && head_q % head_k == 0 && supported_dims(dim, dim_v) && batch > 0) {
+        const Plan pl = make_plan(max_seq_k, batch, head_q, head_k, dim, dim_v, v != nullptr, total_k);
+        if (pl.ws_bytes > kScratchBytes)
+            return fail(DA_ERR_WORKSPACE,
+                        "this shape needs %zu bytes of split workspace, more than the %zu bytes of the static array "
+                        "da_decoding_attn_noalloc works in; use da_decoding_attn_ex with a workspace of your own",
+                        pl.ws_bytes, kScratchBytes);
+    }
+    void* ws = nullptr;
+    const int rc = scratch_on_current_device(&ws);
+    if (rc != DA_OK) return rc;
+    return run_attention(q, k, v, o, cu_seq_k, Paging{}, KvFormat{}, max_seq_k, batch, head_q, head_k, dim, dim_v, is_alibi,
+                         is_bf16, softmax_scale, alibi_slopes, total_k, ws, kScratchBytes, hip_stream);
 }
 
 int da_decoding_attn(const void* q, const void* k, const void* v, void* o, const int32_t* cu_seq_k, size_t max_seq_k,

@@ -63,6 +63,20 @@ int da_decoding_attn_ex(const void *q, const void *k, const void *v, void *o, co
                         void *workspace, size_t workspace_bytes, void *hip_stream);
 
 /*
+ * da_decoding_attn_ex for callers that cannot allocate: code under HIP graph capture, tight serving loops, harnesses
+ * that forbid hipMalloc.  No counterpart in the reference.  The split partials go to a static device array of
+ * da_noalloc_workspace_limit() bytes (80 MiB) that every GPU the library is loaded on holds until the process ends;
+ * the call allocates nothing, on the device or through any library, and returns DA_ERR_WORKSPACE (nothing enqueued)
+ * for a shape whose plan needs more.  All calls on one GPU share that array: calls that overlap on one GPU (two
+ * streams, two threads) race on it; calls on one stream do not.
+ */
+int da_decoding_attn_noalloc(const void *q, const void *k, const void *v, void *o, const int32_t *cu_seq_k,
+                             size_t max_seq_k, size_t batch, size_t head_q, size_t head_k, size_t dim, size_t dim_v,
+                             int is_alibi, int is_bf16, float softmax_scale, const float *alibi_slopes, size_t total_k,
+                             void *hip_stream);
+size_t da_noalloc_workspace_limit(void);
+
+/*
  * Bytes of workspace da_decoding_attn_ex needs for this shape (0 when the sequence is not split).
  * No counterpart in the reference, whose kernel never splits a sequence
  * (csrc/kernel/decoding_attn/decoding_fwd_launch_template.h:12-31).
