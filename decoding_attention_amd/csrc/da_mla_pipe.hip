@@ -456,10 +456,14 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_num_vgpr(kScV))) void la
 
     // ---- phase A: S(t+1) = K(t+1) Q^T beside the softmax of S(t) and the loads of tile t+3 ------------------------
     // QK: the matrix steps (else only the softmax runs: last trip); SM: the softmax (else only the matrix steps:
-    // prologue); DMA: the nine loads of a whole tile go out behind steps 1, 5, ..., 33.
+    // prologue); DMA >= 0: the nine loads of a whole tile go out behind steps DMA, DMA + 4, ..., DMA + 32.  (A
+    // direct-to-LDS load blocks its wave until the memory path accepts it, ~100 clocks at this kernel's 4 TB/s; giving
+    // each of the four waves another DMA, so that their loads do not come together, measured slower, 2970 against
+    // 2800 clocks per tile.)
     auto phase_a = [&](auto qk_c, auto sm_c, auto dma_c, uint32_t tb, uint32_t tv, const uint8_t* base,
                        const uint8_t* base1, uint32_t dma_lds) {
-        constexpr bool QK = decltype(qk_c)::value, SM = decltype(sm_c)::value, DMA = decltype(dma_c)::value;
+        constexpr bool QK = decltype(qk_c)::value, SM = decltype(sm_c)::value;
+        constexpr int DMA = decltype(dma_c)::value;
         constexpr bool VNEXT = SM;  // a trip with a softmax continues with phase B
         if constexpr (QK) {
             // the ring was primed by the caller with steps 0 .. kRing-1
@@ -479,7 +483,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_num_vgpr(kScV))) void la
                     constexpr int per = (SMN + 27) / 28;  // spread over the first 28 steps (the last 8 carry two reads)
                     static_for<(g * per < SMN ? g * per : SMN), ((g + 1) * per < SMN ? (g + 1) * per : SMN)>(sm_op);
                 }
-                if constexpr (DMA && g % 4 == 1) issue_load_fast(std::integral_constant<int, g / 4>{}, base, base1, dma_lds);
+                if constexpr (DMA >= 0 && g % 4 == (DMA >= 0 ? DMA : 0)) issue_load_fast(std::integral_constant<int, g / 4>{}, base, base1, dma_lds);
             });
         } else {
             static_for<0, SMN>(sm_op);
@@ -572,7 +576,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_num_vgpr(kScV))) void la
 #endif
     {
         prime_k(base_b);
-        phase_a(std::true_type{}, std::false_type{}, std::false_type{}, base_b, base_v, nullptr, nullptr, 0);
+        phase_a(std::true_type{}, std::false_type{}, std::integral_constant<int, -1>{}, base_b, base_v, nullptr, nullptr, 0);
 #pragma unroll
         for (int j = 0; j < NKA; ++j) ka[j] += (uint32_t)BUF;  // on to buffer 1
         // the compiler does not see the matrix instructions inside the assembly: cover the result latency of the
@@ -606,7 +610,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_num_vgpr(kScV))) void la
             __syncthreads();    // every wave's share of tile t+1 is in LDS, and every wave is done with tile t-1
             prime_k(base_b + nxt);
             softmax_head(t, std::true_type{});
-            phase_a(std::true_type{}, std::true_type{}, std::true_type{}, base_b + nxt, base_v + cur, kt3,
+            phase_a(std::true_type{}, std::true_type{}, std::integral_constant<int, 1>{}, base_b + nxt, base_v + cur, kt3,
                     kt3 + 16 * k_row_bytes, smem_off + dst);
             kt3 += kTile * k_row_bytes;
             const uint32_t nn = dst == (uint32_t)((NB - 1) * BUF) ? 0u : dst + (uint32_t)BUF;  // buffer after dst = that of tile t+4
@@ -664,10 +668,11 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_num_vgpr(kScV))) void la
         pr_top += pr_s1 - pr_s0;
 #endif
         if (fast)
-            phase_a(std::true_type{}, std::true_type{}, std::true_type{}, base_b + nxt, base_v + cur, tr.base, tr.base1,
-                    smem_off + (uint32_t)(((t + NB - 1) & (NB - 1)) * BUF));
+            phase_a(std::true_type{}, std::true_type{}, std::integral_constant<int, 1>{}, base_b + nxt, base_v + cur, tr.base,
+                    tr.base1, smem_off + (uint32_t)(((t + NB - 1) & (NB - 1)) * BUF));
         else
-            phase_a(std::true_type{}, std::true_type{}, std::false_type{}, base_b + nxt, base_v + cur, nullptr, nullptr, 0);
+            phase_a(std::true_type{}, std::true_type{}, std::integral_constant<int, -1>{}, base_b + nxt, base_v + cur, nullptr,
+                    nullptr, 0);
 #if DA_PIPE_PROBE > 1
         const long long pr_s2 = clock64();
         pr_a += pr_s2 - pr_s1;
@@ -683,7 +688,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_num_vgpr(kScV))) void la
     {
         const uint32_t cur = (uint32_t)((t & (NB - 1)) * BUF);
         softmax_head(t, std::false_type{});
-        phase_a(std::false_type{}, std::true_type{}, std::false_type{}, 0, base_v + cur, nullptr, nullptr, 0);
+        phase_a(std::false_type{}, std::true_type{}, std::integral_constant<int, -1>{}, 0, base_v + cur, nullptr, nullptr, 0);
         phase_b(std::integral_constant<int, kRing - 1>{}, std::false_type{}, base_v + cur, 0);
     }
 
