@@ -30,8 +30,18 @@ if ROOT not in sys.path:
 HBM_PEAK_GBPS = 8000.0      # MI355X HBM3E, published
 MFMA_PEAK_TFLOPS = 2500.0   # MI355X dense fp16/bf16 MFMA, published
 # HBM bytes per call from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of `bench.py --only gqa|mla`, each counter
-# scaled by what it reads for a 1 GiB device copy (profiles/*_hbm_traffic.md); valid for the default launch plan.
-MEASURED_TRAFFIC_BYTES = {"gqa": 1079830528, "mla": 471680000}
+# scaled by what it reads for a 1 GiB device copy (profiles/*_hbm_traffic.md).  A figure belongs to the launch plan
+# it was measured under; when the library plans the workload differently, the bench line carries null instead.
+MEASURED_TRAFFIC = {
+    "gqa": {"bytes": 1079830528, "plan": {"kind": 3, "nsplit": 2, "chunk": 2048, "heads_per_group": 16}},
+    "mla": {"bytes": 393961472, "plan": {"kind": 2, "nsplit": 4, "chunk": 1024, "heads_per_group": 128},
+            "partials": "16-bit"},
+}
+
+
+def measured_traffic(key, plan):
+    rec = MEASURED_TRAFFIC[key]
+    return rec["bytes"] if all(plan.get(k) == v for k, v in rec["plan"].items()) else None
 
 
 def _time_calls(torch, fn_list, steps, warmup):
@@ -179,37 +189,50 @@ def cpu_baseline(torch, w, budget_s=20.0):
     }
 
 
-def sweep_kernel_us(torch, w, reps=30):
-    """Average duration of the sweep kernel alone (the call without its merge kernel), timed with events on the
-    launch stream: the dominant kernel of the call, as a profiler's kernel trace reports it."""
+def call_and_kernel_us(torch, w, reps=50, warmup=5):
+    """Mean duration of the whole call and of its sweep kernel alone, from one loop that alternates the two on the
+    launch stream with an event between every launch (so both see the same clocks, and kernel <= call).  The call
+    is the C-ABI entry with a caller-owned workspace; the kernel alone is the probe library's sweep-only entry
+    (the same code without the merge launch).  Inputs rotate over several device copies as in measure()."""
     from decoding_attention_amd import _lib
 
-    lib = _lib.load()
-    wd = w.to(torch.device("cuda:0"))
+    lib, probe = _lib.load(), _lib.load_probe()
+    dev = torch.device("cuda:0")
+    copies = _device_copies(torch, w, dev)
     total = int(w.k.shape[0])
-    o = torch.empty(w.batch, w.head_q, w.dim_v, dtype=w.q.dtype, device="cuda:0")
+    o = torch.empty(w.batch, w.head_q, w.dim_v, dtype=w.q.dtype, device=dev)
     n = lib.da_workspace_bytes(w.max_seq_k, w.batch, w.head_q, w.head_k, w.dim, w.dim_v, total)
-    ws = torch.empty(max(n, 16), dtype=torch.uint8, device="cuda:0")
+    ws = torch.empty(max(n, 16), dtype=torch.uint8, device=dev)
     stream = torch.cuda.current_stream().cuda_stream
+    bf16 = int(w.q.dtype == torch.bfloat16)
 
-    def launch():
-        rc = lib.da_probe_sweep_only(wd.q.data_ptr(), wd.k.data_ptr(), None if wd.v is None else wd.v.data_ptr(),
-                                     o.data_ptr(), wd.cu_seq_k.data_ptr(), w.max_seq_k, w.batch, w.head_q, w.head_k,
-                                     w.dim, w.dim_v, int(w.is_alibi), int(w.q.dtype == torch.bfloat16), total,
-                                     ws.data_ptr(), n, stream)
+    def full(c):
+        rc = lib.da_decoding_attn_ex(c.q.data_ptr(), c.k.data_ptr(), None if c.v is None else c.v.data_ptr(),
+                                     o.data_ptr(), c.cu_seq_k.data_ptr(), w.max_seq_k, w.batch, w.head_q, w.head_k,
+                                     w.dim, w.dim_v, int(w.is_alibi), bf16, 0.0, None, total, ws.data_ptr(), n, stream)
         assert rc == 0, _lib.last_error()
 
-    for _ in range(3):
-        launch()
+    def sweep(c):
+        rc = probe.da_probe_sweep_only(c.q.data_ptr(), c.k.data_ptr(), None if c.v is None else c.v.data_ptr(),
+                                       o.data_ptr(), c.cu_seq_k.data_ptr(), w.max_seq_k, w.batch, w.head_q, w.head_k,
+                                       w.dim, w.dim_v, int(w.is_alibi), bf16, total, ws.data_ptr(), n, stream)
+        assert rc == 0, probe.da_last_error().decode("utf-8", "replace")
+
+    for i in range(warmup):
+        full(copies[i % len(copies)])
+        sweep(copies[i % len(copies)])
     torch.cuda.synchronize()
-    start = torch.cuda.Event(enable_timing=True)
-    end = torch.cuda.Event(enable_timing=True)
-    start.record()
-    for _ in range(reps):
-        launch()
-    end.record()
+    ev = [torch.cuda.Event(enable_timing=True) for _ in range(2 * reps + 1)]
+    ev[0].record()
+    for i in range(reps):
+        full(copies[(2 * i) % len(copies)])
+        ev[2 * i + 1].record()
+        sweep(copies[(2 * i + 1) % len(copies)])
+        ev[2 * i + 2].record()
     torch.cuda.synchronize()
-    return start.elapsed_time(end) / reps * 1e3
+    call_ms = sum(ev[2 * i].elapsed_time(ev[2 * i + 1]) for i in range(reps)) / reps
+    kern_ms = sum(ev[2 * i + 1].elapsed_time(ev[2 * i + 2]) for i in range(reps)) / reps
+    return call_ms * 1e3, kern_ms * 1e3
 
 
 def stream_read_GBps(torch, nbytes=1 << 30, reps=20):
@@ -217,7 +240,7 @@ def stream_read_GBps(torch, nbytes=1 << 30, reps=20):
     only reads (the practical ceiling for the bandwidth-bound attention kernels on this GPU)."""
     from decoding_attention_amd import _lib
 
-    lib = _lib.load()
+    lib = _lib.load_probe()
     buf = torch.empty(nbytes, dtype=torch.uint8, device="cuda:0").fill_(1)
     stream = torch.cuda.current_stream().cuda_stream
     for _ in range(3):
@@ -232,6 +255,31 @@ def stream_read_GBps(torch, nbytes=1 << 30, reps=20):
     torch.cuda.synchronize()
     ms = start.elapsed_time(end) / reps
     return lib.da_probe_stream_read_bytes(nbytes) / (ms * 1e-3) / 1e9
+
+
+def mfma_sustained_TFLOPs(torch, operand_std=1.0, iters=2000, reps=10):
+    """Matrix rate the chip sustains under its power limit: a kernel of nothing but fp16 matrix instructions on every
+    SIMD (each fed by one LDS read), operands N(0, operand_std) -- the practical ceiling for the latent kernel's
+    matrix work.  With operand_std = 0 (all zeros) the same kernel runs near the nominal clock."""
+    from decoding_attention_amd import _lib
+
+    probe = _lib.load_probe()
+    g = torch.Generator(device="cpu").manual_seed(0)
+    ops = (torch.randn(16384, generator=g) * operand_std).to(torch.float16).to("cuda:0")
+    sink = torch.empty(65536, dtype=torch.float32, device="cuda:0")
+    stream = torch.cuda.current_stream().cuda_stream
+    for _ in range(3):
+        assert probe.da_probe_mfma_rate(ops.data_ptr(), iters, sink.data_ptr(), stream) == 0
+    torch.cuda.synchronize()
+    start = torch.cuda.Event(enable_timing=True)
+    end = torch.cuda.Event(enable_timing=True)
+    start.record()
+    for _ in range(reps):
+        probe.da_probe_mfma_rate(ops.data_ptr(), iters, sink.data_ptr(), stream)
+    end.record()
+    torch.cuda.synchronize()
+    ms = start.elapsed_time(end) / reps
+    return probe.da_probe_mfma_rate_flops(iters) / (ms * 1e-3) / 1e12
 
 
 def run_default(args):
@@ -252,7 +300,7 @@ def run_default(args):
         del src, dst
     gqa_w = wl.config_gqa_fixed(seed=0)
     if args.only == "mla":
-        mla = measure(torch, wl.config_mla(64, 4096), args.steps, args.warmup)
+        mla = measure(torch, wl.config_mla(64, 4096), max(50, args.steps), max(5, args.warmup))
         print(json.dumps({"only": "mla", **mla}))
         return 0
     gqa = measure(torch, gqa_w, args.steps, args.warmup)
@@ -261,11 +309,16 @@ def run_default(args):
         return 0
     mla = None
     if not args.no_mla:
+        # (under this kernel the chip's clock moves in slow waves, 82-119 us per launch over some hundred launches in
+        # a kernel trace: a long warm-up and a long run, so that the mean is the sustained one)
         mla_w = wl.config_mla(64, 4096)
-        mla = measure(torch, mla_w, max(5, args.steps // 2), max(2, args.warmup // 2))
-        mla["kernel_us"] = sweep_kernel_us(torch, mla_w)
+        mla = measure(torch, mla_w, max(300, args.steps), max(100, args.warmup))
+        mla["interleaved_call_us"], mla["kernel_us"] = call_and_kernel_us(torch, mla_w, reps=max(150, args.steps),
+                                                                           warmup=max(10, args.warmup))
+        mfma_rand = mfma_sustained_TFLOPs(torch, 1.0)
+        mfma_zero = mfma_sustained_TFLOPs(torch, 0.0)
     stream_gbps = stream_read_GBps(torch)
-    sweep_us = sweep_kernel_us(torch, gqa_w)
+    gqa_call_us, sweep_us = call_and_kernel_us(torch, gqa_w, reps=max(30, args.steps), warmup=max(5, args.warmup))
     sweep_gbps = gqa["algorithmic_bytes"] / (sweep_us * 1e-6) / 1e9
     cpu = None if args.no_cpu else cpu_baseline(torch, gqa_w, args.cpu_budget)
 
@@ -291,8 +344,8 @@ def run_default(args):
         # the dominant kernel (the grouped-head sweep) on its own: algorithmic bytes of the call over its average
         # launch duration, timed in this run with events on the launch stream
         "roofline": {"bound": "hbm", "achieved": sweep_gbps, "peak": HBM_PEAK_GBPS, "unit": "GB/s",
-                     "frac": sweep_gbps / HBM_PEAK_GBPS, "traffic": MEASURED_TRAFFIC_BYTES["gqa"],
-                     "kernel": "gqa_mfma_kernel", "kernel_us": sweep_us,
+                     "frac": sweep_gbps / HBM_PEAK_GBPS, "traffic": measured_traffic("gqa", gqa["plan"]),
+                     "kernel": "gqa_mfma_kernel", "kernel_us": sweep_us, "interleaved_call_us": gqa_call_us,
                      "whole_call": {"achieved": gqa["hbm_GBps"], "frac": gqa["hbm_frac_of_peak"],
                                     "kernels": "gqa_mfma_kernel + reduce_kernel"},
                      # measured in this run: a kernel that only streams 1 GiB from HBM, and the sweep against it
@@ -308,15 +361,21 @@ def run_default(args):
             "tflops": mla["tflops"], "pct_mfma_peak": 100.0 * mla["mfma_frac_of_peak"],
             "algorithmic_bytes": mla["algorithmic_bytes"], "algorithmic_flops": mla["algorithmic_flops"],
             "input_copies_rotated": mla["input_copies_rotated"], "plan": mla["plan"],
-            # both for the latent MFMA kernel alone (kernel_us, events on the launch stream, back-to-back launches)
+            # both for the latent MFMA kernel alone: kernel_us from a loop that alternates the whole call and the kernel
+            # alone, an event between every launch (interleaved_call_us is the whole call in that same loop)
             "roofline": {"bound": "hbm", "achieved": mla["algorithmic_bytes"] / (mla["kernel_us"] * 1e-6) / 1e9,
                          "peak": HBM_PEAK_GBPS, "unit": "GB/s",
                          "frac": mla["algorithmic_bytes"] / (mla["kernel_us"] * 1e-6) / 1e9 / HBM_PEAK_GBPS,
-                         "traffic": MEASURED_TRAFFIC_BYTES["mla"], "kernel": "mfma_latent_kernel",
-                         "kernel_us": mla["kernel_us"]},
+                         "traffic": measured_traffic("mla", mla["plan"]), "kernel": "latent_pipe_kernel",
+                         "kernel_us": mla["kernel_us"], "interleaved_call_us": mla["interleaved_call_us"]},
             "roofline_mfma": {"bound": "mfma", "achieved": mla["algorithmic_flops"] / (mla["kernel_us"] * 1e-6) / 1e12,
                               "peak": MFMA_PEAK_TFLOPS, "unit": "TFLOP/s",
-                              "frac": mla["algorithmic_flops"] / (mla["kernel_us"] * 1e-6) / 1e12 / MFMA_PEAK_TFLOPS},
+                              "frac": mla["algorithmic_flops"] / (mla["kernel_us"] * 1e-6) / 1e12 / MFMA_PEAK_TFLOPS,
+                              # measured in this run: nothing but matrix instructions on every SIMD, with N(0,1)
+                              # operands (what the power limit leaves) and with zeros (near the nominal clock)
+                              "sustained_TFLOPs_random_operands": mfma_rand,
+                              "sustained_TFLOPs_zero_operands": mfma_zero,
+                              "frac_of_sustained": mla["algorithmic_flops"] / (mla["kernel_us"] * 1e-6) / 1e12 / mfma_rand},
         }
     print(json.dumps(line))
     return 0

@@ -25,9 +25,6 @@ EXPORTED_SYMBOLS = (
     "da_decoding_attn_paged_int8kv",
     "da_workspace_bytes_int8kv",
     "da_plan",
-    "da_probe_stream_read",
-    "da_probe_sweep_only",
-    "da_probe_stream_read_bytes",
     "da_supported_head_dims",
     "da_last_error",
     "da_version",
@@ -87,12 +84,6 @@ def load():
     lib.da_decoding_attn_paged_int8kv.argtypes = lib.da_decoding_attn_paged_fp8kv.argtypes
     lib.da_workspace_bytes_int8kv.restype = sz
     lib.da_workspace_bytes_int8kv.argtypes = lib.da_workspace_bytes_fp8kv.argtypes
-    lib.da_probe_stream_read.restype = ci
-    lib.da_probe_stream_read.argtypes = [vp, sz, vp, vp]
-    lib.da_probe_sweep_only.restype = ci
-    lib.da_probe_sweep_only.argtypes = [vp, vp, vp, vp, vp, sz, sz, sz, sz, sz, sz, ci, ci, sz, vp, sz, vp]
-    lib.da_probe_stream_read_bytes.restype = sz
-    lib.da_probe_stream_read_bytes.argtypes = [sz]
     ip = ctypes.POINTER(ci)
     lib.da_plan.restype = ci
     lib.da_plan.argtypes = [sz, sz, sz, sz, sz, sz, ci, sz, ip, ip, ip, ip]
@@ -103,6 +94,35 @@ def load():
     lib.da_version.restype = ci
     lib.da_version.argtypes = []
     _lib = lib
+    return lib
+
+
+PROBE_LIB_PATH = os.path.join(PKG_DIR, "libdecoding_attn_probe.so")
+_probe = None
+
+
+def load_probe():
+    """The benchmark's measurement aids (include/decoding_attn_probe.h): a second build of the library with the
+    sweep-only entry point and the streaming-read kernel.  Not part of the drop-in ABI; only bench.py loads it."""
+    global _probe
+    if _probe is not None:
+        return _probe
+    if not os.path.exists(PROBE_LIB_PATH):
+        raise LibraryNotBuilt(f"{PROBE_LIB_PATH} is missing: build it with `python -m decoding_attention_amd.build`")
+    lib = ctypes.CDLL(PROBE_LIB_PATH)
+    vp, sz, ci = ctypes.c_void_p, ctypes.c_size_t, ctypes.c_int
+    lib.da_probe_stream_read.restype = ci
+    lib.da_probe_stream_read.argtypes = [vp, sz, vp, vp]
+    lib.da_probe_sweep_only.restype = ci
+    lib.da_probe_sweep_only.argtypes = [vp, vp, vp, vp, vp, sz, sz, sz, sz, sz, sz, ci, ci, sz, vp, sz, vp]
+    lib.da_probe_stream_read_bytes.restype = sz
+    lib.da_probe_stream_read_bytes.argtypes = [sz]
+    lib.da_probe_mfma_rate.restype = ci
+    lib.da_probe_mfma_rate.argtypes = [vp, ci, vp, vp]
+    lib.da_probe_mfma_rate_flops.restype = ctypes.c_double
+    lib.da_probe_mfma_rate_flops.argtypes = [ci]
+    lib.da_last_error.restype = ctypes.c_char_p
+    _probe = lib
     return lib
 
 

@@ -25,8 +25,11 @@ SOURCES = [
     "da_sweep_kv8.hip",
     "da_gqa_mfma_kv8.hip",
     "da_gqa_mfma_i8.hip",
-    "da_probe.hip",
 ]
+
+# libdecoding_attn_probe.so (measurement aids of bench.py, include/decoding_attn_probe.h): the same objects, with
+# da_api.hip compiled once more with the sweep-only entry point, plus the streaming-read kernel.
+PROBE_LIB_PATH = os.path.join(PKG_DIR, "libdecoding_attn_probe.so")
 
 # packed-fp32 VALU forms are switched off on purpose: only scalar fp32 arithmetic is emitted.
 HIPCC_FLAGS = [
@@ -51,9 +54,10 @@ EXTRA_FLAGS = {
 ISA_CHECKED = {"da_mla_pipe.hip"}
 
 
-def _compile(src):
-    obj = os.path.join(OBJ_DIR, os.path.splitext(src)[0] + ".o")
-    cmd = [_hipcc()] + HIPCC_FLAGS + EXTRA_FLAGS.get(src, []) + ["-c", os.path.join(CSRC, src), "-o", obj]
+def _compile(src, obj_name=None, defines=()):
+    obj = os.path.join(OBJ_DIR, (obj_name or os.path.splitext(src)[0]) + ".o")
+    cmd = ([_hipcc()] + HIPCC_FLAGS + EXTRA_FLAGS.get(src, []) + [f"-D{d}" for d in defines] +
+           ["-c", os.path.join(CSRC, src), "-o", obj])
     if os.environ.get("DA_SAVE_TEMPS"):
         cmd += ["-save-temps=obj"]
     res = subprocess.run(cmd, capture_output=True, text=True)
@@ -82,6 +86,15 @@ def build(force=True, verbose=False):
     res = subprocess.run(cmd, capture_output=True, text=True)
     if res.returncode != 0:
         raise RuntimeError(f"link failed:\n{res.stdout}\n{res.stderr}")
+    # the probe library: every object but da_api.o, da_api.hip with the probe entry point, the streaming-read kernel
+    api_probe, _ = _compile("da_api.hip", obj_name="da_api_probe", defines=("DA_BUILD_PROBES",))
+    stream_probe, _ = _compile("da_probe.hip")
+    api_obj = os.path.join(OBJ_DIR, "da_api.o")
+    cmd = ([_hipcc(), "--offload-arch=gfx950", "-shared", "-fPIC", "-o", PROBE_LIB_PATH] +
+           [o for o in objs if o != api_obj] + [api_probe, stream_probe])
+    res = subprocess.run(cmd, capture_output=True, text=True)
+    if res.returncode != 0:
+        raise RuntimeError(f"link of the probe library failed:\n{res.stdout}\n{res.stderr}")
     return LIB_PATH
 
 

@@ -15,6 +15,9 @@
 #include <utility>
 
 #include "../../include/decoding_attn_hip.h"
+#ifdef DA_BUILD_PROBES
+#include "../../include/decoding_attn_probe.h"
+#endif
 #include "da_gqa_mfma.h"
 #include "da_mla.h"
 #include "da_sweep_launch.h"
@@ -669,6 +672,8 @@ int da_decoding_attn_ex(const void* q, const void* k, const void* v, void* o, co
                          is_bf16, softmax_scale, alibi_slopes, total_k, workspace, workspace_bytes, hip_stream);
 }
 
+#ifdef DA_BUILD_PROBES
+// (libdecoding_attn_probe.so only, declared in include/decoding_attn_probe.h)
 int da_probe_sweep_only(const void* q, const void* k, const void* v, void* o, const int32_t* cu_seq_k, size_t max_seq_k,
                         size_t batch, size_t head_q, size_t head_k, size_t dim, size_t dim_v, int is_alibi, int is_bf16,
                         size_t total_k, void* workspace, size_t workspace_bytes, void* hip_stream) {
@@ -677,6 +682,7 @@ int da_probe_sweep_only(const void* q, const void* k, const void* v, void* o, co
     return run_attention(q, k, v, o, cu_seq_k, Paging{}, kf, max_seq_k, batch, head_q, head_k, dim, dim_v, is_alibi,
                          is_bf16, 0.0f, nullptr, total_k, workspace, workspace_bytes, hip_stream);
 }
+#endif
 
 int da_decoding_attn_paged(const void* q, const void* k_pages, const void* v_pages, void* o,
                            const int32_t* block_table, const int32_t* seq_lens, size_t max_seq_k, size_t batch,

@@ -210,46 +210,12 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_num_vgpr(kScV))) void la
         return;
     }
 
-    // Q rows of this wave's heads as B-operands: lane (n, half) holds Q[head n][ks*16 + half*8 .. +8).  The wave's
-    // 32 x 576 block of Q is staged like a K tile (whole-row direct-to-LDS loads, same swizzle, into the wave's own
-    // buffer) and read back with the K-row read pattern, which is the same operand layout.
     const int q_last = max(nh, 1) - 1;
     const int hq = min(h_base + min(n, q_last), p.head_q - 1);
     const uint32_t lane16 = lane * 16;
     const int rb = lane >> 3;  // region B: row within the group of eight, chunk lane & 7
-    {
-        const uint8_t* const qb = reinterpret_cast<const uint8_t*>(p.q) + (size_t)b * p.head_q * (D * 2);
-        const uint32_t qbuf = smem_off + wave * BUF;
-        static_for<0, kTile>([&](auto rc) {
-            constexpr int row = decltype(rc)::value;
-            const int head = min(h_base + min(row, q_last), p.head_q - 1);  // wave-uniform
-            lds_dma16(qb, (uint32_t)head * (uint32_t)(D * 2) + (lane16 ^ (uint32_t)(swz_a(row) * 16)),
-                      qbuf + (uint32_t)(row * ROW_A));
-        });
-        static_for<0, kTile / 8>([&](auto jc) {
-            constexpr int j = decltype(jc)::value;
-            const int row = j * 8 + rb;
-            const int head = min(h_base + min(row, q_last), p.head_q - 1);
-            lds_dma16(qb, (uint32_t)head * (uint32_t)(D * 2) + (uint32_t)(DV * 2 + (((lane & 7) ^ swz_b(row)) * 16)),
-                      qbuf + (uint32_t)(OFF_B + j * 1024));
-        });
-        wait_vmcnt<0>();
-        const uint32_t qa = qbuf + n * ROW_A + ((swz_a(n) ^ half) * 16);
-        const uint32_t qbb = qbuf + OFF_B + n * ROW_B + ((swz_b(n) ^ half) * 16);
-        static_for<0, KS>([&](auto ic) {
-            constexpr int ks = decltype(ic)::value;
-            uint32_t tmp;
-            if constexpr (ks < 32)
-                ring_read_b128<kQV + 4 * ks, 32 * (ks & 7), (ks >> 3) * 256>(qa, tmp);
-            else
-                ring_read_b128<kQV + 4 * ks, 32 * (ks - 32), 0>(qbb, tmp);
-            if constexpr (ks % 12 == 11) wait_lgkm_n<0>();  // the counter of outstanding reads is 4 bits wide
-        });
-    }
-    __syncthreads();  // the tile buffers are free for K once every wave has its Q in registers
     const float slope = p.is_alibi ? alibi_slope_log2(p.slopes, hq, p.head_q) : 0.0f;
 
-    static_for<0, CT * 16>([&](auto ic) { asm volatile("v_accvgpr_write_b32 a[%0], 0" ::"n"(decltype(ic)::value)); });
     float m = kNegBig, l = 0.0f;
 
     const uint8_t* const kbytes = reinterpret_cast<const uint8_t*>(p.k) + (size_t)hk * D * 2;
@@ -327,15 +293,79 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_num_vgpr(kScV))) void la
     };
 
     const int ntiles = (c1 - c0 + kTile - 1) / kTile;
-    // tiles 0 .. 2 go out at once (buffers 0 .. 2); tile t + 3 follows in trip t
+    auto issue_any = [&](int i) {
+        if constexpr (PG)
+            issue_tile_pg(c0 + i * kTile, i);
+        else
+            issue_tile(c0 + i * kTile, i);
+    };
+    // Tile 0 goes out at once (buffer 0), tile 1 behind the second round of Q, tile 2 when Q is through, tile t + 3
+    // in trip t: the first trip needs Q and tile 0 only, and every work-group of the grid asks for them at the same
+    // moment, so nothing else competes with them.
+    if (0 < ntiles) issue_any(0);
+
+    // Q rows of this wave's heads as B-operands: lane (n, half) holds Q[head n][ks*16 + half*8 .. +8).  The wave's
+    // 32 x 576 block of Q is staged like a K tile (whole-row direct-to-LDS loads, same swizzle) and read back with
+    // the K-row read pattern, which is the same operand layout.  Q passes through buffers 2 and 3, two blocks at a
+    // time, so that the first K tiles can be on their way meanwhile (all four blocks at once would need the whole
+    // LDS).
+    // this wave's share (region-A rows wave + 4 q, region-B rows 8 wave .. 8 wave + 7) of the Q block of wave `blk`
+    // (its 32 heads), into tile buffer 2 + blk % 2: the four waves fetch a block together, as they fetch a K tile,
+    // because a direct-to-LDS load holds its wave for ~100 clocks (36 of them in a row would be the prologue's longest
+    // stretch)
+    auto issue_q_share = [&](int blk) {
+        const uint8_t* const qb = reinterpret_cast<const uint8_t*>(p.q) + (size_t)b * p.head_q * (D * 2);
+        const int first = hk * p.ratio + grp * 32 * NWV + blk * 32;  // first head of the block
+        const int last_row = max(min(32, wg_heads - blk * 32), 1) - 1;  // rows past the block's live heads repeat one
+        const uint32_t qbuf = smem_off + (uint32_t)((2 + (blk & 1)) * BUF);
 #pragma unroll
-    for (int i = 0; i < NB - 1; ++i)
-        if (i < ntiles) {
-            if constexpr (PG)
-                issue_tile_pg(c0 + i * kTile, i);
-            else
-                issue_tile(c0 + i * kTile, i);
+        for (int q = 0; q < NLA; ++q) {
+            const int row = wave + NWV * q;  // wave-uniform
+            const int head = min(first + min(row, last_row), p.head_q - 1);
+            lds_dma16(qb, (uint32_t)head * (uint32_t)(D * 2) + (lane16 ^ (uint32_t)(swz_a(row) * 16)),
+                      qbuf + (uint32_t)(row * ROW_A));
         }
+        {
+            const int row = wave * 8 + rb;
+            const int head = min(first + min(row, last_row), p.head_q - 1);
+            lds_dma16(qb, (uint32_t)head * (uint32_t)(D * 2) + (uint32_t)(DV * 2 + (((lane & 7) ^ swz_b(row)) * 16)),
+                      qbuf + (uint32_t)(OFF_B + wave * 1024));
+        }
+    };
+    auto read_q = [&]() {
+        const uint32_t qbuf = smem_off + (uint32_t)((2 + (wave & 1)) * BUF);
+        const uint32_t qa = qbuf + n * ROW_A + ((swz_a(n) ^ half) * 16);
+        const uint32_t qbb = qbuf + OFF_B + n * ROW_B + ((swz_b(n) ^ half) * 16);
+        static_for<0, KS>([&](auto ic) {
+            constexpr int ks = decltype(ic)::value;
+            uint32_t tmp;
+            if constexpr (ks < 32)
+                ring_read_b128<kQV + 4 * ks, 32 * (ks & 7), (ks >> 3) * 256>(qa, tmp);
+            else
+                ring_read_b128<kQV + 4 * ks, 32 * (ks - 32), 0>(qbb, tmp);
+            if constexpr (ks % 12 == 11) wait_lgkm_n<0>();  // the counter of outstanding reads is 4 bits wide
+        });
+    };
+    issue_q_share(0);
+    issue_q_share(1);
+    // (while the loads are on their way) the output tiles start at zero
+    static_for<0, CT * 16>([&](auto ic) { asm volatile("v_accvgpr_write_b32 a[%0], 0" ::"n"(decltype(ic)::value)); });
+    wait_vmcnt<0>();
+    __syncthreads();  // the Q blocks of waves 0 and 1 (and tile 0) are in LDS
+    if ((wave >> 1) == 0) read_q();
+    __syncthreads();  // ... and in registers: buffers 2 and 3 take the blocks of waves 2 and 3
+    issue_q_share(2);
+    issue_q_share(3);
+    if (1 < ntiles) {
+        issue_any(1);
+        wait_vmcnt<NLW>();  // (loads complete in order: tile 1's may stay outstanding)
+    } else {
+        wait_vmcnt<0>();
+    }
+    __syncthreads();
+    if ((wave >> 1) == 1) read_q();
+    __syncthreads();  // buffers 2 and 3 are free for K
+    if (2 < ntiles) issue_any(2);
 
     // The fast form of a tile's loads, for whole tiles (no row past the end) between the matrix steps of phase A: the
     // row part of the address is added to the tile's base in scalar registers, the lane part is one XOR.

@@ -188,25 +188,6 @@ int da_supported_head_dims(size_t dim, size_t dim_v);
  * DA_CHECK / DA_CHECK_CUDART_ERROR macros (csrc/common/common.h:17-49). */
 const char *da_last_error(void);
 
-/*
- * Measurement aid (no counterpart in the reference): enqueue a plain streaming read of `bytes` bytes at `buf`
- * (device memory, 16-byte aligned, at least 128 MiB).  It reads da_probe_stream_read_bytes(bytes) of them, in
- * contiguous slabs with 16-byte loads.  Timing it gives the bandwidth HBM delivers to a kernel that only reads,
- * the practical ceiling for the bandwidth-bound attention kernels.  `sink` may be NULL.
- */
-int da_probe_stream_read(const void *buf, size_t bytes, void *sink, void *hip_stream);
-
-/*
- * Measurement aid (no counterpart in the reference): da_decoding_attn_ex without its merge kernel, so that the sweep
- * kernel of a call can be timed on its own with events.  When the plan splits the sequences the output rows are not
- * written (the partials stay in the workspace); never use it for results.
- */
-int da_probe_sweep_only(const void *q, const void *k, const void *v, void *o, const int32_t *cu_seq_k,
-                        size_t max_seq_k, size_t batch, size_t head_q, size_t head_k, size_t dim, size_t dim_v,
-                        int is_alibi, int is_bf16, size_t total_k, void *workspace, size_t workspace_bytes,
-                        void *hip_stream);
-size_t da_probe_stream_read_bytes(size_t bytes);
-
 /* Library version, major * 10000 + minor * 100 + patch (reference decoding_attn/__init__.py:15 holds "0.1.0"). */
 int da_version(void);
 
