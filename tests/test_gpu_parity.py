@@ -10,7 +10,7 @@ import torch
 
 from decoding_attention_amd import _lib, decoding_attn_fwd, fwd
 from decoding_attention_amd import workloads as wl
-from gpu_util import TOL, check_against_oracle, run_hip, run_oracle, sub_workload
+from gpu_util import TOL, check_against_oracle, run_hip, run_hip_ex, run_oracle, sub_workload
 
 pytestmark = pytest.mark.gpu
 DTYPES = [torch.float16, torch.bfloat16]
@@ -45,10 +45,22 @@ def test_reference_grid_mla(head_q, batch, seq_k, dtype):
     check_against_oracle(w, run_hip(w))
 
 
-@pytest.mark.parametrize("batch,seq_k", [(1, 128), (8, 128), (32, 128), (1, 512), (1, 1536), (1, 4096), (1, 8192)])
+@pytest.mark.parametrize("batch,seq_k", [(1, 128), (8, 128), (32, 128), (128, 128), (512, 128), (1, 512), (1, 1536),
+                                          (1, 4096), (1, 8192)])
 def test_config1_mha_sweep_points(batch, seq_k):
+    """Every point of the two sweeps (batch 2048 below), every row against the oracle."""
     w = wl.config_mha_sweep(batch, seq_k)
     check_against_oracle(w, run_hip(w))
+
+
+def test_config1_mha_sweep_batch_2048():
+    """The largest point of the batch sweep: all 2048 x 32 rows finite, every 16th sequence against the oracle."""
+    w = wl.config_mha_sweep(2048, 128)
+    o = run_hip(w)
+    assert torch.isfinite(o.float()).all()
+    rows = list(range(0, 2048, 16)) + [2047]
+    _, ref32 = run_oracle(sub_workload(w, rows))
+    assert (o[rows].float() - ref32).abs().max().item() <= TOL[torch.float16]
 
 
 def test_config2_gqa_varlen_scaled():
@@ -56,52 +68,65 @@ def test_config2_gqa_varlen_scaled():
     check_against_oracle(w, run_hip(w))
 
 
-def test_config2_gqa_varlen_full_size_spot_checked():
+def test_config2_gqa_varlen_full_size_every_row():
+    """BASELINE's ragged batch (64 sequences of 1..8192 tokens, balanced grid): every row against the oracle."""
     w = wl.config_gqa_varlen(seed=0)
-    o = run_hip(w)
-    assert torch.isfinite(o.float()).all()
-    order = sorted(range(w.batch), key=lambda b: w.lengths[b])
-    rows = [order[0], order[1], order[len(order) // 2], order[-1]]  # shortest, median, longest
-    sub = sub_workload(w, rows)
-    _, ref32 = run_oracle(sub)
-    assert (o[rows].float() - ref32).abs().max().item() <= TOL[torch.bfloat16]
+    check_against_oracle(w, run_hip(w))
 
 
-def test_config2_gqa_fixed_4096_spot_checked():
+def test_config2_gqa_varlen_full_size_without_token_count():
+    """The same batch as a caller of the reference-signature entry sees it planned (no token count: fixed splits)."""
+    w = wl.config_gqa_varlen(seed=0)
+    check_against_oracle(w, run_hip_ex(w, 0))
+
+
+def test_config2_gqa_fixed_4096_every_row():
     w = wl.config_gqa_fixed(seed=0)
-    o = run_hip(w)
-    rows = [0, 31, 63]
-    _, ref32 = run_oracle(sub_workload(w, rows))
-    assert (o[rows].float() - ref32).abs().max().item() <= TOL[torch.bfloat16]
+    check_against_oracle(w, run_hip(w))
+
+
+@pytest.mark.parametrize("batch", [40, 48, 100])
+def test_gqa_batches_that_refill_the_grid(batch):
+    """Batch sizes whose first plan fills its last round of CUs poorly and is re-planned: every row."""
+    w = wl.config_gqa_fixed(seed=batch, batch=batch)
+    check_against_oracle(w, run_hip(w))
 
 
 def test_config3_mqa_alibi_scaled_and_full():
     w = wl.config_mqa_alibi(seed=2, batch=4, seq_k=1024)
     check_against_oracle(w, run_hip(w))
-    w = wl.config_mqa_alibi(seed=0)
-    o = run_hip(w)
-    rows = [0, 17]
-    _, ref32 = run_oracle(sub_workload(w, rows))
-    assert (o[rows].float() - ref32).abs().max().item() <= TOL[torch.float16]
+    w = wl.config_mqa_alibi(seed=0)  # BASELINE's shape (batch 32, 4096 tokens): every row
+    check_against_oracle(w, run_hip(w))
 
 
-@pytest.mark.parametrize("batch,seq_k", [(1, 4096), (16, 512), (2, 16384)])
+@pytest.mark.parametrize("batch,seq_k", [(1, 4096), (16, 512), (16, 1024), (16, 2048), (16, 4096), (2, 16384)])
 def test_config4_mla_points(batch, seq_k):
+    """Points of BASELINE's two latent sweeps that the oracle does whole in seconds: every row."""
+    w = wl.config_mla(batch, seq_k)
+    check_against_oracle(w, run_hip(w))
+
+
+@pytest.mark.parametrize("batch,seq_k,step", [(16, 8192, 3), (16, 16384, 5), (128, 4096, 16)])
+def test_config4_mla_large_points(batch, seq_k, step):
+    """The largest points of the two sweeps: every output finite, every step-th sequence (and the last) against the
+    oracle."""
     w = wl.config_mla(batch, seq_k)
     o = run_hip(w)
-    rows = [0] if batch == 1 else [0, batch - 1]
-    sub = sub_workload(w, rows)
-    _, ref32 = run_oracle(sub)
-    assert (o[rows].float() - ref32).abs().max().item() <= TOL[torch.float16]
-
-
-def test_config4_mla_b64_full_size_spot_checked():
-    w = wl.config_mla(64, 4096)
-    o = run_hip(w)
     assert torch.isfinite(o.float()).all()
-    rows = [5, 63]
+    rows = sorted(set(range(0, batch, step)) | {batch - 1})
     _, ref32 = run_oracle(sub_workload(w, rows))
     assert (o[rows].float() - ref32).abs().max().item() <= TOL[torch.float16]
+
+
+def test_config4_mla_b64_full_size_every_row():
+    """BASELINE's headline latent shape (batch 64, 4096 tokens, 4 sequence splits of 16-bit partials): every row."""
+    w = wl.config_mla(64, 4096)
+    check_against_oracle(w, run_hip(w))
+
+
+def test_config4_mla_b64_bf16_every_row():
+    w = wl.config_mla(64, 4096, dtype=torch.bfloat16)
+    check_against_oracle(w, run_hip(w))
 
 
 @pytest.mark.parametrize("dtype", DTYPES, ids=_name)
