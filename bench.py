@@ -13,9 +13,10 @@ cu_seq_k) divided by the mean time of one call, inputs resident in HBM.  Calls a
 stream the kernels are launched on.  Working sets below 512 MB are rotated over several input copies so the
 256 MB Infinity Cache cannot serve them.
 
-`--sweep` prints the reference's two sweeps (batch sweep at seq_k 128, sequence sweep at batch 1, and the
-MLA equivalents) in the reference's log format
-(reference benchmarks/python/benchmark_decoding_attn.py:248-249, formulas :52-57).
+`--sweep mha|mla` prints the reference's two sweeps for that head shape (its `Benchmark Seq` section at batch 1,
+then its `Benchmark Batch` section, with the reference's full lists) in the reference's log format, which the
+reference's plot script reads (reference benchmarks/python/benchmark_decoding_attn.py:248-249 and :303-330,
+formulas :52-57); `--sweep baseline` the remaining benchmark shapes; `--sweep all` all three.
 """
 import argparse
 import json
@@ -34,7 +35,7 @@ MFMA_PEAK_TFLOPS = 2500.0   # MI355X dense fp16/bf16 MFMA, published
 # it was measured under; when the library plans the workload differently, the bench line carries null instead.
 MEASURED_TRAFFIC = {
     "gqa": {"bytes": 1079830528, "plan": {"kind": 3, "nsplit": 2, "chunk": 2048, "heads_per_group": 16}},
-    "mla": {"bytes": 393961472, "plan": {"kind": 2, "nsplit": 4, "chunk": 1024, "heads_per_group": 128},
+    "mla": {"bytes": 388052992, "plan": {"kind": 2, "nsplit": 4, "chunk": 1024, "heads_per_group": 128},
             "partials": "16-bit"},
 }
 
@@ -381,41 +382,97 @@ def run_default(args):
     return 0
 
 
-def run_sweep(args):
-    """The reference's sweeps, printed in its log format (one line per shape)."""
+# The reference's sweep lists (benchmarks/python/benchmark_decoding_attn.py:303-330): sequence lengths at batch 1,
+# then batches at one length, for the head shape given on its command line (run_python.sh:25-31: MHA 32/32 x 128,
+# MLA 128/1 x 576/512).
+REF_SWEEPS = {
+    "mha": {"heads": (32, 32, 128, 128),
+            "seq_ks": [1, 8, 16, 32, 64, 128, 256, 512, 1024, 2048, 3072, 4096, 5120, 6144, 7168, 8192],
+            "batch_seq_k": 128},
+    "mla": {"heads": (128, 1, 576, 512),
+            "seq_ks": [256, 512, 1024, 2048, 3072, 4096, 5120, 6144, 7168, 8192],
+            "batch_seq_k": 4096},
+}
+REF_BATCHES = [1, 2, 4, 8, 16, 32, 64, 128, 256, 512, 768, 1024, 1536, 2048]
+SEQ_MARKER = "------------------------------- Benchmark Seq -------------------------------"
+BATCH_MARKER = "------------------------------- Benchmark Batch -------------------------------"
+
+
+def reference_log_line(batch, seq_k, ms, tflops, gbps):
+    """One result in the reference's log format (benchmarks/python/benchmark_decoding_attn.py:248-249): its plot
+    script (tools/performance/python/performance.py:82-104) splits the line at spaces and reads token 0 as the
+    method, token 1 as batch-seq_k, token 7 as TFLOPS and token 10 as GB/s."""
+    return (f"Decoding-Attention {batch}-{seq_k} profiling time: {ms:.4f} ms, throughput: {tflops:.4f} TFLOPS, "
+            f"bandwidth: {gbps:.3f} GB/s")
+
+
+def sweep_sections(kind):
+    """The shapes `--sweep kind` measures, as (section marker or None, tag, workload arguments) in print order.
+    `mha` and `mla` are the reference's two sections with its full lists; `baseline` holds the benchmark shapes
+    those lists leave out (the ragged and fixed GQA batches, MQA with ALiBi, sequence length 1536, and the latent
+    form's length sweep at batch 16)."""
+    out = []
+    for fam in ("mha", "mla"):
+        if kind in (fam, "all"):
+            r = REF_SWEEPS[fam]
+            out += [(SEQ_MARKER if i == 0 else None, f"{fam}-seq", (fam, 1, sk)) for i, sk in enumerate(r["seq_ks"])]
+            out += [(BATCH_MARKER if i == 0 else None, f"{fam}-batch", (fam, b, r["batch_seq_k"]))
+                    for i, b in enumerate(REF_BATCHES)]
+    if kind in ("baseline", "gqa", "all"):
+        title = "------------------------------- Other shapes -------------------------------"
+        out += [(title, "gqa-varlen", ("gqa-varlen",)), (None, "gqa-fixed", ("gqa-fixed",)),
+                (None, "mqa-alibi", ("mqa-alibi",)), (None, "mha-seq", ("mha", 1, 1536))]
+        out += [(None, "mla-seq-b16", ("mla", 16, sk)) for sk in (512, 1024, 2048, 4096, 8192, 16384)]
+    return out
+
+
+def _sweep_workload(torch, wl, spec, device):
+    if spec[0] == "mha":
+        hq, hk, d, dv = REF_SWEEPS["mha"]["heads"]
+        return wl.make_workload(spec[1], hq, hk, d, dv, spec[2], torch.float16, device=device)
+    if spec[0] == "mla":
+        hq, hk, d, dv = REF_SWEEPS["mla"]["heads"]
+        return wl.make_workload(spec[1], hq, hk, d, dv, spec[2], torch.float16, device=device)
+    return {"gqa-varlen": wl.config_gqa_varlen, "gqa-fixed": wl.config_gqa_fixed, "mqa-alibi": wl.config_mqa_alibi}[spec[0]]()
+
+
+def run_sweep(args, measure_fn=None, workload_fn=None, out=None):
+    """The reference's sweeps, printed in its log format: per head shape a header line, the `Benchmark Seq` marker
+    and one line per sequence length, the `Benchmark Batch` marker and one line per batch (the reference's plot script
+    cuts the log at the second marker; give it the log of one family, `--sweep mha` or `--sweep mla`).  Lines that
+    start with four spaces carry this build's own figures and are skipped by that script (no `TFLOPS` in them)."""
     import torch
 
     from decoding_attention_amd import workloads as wl
 
-    shapes = []
-    if args.sweep in ("mha", "all"):
-        shapes += [("mha-batch", wl.config_mha_sweep(b, 128)) for b in (1, 8, 32, 128, 512, 2048)]
-        shapes += [("mha-seq", wl.config_mha_sweep(1, s)) for s in (128, 512, 1536, 4096, 8192)]
-    if args.sweep in ("mla", "all"):
-        shapes += [("mla-batch", wl.config_mla(b, 4096)) for b in (1, 16, 64, 128)]
-        shapes += [("mla-seq", wl.config_mla(16, s)) for s in (512, 1024, 2048, 4096, 8192, 16384)]
-    if args.sweep in ("gqa", "all"):
-        shapes += [("gqa-varlen", wl.config_gqa_varlen()), ("gqa-fixed", wl.config_gqa_fixed()),
-                   ("mqa-alibi", wl.config_mqa_alibi())]
+    out = out or sys.stdout
+    measure_fn = measure_fn or measure  # (tests of the log format pass their own, and shapes without data)
+    workload_fn = workload_fn or (lambda spec: _sweep_workload(torch, wl, spec, "cuda:0"))
+    shapes = [(m, tag, spec, {}) for m, tag, spec in sweep_sections(args.sweep)]
     if args.sweep == "paged":  # the benchmark shapes over shuffled pages of 64, 16 and 1 tokens, beside the packed layout
         for w in (wl.config_gqa_fixed(), wl.config_gqa_varlen(), wl.config_mqa_alibi(), wl.config_mla(64, 4096)):
-            shapes += [("packed", w), ("paged-64", w), ("paged-16", w), ("paged-1", w)]
+            shapes += [(None, "packed", w, {})] + [(None, f"paged-{n}", w, {"page_size": n}) for n in (64, 16, 1)]
     if args.sweep == "fp8":  # 16-bit against FP8 and int8 K/V on the bandwidth-bound shapes and the latent form
         for w in (wl.config_gqa_fixed(), wl.config_mha_sweep(512, 128), wl.config_mha_sweep(1, 8192),
                   wl.config_mqa_alibi(), wl.config_mla(64, 4096), wl.config_mla(16, 4096)):
-            shapes += [("kv16", w), ("kv-fp8", w), ("kv-int8", w)]
+            shapes += [(None, "kv16", w, {}), (None, "kv-fp8", w, {"kv_fp8": True}), (None, "kv-int8", w, {"kv_int8": True})]
     results = []
-    for tag, w in shapes:
-        r = measure(torch, w, args.steps, args.warmup, page_size=int(tag[6:]) if tag.startswith("paged-") else 0,
-                    kv_fp8=tag == "kv-fp8", kv_int8=tag == "kv-int8")
+    for marker, tag, spec, kw in shapes:
+        if marker == SEQ_MARKER:
+            hq, hk, d, dv = REF_SWEEPS[spec[0]]["heads"]
+            print(f"Benchmark Decoding Attention: head q: {hq}, head k: {hk}, dim: {d}, dim v: {dv}, is alibi: False, "
+                  f"is bf16: False, warmup iterations: {args.warmup}, profiling iterations: {args.steps}", file=out)
+        if marker:
+            print(marker, file=out, flush=True)
+        w = workload_fn(spec) if isinstance(spec, tuple) else spec
+        r = measure_fn(torch, w, args.steps, args.warmup, **kw)
         ms = r["us_per_call"] / 1e3
         sk = w.max_seq_k
         ref_bytes = wl.reference_formula_bytes(w.batch, w.head_q, w.head_k, w.dim, w.dim_v, sk)
-        print(f"Decoding-Attention {w.batch}-{sk} profiling time: {ms:.4f} ms, throughput: {r['tflops']:.4f} TFLOPS, "
-              f"bandwidth: {ref_bytes / (ms * 1e-3) / 1e9:.3f} GB/s", flush=True)
+        print(reference_log_line(w.batch, sk, ms, r["tflops"], ref_bytes / (ms * 1e-3) / 1e9), file=out, flush=True)
         print(f"    [{tag}] {w.name}: {r['us_per_call']:.1f} us/call (min {r['us_isolated_call_min']:.1f}), "
               f"{r['hbm_GBps'] / 1e3:.3f} TB/s of real traffic = {100 * r['hbm_frac_of_peak']:.1f}% of "
-              f"{HBM_PEAK_GBPS / 1e3:.0f} TB/s, plan {r['plan']}", flush=True)
+              f"{HBM_PEAK_GBPS / 1e3:.0f} TB/s, plan {r['plan']}", file=out, flush=True)
         r["tag"] = tag
         results.append(r)
         del w
@@ -437,7 +494,7 @@ def main():
     ap.add_argument("--calibrate-copy", action="store_true", help="first run three 1 GiB device copies (a known "
                     "traffic figure for scaling profiler byte counters)")
     ap.add_argument("--cpu-budget", type=float, default=15.0, help="seconds of single-thread CPU work to sample")
-    ap.add_argument("--sweep", choices=["mha", "mla", "gqa", "all", "paged", "fp8"], help="print the reference's sweeps instead "
+    ap.add_argument("--sweep", choices=["mha", "mla", "baseline", "gqa", "all", "paged", "fp8"], help="print the reference's sweeps instead "
                     "(paged / fp8: benchmark shapes over a paged or an 8-bit, FP8 and int8, K/V cache)")
     ap.add_argument("--json-out", help="with --sweep: also write the results as JSON")
     args = ap.parse_args()

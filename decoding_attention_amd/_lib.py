@@ -14,6 +14,7 @@ EXPORTED_SYMBOLS = (
     "da_decoding_attn",
     "da_decoding_attn_ex",
     "da_workspace_bytes",
+    "da_release_workspaces",
     "da_decoding_attn_noalloc",
     "da_noalloc_workspace_limit",
     "da_decoding_attn_paged",
@@ -60,6 +61,8 @@ def load():
     lib.da_decoding_attn_ex.argtypes = [vp, vp, vp, vp, vp, sz, sz, sz, sz, sz, sz, ci, ci, cf, vp, sz, vp, sz, vp]
     lib.da_workspace_bytes.restype = sz
     lib.da_workspace_bytes.argtypes = [sz, sz, sz, sz, sz, sz, sz]
+    lib.da_release_workspaces.restype = ci
+    lib.da_release_workspaces.argtypes = []
     lib.da_decoding_attn_noalloc.restype = ci
     lib.da_decoding_attn_noalloc.argtypes = [vp, vp, vp, vp, vp, sz, sz, sz, sz, sz, sz, ci, ci, cf, vp, sz, vp]
     lib.da_noalloc_workspace_limit.restype = sz

@@ -289,6 +289,11 @@ Plan make_plan(size_t max_seq_k, size_t batch, size_t head_q, size_t head_k, siz
     // longer split loses again, batch 32 x 16384 tokens 360 -> 377 us with 4096-token splits)
     if (pl.kind == kKindGroup && !latent_group && total_k > 0 && !ragged && !kv_8bit && (packed || page_size >= 16))
         by_cap = base >= 512 ? 1 : ((long long)max_seq_k + 2047) / 2048;
+    // ... and without a token count (the reference-signature entry point) the same kernel at d = 128 caps at 2048
+    // tokens: as good as the counted plan on a uniform batch and better than the 1024 cap on a ragged one (measured,
+    // 32/8 heads, batch 64: 4096 tokens each 184.6 -> 181.6 us, 181.4 with the count; 1..8192 tokens 264.7 -> 246.1 us)
+    if (pl.kind == kKindGroup && !latent_group && total_k == 0 && dim == 128 && !kv_8bit && (packed || page_size >= 16))
+        by_cap = ((long long)max_seq_k + 2047) / 2048;
     // (one round of long splits beats two rounds with the second nearly empty)
     if (latent_group && base <= target_wgs && base * by_cap > target_wgs) by_cap = 1;
     long long ns = std::max(std::min(want, by_len), std::min(by_cap, by_len));
@@ -346,6 +351,12 @@ struct CachedWs {
 };
 std::mutex g_ws_mutex;
 std::map<std::pair<int, void*>, CachedWs> g_ws;
+bool g_ws_exit_hook = false;
+int release_cached_workspaces(bool report);
+// Registered when the first workspace is allocated, so after the HIP runtime set itself up: exit handlers run in
+// reverse order of registration, which hands the workspaces back while the runtime is still there (at process exit,
+// and when the library is unloaded, where the handlers of a shared object run too).
+void release_at_exit() { (void)release_cached_workspaces(false); }
 
 // Workspace of the reference-signature entry point: one buffer per (device, stream), grown on demand.
 int cached_workspace(size_t bytes, hipStream_t stream, void** out) {
@@ -368,9 +379,34 @@ int cached_workspace(size_t bytes, hipStream_t stream, void** out) {
             return fail(DA_ERR_HIP, "hipMalloc(workspace, %zu): %s", want, hipGetErrorString(e));
         }
         w.bytes = want;
+        if (!g_ws_exit_hook) {
+            g_ws_exit_hook = true;
+            (void)std::atexit(release_at_exit);
+        }
     }
     *out = w.ptr;
     return DA_OK;
+}
+
+// Free every cached workspace (the caller vouches that no enqueued call still uses one).  Errors are reported for an
+// explicit release and ignored at exit or unload.
+int release_cached_workspaces(bool report) {
+    std::lock_guard<std::mutex> lock(g_ws_mutex);
+    int rc = DA_OK;
+    if (g_ws.empty()) return rc;  // (and no call into the HIP runtime: it may be gone already)
+    int prev = 0;
+    const bool have_prev = hipGetDevice(&prev) == hipSuccess;
+    for (auto& kv : g_ws) {
+        if (!kv.second.ptr) continue;
+        hipError_t e = hipSetDevice(kv.first.first);
+        if (e == hipSuccess) e = hipFree(kv.second.ptr);
+        if (e != hipSuccess && report) rc = fail(DA_ERR_HIP, "hipFree(workspace): %s", hipGetErrorString(e));
+        kv.second.ptr = nullptr;
+        kv.second.bytes = 0;
+    }
+    g_ws.clear();
+    if (have_prev) (void)hipSetDevice(prev);
+    return rc;
 }
 
 bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
@@ -511,7 +547,8 @@ int run_attention(const void* q, const void* k, const void* v, void* o, const in
                     dim, dim_v);
     if (!aligned16(q) || !aligned16(k) || (v && !aligned16(v)))
         return fail(DA_ERR_INVALID_ARGUMENT, "q, k and v must be 16-byte aligned");
-    if ((reinterpret_cast<uintptr_t>(o) & 1u) != 0) return fail(DA_ERR_INVALID_ARGUMENT, "o must be 2-byte aligned");
+    // (every finishing path stores 8 or 16 bytes of a row at a time; rows are multiples of 128 bytes)
+    if (!aligned16(o)) return fail(DA_ERR_INVALID_ARGUMENT, "o must be 16-byte aligned");
     if (max_seq_k > (size_t)INT32_MAX || batch > 65535 || head_q > 65535)
         return fail(DA_ERR_INVALID_ARGUMENT, "shape out of range (max_seq_k %zu, batch %zu, head_q %zu; grid limit 65535)",
                     max_seq_k, batch, head_q);
@@ -750,6 +787,8 @@ int da_decoding_attn_paged_int8kv(const void* q, const void* k_pages, const void
                          batch, head_q, head_k, dim, dim_v, is_alibi, is_bf16, softmax_scale, alibi_slopes, total_k,
                          workspace, workspace_bytes, hip_stream);
 }
+
+int da_release_workspaces(void) { return release_cached_workspaces(true); }
 
 size_t da_noalloc_workspace_limit(void) { return kScratchBytes; }
 

@@ -55,15 +55,17 @@ def get_cu_seq(seqs: torch.Tensor) -> torch.Tensor:
 
 
 def make_workload(batch, head_q, head_k, dim, dim_v, seq_k, dtype, *, seed=0, varlen=False, latent=None,
-                  is_alibi=False, name=None, min_len=1) -> Workload:
+                  is_alibi=False, name=None, min_len=1, device="cpu") -> Workload:
     """Build one workload.
 
     ``seq_k`` is the common length, or the inclusive upper bound of uniform random lengths
     when ``varlen`` is set.  ``latent`` (default: dim != dim_v) makes V alias K[..., :dim_v].
+    ``device`` other than the CPU draws q/k/v there (a different random stream: for timing, not for the parity
+    tests, whose inputs are the CPU stream's).
     """
     if latent is None:
         latent = dim != dim_v
-    g = torch.Generator(device="cpu").manual_seed(seed)
+    g = torch.Generator(device=device).manual_seed(seed)
     if varlen:
         # lengths are drawn last in the stream order, but are needed first to size K/V;
         # use a generator forked from the same seed so that the order stays reproducible.
@@ -72,12 +74,14 @@ def make_workload(batch, head_q, head_k, dim, dim_v, seq_k, dtype, *, seed=0, va
     else:
         lens = torch.full((batch,), seq_k, dtype=torch.int32)
     total_k = int(lens.sum().item())
-    q = torch.randn(batch, head_q, dim, generator=g, dtype=torch.float32).to(dtype)
-    k = torch.randn(total_k, head_k, dim, generator=g, dtype=torch.float32).to(dtype)
+    on_cpu = str(device) == "cpu"
+    draw_dtype = torch.float32 if on_cpu else dtype  # (the CPU stream is fp32 rounded to 16 bits)
+    q = torch.randn(batch, head_q, dim, generator=g, dtype=draw_dtype, device=device).to(dtype)
+    k = torch.randn(total_k, head_k, dim, generator=g, dtype=draw_dtype, device=device).to(dtype)
     v = None
     if not latent:
-        v = torch.randn(total_k, head_k, dim_v, generator=g, dtype=torch.float32).to(dtype)
-    cu = get_cu_seq(lens)
+        v = torch.randn(total_k, head_k, dim_v, generator=g, dtype=draw_dtype, device=device).to(dtype)
+    cu = get_cu_seq(lens).to(device)
     max_seq_k = int(lens.max().item()) if batch > 0 else 0
     if name is None:
         name = f"b{batch}_hq{head_q}_hk{head_k}_d{dim}_dv{dim_v}_sk{seq_k}{'_var' if varlen else ''}_" \
@@ -113,7 +117,7 @@ def to_pages(w: Workload, page_size: int, *, seed=0, combined=False, spare_pages
     shows up in the output (poison=False fills with zeros instead, for integer-typed byte views).  combined=True builds one [pages, 2, page_size, head_k, dim] pool (K and V interleaved
     per page, dim == dim_v) and returns its two halves as views.
     """
-    g = torch.Generator(device="cpu").manual_seed(seed)
+    g = torch.Generator(device=device).manual_seed(seed)
     lens = w.lengths
     blocks = [(n + page_size - 1) // page_size for n in lens]
     max_blocks = max(1, max(blocks))

@@ -36,9 +36,10 @@ extern "C" {
  * Same argument order and meaning; softmax scale is 1/sqrt(dim) (decoding_attn.cpp:54) and the ALiBi slope of
  * head h is 2^(-8(h+1)/head_q) (csrc/kernel/decoding_attn/block_info.h:21).
  *   q [batch, head_q, dim]; k [total_k, head_k, dim]; v [total_k, head_k, dim_v] or NULL (MLA);
- *   o [batch, head_q, dim_v]; cu_seq_k [batch + 1] int32 prefix offsets; q/k/v 16-byte aligned.
+ *   o [batch, head_q, dim_v]; cu_seq_k [batch + 1] int32 prefix offsets; q/k/v/o 16-byte aligned.
  * Split-sequence partials live in a workspace the library keeps per (device, stream) and grows on demand
- * (growth calls hipMalloc; steady-state calls allocate nothing).  Use da_decoding_attn_ex to bring your own.
+ * (growth calls hipMalloc; steady-state calls allocate nothing); da_release_workspaces() frees them, and they are
+ * freed at process exit or when the library is unloaded.  Use da_decoding_attn_ex to bring your own.
  */
 int da_decoding_attn(const void *q, const void *k, const void *v, void *o, const int32_t *cu_seq_k, size_t max_seq_k,
                      size_t batch, size_t head_q, size_t head_k, size_t dim, size_t dim_v, int is_alibi, int is_bf16,
@@ -61,6 +62,13 @@ int da_decoding_attn_ex(const void *q, const void *k, const void *v, void *o, co
                         size_t max_seq_k, size_t batch, size_t head_q, size_t head_k, size_t dim, size_t dim_v,
                         int is_alibi, int is_bf16, float softmax_scale, const float *alibi_slopes, size_t total_k,
                         void *workspace, size_t workspace_bytes, void *hip_stream);
+
+/*
+ * Frees the workspaces da_decoding_attn (and da_decoding_attn_ex with workspace == NULL) keeps per (device, stream),
+ * for long-lived processes that cycle through streams.  The caller must have synchronised every stream whose calls
+ * may still use one.  No counterpart in the reference (its kernel needs no workspace).
+ */
+int da_release_workspaces(void);
 
 /*
  * da_decoding_attn_ex for callers that cannot allocate: code under HIP graph capture, tight serving loops, harnesses

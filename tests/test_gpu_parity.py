@@ -269,6 +269,54 @@ def test_reference_signature_entry_point_with_library_workspace():
     check_against_oracle(w, o.cpu())
 
 
+def test_reference_signature_entry_point_takes_the_plan_of_a_uniform_batch():
+    """BASELINE's GQA shape (batch 64 x 4096 tokens, 32/8 heads) through da_decoding_attn, which is told no token
+    count: the same cut as the counted call (two splits of 2048 tokens), so the same bits and the same time as the
+    Python face; and the library's cached workspace can be released and is allocated again on the next call."""
+    lib = _lib.load()
+    w = wl.config_gqa_fixed(seed=0)
+    dev = torch.device("cuda:0")
+    wd = w.to(dev)
+    o = torch.full((64, 32, 128), float("nan"), dtype=w.q.dtype, device=dev)
+    stream = torch.cuda.current_stream().cuda_stream
+
+    def ref_sig():
+        rc = lib.da_decoding_attn(wd.q.data_ptr(), wd.k.data_ptr(), wd.v.data_ptr(), o.data_ptr(),
+                                  wd.cu_seq_k.data_ptr(), 4096, 64, 32, 8, 128, 128, 0,
+                                  int(w.q.dtype == torch.bfloat16), stream)
+        assert rc == 0, _lib.last_error()
+
+    def python_face():
+        return decoding_attn_fwd(wd.q, wd.k, wd.v, wd.cu_seq_k, wd.max_seq_k, 128, False)
+
+    ref_sig()
+    o_face = python_face()
+    torch.cuda.synchronize()
+    assert torch.equal(o, o_face)
+
+    def us_per_call(fn, reps=100):
+        for _ in range(10):
+            fn()
+        a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        a.record()
+        for _ in range(reps):
+            fn()
+        b.record()
+        b.synchronize()
+        return a.elapsed_time(b) * 1000.0 / reps
+
+    t_ref, t_face = us_per_call(ref_sig), us_per_call(python_face)
+    print(f"GQA b64 sk4096: da_decoding_attn {t_ref:.1f} us/call, Python face {t_face:.1f} us/call")
+    assert t_ref <= t_face * 1.03 + 1.0
+
+    torch.cuda.synchronize()
+    assert lib.da_release_workspaces() == 0, _lib.last_error()
+    o.fill_(float("nan"))
+    ref_sig()
+    torch.cuda.synchronize()
+    assert torch.equal(o, o_face)
+
+
 def test_total_k_hint_changes_the_plan_not_the_result():
     """A ragged batch through da_decoding_attn_ex with and without the token-count hint; both match the oracle."""
     lib = _lib.load()

@@ -49,6 +49,7 @@ def test_argument_errors_without_gpu():
     assert _call_ex(lib, d=80, dv=80) == _lib.DA_ERR_UNSUPPORTED and "unsupported" in _lib.last_error()
     assert _call_ex(lib, d=128, dv=64) == _lib.DA_ERR_UNSUPPORTED
     assert _call_ex(lib, q=24) == _lib.DA_ERR_INVALID_ARGUMENT and "aligned" in _lib.last_error()
+    assert _call_ex(lib, o=24) == _lib.DA_ERR_INVALID_ARGUMENT and "o must be 16-byte aligned" in _lib.last_error()
     assert _call_ex(lib, batch=0) == _lib.DA_OK  # nothing to do, nothing launched
 
 
@@ -91,19 +92,32 @@ def test_plan_total_k_hint_changes_the_splits_and_never_the_kernel():
     assert ragged["nsplit"] * ragged["chunk"] >= sk
 
 
+def test_plan_without_a_token_count_at_d128():
+    """The reference-signature entry point passes no token count: the grouped kernel at d = 128 then cuts a sequence
+    into splits of up to 2048 tokens, on a uniform batch the same cut as the plan that knows the count."""
+    blind = _lib.plan(4096, 64, 32, 8, 128, 128)
+    counted = _lib.plan(4096, 64, 32, 8, 128, 128, total_k=64 * 4096)
+    assert blind["kind"] == counted["kind"] == 3
+    assert (blind["nsplit"], blind["chunk"]) == (counted["nsplit"], counted["chunk"]) == (2, 2048)
+    assert _lib.load().da_release_workspaces() == _lib.DA_OK  # nothing cached, nothing to free, no GPU needed
+
+
 def test_workspace_sizes_of_the_paged_and_fp8_variants():
     lib = _lib.load()
     shape = (4096, 64, 32, 8, 128, 128)
     packed = lib.da_workspace_bytes(*shape, 0)
-    # pages of any size take the packed layout's kernels and plan
-    for page in (1, 8, 16, 64, 256):
+    # pages of 16 tokens and more take the packed layout's kernels and plan; shorter pages keep the shorter splits
+    for page in (16, 64, 256):
         assert lib.da_workspace_bytes_paged(*shape, 0, page) == packed
-    assert lib.da_workspace_bytes_fp8kv(*shape, 0, 0) == packed          # same kernel kind, same plan
+    for page in (1, 8):
+        assert lib.da_workspace_bytes_paged(*shape, 0, page) >= packed
+    # 8-bit K/V: the same kernel kind, with the shorter splits its half-length rows were measured on
+    assert lib.da_workspace_bytes_fp8kv(*shape, 0, 0) >= packed
     # the latent form: the larger of the MFMA kernel's plan (V inside K) and the VALU sweep's (a distinct V buffer)
     mla = (4096, 16, 128, 1, 576, 512)
     assert lib.da_workspace_bytes_fp8kv(*mla, 0, 0) > 0
     assert lib.da_workspace_bytes_fp8kv(128, 4, 6, 4, 64, 64, 0, 0) == 0   # head_q not a multiple of head_k
-    assert lib.da_workspace_bytes_int8kv(*shape, 0, 0) == packed and lib.da_workspace_bytes_int8kv(*mla, 0, 0) > 0
+    assert lib.da_workspace_bytes_int8kv(*shape, 0, 0) == lib.da_workspace_bytes_fp8kv(*shape, 0, 0) and lib.da_workspace_bytes_int8kv(*mla, 0, 0) > 0
 
 
 def test_plan_rejects_bad_shapes():
