@@ -117,7 +117,7 @@ def to_pages(w: Workload, page_size: int, *, seed=0, combined=False, spare_pages
     shows up in the output (poison=False fills with zeros instead, for integer-typed byte views).  combined=True builds one [pages, 2, page_size, head_k, dim] pool (K and V interleaved
     per page, dim == dim_v) and returns its two halves as views.
     """
-    g = torch.Generator(device=device).manual_seed(seed)
+    g = torch.Generator(device="cpu").manual_seed(seed)
     lens = w.lengths
     blocks = [(n + page_size - 1) // page_size for n in lens]
     max_blocks = max(1, max(blocks))
