@@ -190,11 +190,13 @@ def cpu_baseline(torch, w, budget_s=20.0):
     }
 
 
-def call_and_kernel_us(torch, w, reps=50, warmup=5):
-    """Mean duration of the whole call and of its sweep kernel alone, from one loop that alternates the two on the
-    launch stream with an event between every launch (so both see the same clocks, and kernel <= call).  The call
-    is the C-ABI entry with a caller-owned workspace; the kernel alone is the probe library's sweep-only entry
-    (the same code without the merge launch).  Inputs rotate over several device copies as in measure()."""
+def call_and_kernel_us(torch, w, reps=50, warmup=5, group=4):
+    """Mean duration of the whole call and of its sweep kernel alone, from one loop that alternates groups of
+    `group` calls and `group` kernel-alone launches on the launch stream with an event between the groups (so both
+    see the same clocks and kernel <= call; an event costs a few microseconds of stream time, which the group
+    spreads).  The call is the C-ABI entry with a caller-owned workspace; the kernel alone is the probe library's
+    sweep-only entry (the same code without the merge launch).  Inputs rotate over several device copies as in
+    measure()."""
     from decoding_attention_amd import _lib
 
     lib, probe = _lib.load(), _lib.load_probe()
@@ -223,16 +225,22 @@ def call_and_kernel_us(torch, w, reps=50, warmup=5):
         full(copies[i % len(copies)])
         sweep(copies[i % len(copies)])
     torch.cuda.synchronize()
-    ev = [torch.cuda.Event(enable_timing=True) for _ in range(2 * reps + 1)]
+    rounds = max(1, -(-reps // group))
+    ev = [torch.cuda.Event(enable_timing=True) for _ in range(2 * rounds + 1)]
     ev[0].record()
-    for i in range(reps):
-        full(copies[(2 * i) % len(copies)])
+    j = 0
+    for i in range(rounds):
+        for _ in range(group):
+            full(copies[j % len(copies)])
+            j += 1
         ev[2 * i + 1].record()
-        sweep(copies[(2 * i + 1) % len(copies)])
+        for _ in range(group):
+            sweep(copies[j % len(copies)])
+            j += 1
         ev[2 * i + 2].record()
     torch.cuda.synchronize()
-    call_ms = sum(ev[2 * i].elapsed_time(ev[2 * i + 1]) for i in range(reps)) / reps
-    kern_ms = sum(ev[2 * i + 1].elapsed_time(ev[2 * i + 2]) for i in range(reps)) / reps
+    call_ms = sum(ev[2 * i].elapsed_time(ev[2 * i + 1]) for i in range(rounds)) / (rounds * group)
+    kern_ms = sum(ev[2 * i + 1].elapsed_time(ev[2 * i + 2]) for i in range(rounds)) / (rounds * group)
     return call_ms * 1e3, kern_ms * 1e3
 
 

@@ -26,6 +26,7 @@ EXPORTED_SYMBOLS = (
     "da_decoding_attn_paged_int8kv",
     "da_workspace_bytes_int8kv",
     "da_plan",
+    "da_plan_distinct_v",
     "da_supported_head_dims",
     "da_last_error",
     "da_version",
@@ -90,6 +91,8 @@ def load():
     ip = ctypes.POINTER(ci)
     lib.da_plan.restype = ci
     lib.da_plan.argtypes = [sz, sz, sz, sz, sz, sz, ci, sz, ip, ip, ip, ip]
+    lib.da_plan_distinct_v.restype = ci
+    lib.da_plan_distinct_v.argtypes = [sz, sz, sz, sz, sz, sz, sz, sz, ip, ip, ip, ip]
     lib.da_supported_head_dims.restype = ci
     lib.da_supported_head_dims.argtypes = [sz, sz]
     lib.da_last_error.restype = ctypes.c_char_p
@@ -133,12 +136,17 @@ def last_error() -> str:
     return load().da_last_error().decode("utf-8", "replace")
 
 
-def plan(max_seq_k, batch, head_q, head_k, dim, dim_v, is_bf16=False, total_k=0):
-    """Launch plan for a shape: dict(kind, nsplit, chunk, heads_per_group)."""
+def plan(max_seq_k, batch, head_q, head_k, dim, dim_v, is_bf16=False, total_k=0, distinct_v=False, page_size=0):
+    """Launch plan for a shape: dict(kind, nsplit, chunk, heads_per_group).  `distinct_v`: the plan of a call that
+    passes V as its own buffer (packed, or pages of `page_size` tokens)."""
     lib = load()
     kind, ns, ch, rt = ctypes.c_int(), ctypes.c_int(), ctypes.c_int(), ctypes.c_int()
-    rc = lib.da_plan(max_seq_k, batch, head_q, head_k, dim, dim_v, int(is_bf16), int(total_k), ctypes.byref(kind),
-                     ctypes.byref(ns), ctypes.byref(ch), ctypes.byref(rt))
+    if distinct_v:
+        rc = lib.da_plan_distinct_v(max_seq_k, batch, head_q, head_k, dim, dim_v, int(total_k), int(page_size),
+                                    ctypes.byref(kind), ctypes.byref(ns), ctypes.byref(ch), ctypes.byref(rt))
+    else:
+        rc = lib.da_plan(max_seq_k, batch, head_q, head_k, dim, dim_v, int(is_bf16), int(total_k), ctypes.byref(kind),
+                         ctypes.byref(ns), ctypes.byref(ch), ctypes.byref(rt))
     if rc != DA_OK:
         raise RuntimeError(f"da_plan failed ({rc}): {last_error()}")
     return {"kind": kind.value, "nsplit": ns.value, "chunk": ch.value, "heads_per_group": rt.value}

@@ -47,7 +47,7 @@ int env_int(const char* name, int dflt) {
 struct Tunables {
     int target_wgs, mfma_target_wgs, max_chunk, min_chunk, ragged_chunk, force_kind, group_min_ratio, wave_per_head,
         mla_heads, gqa_heads, flat_wgs, flat_min_tokens, flat_paged_min_mb, nsplit, mfma_small_wgs, group_small_wgs,
-        group_small_chunk, mla_group_heads, mla_group_small, fill_rounds, group_target_wgs_d128;
+        group_small_chunk, mla_group_heads, mla_group_small, fill_rounds, group_target_wgs_d128, mla_distinct_v;
     Tunables() {
         target_wgs = env_int("DA_TARGET_WGS", 512);
         mfma_target_wgs = env_int("DA_MFMA_TARGET_WGS", 256);
@@ -63,6 +63,7 @@ struct Tunables {
         mfma_small_wgs = env_int("DA_MFMA_SMALL_WGS", 256);  // latent kernel: below this many 256-token splits, split finer
         // latent form: up to this many query heads take the grouped kernel (0 = never)
         mla_group_heads = env_int("DA_MLA_GROUP_HEADS", 16);
+        mla_distinct_v = env_int("DA_MLA_DISTINCT_V", 1);  // (576, 512) with V in its own buffer on the latent kernel (0 = VALU sweep)
         // ... and any head count while groups x batch x max_seq_k stays within this (twice this for two groups)
         mla_group_small = env_int("DA_MLA_GROUP_SMALL", 65536);
         group_target_wgs_d128 = env_int("DA_GROUP_TARGET_WGS_D128", 256);
@@ -93,6 +94,7 @@ struct Plan {
     int chunk = 0;
     size_t ws_bytes = 0;
     bool wave_per_head = false;  // grouped kernel: the four waves of a work-group take four KV heads
+    bool v_distinct = false;     // latent kernel: the form that fetches V from a buffer of its own
     // Balanced grid (grouped kernel, ragged batch whose total length the caller gave): flat_wgs work-groups
     // per (KV heads, head group), each over flat_tokens consecutive tokens of the concatenated sequences; nsplit
     // is then the most partials one sequence can have, chunk == flat_tokens.
@@ -119,7 +121,9 @@ int rows_per_trip(size_t dim) {
     }
 }
 
-// v_distinct: V is its own buffer (the MFMA kernel reads V out of the K tile, so it needs the aliased form).
+// v_distinct: V is its own buffer.  At (576, 512) the latent kernels read V out of the K tile; a distinct V takes the
+// latent kernel's two-buffer form that stages the V rows beside the K tile (16-bit K/V, packed or in pages of 16 tokens
+// and more; otherwise the VALU sweep).
 // total_k: sum of the key lengths if the caller knows it (0 = unknown).  The planner never reads cu_seq_k (that
 // would need a device synchronisation); when total_k shows that the batch is ragged it cuts the sequences into
 // shorter splits so that the work-groups, whose number is sized for max_seq_k, balance.
@@ -134,8 +138,10 @@ Plan make_plan(size_t max_seq_k, size_t batch, size_t head_q, size_t head_k, siz
     int trip;
     int target_wgs = tun().target_wgs;
     int max_chunk_scale = 1;
-    const bool latent = !v_distinct && da::mla_supported(dim, dim_v, ratio);
     const bool force_sweep = tun().force_kind == kKindSweep;
+    const bool latent_vd = v_distinct && da::mla_supported(dim, dim_v, ratio) && !kv_8bit && !force_sweep &&
+                           (packed || page_size >= 16) && tun().mla_distinct_v;
+    const bool latent = !v_distinct && da::mla_supported(dim, dim_v, ratio);
     // the latent form with up to 16 query heads (a tensor-parallel shard) runs on the grouped kernel, which keeps more
     // bytes in flight per CU than the latent kernel's one-wave form can (its tiles need LDS landing space)
     // (an 8-bit cache: up to twice as many, as two groups that read the same rows; the latent kernel's single
@@ -150,7 +156,7 @@ Plan make_plan(size_t max_seq_k, size_t batch, size_t head_q, size_t head_k, siz
         tun().mla_group_heads > 0 && group_rows <= (groups16 <= 2 ? 2 : 1) * (long long)tun().mla_group_small;
     const bool latent_group = latent && !force_sweep &&
                               (ratio <= (kv_8bit ? 2 * tun().mla_group_heads : tun().mla_group_heads) || latent_small);
-    const bool mfma = latent && !force_sweep && !latent_group;
+    const bool mfma = (latent && !force_sweep && !latent_group) || latent_vd;
     if (latent_group) {
         pl.kind = kKindGroup;
         pl.rt = 16;
@@ -176,11 +182,12 @@ Plan make_plan(size_t max_seq_k, size_t batch, size_t head_q, size_t head_k, siz
         // an 8-bit K cache is converted by the whole work-group: always four waves, those without heads of their
         // own only load and convert (measured, FP8, 32 heads, batch 64 x 4096 tokens: 206 us with one wave)
         if (kv_8bit) pl.rt = 128;
+        pl.v_distinct = latent_vd;
         trip = da::mla_rows_per_trip();
         target_wgs = tun().mfma_target_wgs;  // one 4-wave work-group fills a CU
         // work-groups of one or two waves over 16-bit K take two tile buffers instead of three when there are more
-        // of them than CUs, and then run two to a CU
-        if (pl.rt <= 64 && !kv_8bit) target_wgs *= 2;
+        // of them than CUs, and then run two to a CU (not with a distinct V, whose two buffers fill the LDS)
+        if (pl.rt <= 64 && !kv_8bit && !latent_vd) target_wgs *= 2;
     } else if (dim <= 256 && !force_sweep && (!kv_8bit || dim % 64 == 0) &&
                (ratio >= tun().group_min_ratio ||
                 (tun().group_min_ratio > 1 && (max_seq_k >= 1024 || dim <= 96) &&
@@ -469,6 +476,21 @@ int da_plan(size_t max_seq_k, size_t batch, size_t head_q, size_t head_k, size_t
     return DA_OK;
 }
 
+int da_plan_distinct_v(size_t max_seq_k, size_t batch, size_t head_q, size_t head_k, size_t dim, size_t dim_v,
+                       size_t total_k, size_t page_size, int* kernel_kind, int* nsplit, int* chunk,
+                       int* heads_per_group) {
+    if (head_k == 0 || head_q % head_k != 0)
+        return fail(DA_ERR_INVALID_ARGUMENT, "head_q (%zu) must be a multiple of head_k (%zu)", head_q, head_k);
+    if (!supported_dims(dim, dim_v))
+        return fail(DA_ERR_UNSUPPORTED, "unsupported head dims (dim %zu, dim_v %zu)", dim, dim_v);
+    const Plan pl = make_plan(max_seq_k, batch, head_q, head_k, dim, dim_v, true, total_k, page_size, false);
+    if (kernel_kind) *kernel_kind = pl.kind;
+    if (nsplit) *nsplit = pl.nsplit;
+    if (chunk) *chunk = pl.chunk;
+    if (heads_per_group) *heads_per_group = pl.rt;
+    return DA_OK;
+}
+
 size_t da_workspace_bytes(size_t max_seq_k, size_t batch, size_t head_q, size_t head_k, size_t dim, size_t dim_v,
                           size_t total_k) {
     if (head_k == 0 || head_q % head_k != 0 || !supported_dims(dim, dim_v)) return 0;
@@ -630,6 +652,8 @@ int run_attention(const void* q, const void* k, const void* v, void* o, const in
             e = da::launch_gqa_mfma_kv8(sp, is_bf16 != 0, (int)dim, pl.rt, pl.wave_per_head, grid, stream);
         else
             e = da::launch_sweep_kv8(sp, kf.fmt, is_bf16 != 0, (int)dim, pl.rt, grid, stream);
+    } else if (pl.kind == kKindMfma && pl.v_distinct) {
+        e = da::launch_mla_vd(sp, is_bf16 != 0, pl.rt, grid, stream);
     } else if (pl.kind == kKindMfma) {
         e = da::launch_mla(sp, is_bf16 != 0, pl.rt, grid, stream);
     } else if (pl.kind == kKindGroup) {
@@ -660,7 +684,7 @@ int run_attention(const void* q, const void* k, const void* v, void* o, const in
         rp.flat_wgs = pl.flat_wgs;
         rp.flat_cu = sp.flat_cu;
         rp.early = pl.ws_bytes <= ((size_t)8 << 20) ? 1 : 0;
-        rp.half_partials = da::mla_half_partials(pl.kind == kKindMfma, pl.rt, kf.fmt) ? 1 : 0;
+        rp.half_partials = da::mla_half_partials(pl.kind == kKindMfma && !pl.v_distinct, pl.rt, kf.fmt) ? 1 : 0;
         e = da::launch_reduce(rp, is_bf16 != 0, (int)(batch * head_q), stream);
         if (e != hipSuccess) return fail(DA_ERR_HIP, "merge kernel launch: %s", hipGetErrorString(e));
     }

@@ -15,6 +15,8 @@ hipError_t launch_mla(const SweepParams& p, bool is_bf16, int rt, dim3 grid, hip
 inline bool mla_half_partials(bool latent_kernel, int rt, int kv_fmt) { return latent_kernel && rt == 128 && kv_fmt == 0; }
 // the software-pipelined kernel for work-groups of 128 heads over 16-bit K (da_mla_pipe.hip); launch_mla routes to it
 hipError_t launch_mla_pipe(const SweepParams& p, bool is_bf16, dim3 grid, hipStream_t stream);
+// the (576, 512) shape with V in a buffer of its own (16-bit K/V; packed, or pages of 16 tokens and more)
+hipError_t launch_mla_vd(const SweepParams& p, bool is_bf16, int rt, dim3 grid, hipStream_t stream);
 // the same over an 8-bit K cache of format fmt (kKvFp8 or kKvInt8)
 hipError_t launch_mla_kv8(const SweepParams& p, int fmt, bool is_bf16, int rt, dim3 grid, hipStream_t stream);
 }  // namespace da

@@ -47,7 +47,10 @@ using namespace mla;
 // PG: paged K/V with pages of fewer than 16 tokens (down to 1): every row of a tile has its own page lookup.
 // NB: tile buffers of the 16-bit form.  Three keep two tiles in flight behind the one being read; two (one in
 // flight) halve the LDS footprint, so that two work-groups of one or two waves share a CU.
-template <typename Tag, int D, int DV, int NWV, int KV8, bool PG = false, int NB = kNBuf>
+// VD: V is a buffer of its own ([tokens, head_k, 512], not the leading columns of K).  A tile buffer then starts with
+// the tile's 32 V rows (the layout of the first K region, read by the same transpose reads) followed by the K tile;
+// at 68 KiB a buffer, two of them fit.
+template <typename Tag, int D, int DV, int NWV, int KV8, bool PG = false, int NB = kNBuf, bool VD = false>
 __global__ __launch_bounds__(64 * NWV) void mfma_latent_kernel(const SweepParams p) {
     // (FP8 with PG: the stage is filled a row per load, 36 of the 64 lanes active, instead of 1 KiB per load)
     using MM = Mma<Tag>;
@@ -56,11 +59,15 @@ __global__ __launch_bounds__(64 * NWV) void mfma_latent_kernel(const SweepParams
     static_assert(D == 576 && DV == 512 && (NWV == 1 || NWV == 2 || NWV == 4), "tile layout is specific to (576, 512)");
     constexpr int ROW_A = DV * 2;                        // bytes per row, region A (value columns)
     constexpr int ROW_B = (D - DV) * 2;                  // bytes per row, region B (remaining key columns)
-    constexpr int OFF_B = kTile * ROW_A;                 // region B starts here
-    constexpr int BUF = kTile * D * 2;                   // bytes per tile buffer
+    constexpr int OFF_KA = VD ? kTile * ROW_A : 0;       // K's region A starts here (VD: behind the V rows)
+    constexpr int OFF_B = OFF_KA + kTile * ROW_A;        // region B starts here
+    constexpr int BUF = OFF_B + kTile * ROW_B;           // bytes per tile buffer
+    constexpr int QBUF = kTile * D * 2;                  // bytes of a wave's staged Q block (a K tile without V rows)
+    constexpr int QOFF_B = kTile * ROW_A;
     constexpr int NLA = kTile / NWV;                     // region-A load instructions per tile per wave (one row each)
     constexpr int NLB = (kTile / 8) / NWV;               // region-B load instructions per tile per wave (eight rows each)
-    constexpr int NLW = NLA + NLB;                       // load instructions per tile per wave
+    constexpr int NLW = (VD ? 2 : 1) * NLA + NLB;        // load instructions per tile per wave
+    static_assert(!VD || (KV8 == 0 && !PG && NB == 2), "the distinct-V form: 16-bit K/V, runs of 16 tokens, two buffers");
     constexpr int KS = D / 16;                           // k-steps of Q K^T
     constexpr int CT = DV / 32;                          // 32-column tiles of the output
     // FP8 K cache: stages of the tile's raw bytes, filled 1 KiB per load instruction
@@ -126,7 +133,7 @@ __global__ __launch_bounds__(64 * NWV) void mfma_latent_kernel(const SweepParams
     vec8 qf[KS];
     {
         const uint8_t* const qb = reinterpret_cast<const uint8_t*>(p.q) + (size_t)b * p.head_q * (D * 2);
-        const uint32_t qbuf = smem_off + wave * BUF;
+        const uint32_t qbuf = smem_off + wave * QBUF;
         static_for<0, kTile>([&](auto rc) {
             constexpr int row = decltype(rc)::value;
             const int head = min(h_base + min(row, q_last), p.head_q - 1);  // wave-uniform
@@ -138,11 +145,11 @@ __global__ __launch_bounds__(64 * NWV) void mfma_latent_kernel(const SweepParams
             const int row = j * 8 + rb;
             const int head = min(h_base + min(row, q_last), p.head_q - 1);
             lds_dma16(qb, (uint32_t)head * (uint32_t)(D * 2) + (uint32_t)(DV * 2 + (((lane & 7) ^ swz_b(row)) * 16)),
-                      qbuf + (uint32_t)(OFF_B + j * 1024));
+                      qbuf + (uint32_t)(QOFF_B + j * 1024));
         });
         wait_vmcnt<0>();
         const uint32_t qa = qbuf + n * ROW_A + ((swz_a(n) ^ half) * 16);
-        const uint32_t qbb = qbuf + OFF_B + n * ROW_B + ((swz_b(n) ^ half) * 16);
+        const uint32_t qbb = qbuf + QOFF_B + n * ROW_B + ((swz_b(n) ^ half) * 16);
         static_for<0, KS>([&](auto ic) {
             constexpr int ks = decltype(ic)::value;
             if constexpr (ks < 32)
@@ -165,6 +172,8 @@ __global__ __launch_bounds__(64 * NWV) void mfma_latent_kernel(const SweepParams
     constexpr int KB = KV8 ? 1 : 2;  // bytes per K element in memory
     const uint8_t* const kbytes = reinterpret_cast<const uint8_t*>(p.k) + (size_t)hk * D * KB;
     const size_t k_row_bytes = (size_t)p.k_row * KB;
+    const uint8_t* const vbytes = reinterpret_cast<const uint8_t*>(p.v) + (size_t)hk * p.v_head * 2;  // (VD)
+    const size_t v_row_bytes = (size_t)p.v_row * 2;
     const float sl = p.scale_log2 * head_scale(p.k_scale, hk);  // score scale, log2 units
     const float vs = head_scale(p.v_scale, hk);
 
@@ -175,9 +184,9 @@ __global__ __launch_bounds__(64 * NWV) void mfma_latent_kernel(const SweepParams
     // runs of 16 tokens, each inside one page (pages of paged K/V hold a multiple of 16 tokens and tiles start at
     // multiples of kTile; for the packed layout and larger pages the second run follows the first).  A row past the
     // end re-reads the last valid row, in whichever run that is.
-    auto issue_tile = [&](int tok0, int64_t row0, int64_t row1, int buf) {
-        const uint8_t* const base = kbytes + row0 * KB;
-        const uint8_t* const base1 = kbytes + row1 * KB;
+    auto issue_tile = [&](int tok0, RowRef ref0, RowRef ref1, int buf) {
+        const uint8_t* const base = kbytes + ref0.k * KB;
+        const uint8_t* const base1 = kbytes + ref1.k * KB;
         const int last = c1 - 1 - tok0;
         if constexpr (KV8) {
             // stage `buf`: the tile's bytes in row order, lane l of load j bringing bytes [1024 j + 16 l, +16)
@@ -201,7 +210,19 @@ __global__ __launch_bounds__(64 * NWV) void mfma_latent_kernel(const SweepParams
             const int rc = min(row, last), run = rc >> 4;
             lds_dma16(run ? base1 : base,
                       (uint32_t)(rc - run * 16) * (uint32_t)k_row_bytes + (lane16 ^ (uint32_t)(swz_a(row) * 16)),
-                      smem_off + (uint32_t)(buf * BUF + row * ROW_A));
+                      smem_off + (uint32_t)(buf * BUF + OFF_KA + row * ROW_A));
+        }
+        if constexpr (VD) {
+            const uint8_t* const vbase = vbytes + ref0.v * 2;
+            const uint8_t* const vbase1 = vbytes + ref1.v * 2;
+#pragma unroll
+            for (int q = 0; q < NLA; ++q) {
+                const int row = wave + NWV * q;
+                const int rc = min(row, last), run = rc >> 4;
+                lds_dma16(run ? vbase1 : vbase,
+                          (uint32_t)(rc - run * 16) * (uint32_t)v_row_bytes + (lane16 ^ (uint32_t)(swz_a(row) * 16)),
+                          smem_off + (uint32_t)(buf * BUF + row * ROW_A));
+            }
         }
 #pragma unroll
         for (int q = 0; q < NLB; ++q) {
@@ -294,9 +315,7 @@ __global__ __launch_bounds__(64 * NWV) void mfma_latent_kernel(const SweepParams
     const int ntiles = (c1 - c0 + kTile - 1) / kTile;
     // rows of tokens tok and tok + 16 (the second only looked up when the tile has it: the block table ends with
     // the sequence's last page)
-    auto second_run = [&](int tok, int64_t first) {
-        return tok + 16 < c1 ? row_ref(p, b, start, tok + 16).k : first;
-    };
+    auto second_run = [&](int tok, RowRef first) { return tok + 16 < c1 ? row_ref(p, b, start, tok + 16) : first; };
     constexpr int AHEAD = KV8 ? 3 : NB - 1;  // tiles in flight behind the one being read
     RowPages rows_ahead{};
     if constexpr (PG) {
@@ -304,10 +323,10 @@ __global__ __launch_bounds__(64 * NWV) void mfma_latent_kernel(const SweepParams
         if (NB > 2 && ntiles > 1) issue_tile_pg(c0 + kTile, lookup_rows(c0 + kTile), 1);
         if (ntiles > NB - 1) rows_ahead = lookup_rows(c0 + (NB - 1) * kTile);
     } else {
-        const int64_t r0 = row_ref(p, b, start, c0).k;
+        const RowRef r0 = row_ref(p, b, start, c0);
         issue_tile(c0, r0, second_run(c0, r0), 0);
         if (NB > 2 && ntiles > 1) {
-            const int64_t r1 = row_ref(p, b, start, c0 + kTile).k;
+            const RowRef r1 = row_ref(p, b, start, c0 + kTile);
             issue_tile(c0 + kTile, r1, second_run(c0 + kTile, r1), 1);
         }
     }
@@ -318,7 +337,7 @@ __global__ __launch_bounds__(64 * NWV) void mfma_latent_kernel(const SweepParams
                 issue_tile_pg(c0 + 2 * kTile, rows_ahead, 2);
                 if (ntiles > 3) rows_ahead = lookup_rows(c0 + 3 * kTile);
             } else {
-                const int64_t r0 = row_ref(p, b, start, c0 + 2 * kTile).k;
+                const RowRef r0 = row_ref(p, b, start, c0 + 2 * kTile);
                 issue_tile(c0 + 2 * kTile, r0, second_run(c0 + 2 * kTile, r0), 2);
             }
         }
@@ -343,7 +362,7 @@ __global__ __launch_bounds__(64 * NWV) void mfma_latent_kernel(const SweepParams
     // Per-lane LDS read bases (buffer 0); per-step chunk offsets are XORed in, the rest is instruction offset.
     // K rows: lane (n, half) reads chunk 2 ks + half of row n.
     //   ks < 32: (base_a ^ 32 (ks & 7)) + 256 (ks >> 3)        ks >= 32: base_b ^ 32 (ks - 32)
-    const uint32_t base_a = smem_off + n * ROW_A + ((swz_a(n) ^ half) * 16);
+    const uint32_t base_a = smem_off + OFF_KA + n * ROW_A + ((swz_a(n) ^ half) * 16);
     const uint32_t base_b = smem_off + OFF_B + n * ROW_B + ((swz_b(n) ^ half) * 16);
     // V^T: as a source lane of the transpose read this lane addresses row half*4 + q (+16 s2, +8 for the second
     // read), 8 bytes at chunk 4 c + 2 b1 + b0 of it, q = (lane & 15) >> 2, b1 = lane bit 4, b0 = lane bit 1:
@@ -378,8 +397,8 @@ __global__ __launch_bounds__(64 * NWV) void mfma_latent_kernel(const SweepParams
             } else {
             if (t + 3 < ntiles) {
                 const int tk = c0 + (t + 3) * kTile;
-                const int64_t r0 = row_in_page(p, start, tk, page_ahead).k;
-                issue_tile(tk, r0, tk + 16 < c1 ? row_in_page(p, start, tk + 16, page_ahead1).k : r0, buf_next);
+                const RowRef r0 = row_in_page(p, start, tk, page_ahead);
+                issue_tile(tk, r0, tk + 16 < c1 ? row_in_page(p, start, tk + 16, page_ahead1) : r0, buf_next);
             }
             if (t + 4 < ntiles) {
                 const int tk = c0 + (t + 4) * kTile;
@@ -411,8 +430,8 @@ __global__ __launch_bounds__(64 * NWV) void mfma_latent_kernel(const SweepParams
             } else {
             if (t + 3 < ntiles) {
                 const int tk = c0 + (t + 3) * kTile;
-                const int64_t r0 = row_in_page(p, start, tk, page_ahead).k;
-                issue_tile(tk, r0, tk + 16 < c1 ? row_in_page(p, start, tk + 16, page_ahead1).k : r0, buf_next);
+                const RowRef r0 = row_in_page(p, start, tk, page_ahead);
+                issue_tile(tk, r0, tk + 16 < c1 ? row_in_page(p, start, tk + 16, page_ahead1) : r0, buf_next);
             }
             if (t + 4 < ntiles) {
                 const int tk = c0 + (t + 4) * kTile;
@@ -432,8 +451,8 @@ __global__ __launch_bounds__(64 * NWV) void mfma_latent_kernel(const SweepParams
         } else {
         if (t + AHEAD < ntiles) {
             const int tk = c0 + (t + AHEAD) * kTile;
-            const int64_t r0 = row_in_page(p, start, tk, page_ahead).k;
-            issue_tile(tk, r0, tk + 16 < c1 ? row_in_page(p, start, tk + 16, page_ahead1).k : r0, buf_next);
+            const RowRef r0 = row_in_page(p, start, tk, page_ahead);
+            issue_tile(tk, r0, tk + 16 < c1 ? row_in_page(p, start, tk + 16, page_ahead1) : r0, buf_next);
         }
         if (t + AHEAD + 1 < ntiles) {
             const int tk = c0 + (t + AHEAD + 1) * kTile;
@@ -596,23 +615,23 @@ __global__ __launch_bounds__(64 * NWV) void mfma_latent_kernel(const SweepParams
 
 // kNBuf tile buffers (FP8: two of them and three stages of raw bytes); the prologue stages each wave's Q block in a
 // buffer of its own.
-template <int D, int NWV, int KV8, int NB>
+template <int D, int DV, int NWV, int KV8, int NB, bool VD>
 constexpr size_t lds_bytes() {
     constexpr size_t buf = (size_t)kTile * D * 2;
     constexpr size_t stg = (size_t)((kTile * D / 1024 + NWV - 1) / NWV) * NWV * 1024;
-    constexpr size_t tiles = KV8 ? 2 * buf + 3 * stg : (size_t)NB * buf;
+    constexpr size_t tiles = KV8 ? 2 * buf + 3 * stg : (size_t)NB * (buf + (VD ? (size_t)kTile * DV * 2 : 0));
     constexpr size_t qstage = (size_t)NWV * buf;
     return tiles > qstage ? tiles : qstage;
 }
 
-template <typename Tag, int D, int DV, int NWV, int KV8, bool PG, int NB>
+template <typename Tag, int D, int DV, int NWV, int KV8, bool PG, int NB, bool VD = false>
 hipError_t launch_form(const SweepParams& p, dim3 grid, hipStream_t stream) {
-    auto kern = mfma_latent_kernel<Tag, D, DV, NWV, KV8, PG, NB>;
+    auto kern = mfma_latent_kernel<Tag, D, DV, NWV, KV8, PG, NB, VD>;
     static std::atomic<uint64_t> devices_done{0};
-    const hipError_t attr_err =
-        ensure_lds_limit(reinterpret_cast<const void*>(kern), lds_bytes<D, NWV, KV8, NB>(), devices_done);
+    constexpr size_t lds = lds_bytes<D, DV, NWV, KV8, NB, VD>();
+    static_assert(lds <= 160 * 1024, "LDS of one CU");
+    const hipError_t attr_err = ensure_lds_limit(reinterpret_cast<const void*>(kern), lds, devices_done);
     if (attr_err != hipSuccess) return attr_err;
-    constexpr size_t lds = lds_bytes<D, NWV, KV8, NB>();
     hipLaunchKernelGGL(kern, grid, dim3(64 * NWV), lds, stream, p);
     return hipGetLastError();
 }
@@ -664,6 +683,22 @@ int mla_rows_per_trip() { return kTile; }
 
 hipError_t launch_mla(const SweepParams& p, bool is_bf16, int rt, dim3 grid, hipStream_t stream) {
     return is_bf16 ? launch_tag<bf16_tag, 0>(p, rt, grid, stream) : launch_tag<f16_tag, 0>(p, rt, grid, stream);
+}
+
+hipError_t launch_mla_vd(const SweepParams& p, bool is_bf16, int rt, dim3 grid, hipStream_t stream) {
+    if (p.block_table != nullptr && p.page_shift < 4) return hipErrorInvalidValue;  // (tiles come as runs of 16 tokens)
+    switch (rt) {
+        case 32:
+            return is_bf16 ? launch_form<bf16_tag, 576, 512, 1, 0, false, 2, true>(p, grid, stream)
+                           : launch_form<f16_tag, 576, 512, 1, 0, false, 2, true>(p, grid, stream);
+        case 64:
+            return is_bf16 ? launch_form<bf16_tag, 576, 512, 2, 0, false, 2, true>(p, grid, stream)
+                           : launch_form<f16_tag, 576, 512, 2, 0, false, 2, true>(p, grid, stream);
+        case 128:
+            return is_bf16 ? launch_form<bf16_tag, 576, 512, 4, 0, false, 2, true>(p, grid, stream)
+                           : launch_form<f16_tag, 576, 512, 4, 0, false, 2, true>(p, grid, stream);
+        default: return hipErrorInvalidValue;
+    }
 }
 
 hipError_t launch_mla_kv8(const SweepParams& p, int fmt, bool is_bf16, int rt, dim3 grid, hipStream_t stream) {

@@ -189,6 +189,16 @@ size_t da_workspace_bytes_int8kv(size_t max_seq_k, size_t batch, size_t head_q, 
 int da_plan(size_t max_seq_k, size_t batch, size_t head_q, size_t head_k, size_t dim, size_t dim_v, int is_bf16,
             size_t total_k, int *kernel_kind, int *nsplit, int *chunk, int *heads_per_group);
 
+/*
+ * The same for a call that passes V as a buffer of its own (v != NULL), over the packed layout (page_size 0) or
+ * pages of page_size tokens.  It differs from da_plan at (576, 512) only: V outside K takes the latent MFMA kernel's
+ * form that stages the V rows beside each K tile (kind 2; it moves both buffers, 1.9x the bytes of the aliased
+ * call), except over pages of fewer than 16 tokens, which take the VALU sweep (kind 1, several times slower).
+ */
+int da_plan_distinct_v(size_t max_seq_k, size_t batch, size_t head_q, size_t head_k, size_t dim, size_t dim_v,
+                       size_t total_k, size_t page_size, int *kernel_kind, int *nsplit, int *chunk,
+                       int *heads_per_group);
+
 /* 1 when (dim, dim_v) is a supported pair: the reference's DA_HEADDIM_SWITCH set (csrc/common/common.h:73-96). */
 int da_supported_head_dims(size_t dim, size_t dim_v);
 

@@ -1,0 +1,124 @@
+"""The (576, 512) shape with V passed as a buffer of its own (the reference's binding always passes a V tensor,
+reference csrc/torch/decoding_torch.cpp:24-74; its kernel reads whatever buffer it is given).  Such a call takes the
+latent MFMA kernel's form that stages the V rows beside each K tile; over pages of fewer than 16 tokens it takes the
+VALU sweep.  V here is random and unrelated to K, so a kernel that read the leading columns of K instead would fail.
+
+Tolerances as in test_gpu_parity.py (max-abs 2e-3 fp16 / 1e-2 bf16 against the fp32-accumulated oracle).
+"""
+import pytest
+import torch
+
+from decoding_attention_amd import _lib, decoding_attn_fwd, decoding_attn_paged_fwd
+from decoding_attention_amd import workloads as wl
+from gpu_util import TOL, check_against_oracle, run_hip, run_oracle, sub_workload
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+DTYPES = [torch.float16, torch.bfloat16]
+
+
+def _name(dtype):
+    return "bf16" if dtype == torch.bfloat16 else "fp16"
+
+
+def _workload(batch, head_q, seq_k, dtype, **kw):
+    return wl.make_workload(batch, head_q, 1, 576, 512, seq_k, dtype, latent=False, **kw)
+
+
+def test_plan_of_a_distinct_v_call():
+    """V outside K stays on the matrix-instruction kernel (kind 2) wherever it can fetch a tile as runs of 16 tokens;
+    only pages shorter than that fall to the VALU sweep (kind 1).  The aliased call's plan is unchanged."""
+    for batch, sk in ((64, 4096), (1, 512), (16, 16384), (256, 1024)):
+        assert _lib.plan(sk, batch, 128, 1, 576, 512, distinct_v=True)["kind"] == 2
+        assert _lib.plan(sk, batch, 128, 1, 576, 512, distinct_v=True, page_size=16)["kind"] == 2
+        assert _lib.plan(sk, batch, 128, 1, 576, 512, distinct_v=True, page_size=8)["kind"] == 1
+    assert _lib.plan(4096, 64, 128, 1, 576, 512)["kind"] == 2
+    assert _lib.plan(4096, 64, 16, 1, 576, 512, distinct_v=True)["kind"] == 2
+    p = _lib.plan(4096, 64, 128, 1, 576, 512, distinct_v=True)
+    assert (p["nsplit"], p["heads_per_group"]) == (4, 128)
+    # at the other head dims V is always distinct and the two entries agree
+    assert _lib.plan(4096, 64, 32, 8, 128, 128, distinct_v=True) == _lib.plan(4096, 64, 32, 8, 128, 128)
+
+
+@pytest.mark.parametrize("dtype", DTYPES, ids=_name)
+@pytest.mark.parametrize("head_q", [8, 16, 32, 64, 96, 128])
+@pytest.mark.parametrize("batch,seq_k", [(2, 300), (16, 1024), (1, 4096)])
+def test_distinct_v_matches_the_oracle(batch, seq_k, head_q, dtype):
+    w = _workload(batch, head_q, seq_k, dtype, seed=head_q + batch + seq_k)
+    check_against_oracle(w, run_hip(w))
+
+
+@pytest.mark.parametrize("dtype", DTYPES, ids=_name)
+def test_distinct_v_ragged_with_empty_sequences_and_alibi(dtype):
+    lens = torch.tensor([0, 1, 65, 300, 0, 1031, 16, 17, 32, 33], dtype=torch.int32)
+    g = torch.Generator().manual_seed(7)
+    total = int(lens.sum())
+    q = torch.randn(len(lens), 128, 576, generator=g).to(dtype)
+    k = torch.randn(total, 1, 576, generator=g).to(dtype)
+    v = torch.randn(total, 1, 512, generator=g).to(dtype)
+    for alibi in (False, True):
+        w = wl.Workload("ragged_distinct_v", q, k, v, wl.get_cu_seq(lens), int(lens.max()), 512, alibi, lens.tolist())
+        o = run_hip(w)
+        check_against_oracle(w, o)
+        assert (o[0].float() == 0).all() and (o[4].float() == 0).all()
+        # one token: the output is that token's V row, whatever K holds
+        assert torch.equal(o[1, 7].view(torch.int16), v[0, 0].view(torch.int16))
+
+
+@pytest.mark.parametrize("page_size", [1, 8, 16, 64])
+@pytest.mark.parametrize("head_q", [16, 128])
+def test_distinct_v_over_pages(head_q, page_size):
+    """Pages of 16 tokens and more: the same kernel and plan as the packed call, same bits.  Shorter pages: the VALU
+    sweep, within the tolerance of the oracle."""
+    w = _workload(5, head_q, 900, torch.float16, seed=11, varlen=True)
+    pk = wl.to_pages(w, page_size, seed=3).to(DEV)
+    wd = w.to(DEV)
+    paged = decoding_attn_paged_fwd(wd.q, pk.k_pages, pk.v_pages, pk.block_table, pk.seq_lens, w.max_seq_k, 512,
+                                    False).cpu()
+    torch.cuda.synchronize()
+    check_against_oracle(w, paged)
+    if page_size >= 16:
+        from gpu_util import run_hip_ex
+        dense = run_hip_ex(w, 0)
+        assert torch.equal(dense.view(torch.int16), paged.view(torch.int16))
+
+
+def test_distinct_v_that_equals_the_leading_columns_gives_the_aliased_result():
+    """V = a copy of K[..., :512] in its own buffer: the distinct-V kernel must land where the aliased kernel does
+    (both within the tolerance of one oracle result; the two kernels round their partial results differently)."""
+    w = wl.config_mla(4, 2048, seed=9)
+    v = w.k[:, :, :512].contiguous()
+    wv = wl.Workload("copied_v", w.q, w.k, v, w.cu_seq_k, w.max_seq_k, 512, False, w.lengths)
+    o_alias, o_copy = run_hip(w), run_hip(wv)
+    check_against_oracle(w, o_copy)
+    assert (o_alias.float() - o_copy.float()).abs().max().item() <= TOL[torch.float16]
+
+
+def test_distinct_v_full_size_and_cost_against_the_aliased_call():
+    """Batch 64 x 4096 tokens, 128 heads: sampled sequences against the oracle, every row finite; and the call's time
+    beside the aliased call's.  It moves K and V (302 + 268 MB, 588 MB with Q, O and the split partials) where the
+    aliased call moves K alone, and must stay within twice its time."""
+    w = _workload(64, 128, 4096, torch.float16, seed=1)
+    wd = w.to(DEV)
+    o = decoding_attn_fwd(wd.q, wd.k, wd.v, wd.cu_seq_k, wd.max_seq_k, 512, False)
+    torch.cuda.synchronize()
+    assert torch.isfinite(o.float()).all()
+    rows = [0, 13, 31, 63]
+    _, ref32 = run_oracle(sub_workload(w, rows))
+    assert (o[rows].cpu().float() - ref32).abs().max().item() <= TOL[torch.float16]
+
+    def us_per_call(fn, reps=60):
+        for _ in range(10):
+            fn()
+        a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        a.record()
+        for _ in range(reps):
+            fn()
+        b.record()
+        b.synchronize()
+        return a.elapsed_time(b) * 1000.0 / reps
+
+    t_distinct = us_per_call(lambda: decoding_attn_fwd(wd.q, wd.k, wd.v, wd.cu_seq_k, wd.max_seq_k, 512, False))
+    t_alias = us_per_call(lambda: decoding_attn_fwd(wd.q, wd.k, None, wd.cu_seq_k, wd.max_seq_k, 512, False))
+    print(f"(576, 512) batch 64 x 4096: distinct V {t_distinct:.1f} us/call, V inside K {t_alias:.1f} us/call")
+    assert t_distinct <= 2.0 * t_alias
