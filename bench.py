@@ -490,6 +490,89 @@ def run_sweep(args, measure_fn=None, workload_fn=None, out=None):
     return 0
 
 
+# Shapes of the latent form whose launch plan `--sweep latent-plan` derives: the benchmark's two sweeps (batch at 4096
+# tokens, length at batch 16) and the reference's lists around them.
+LATENT_PLAN_SHAPES = ([(b, 4096) for b in (1, 2, 4, 8, 16, 32, 64, 128, 256)] +
+                      [(16, sk) for sk in (512, 1024, 2048, 8192, 16384)] + [(1, sk) for sk in (512, 2048, 8192)] +
+                      [(4, 16384), (8, 8192), (32, 1024), (64, 1024), (100, 4096)])
+
+
+def run_latent_plan_sweep(args):
+    """Every shape of LATENT_PLAN_SHAPES (128 heads over one latent head, fp16) timed under the library's own plan
+    and under forced alternatives: the grouped kernel's latent form, and the latent kernel with 64 or 128 heads per
+    work-group at each split count.  The planner's thresholds for the latent path are read off this log.  Runs on the
+    probe library (the same code with a setter for the planner's tunables)."""
+    import ctypes
+
+    import torch
+
+    from decoding_attention_amd import _lib
+    from decoding_attention_amd import workloads as wl
+
+    probe = _lib.load_probe()
+    dev = torch.device("cuda:0")
+    stream = torch.cuda.current_stream().cuda_stream
+    defaults = {"DA_NSPLIT": 0, "DA_MLA_HEADS": 0, "DA_MLA_GROUP_SMALL": 65536}
+
+    def set_tunables(**kw):
+        for name, value in {**defaults, **kw}.items():
+            assert probe.da_probe_set_tunable(name.encode(), int(value)) == 0
+
+    def plan_of(w):
+        kind, ns, ch, rt = (ctypes.c_int() for _ in range(4))
+        assert probe.da_plan(w.max_seq_k, w.batch, 128, 1, 576, 512, 0, int(w.k.shape[0]), ctypes.byref(kind),
+                             ctypes.byref(ns), ctypes.byref(ch), ctypes.byref(rt)) == 0
+        return kind.value, rt.value, ns.value, ch.value
+
+    def time_us(copies, w):
+        total = int(w.k.shape[0])
+        n = probe.da_workspace_bytes(w.max_seq_k, w.batch, 128, 1, 576, 512, total)
+        ws = torch.empty(max(n, 16), dtype=torch.uint8, device=dev)
+        o = torch.empty(w.batch, 128, 512, dtype=torch.float16, device=dev)
+
+        def call(c):
+            rc = probe.da_decoding_attn_ex(c.q.data_ptr(), c.k.data_ptr(), None, o.data_ptr(), c.cu_seq_k.data_ptr(),
+                                           w.max_seq_k, w.batch, 128, 1, 576, 512, 0, 0, 0.0, None, total,
+                                           ws.data_ptr(), n, stream)
+            assert rc == 0, probe.da_last_error().decode("utf-8", "replace")
+
+        mean_ms, _ = _time_calls(torch, [lambda c=c: call(c) for c in copies], args.steps, args.warmup)
+        return mean_ms * 1e3
+
+    print("shape: candidates as kernel/heads-per-work-group/splits = us per call; kernel g = grouped (16 heads per "
+          "group), l = latent", flush=True)
+    for batch, sk in LATENT_PLAN_SHAPES:
+        w = wl.make_workload(batch, 128, 1, 576, 512, sk, torch.float16, device="cuda:0")
+        copies = _device_copies(torch, w, dev)
+        set_tunables()
+        kind, rt, ns, ch = plan_of(w)
+        chosen = f"{'g' if kind == 3 else 'l'}/{rt}/{ns}"
+        results = {}
+        # the grouped kernel's latent form, its own split count
+        set_tunables(DA_MLA_GROUP_SMALL=1 << 30)
+        k2, rt2, ns2, _ = plan_of(w)
+        if k2 == 3:
+            results[f"g/{rt2}/{ns2}"] = time_us(copies, w)
+        for heads in (64, 128):
+            for nsplit in (1, 2, 3, 4, 6, 8, 12, 16, 24, 32):
+                if sk // nsplit < 128 or batch * nsplit * (128 // heads) > 1024:
+                    continue
+                set_tunables(DA_MLA_GROUP_SMALL=0, DA_MLA_HEADS=heads, DA_NSPLIT=nsplit)
+                k3, rt3, ns3, _ = plan_of(w)
+                key = f"l/{rt3}/{ns3}"
+                if k3 == 2 and key not in results:
+                    results[key] = time_us(copies, w)
+        set_tunables()
+        if chosen not in results:
+            results[chosen] = time_us(copies, w)
+        best = min(results, key=results.get)
+        ranked = ", ".join(f"{k} = {v:.1f}" for k, v in sorted(results.items(), key=lambda kv: kv[1])[:6])
+        print(f"b{batch} x {sk}: planner {chosen} = {results[chosen]:.1f} us; best {best} = {results[best]:.1f} us "
+              f"(planner / best = {results[chosen] / results[best]:.3f}); fastest six: {ranked}", flush=True)
+        del w, copies
+    return 0
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -502,7 +585,7 @@ def main():
     ap.add_argument("--calibrate-copy", action="store_true", help="first run three 1 GiB device copies (a known "
                     "traffic figure for scaling profiler byte counters)")
     ap.add_argument("--cpu-budget", type=float, default=15.0, help="seconds of single-thread CPU work to sample")
-    ap.add_argument("--sweep", choices=["mha", "mla", "baseline", "gqa", "all", "paged", "fp8"], help="print the reference's sweeps instead "
+    ap.add_argument("--sweep", choices=["mha", "mla", "baseline", "gqa", "all", "paged", "fp8", "latent-plan"], help="print the reference's sweeps instead "
                     "(paged / fp8: benchmark shapes over a paged or an 8-bit, FP8 and int8, K/V cache)")
     ap.add_argument("--json-out", help="with --sweep: also write the results as JSON")
     args = ap.parse_args()
@@ -510,6 +593,8 @@ def main():
         print("bench.py measures one GPU: the op has no multi-GPU path (sequences and KV heads shard without "
               "communication); run with --gpus 1", file=sys.stderr)
         return 2
+    if args.sweep == "latent-plan":
+        return run_latent_plan_sweep(args)
     if args.sweep:
         return run_sweep(args)
     return run_default(args)

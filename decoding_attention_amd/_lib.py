@@ -55,6 +55,13 @@ def load():
             f"{LIB_PATH} is missing: build it with `python -m decoding_attention_amd.build` "
             "(hipcc, --offload-arch=gfx950). There is no CPU or PyTorch fallback.")
     lib = ctypes.CDLL(LIB_PATH)
+    _declare(lib)
+    _lib = lib
+    return lib
+
+
+def _declare(lib):
+    """Prototypes of the drop-in ABI (include/decoding_attn_hip.h)."""
     vp, sz, ci, cf = ctypes.c_void_p, ctypes.c_size_t, ctypes.c_int, ctypes.c_float
     lib.da_decoding_attn.restype = ci
     lib.da_decoding_attn.argtypes = [vp, vp, vp, vp, vp, sz, sz, sz, sz, sz, sz, ci, ci, vp]
@@ -99,8 +106,6 @@ def load():
     lib.da_last_error.argtypes = []
     lib.da_version.restype = ci
     lib.da_version.argtypes = []
-    _lib = lib
-    return lib
 
 
 PROBE_LIB_PATH = os.path.join(PKG_DIR, "libdecoding_attn_probe.so")
@@ -116,7 +121,10 @@ def load_probe():
     if not os.path.exists(PROBE_LIB_PATH):
         raise LibraryNotBuilt(f"{PROBE_LIB_PATH} is missing: build it with `python -m decoding_attention_amd.build`")
     lib = ctypes.CDLL(PROBE_LIB_PATH)
+    _declare(lib)  # (the probe library is the same code: it exports the drop-in entry points too)
     vp, sz, ci = ctypes.c_void_p, ctypes.c_size_t, ctypes.c_int
+    lib.da_probe_set_tunable.restype = ci
+    lib.da_probe_set_tunable.argtypes = [ctypes.c_char_p, ci]
     lib.da_probe_stream_read.restype = ci
     lib.da_probe_stream_read.argtypes = [vp, sz, vp, vp]
     lib.da_probe_sweep_only.restype = ci
@@ -127,7 +135,6 @@ def load_probe():
     lib.da_probe_mfma_rate.argtypes = [vp, ci, vp, vp]
     lib.da_probe_mfma_rate_flops.restype = ctypes.c_double
     lib.da_probe_mfma_rate_flops.argtypes = [ci]
-    lib.da_last_error.restype = ctypes.c_char_p
     _probe = lib
     return lib
 

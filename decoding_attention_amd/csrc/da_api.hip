@@ -76,10 +76,11 @@ struct Tunables {
         group_min_ratio = env_int("DA_GROUP_MIN_RATIO", 2);  // smallest head group that takes the grouped MFMA sweep
     }
 };
-const Tunables& tun() {
+Tunables& tun_storage() {
     static Tunables t;
     return t;
 }
+const Tunables& tun() { return tun_storage(); }
 
 constexpr int kKindSweep = 1;
 constexpr int kKindMfma = 2;
@@ -150,10 +151,15 @@ Plan make_plan(size_t max_seq_k, size_t batch, size_t head_q, size_t head_k, siz
     // rows: the latent kernel's work-groups pay ~6 us to stage Q before their first tile, which a few tiles do not
     // win back (measured, 128 heads: batch 1 x 8192 tokens 34.4 -> 24.8 us, batch 16 x 512 29.8 -> 23.4; 32 heads:
     // batch 1 x 16384 33.4 -> 23.0; past the bound below the re-read rows cost more than the staging).
+    // (65 heads and more over 16-bit K run on the software-pipelined latent kernel, which wins from a quarter of that
+    // bound on: 128 heads, batch 1 x 4096 tokens 21.6 -> 19.8 us, batch 2 x 4096 26.2 -> 24.3, batch 16 x 512 27.1 ->
+    // 24.6; batch 1 x 512 stays, 16.5 against 17.7, batch 1 x 2048 is a tie)
+    const bool pipe_kernel = latent && ratio > 64 && !kv_8bit;
     const long long groups16 = (ratio + 15) / 16;
     const long long group_rows = groups16 * (long long)batch * (long long)max_seq_k;
-    const bool latent_small =
-        tun().mla_group_heads > 0 && group_rows <= (groups16 <= 2 ? 2 : 1) * (long long)tun().mla_group_small;
+    const long long small_bound =
+        pipe_kernel ? (long long)tun().mla_group_small / 4 : (groups16 <= 2 ? 2 : 1) * (long long)tun().mla_group_small;
+    const bool latent_small = tun().mla_group_heads > 0 && group_rows <= small_bound;
     const bool latent_group = latent && !force_sweep &&
                               (ratio <= (kv_8bit ? 2 * tun().mla_group_heads : tun().mla_group_heads) || latent_small);
     const bool mfma = (latent && !force_sweep && !latent_group) || latent_vd;
@@ -174,8 +180,11 @@ Plan make_plan(size_t max_seq_k, size_t batch, size_t head_q, size_t head_k, siz
         // heads per (sequence, split) beat one of 128 (measured: batch 1, seq 4096: 35 -> 31 us).  The same holds for
         // up to four long sequences (batch 1 x 65536 tokens 64.2 -> 55.7 us, batch 2 x 32768 63.7 -> 56.3, batch 4 x
         // 16384 63.5 -> 56.8; batch 8 x 8192 and larger batches lose, 53.2 -> 57.6).
+        // (the compiler-scheduled four-wave form, i.e. an 8-bit cache or a distinct V: the pipelined kernel is faster
+        // with 128 heads at every size; batch 8 x 4096 tokens 38.7 -> 30.0 us, batch 16 x 2048 38.9 -> 29.8, batch 4 x
+        // 16384 54.4 -> 41.1, batch 32 x 1024 39.2 -> 30.3)
         const long long tiles256 = (long long)batch * (long long)(max_seq_k / 256);
-        if (pl.rt == 128 && (tiles256 <= 128 || (batch <= 4 && tiles256 <= 512))) pl.rt = 64;
+        if (pl.rt == 128 && !pipe_kernel && (tiles256 <= 128 || (batch <= 4 && tiles256 <= 512))) pl.rt = 64;
         if ((tun().mla_heads == 32 || tun().mla_heads == 64 || tun().mla_heads == 128) && tun().mla_heads <= 128 &&
             tun().mla_heads >= 32)
             pl.rt = std::min(tun().mla_heads, da::mla_heads_per_group(ratio));
@@ -284,6 +293,13 @@ Plan make_plan(size_t max_seq_k, size_t batch, size_t head_q, size_t head_k, siz
     // 40 x 8192, 280 work-groups 209 us, 240 work-groups 146 us; 16 heads, batch 150 x 4096, 300 work-groups 183 us,
     // 150 work-groups 153 us).
     if ((latent_group || mfma) && base > 0) want = std::max<long long>(1, target_wgs / base);
+    // The pipelined latent kernel with splits under 512 tokens: three quarters of the CUs do better than all of them
+    // (a work-group's fixed cost, Q in and partials out, is then most of its time, and fewer splits mean fewer
+    // partials; the chip also clocks higher).  Measured, 128 heads: batch 16 x 4096 tokens, 16 -> 12 splits, 40.4 ->
+    // 37.3 us; batch 8 x 8192, 32 -> 24, 40.8 -> 37.9; batch 64 x 1024, 4 -> 3, 41.1 -> 38.6; from 512-token splits
+    // up the full grid wins or ties (batch 64 x 4096, 4 splits 87.3 us, 3 splits 91.6; batch 32 x 4096, 8 and 6 tie).
+    if (mfma && pipe_kernel && pl.rt == 128 && base > 0 && want > 1 && (long long)max_seq_k / want < 512)
+        want = std::max<long long>(1, (target_wgs * 3 / 4) / base);
     const long long by_len = std::max<long long>(1, (long long)max_seq_k / min_chunk);
     // sweep work-groups are also kept short (shorter still for a ragged batch); the latent MFMA kernel's partials
     // are too large (heads x dim_v floats per split) to split more than occupancy asks for
@@ -742,6 +758,22 @@ int da_probe_sweep_only(const void* q, const void* k, const void* v, void* o, co
     kf.sweep_only = true;
     return run_attention(q, k, v, o, cu_seq_k, Paging{}, kf, max_seq_k, batch, head_q, head_k, dim, dim_v, is_alibi,
                          is_bf16, 0.0f, nullptr, total_k, workspace, workspace_bytes, hip_stream);
+}
+
+// Overrides one planner tunable of this (probe) library in the running process, for sweeps over plans; not
+// thread-safe against concurrent calls.
+int da_probe_set_tunable(const char* name, int value) {
+    if (!name) return DA_ERR_INVALID_ARGUMENT;
+    Tunables& t = tun_storage();
+    const std::string n(name);
+    if (n == "DA_NSPLIT") t.nsplit = value;
+    else if (n == "DA_MLA_HEADS") t.mla_heads = value;
+    else if (n == "DA_MLA_GROUP_SMALL") t.mla_group_small = value;
+    else if (n == "DA_MLA_GROUP_HEADS") t.mla_group_heads = value;
+    else if (n == "DA_MFMA_TARGET_WGS") t.mfma_target_wgs = value;
+    else if (n == "DA_MFMA_SMALL_WGS") t.mfma_small_wgs = value;
+    else return fail(DA_ERR_INVALID_ARGUMENT, "unknown tunable %s", name);
+    return DA_OK;
 }
 #endif
 

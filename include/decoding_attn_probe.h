@@ -1,6 +1,6 @@
 /*
  * Measurement aids of the benchmark (bench.py), exported by libdecoding_attn_probe.so only: a second build of the
- * library's sources with these two entry points added.  None of this is part of the drop-in ABI
+ * library's sources with these entry points added.  None of this is part of the drop-in ABI
  * (decoding_attn_hip.h) and nothing here has a counterpart in the reference.
  */
 #ifndef DECODING_ATTN_PROBE_H_
@@ -43,6 +43,13 @@ int da_probe_sweep_only(const void *q, const void *k, const void *v, void *o, co
                         size_t max_seq_k, size_t batch, size_t head_q, size_t head_k, size_t dim, size_t dim_v,
                         int is_alibi, int is_bf16, size_t total_k, void *workspace, size_t workspace_bytes,
                         void *hip_stream);
+
+/*
+ * Overrides one planner tunable (by the name of its environment variable: DA_NSPLIT, DA_MLA_HEADS,
+ * DA_MLA_GROUP_SMALL, DA_MLA_GROUP_HEADS, DA_MFMA_TARGET_WGS, DA_MFMA_SMALL_WGS) for later calls into this library in
+ * this process, so that one process can time a shape under several launch plans (bench.py --sweep latent-plan).
+ */
+int da_probe_set_tunable(const char *name, int value);
 
 #ifdef __cplusplus
 }

@@ -115,17 +115,23 @@ def test_latent_form_with_fp8_cache(batch, head_q, seq_k, dtype, is_alibi):
     assert (o.float() - ref).abs().max().item() <= TOL[dtype]
 
 
-def test_latent_fp8_unit_scales_equal_the_16_bit_call_bit_for_bit():
+@pytest.mark.parametrize("head_q", [64, 128])
+def test_latent_fp8_unit_scales_equal_the_16_bit_call(head_q):
     """FP8 values convert exactly and the tiles are converted before any arithmetic: with unit scales the FP8 call
-    is the 16-bit call on the same values, same kernel, same order of operations."""
+    is the 16-bit call on the same values.  Up to 64 heads both run the same kernel in the same order of operations:
+    same bits.  With 128 heads the 16-bit call runs on the software-pipelined kernel (other rounding of the split
+    partials): equal within the output tolerance."""
     # (large enough for the planner to pick the latent kernel, whose property this is)
-    w, k8, _, ks, _ = _case(6, 128, 1, 576, 512, 3000, torch.float16, latent=True, unit=True, seed=9)
-    assert _lib.plan(w.max_seq_k, 6, 128, 1, 576, 512)["kind"] == 2
+    w, k8, _, ks, _ = _case(6, head_q, 1, 576, 512, 3000, torch.float16, latent=True, unit=True, seed=9)
+    assert _lib.plan(w.max_seq_k, 6, head_q, 1, 576, 512)["kind"] == 2
     k16 = k8.to(torch.float16).to(DEV)
     args = (w.cu_seq_k.to(DEV), w.max_seq_k, 512, False)
     o8 = decoding_attn_fwd(w.q.to(DEV), k8.to(DEV), None, *args, k_scale=ks.to(DEV), v_scale=ks.to(DEV))
     o16 = decoding_attn_fwd(w.q.to(DEV), k16, None, *args)
-    assert torch.equal(o8.view(torch.int16), o16.view(torch.int16))
+    if head_q <= 64:
+        assert torch.equal(o8.view(torch.int16), o16.view(torch.int16))
+    else:
+        assert (o8.float() - o16.float()).abs().max().item() <= TOL[torch.float16]
 
 
 @pytest.mark.parametrize("page_size", [1, 4, 16, 32, 64])

@@ -121,13 +121,16 @@ def test_latent_form_with_int8_cache(batch, head_q, seq_k, dtype, is_alibi):
     assert (o.float() - _reference(w, k8, None, ks, ks)).abs().max().item() <= TOL[dtype]
 
 
+@pytest.mark.parametrize("head_q", [64, 128])
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
-def test_latent_int8_unit_scales_equal_the_16_bit_call_bit_for_bit(dtype):
+def test_latent_int8_unit_scales_equal_the_16_bit_call(dtype, head_q):
     """The tiles are converted, exactly, before any arithmetic: with unit scales the int8 call is the 16-bit call on
-    the same integers, same kernel, same order of operations.  All 256 byte values occur."""
+    the same integers.  Up to 64 heads both run the same kernel in the same order of operations: same bits.  With 128
+    heads the 16-bit call runs on the software-pipelined kernel (other rounding of the split partials): equal within
+    the output tolerance.  All 256 byte values occur."""
     # (large enough for the planner to pick the latent kernel, whose property this is)
-    w = wl.make_workload(6, 128, 1, 576, 512, 3000, dtype, seed=9, varlen=True, latent=True)
-    assert _lib.plan(w.max_seq_k, 6, 128, 1, 576, 512)["kind"] == 2
+    w = wl.make_workload(6, head_q, 1, 576, 512, 3000, dtype, seed=9, varlen=True, latent=True)
+    assert _lib.plan(w.max_seq_k, 6, head_q, 1, 576, 512)["kind"] == 2
     g = torch.Generator().manual_seed(10)
     k8 = torch.round(torch.randn(w.k.shape, generator=g) * 0.7).to(torch.int8)
     k8.view(-1)[::211] = torch.arange(-128, 128, dtype=torch.int8).repeat(k8.numel() // 211 // 256 + 1)[
@@ -137,7 +140,12 @@ def test_latent_int8_unit_scales_equal_the_16_bit_call_bit_for_bit(dtype):
     o8 = decoding_attn_fwd(w.q.to(DEV), k8.to(DEV), None, *args)
     o16 = decoding_attn_fwd(w.q.to(DEV), k8.to(dtype).to(DEV), None, *args)
     assert torch.isfinite(o8.float()).all()
-    assert torch.equal(o8.view(torch.int16), o16.view(torch.int16))
+    if head_q <= 64:
+        assert torch.equal(o8.view(torch.int16), o16.view(torch.int16))
+    else:
+        # (integer values up to 128 in magnitude: outputs of order 1, so the tolerance is relative)
+        scale = max(1.0, o16.float().abs().max().item())
+        assert (o8.float() - o16.float()).abs().max().item() <= TOL[dtype] * scale
 
 
 @pytest.mark.parametrize("page_size", [1, 4, 16, 32, 64])

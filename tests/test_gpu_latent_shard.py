@@ -103,6 +103,6 @@ def test_value_passed_as_a_view_of_the_key_rows(head_q):
 def test_small_problems_of_any_head_count_as_groups_of_16(head_q, dtype):
     """Small latent problems run on the grouped kernel whatever the head count, ceil(heads / 16) groups per sequence,
     the last one partly idle when 16 does not divide the head count."""
-    w = _latent(3, head_q, 700, dtype, seed=head_q, is_alibi=head_q == 40)
+    w = _latent(3, head_q, 600, dtype, seed=head_q, is_alibi=head_q == 40)
     assert _lib.plan(w.max_seq_k, 3, head_q, 1, 576, 512)["kind"] == 3
     check_against_oracle(w, run_hip(w))
