@@ -24,10 +24,14 @@
 // cannot afford.  What the compiler allocates: the score tile being accumulated, addresses and scalars.
 //
 // LDS fragments for the matrix steps run through a ring of eight register sets, requested eight steps ahead of
-// their use across the A -> B boundary; the ring drains at the end of a trip (the next trip's K tile is only known
-// to be in LDS after the trip's barrier), and the scaling and maximum of S(t+1) are computed while it refills.
-// One barrier per trip: behind it every wave's share of tile t+1 has landed and every wave is done with tile t-1,
-// whose buffer then receives tile t+3.
+// their use across the A -> B boundary and, in the steady-state loop, across the trip boundary as well: the barrier
+// that makes tile t+2 visible to every wave sits eight matrix steps before the end of trip t's phase B (each wave
+// first waits for its own loads of that tile), and the last eight steps request the first K fragments of tile t+2,
+// so the matrix pipe finds its operands waiting when trip t+1 starts.  A second, plain barrier at the top of a trip
+// keeps the loads of tile t+3 behind every wave's last read of tile t-1, whose buffer they fill.  (A trip has 68
+// steps, four more than a multiple of eight, so steady-state trips come in pairs with the ring slots offset by
+// four in the second.)  The other trips (the first, the last ones of a split, ALiBi, paged rows) start with an empty
+// ring behind one barrier, and the scaling and maximum of S(t+1) are computed while it refills.
 //
 // Mathematics as in the reference kernel (csrc/kernel/decoding_attn/decoding_fwd_kernel.h:50-235 with the latent
 // aliasing of csrc/ops/decoding_attn.cpp:30-37); the structure is unrelated.
@@ -379,7 +383,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_num_vgpr(kScV))) void la
     const uint32_t voff_b = (uint32_t)(((wave & 1) * 8 + rb) * (int)k_row_bytes) +
                             (uint32_t)(DV * 2 + (((lane & 7) ^ swz_b(wave * 8 + rb)) * 16));
     const uint32_t lane16w = lane16 ^ (uint32_t)(wave << 6);  // lane16 ^ 16 * (swizzle bits from row & 3 = wave)
-    auto issue_load_fast = [&](auto qc, const uint8_t* base, const uint8_t* base1, uint32_t lds_buf) {
+    auto issue_load_fast = [&](auto qc, const uint8_t* base, const uint8_t* base1, uint32_t lds_buf) __attribute__((always_inline)) {
         constexpr int q = decltype(qc)::value;
         if constexpr (q < NLA) {
             // row = wave + 4 q: swizzle = wave << 2 | (q & 3)
@@ -423,19 +427,23 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_num_vgpr(kScV))) void la
 
     // read for k-step ks of the K tile whose region-B base is tb (region A: ka[]; the PG form, short of registers for
     // its row addresses, keeps one base, ka[0], and XORs in front of every read)
-    auto read_k = [&](auto ksc, uint32_t tb) {
+    // RO: where the trip's first step sits in the ring.  A trip has 68 steps, four more than a multiple of the ring's
+    // eight slots, so when the ring runs on from one trip into the next (steady-state loop) trips alternate between
+    // RO = 0 and RO = 4; a trip that starts with an empty ring starts at 0.
+    auto read_k = [&](auto ksc, uint32_t tb, auto ro_c) __attribute__((always_inline)) {
         constexpr int ks = decltype(ksc)::value;
+        constexpr int slot = (ks + decltype(ro_c)::value) % kRing;
         if constexpr (ks < 32 && PG)
-            ring_read_b128<kRingV + 4 * (ks % kRing), 32 * (ks & 7), (ks >> 3) * 256>(ka[0], xt);
+            ring_read_b128<kRingV + 4 * slot, 32 * (ks & 7), (ks >> 3) * 256>(ka[0], xt);
         else if constexpr (ks < 32)
-            ring_read_b128<kRingV + 4 * (ks % kRing), 0, (ks >> 3) * 256>(ka[ks & 7], xt);
+            ring_read_b128<kRingV + 4 * slot, 0, (ks >> 3) * 256>(ka[ks & 7], xt);
         else
-            ring_read_b128<kRingV + 4 * (ks % kRing), 32 * (ks - 32), 0>(tb, xt);
+            ring_read_b128<kRingV + 4 * slot, 32 * (ks - 32), 0>(tb, xt);
     };
     // reads for step i of O += V^T P^T (column tile i / 2, token half i % 2) of the tile at tv; ring slot (KS + i) % kRing
-    auto read_v = [&](auto ic, uint32_t tv) {
+    auto read_v = [&](auto ic, uint32_t tv, auto ro_c) __attribute__((always_inline)) {
         constexpr int i = decltype(ic)::value;
-        constexpr int c = i >> 1, s2 = i & 1, slot = (KS + i) % kRing;
+        constexpr int c = i >> 1, s2 = i & 1, slot = (KS + i + decltype(ro_c)::value) % kRing;
         if constexpr (s2 == 0) {
             if constexpr (c == 0)
                 asm volatile("v_mov_b32 %0, %1" : "=v"(xa) : "v"(tv));
@@ -453,7 +461,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_num_vgpr(kScV))) void la
     constexpr int SMP = kBf16 ? 7 : 5;  // instructions per pair
     constexpr int SMN = 8 * SMP;        // in all
     float tlo, thi;
-    auto sm_op = [&](auto jc) {
+    auto sm_op = [&](auto jc) __attribute__((always_inline)) {
         constexpr int j = decltype(jc)::value;
         constexpr int k = j / SMP, o = j % SMP;
         if constexpr (o == 0) sc_exp2<2 * k>();
@@ -472,7 +480,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_num_vgpr(kScV))) void la
     };
     // maximum of the raw scores in sacc, between the matrix steps of phase B (its first instruction well behind the
     // last matrix instruction that wrote sacc): eleven instructions
-    auto mx_op = [&](auto jc) {
+    auto mx_op = [&](auto jc) __attribute__((always_inline)) {
         constexpr int j = decltype(jc)::value;
         if constexpr (j == 0) asm volatile("v_max3_f32 %0, %1, %2, %3" : "=v"(mxr) : "v"(sacc[0]), "v"(sacc[1]), "v"(sacc[2]));
         if constexpr (j >= 1 && j <= 6)
@@ -491,9 +499,10 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_num_vgpr(kScV))) void la
     // each of the four waves another DMA, so that their loads do not come together, measured slower, 2970 against
     // 2800 clocks per tile.)
     auto phase_a = [&](auto qk_c, auto sm_c, auto dma_c, uint32_t tb, uint32_t tv, const uint8_t* base,
-                       const uint8_t* base1, uint32_t dma_lds) {
+                       const uint8_t* base1, uint32_t dma_lds, auto ro_c) __attribute__((always_inline)) {
         constexpr bool QK = decltype(qk_c)::value, SM = decltype(sm_c)::value;
         constexpr int DMA = decltype(dma_c)::value;
+        constexpr int RO = decltype(ro_c)::value;
         constexpr bool VNEXT = SM;  // a trip with a softmax continues with phase B
         if constexpr (QK) {
             // the ring was primed by the caller with steps 0 .. kRing-1
@@ -504,11 +513,11 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_num_vgpr(kScV))) void la
                 constexpr int nk = (last_issued < KS ? last_issued : KS - 1) - g;           // K reads among them
                 constexpr int nv = last_issued >= KS ? last_issued - KS + 1 : 0;            // V steps among them
                 wait_lgkm_n<nk + 2 * nv>();
-                mma_s<Tag, kRingV + 4 * (g % kRing), kQV + 4 * g, g == 0>(sacc);
+                mma_s<Tag, kRingV + 4 * ((g + RO) % kRing), kQV + 4 * g, g == 0>(sacc);
                 if constexpr (g + kRing < KS)
-                    read_k(std::integral_constant<int, g + kRing>{}, tb);
+                    read_k(std::integral_constant<int, g + kRing>{}, tb, ro_c);
                 else if constexpr (VNEXT)
-                    read_v(std::integral_constant<int, g + kRing - KS>{}, tv);
+                    read_v(std::integral_constant<int, g + kRing - KS>{}, tv, ro_c);
                 if constexpr (SM) {
                     constexpr int per = (SMN + 27) / 28;  // spread over the first 28 steps (the last 8 carry two reads)
                     static_for<(g * per < SMN ? g * per : SMN), ((g + 1) * per < SMN ? (g + 1) * per : SMN)>(sm_op);
@@ -518,23 +527,40 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_num_vgpr(kScV))) void la
         } else {
             static_for<0, SMN>(sm_op);
             // prime the ring with V steps 0 .. kRing-2 (two reads each; the counter of outstanding reads is 4 bits)
-            static_for<0, kRing - 1>([&](auto ic) { read_v(ic, tv); });
+            static_for<0, kRing - 1>([&](auto ic) { read_v(ic, tv, ro_c); });
         }
     };
 
     // ---- phase B: O += V(t)^T P(t)^T --------------------------------------------------------------------------------
     // AHEAD: V steps requested ahead (kRing behind a phase A with matrix steps, kRing - 1 otherwise); MX: the maximum
     // of the scores in sacc is taken on the way (steps 4 .. 14)
-    auto phase_b = [&](auto ahead_c, auto mx_c, uint32_t tv, uint32_t ka_delta) {
+    // NEXTK (steady-state loop; AHEAD = kRing): the ring runs on into the next trip.  Behind step NV - kRing's matrix
+    // instruction the wave waits for its own loads of tile t+2 and meets the other waves at a barrier, after which that
+    // tile is in LDS for everyone; the last kRing steps then request the first kRing K fragments of tile t+2 (region-B
+    // base tb_next; ka[] has moved there by then), which the next trip's phase A finds on their way.
+    auto phase_b = [&](auto ahead_c, auto mx_c, uint32_t tv, uint32_t ka_delta, auto ro_c, auto nextk_c, uint32_t tb_next) __attribute__((always_inline)) {
         constexpr int AHEAD = decltype(ahead_c)::value;
         constexpr bool MX = decltype(mx_c)::value;
+        constexpr int RO = decltype(ro_c)::value;
+        constexpr bool NEXTK = decltype(nextk_c)::value;
+        static_assert(!NEXTK || (AHEAD == kRing && MX && 16 + NKA <= NV - kRing), "the K addresses move before they are used");
         static_for<0, NV>([&](auto ic) {
             constexpr int i = decltype(ic)::value;
-            constexpr int slot = (KS + i) % kRing;
+            constexpr int slot = (KS + i + RO) % kRing;
             constexpr int left = NV - 1 - i;
-            wait_lgkm_n<2 * (left < AHEAD - 1 ? left : AHEAD - 1)>();
+            // reads outstanding behind step i's: V steps (two reads each), then, NEXTK, K steps of the next tile (one each)
+            constexpr int nv = left < AHEAD - 1 ? left : AHEAD - 1;
+            constexpr int nk = NEXTK ? AHEAD - 1 - nv : 0;
+            wait_lgkm_n<2 * nv + nk>();
             mma_o<Tag, kRingV + 4 * slot, kScV + 4 * (i & 1), 16 * (i >> 1)>();
-            if constexpr (i + AHEAD < NV) read_v(std::integral_constant<int, i + AHEAD>{}, tv);
+            if constexpr (NEXTK && i == NV - AHEAD) {
+                wait_vmcnt<NLW>();  // this wave's share of tile t+2 has landed (tile t+3's loads may be outstanding)
+                asm volatile("s_barrier" ::: "memory");
+            }
+            if constexpr (i + AHEAD < NV)
+                read_v(std::integral_constant<int, i + AHEAD>{}, tv, ro_c);
+            else if constexpr (NEXTK)
+                read_k(std::integral_constant<int, i + AHEAD - NV>{}, tb_next, std::integral_constant<int, (KS + NV + RO) % kRing>{});
             if constexpr (MX && i >= 4 && i < 15) mx_op(std::integral_constant<int, i - 4>{});
             // the K read addresses move on to the buffer of the tile after next
             if constexpr (MX && i >= 16 && i < 16 + NKA)
@@ -545,7 +571,10 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_num_vgpr(kScV))) void la
     // the first kRing reads of a K tile (its region-A addresses were moved to it in the preceding phase B)
 #pragma unroll
     for (int j = 0; j < NKA; ++j) ka[j] = base_a ^ (uint32_t)(32 * j);
-    auto prime_k = [&](uint32_t tb) { static_for<0, kRing>([&](auto gc) { read_k(gc, tb); }); };
+    constexpr std::integral_constant<int, 0> ro0{};
+    constexpr std::integral_constant<int, (KS + NV) % kRing> ro1{};  // the trip behind one that started at 0
+    static_assert((2 * (KS + NV)) % kRing == 0, "two trips are a whole number of turns of the ring");
+    auto prime_k = [&](uint32_t tb) __attribute__((always_inline)) { static_for<0, kRing>([&](auto gc) { read_k(gc, tb, ro0); }); };
 
     // The part of the softmax of tile t that precedes phase A: running maximum (moved only when exceeded by kLazy;
     // then the denominator and the output tiles are rescaled) and sc = scores - maximum in log2 units.  Whole tiles
@@ -554,7 +583,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_num_vgpr(kScV))) void la
     const bool gen_all = p.is_alibi || !(sl >= 0.0f);
     // PLAIN (compile-time): the caller knows that this is a whole tile of a launch without ALiBi and with a
     // non-negative scale
-    auto softmax_head = [&](int t, auto plain_c) {
+    auto softmax_head = [&](int t, auto plain_c) __attribute__((always_inline)) {
         constexpr bool PLAIN = decltype(plain_c)::value;
         const int tok0 = c0 + t * kTile;
         const bool gen = !PLAIN && (gen_all || tok0 + kTile > c1);
@@ -606,7 +635,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_num_vgpr(kScV))) void la
 #endif
     {
         prime_k(base_b);
-        phase_a(std::true_type{}, std::false_type{}, std::integral_constant<int, -1>{}, base_b, base_v, nullptr, nullptr, 0);
+        phase_a(std::true_type{}, std::false_type{}, std::integral_constant<int, -1>{}, base_b, base_v, nullptr, nullptr, 0, ro0);
 #pragma unroll
         for (int j = 0; j < NKA; ++j) ka[j] += (uint32_t)BUF;  // on to buffer 1
         // the compiler does not see the matrix instructions inside the assembly: cover the result latency of the
@@ -632,25 +661,57 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_num_vgpr(kScV))) void la
 #ifdef DA_PIPE_PROBE
     long long pr_top = 0, pr_a = 0, pr_b = 0, pr_x0 = 0, pr_x1 = 0, pr_x2 = 0;
 #endif
-    // The common case on its own, with nothing left to decide per trip: packed rows, no ALiBi, a whole tile t+3.
-    if (!PG && packed && !gen_all) {
+    // The common case on its own, with nothing left to decide per trip: packed rows, no ALiBi, a whole tile t+3.  Here
+    // the fragment ring never drains: the barrier that makes tile t+2 visible sits eight matrix steps before the end
+    // of trip t's phase B, whose last steps already request the first K fragments of tile t+2 (phase_b, NEXTK).  A
+    // second, plain barrier at the top of a trip keeps the loads of tile t+3 behind every wave's last read of tile
+    // t-1, whose buffer they fill.  Trips come in pairs (see RO at read_k).
+    bool primed = false;  // the ring holds the first K fragments of tile t+1, which is in LDS for every wave
+    if (!PG && packed && !gen_all && t + NB < nfull) {
         uint32_t cur = 0, nxt = (uint32_t)BUF, dst = (uint32_t)((NB - 1) * BUF);  // buffers of tiles t, t+1, t+3
-        for (; t + NB - 1 < nfull; ++t) {
-            wait_vmcnt<NLW>();  // tile t+1 landed; tile t+2 may still be in flight
-            __syncthreads();    // every wave's share of tile t+1 is in LDS, and every wave is done with tile t-1
-            prime_k(base_b + nxt);
+        wait_vmcnt<NLW>();  // tile 1 landed; tile 2 may still be in flight
+        __syncthreads();
+        prime_k(base_b + nxt);
+        auto steady_trip = [&](auto ro_c) __attribute__((always_inline)) {
+#if DA_PIPE_PROBE > 1
+            const long long pr_s0 = clock64();
+#endif
             softmax_head(t, std::true_type{});
+#if DA_PIPE_PROBE > 1
+            const long long pr_s0b = clock64();
+#endif
+            asm volatile("s_barrier" ::: "memory");  // every wave is done with tile t-1
+#if DA_PIPE_PROBE > 1
+            const long long pr_s1 = clock64();
+            pr_x2 += pr_s1 - pr_s0b;
+            pr_top += pr_s1 - pr_s0;
+#endif
             phase_a(std::true_type{}, std::true_type{}, std::integral_constant<int, 1>{}, base_b + nxt, base_v + cur, kt3,
-                    kt3 + 16 * k_row_bytes, smem_off + dst);
+                    kt3 + 16 * k_row_bytes, smem_off + dst, ro_c);
+#if DA_PIPE_PROBE > 1
+            const long long pr_s2 = clock64();
+            pr_a += pr_s2 - pr_s1;
+#endif
             kt3 += kTile * k_row_bytes;
             const uint32_t nn = dst == (uint32_t)((NB - 1) * BUF) ? 0u : dst + (uint32_t)BUF;  // buffer after dst = that of tile t+4
             // (tile t+2 lies in the buffer behind nxt)
             const uint32_t nx2 = nxt == (uint32_t)((NB - 1) * BUF) ? 0u : nxt + (uint32_t)BUF;
-            phase_b(std::integral_constant<int, kRing>{}, std::true_type{}, base_v + cur, nx2 - nxt);
+            phase_b(std::integral_constant<int, kRing>{}, std::true_type{}, base_v + cur, nx2 - nxt, ro_c, std::true_type{},
+                    base_b + nx2);
+#if DA_PIPE_PROBE > 1
+            pr_b += clock64() - pr_s2;
+#endif
             cur = nxt;
             nxt = nx2;
             dst = nn;
+            ++t;
+        };
+        // (both trips of a pair load a whole tile: t + 3 and t + 4 lie below nfull)
+        for (; t + NB < nfull;) {
+            steady_trip(ro0);
+            steady_trip(ro1);
         }
+        primed = true;
     }
     for (; t + 1 < ntiles; ++t) {
 #if DA_PIPE_PROBE > 1
@@ -671,21 +732,19 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_num_vgpr(kScV))) void la
 #if DA_PIPE_PROBE > 1
         const long long pr_s0a = clock64();
 #endif
-        if (t + 2 < ntiles)
-            wait_vmcnt<NLW>();  // tile t+1 landed; tile t+2 may still be in flight
-        else
-            wait_vmcnt<0>();
-#if DA_PIPE_PROBE > 1
-        const long long pr_s0b = clock64();
-#endif
-        __syncthreads();  // every wave's share of tile t+1 is in LDS, and every wave is done with tile t-1
-#if DA_PIPE_PROBE > 1
-        const long long pr_s0c = clock64();
-        pr_x0 += pr_s0a - pr_s0;
-        pr_x1 += pr_s0b - pr_s0a;
-        pr_x2 += pr_s0c - pr_s0b;
-#endif
-        prime_k(base_b + nxt);
+        if (primed) {
+            // behind the steady-state loop: tile t+1 is in LDS for every wave and its first K fragments are on their
+            // way; what is left to wait for is every wave's last read of tile t-1
+            __syncthreads();
+            primed = false;
+        } else {
+            if (t + 2 < ntiles)
+                wait_vmcnt<NLW>();  // tile t+1 landed; tile t+2 may still be in flight
+            else
+                wait_vmcnt<0>();
+            __syncthreads();  // every wave's share of tile t+1 is in LDS, and every wave is done with tile t-1
+            prime_k(base_b + nxt);
+        }
         if (!fast && t + NB - 1 < ntiles) {
             if constexpr (PG)
                 issue_tile_pg(c0 + (t + NB - 1) * kTile, (t + NB - 1) & (NB - 1));
@@ -699,17 +758,17 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_num_vgpr(kScV))) void la
 #endif
         if (fast)
             phase_a(std::true_type{}, std::true_type{}, std::integral_constant<int, 1>{}, base_b + nxt, base_v + cur, tr.base,
-                    tr.base1, smem_off + (uint32_t)(((t + NB - 1) & (NB - 1)) * BUF));
+                    tr.base1, smem_off + (uint32_t)(((t + NB - 1) & (NB - 1)) * BUF), ro0);
         else
             phase_a(std::true_type{}, std::true_type{}, std::integral_constant<int, -1>{}, base_b + nxt, base_v + cur, nullptr,
-                    nullptr, 0);
+                    nullptr, 0, ro0);
 #if DA_PIPE_PROBE > 1
         const long long pr_s2 = clock64();
         pr_a += pr_s2 - pr_s1;
 #endif
         // (tile t+2 lies in buffer (t+2) % NB)
         phase_b(std::integral_constant<int, kRing>{}, std::true_type{}, base_v + cur,
-                (uint32_t)(((t + 2) & (NB - 1)) * BUF) - nxt);
+                (uint32_t)(((t + 2) & (NB - 1)) * BUF) - nxt, ro0, std::false_type{}, 0);
 #if DA_PIPE_PROBE > 1
         pr_b += clock64() - pr_s2;
 #endif
@@ -718,8 +777,8 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_num_vgpr(kScV))) void la
     {
         const uint32_t cur = (uint32_t)((t & (NB - 1)) * BUF);
         softmax_head(t, std::false_type{});
-        phase_a(std::false_type{}, std::true_type{}, std::integral_constant<int, -1>{}, 0, base_v + cur, nullptr, nullptr, 0);
-        phase_b(std::integral_constant<int, kRing - 1>{}, std::false_type{}, base_v + cur, 0);
+        phase_a(std::false_type{}, std::true_type{}, std::integral_constant<int, -1>{}, 0, base_v + cur, nullptr, nullptr, 0, ro0);
+        phase_b(std::integral_constant<int, kRing - 1>{}, std::false_type{}, base_v + cur, 0, ro0, std::false_type{}, 0);
     }
 
 #ifdef DA_PIPE_PROBE
@@ -807,6 +866,8 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_num_vgpr(kScV))) void la
             pa[8] = (float)(pr_w1 & 0xffffff);
             pa[9] = (float)(pr_w2 & 0xffffff);
             pa[10] = (float)(pr_wq & 0xffffff);
+            pa[11] = (float)pr_x1;
+            pa[12] = (float)pr_x2;
         }
     }
 #endif
