@@ -211,12 +211,15 @@ Plan make_plan(size_t max_seq_k, size_t batch, size_t head_q, size_t head_k, siz
         if (tun().gqa_heads == 16 || tun().gqa_heads == 32) pl.rt = tun().gqa_heads;
         pl.wave_per_head = head_k % 4 == 0 && tun().wave_per_head;
         trip = pl.wave_per_head ? da::kGqaTile : 4 * da::kGqaTile;
-        // d = 128: one work-group per CU already saturates HBM, and half as many splits halve the merge (measured,
-        // 256 against 512 work-groups: 32/8 heads, batch 64 x 4096 tokens 183.8 -> 181.8 us, batch 128 x 2048 183.6 ->
-        // 178.0; MQA 32/1, batch 64 x 4096 35.8 -> 31.5; 16/2 heads, batch 32 x 4096 30.6 -> 27.6)
+        // d = 128, four waves sharing one KV head's tokens (MQA and other head counts that are no multiple of four): one
+        // work-group per CU already saturates what this form can pull, and half as many splits halve the merge
+        // (measured, 256 against 512 work-groups: MQA 32/1, batch 64 x 4096 tokens 35.7 -> 29.6 us; 16/2 heads, batch 32
+        // x 4096 a tie).  With one wave per KV head the usual 512 do better since the K/V loads are non-temporal
+        // (32/8 heads, batch 64 x 4096 tokens 170.4 -> 166.1 us, batch 128 x 2048 167.4 -> 165.0; with ordinary loads it
+        // was the other way round, 181.8 against 183.8).
         // (16-bit K/V in whole tiles or 16-token runs only: the 8-bit forms and the per-row page lookups keep fewer
         // bytes in flight per work-group and need the 512; FP8, batch 64 x 4096 tokens: 96 us against 110)
-        if (dim == 128 && !kv_8bit && (packed || page_size >= 16)) target_wgs = tun().group_target_wgs_d128;
+        if (dim == 128 && !kv_8bit && (packed || page_size >= 16) && !pl.wave_per_head) target_wgs = tun().group_target_wgs_d128;
     } else {
         pl.kind = kKindSweep;
         const int max_rt = dim > 256 ? 2 : 4;

@@ -198,7 +198,7 @@ __global__ __launch_bounds__(64 * NWV) void mfma_latent_kernel(const SweepParams
                 const uint32_t row = off / (uint32_t)D, within = off - row * (uint32_t)D;
                 // rows 0..15 fill loads 0..8 exactly, rows 16..31 loads 9..17: the run is wave-uniform
                 const int run = min(j >= 16 * D / 1024 ? 1 : 0, last >> 4);
-                lds_dma16(run ? base1 : base,
+                lds_dma16<true>(run ? base1 : base,
                           (uint32_t)(min((int)row, last) - run * 16) * (uint32_t)k_row_bytes + within,
                           smem_off + (uint32_t)(STG0 + buf * STG + (wave + NWV * q) * 1024));
             }
@@ -208,7 +208,7 @@ __global__ __launch_bounds__(64 * NWV) void mfma_latent_kernel(const SweepParams
         for (int q = 0; q < NLA; ++q) {
             const int row = wave + NWV * q;  // wave-uniform
             const int rc = min(row, last), run = rc >> 4;
-            lds_dma16(run ? base1 : base,
+            lds_dma16<true>(run ? base1 : base,
                       (uint32_t)(rc - run * 16) * (uint32_t)k_row_bytes + (lane16 ^ (uint32_t)(swz_a(row) * 16)),
                       smem_off + (uint32_t)(buf * BUF + OFF_KA + row * ROW_A));
         }
@@ -219,7 +219,7 @@ __global__ __launch_bounds__(64 * NWV) void mfma_latent_kernel(const SweepParams
             for (int q = 0; q < NLA; ++q) {
                 const int row = wave + NWV * q;
                 const int rc = min(row, last), run = rc >> 4;
-                lds_dma16(run ? vbase1 : vbase,
+                lds_dma16<true>(run ? vbase1 : vbase,
                           (uint32_t)(rc - run * 16) * (uint32_t)v_row_bytes + (lane16 ^ (uint32_t)(swz_a(row) * 16)),
                           smem_off + (uint32_t)(buf * BUF + row * ROW_A));
             }
@@ -229,7 +229,7 @@ __global__ __launch_bounds__(64 * NWV) void mfma_latent_kernel(const SweepParams
             const int j = wave + NWV * q;
             const int row = j * 8 + rb;
             const int run = min(j >> 1, last >> 4);  // the eight rows of a load lie in one run, clamped or not
-            lds_dma16(run ? base1 : base, (uint32_t)(min(row, last) - run * 16) * (uint32_t)k_row_bytes +
+            lds_dma16<true>(run ? base1 : base, (uint32_t)(min(row, last) - run * 16) * (uint32_t)k_row_bytes +
                                               (uint32_t)(DV * 2 + (((lane & 7) ^ swz_b(row)) * 16)),
                       smem_off + (uint32_t)(buf * BUF + OFF_B + j * 1024));
         }
@@ -262,14 +262,14 @@ __global__ __launch_bounds__(64 * NWV) void mfma_latent_kernel(const SweepParams
 #pragma unroll
             for (int q = 0; q < NLA; ++q) {
                 const int row = wave * NLA + q;
-                if (lane < D / 16) lds_dma16(kbytes + rowoff[q], lane16, smem_off + (uint32_t)(STG0 + buf * STG + row * D));
+                if (lane < D / 16) lds_dma16<true>(kbytes + rowoff[q], lane16, smem_off + (uint32_t)(STG0 + buf * STG + row * D));
             }
             return;
         }
 #pragma unroll
         for (int q = 0; q < NLA; ++q) {
             const int row = wave * NLA + q;
-            lds_dma16(kbytes + rowoff[q], lane16 ^ (uint32_t)(swz_a(row) * 16),
+            lds_dma16<true>(kbytes + rowoff[q], lane16 ^ (uint32_t)(swz_a(row) * 16),
                       smem_off + (uint32_t)(buf * BUF + row * ROW_A));
         }
 #pragma unroll
@@ -279,7 +279,7 @@ __global__ __launch_bounds__(64 * NWV) void mfma_latent_kernel(const SweepParams
             int64_t mine = rowoff[8 * q];
 #pragma unroll
             for (int i = 1; i < 8; ++i) mine = rb == i ? rowoff[8 * q + i] : mine;
-            lds_dma16_v(kbytes + mine + (DV * 2 + (((lane & 7) ^ swz_b(row)) * 16)),
+            lds_dma16_v<true>(kbytes + mine + (DV * 2 + (((lane & 7) ^ swz_b(row)) * 16)),
                         smem_off + (uint32_t)(buf * BUF + OFF_B + j * 1024));
         }
     };

@@ -240,12 +240,12 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_num_vgpr(kScV))) void la
             asm volatile("v_xor_b32 %0, %1, %2\n\tv_add_u32 %0, %3, %0"
                          : "=&v"(off)
                          : "s"((uint32_t)(swz_a(row) * 16)), "v"(lane16), "s"((uint32_t)(rc - run * 16) * (uint32_t)k_row_bytes));
-            lds_dma16(run ? base1 : base, off, smem_off + (uint32_t)(buf * BUF + row * ROW_A));
+            lds_dma16<true>(run ? base1 : base, off, smem_off + (uint32_t)(buf * BUF + row * ROW_A));
         } else {
             const int j = wave;
             const int row = j * 8 + rb;
             const int run = min(j >> 1, last >> 4);  // the eight rows of a load lie in one run, clamped or not
-            lds_dma16(run ? base1 : base, (uint32_t)(min(row, last) - run * 16) * (uint32_t)k_row_bytes +
+            lds_dma16<true>(run ? base1 : base, (uint32_t)(min(row, last) - run * 16) * (uint32_t)k_row_bytes +
                                               (uint32_t)(DV * 2 + (((lane & 7) ^ swz_b(row)) * 16)),
                       smem_off + (uint32_t)(buf * BUF + OFF_B + j * 1024));
         }
@@ -282,7 +282,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_num_vgpr(kScV))) void la
 #pragma unroll
         for (int q = 0; q < NLA; ++q) {
             const int row = wave * NLA + q;
-            lds_dma16(kbytes + rowoff[q], lane16 ^ (uint32_t)(swz_a(row) * 16),
+            lds_dma16<true>(kbytes + rowoff[q], lane16 ^ (uint32_t)(swz_a(row) * 16),
                       smem_off + (uint32_t)(buf * BUF + row * ROW_A));
         }
         {
@@ -291,7 +291,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_num_vgpr(kScV))) void la
             int64_t mine = rowoff[0];
 #pragma unroll
             for (int i = 1; i < 8; ++i) mine = rb == i ? rowoff[i] : mine;
-            lds_dma16_v(kbytes + mine + (DV * 2 + (((lane & 7) ^ swz_b(row)) * 16)),
+            lds_dma16_v<true>(kbytes + mine + (DV * 2 + (((lane & 7) ^ swz_b(row)) * 16)),
                         smem_off + (uint32_t)(buf * BUF + OFF_B + j * 1024));
         }
     };
@@ -392,10 +392,10 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_num_vgpr(kScV))) void la
                 off = lane16w;
             else
                 asm volatile("v_xor_b32 %0, %1, %2" : "=v"(off) : "n"((q & 3) * 16), "v"(lane16w));
-            lds_dma16((q < 4 ? base : base1) + rowoff[q & 3], off,
+            lds_dma16<true>((q < 4 ? base : base1) + rowoff[q & 3], off,
                       lds_buf + (uint32_t)(q * NWV * ROW_A) + (uint32_t)(wave * ROW_A));
         } else {
-            lds_dma16((wave >> 1) ? base1 : base, voff_b, lds_buf + (uint32_t)OFF_B + (uint32_t)(wave * 1024));
+            lds_dma16<true>((wave >> 1) ? base1 : base, voff_b, lds_buf + (uint32_t)OFF_B + (uint32_t)(wave * 1024));
         }
     };
 

@@ -9,15 +9,17 @@
 
 namespace {
 
-// Each work-group reads one contiguous slab with 16-byte loads, eight in flight per lane.
-__global__ __launch_bounds__(256) void stream_read_kernel(const uint4* __restrict__ p, size_t per_block, uint32_t* sink) {
+// Each work-group reads one contiguous slab with 16-byte loads, eight in flight per lane, marked non-temporal as the
+// attention kernels' K/V loads are (6.2-6.3 TB/s with ordinary loads, 7.0-7.1 TB/s with the hint, on this GPU).
+typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
+__global__ __launch_bounds__(256) void stream_read_kernel(const u32x4* __restrict__ p, size_t per_block, uint32_t* sink) {
     constexpr int U = 8;
-    const uint4* b = p + (size_t)blockIdx.x * per_block;
+    const u32x4* b = p + (size_t)blockIdx.x * per_block;
     uint32_t acc = 0;
     for (size_t i = threadIdx.x; i + (size_t)(U - 1) * 256 < per_block; i += (size_t)256 * U) {
-        uint4 a[U];
+        u32x4 a[U];
 #pragma unroll
-        for (int u = 0; u < U; ++u) a[u] = b[i + (size_t)u * 256];
+        for (int u = 0; u < U; ++u) a[u] = __builtin_nontemporal_load(&b[i + (size_t)u * 256]);
 #pragma unroll
         for (int u = 0; u < U; ++u) acc ^= a[u].x ^ a[u].y ^ a[u].z ^ a[u].w;
     }
@@ -88,7 +90,7 @@ extern "C" int da_probe_stream_read(const void* buf, size_t bytes, void* sink, v
     const size_t per_block = bytes / 16 / kBlocks / kGrain * kGrain;
     if (per_block == 0) return DA_ERR_INVALID_ARGUMENT;  // needs at least 128 MiB
     hipLaunchKernelGGL(stream_read_kernel, dim3(kBlocks), dim3(256), 0, reinterpret_cast<hipStream_t>(hip_stream),
-                       reinterpret_cast<const uint4*>(buf), per_block, reinterpret_cast<uint32_t*>(sink));
+                       reinterpret_cast<const u32x4*>(buf), per_block, reinterpret_cast<uint32_t*>(sink));
     return hipGetLastError() == hipSuccess ? DA_OK : DA_ERR_HIP;
 }
 

@@ -94,9 +94,9 @@ __global__ __launch_bounds__(256) void sweep_kernel(const SweepParams p) {
     const float vs = head_scale(p.v_scale, hk);
     auto load8 = [](const uint8_t* ptr) __attribute__((always_inline)) {  // eight elements as 16-bit pairs
         if constexpr (KV8)
-            return kv8x8_to_16<Tag, KV8>(*reinterpret_cast<const uint2*>(ptr));
+            return kv8x8_to_16<Tag, KV8>(stream_load8(ptr));
         else
-            return *reinterpret_cast<const uint4*>(ptr);
+            return stream_load16(ptr);
     };
 
     const int ntiles = (c1 - c0 + TILE - 1) / TILE;

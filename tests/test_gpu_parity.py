@@ -271,7 +271,7 @@ def test_reference_signature_entry_point_with_library_workspace():
 
 def test_reference_signature_entry_point_takes_the_plan_of_a_uniform_batch():
     """BASELINE's GQA shape (batch 64 x 4096 tokens, 32/8 heads) through da_decoding_attn, which is told no token
-    count: the same cut as the counted call (two splits of 2048 tokens), so the same bits and the same time as the
+    count: the same cut as the counted call (four splits of 1024 tokens), so the same bits and the same time as the
     Python face; and the library's cached workspace can be released and is allocated again on the next call."""
     lib = _lib.load()
     w = wl.config_gqa_fixed(seed=0)

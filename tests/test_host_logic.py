@@ -98,7 +98,11 @@ def test_plan_without_a_token_count_at_d128():
     blind = _lib.plan(4096, 64, 32, 8, 128, 128)
     counted = _lib.plan(4096, 64, 32, 8, 128, 128, total_k=64 * 4096)
     assert blind["kind"] == counted["kind"] == 3
-    assert (blind["nsplit"], blind["chunk"]) == (counted["nsplit"], counted["chunk"]) == (2, 2048)
+    assert (blind["nsplit"], blind["chunk"]) == (counted["nsplit"], counted["chunk"]) == (4, 1024)
+    # a long sequence of a small batch: the cap, not the work-group target, sets the cut
+    assert _lib.plan(16384, 64, 32, 8, 128, 128)["chunk"] == 2048
+    # MQA (four waves share the one KV head's tokens): 256 work-groups
+    assert _lib.plan(4096, 64, 32, 1, 128, 128, total_k=64 * 4096)["nsplit"] == 4
     assert _lib.load().da_release_workspaces() == _lib.DA_OK  # nothing cached, nothing to free, no GPU needed
 
 
