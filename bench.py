@@ -34,8 +34,8 @@ MFMA_PEAK_TFLOPS = 2500.0   # MI355X dense fp16/bf16 MFMA, published
 # scaled by what it reads for a 1 GiB device copy (profiles/*_hbm_traffic.md).  A figure belongs to the launch plan
 # it was measured under; when the library plans the workload differently, the bench line carries null instead.
 MEASURED_TRAFFIC = {
-    "gqa": {"bytes": 1079830528, "plan": {"kind": 3, "nsplit": 2, "chunk": 2048, "heads_per_group": 16}},
-    "mla": {"bytes": 388052992, "plan": {"kind": 2, "nsplit": 4, "chunk": 1024, "heads_per_group": 128},
+    "gqa": {"bytes": 1092312678, "plan": {"kind": 3, "nsplit": 4, "chunk": 1024, "heads_per_group": 16}},
+    "mla": {"bytes": 388134502, "plan": {"kind": 2, "nsplit": 4, "chunk": 1024, "heads_per_group": 128},
             "partials": "16-bit"},
 }
 

@@ -98,12 +98,6 @@ __device__ __forceinline__ uint4 stream_load16(const void* p) {
     return make_uint4(v.x, v.y, v.z, v.w);
 }
 
-__device__ __forceinline__ uint2 stream_load8(const void* p) {
-    typedef unsigned int u32x2 __attribute__((ext_vector_type(2)));
-    const u32x2 v = __builtin_nontemporal_load(reinterpret_cast<const u32x2*>(p));
-    return make_uint2(v.x, v.y);
-}
-
 // Formats of an 8-bit K/V cache (template argument KV8 of the kernels; 0 = 16-bit K/V).
 constexpr int kKvFp8 = 1;   // OCP e4m3
 constexpr int kKvInt8 = 2;  // two's-complement integers

@@ -94,7 +94,7 @@ __global__ __launch_bounds__(256) void sweep_kernel(const SweepParams p) {
     const float vs = head_scale(p.v_scale, hk);
     auto load8 = [](const uint8_t* ptr) __attribute__((always_inline)) {  // eight elements as 16-bit pairs
         if constexpr (KV8)
-            return kv8x8_to_16<Tag, KV8>(stream_load8(ptr));
+            return kv8x8_to_16<Tag, KV8>(*reinterpret_cast<const uint2*>(ptr));  // (8-byte loads run slower with the non-temporal hint: MHA batch 512 x 128 tokens, FP8, 105 -> 131 us)
         else
             return stream_load16(ptr);
     };
