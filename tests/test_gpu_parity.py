@@ -106,6 +106,29 @@ def test_config4_mla_points(batch, seq_k):
     check_against_oracle(w, run_hip(w))
 
 
+@pytest.mark.parametrize("dtype", DTYPES, ids=_name)
+def test_latent_kernel_every_trip_count(dtype):
+    """256 unsplit sequences of 129 .. 420 tokens, 128 heads: one work-group per sequence, so every count of whole
+    tiles from 4 to 13 occurs with and without a partial last tile, on both sides of where the pipelined kernel's
+    steady-state loop (pairs of trips) starts and hands over to its general loop.  Every 5th sequence and the ten
+    shortest and longest against the oracle, every row finite."""
+    lens = torch.tensor([129 + (i * 37) % 292 for i in range(256)], dtype=torch.int32)
+    g = torch.Generator().manual_seed(17)
+    total = int(lens.sum())
+    q = torch.randn(256, 128, 576, generator=g).to(dtype)
+    k = torch.randn(total, 1, 576, generator=g).to(dtype)
+    w = wl.Workload("trip_counts", q, k, None, wl.get_cu_seq(lens), int(lens.max()), 512, False, lens.tolist())
+    p = _lib.plan(w.max_seq_k, 256, 128, 1, 576, 512, total_k=total)
+    assert (p["kind"], p["nsplit"], p["heads_per_group"]) == (2, 1, 128)
+    assert {int(n) // 32 for n in lens.tolist()} >= set(range(4, 14))
+    o = run_hip(w)
+    assert torch.isfinite(o.float()).all()
+    order = sorted(range(256), key=lambda i: int(lens[i]))
+    rows = sorted(set(list(range(0, 256, 5)) + order[:10] + order[-10:]))
+    _, ref32 = run_oracle(sub_workload(w, rows))
+    assert (o[rows].float() - ref32).abs().max().item() <= TOL[dtype]
+
+
 @pytest.mark.parametrize("batch,seq_k,step", [(16, 8192, 3), (16, 16384, 5), (128, 4096, 16)])
 def test_config4_mla_large_points(batch, seq_k, step):
     """The largest points of the two sweeps: every output finite, every step-th sequence (and the last) against the
