@@ -40,14 +40,16 @@ def _replay_matches_eager(run, tensors_to_perturb, out_of):
         assert torch.equal(got.view(torch.int16), want.view(torch.int16)), f"replay {step}"
 
 
-@pytest.mark.parametrize("shape", ["gqa_split", "mha_unsplit", "mla"])
+@pytest.mark.parametrize("shape", ["gqa_split", "mha_unsplit", "mla", "mla_distinct_v"])
 def test_packed_call_replays_from_a_graph(shape):
     if shape == "gqa_split":
         w = wl.make_workload(8, 32, 8, 128, 128, 2048, torch.bfloat16, seed=4, varlen=True)
     elif shape == "mha_unsplit":
         w = wl.make_workload(64, 8, 8, 128, 128, 128, torch.float16, seed=4)
+    elif shape == "mla":
+        w = wl.config_mla(4, 700, seed=4)  # the pipelined latent kernel, five tiles per split
     else:
-        w = wl.config_mla(4, 700, seed=4)
+        w = wl.make_workload(4, 128, 1, 576, 512, 700, torch.float16, seed=4, latent=False)  # V in its own buffer
     wd = w.to(DEV)
 
     def run():
