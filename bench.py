@@ -90,7 +90,7 @@ def _device_copies(torch, w, dev, min_total_bytes=768 << 20):
     return copies
 
 
-def measure(torch, w, steps, warmup, page_size=0, kv_fp8=False, kv_int8=False):
+def measure(torch, w, steps, warmup, page_size=0, kv_fp8=False, kv_int8=False, kv_int4=False):
     from decoding_attention_amd import _lib, decoding_attn_fwd
     from decoding_attention_amd import workloads as wl
 
@@ -99,13 +99,16 @@ def measure(torch, w, steps, warmup, page_size=0, kv_fp8=False, kv_int8=False):
     outs = []
 
     def make(c):
-        if kv_fp8 or kv_int8:  # K/V as FP8 (e4m3) or int8 with per-head scales; q and o stay 16-bit
+        if kv_fp8 or kv_int8 or kv_int4:  # K/V as FP8 (e4m3), int8 or int4 with per-head scales; q and o stay 16-bit
             def quantise(x, step):
+                if kv_int4:
+                    from decoding_attention_amd import pack_int4
+                    return pack_int4(torch.round(x.float() / step).clamp(-8, 7).to(torch.int8))
                 if kv_int8:
                     return torch.round(x.float() / step).clamp(-128, 127).to(torch.int8)
                 return (x.float() / step).to(torch.float8_e4m3fn)
 
-            step = 4.0 / 127 if kv_int8 else 0.02
+            step = 3.0 / 7 if kv_int4 else (4.0 / 127 if kv_int8 else 0.02)
             ks = torch.full((w.head_k,), step, device=dev)
             k8 = quantise(c.k, step)
             v8 = None if c.v is None else quantise(c.v, step)  # (latent form: V is in K)
@@ -133,9 +136,10 @@ def measure(torch, w, steps, warmup, page_size=0, kv_fp8=False, kv_int8=False):
     mean_ms, min_ms = _time_calls(torch, fns, steps, warmup)
     assert torch.isfinite(outs[0].float()).all()
     nbytes = wl.workload_bytes(w)
-    if kv_fp8 or kv_int8:  # one byte per K/V element
+    if kv_fp8 or kv_int8 or kv_int4:  # one byte (half a byte) per K/V element
+        kv_elems = int(w.k.numel() + (w.v.numel() if w.v is not None else 0))
         nbytes = wl.algorithmic_bytes(w.batch, w.head_q, w.head_k, w.dim, w.dim_v, int(w.k.shape[0]), w.v is not None,
-                                      elem_bytes=2) - int(w.k.numel() + (w.v.numel() if w.v is not None else 0))
+                                      elem_bytes=2) - (kv_elems * 3 // 2 if kv_int4 else kv_elems)
     flops = wl.workload_flops(w)
     plan = _lib.plan(w.max_seq_k, w.batch, w.head_q, w.head_k, w.dim, w.dim_v, total_k=int(w.k.shape[0]))
     return {
@@ -460,10 +464,12 @@ def run_sweep(args, measure_fn=None, workload_fn=None, out=None):
     if args.sweep == "paged":  # the benchmark shapes over shuffled pages of 64, 16 and 1 tokens, beside the packed layout
         for w in (wl.config_gqa_fixed(), wl.config_gqa_varlen(), wl.config_mqa_alibi(), wl.config_mla(64, 4096)):
             shapes += [(None, "packed", w, {})] + [(None, f"paged-{n}", w, {"page_size": n}) for n in (64, 16, 1)]
-    if args.sweep == "fp8":  # 16-bit against FP8 and int8 K/V on the bandwidth-bound shapes and the latent form
+    if args.sweep == "fp8":  # 16-bit against FP8, int8 and int4 K/V on the bandwidth-bound shapes and the latent form
         for w in (wl.config_gqa_fixed(), wl.config_mha_sweep(512, 128), wl.config_mha_sweep(1, 8192),
                   wl.config_mqa_alibi(), wl.config_mla(64, 4096), wl.config_mla(16, 4096)):
             shapes += [(None, "kv16", w, {}), (None, "kv-fp8", w, {"kv_fp8": True}), (None, "kv-int8", w, {"kv_int8": True})]
+            if w.dim != 576:  # (the latent kernel has no int4 form)
+                shapes += [(None, "kv-int4", w, {"kv_int4": True})]
     results = []
     for marker, tag, spec, kw in shapes:
         if marker == SEQ_MARKER:

@@ -25,6 +25,9 @@ EXPORTED_SYMBOLS = (
     "da_decoding_attn_int8kv",
     "da_decoding_attn_paged_int8kv",
     "da_workspace_bytes_int8kv",
+    "da_decoding_attn_int4kv",
+    "da_decoding_attn_paged_int4kv",
+    "da_workspace_bytes_int4kv",
     "da_plan",
     "da_plan_distinct_v",
     "da_supported_head_dims",
@@ -95,6 +98,12 @@ def _declare(lib):
     lib.da_decoding_attn_paged_int8kv.argtypes = lib.da_decoding_attn_paged_fp8kv.argtypes
     lib.da_workspace_bytes_int8kv.restype = sz
     lib.da_workspace_bytes_int8kv.argtypes = lib.da_workspace_bytes_fp8kv.argtypes
+    lib.da_decoding_attn_int4kv.restype = ci
+    lib.da_decoding_attn_int4kv.argtypes = lib.da_decoding_attn_fp8kv.argtypes
+    lib.da_decoding_attn_paged_int4kv.restype = ci
+    lib.da_decoding_attn_paged_int4kv.argtypes = lib.da_decoding_attn_paged_fp8kv.argtypes
+    lib.da_workspace_bytes_int4kv.restype = sz
+    lib.da_workspace_bytes_int4kv.argtypes = lib.da_workspace_bytes_fp8kv.argtypes
     ip = ctypes.POINTER(ci)
     lib.da_plan.restype = ci
     lib.da_plan.argtypes = [sz, sz, sz, sz, sz, sz, ci, sz, ip, ip, ip, ip]

@@ -25,6 +25,7 @@ SOURCES = [
     "da_sweep_kv8.hip",
     "da_gqa_mfma_kv8.hip",
     "da_gqa_mfma_i8.hip",
+    "da_gqa_mfma_i4.hip",
 ]
 
 # libdecoding_attn_probe.so (measurement aids of bench.py, include/decoding_attn_probe.h): the same objects, with

@@ -550,8 +550,8 @@ struct Paging {
     size_t page_size = 0, max_blocks = 0, k_page = 0, v_page = 0;
 };
 
-// Element format of K/V: 16-bit like Q (fmt 0), or 8-bit (da::kKvFp8, da::kKvInt8) with per-KV-head de-quantisation
-// factors (null = 1).
+// Element format of K/V: 16-bit like Q (fmt 0), or 8-bit (da::kKvFp8, da::kKvInt8) or 4-bit (da::kKvInt4) with
+// per-KV-head de-quantisation factors (null = 1).
 struct KvFormat {
     bool sweep_only = false;  // measurement: leave the split partials in the workspace, do not merge them
     int fmt = 0;
@@ -600,6 +600,10 @@ int run_attention(const void* q, const void* k, const void* v, void* o, const in
                               pg.table ? pg.page_size : 0, kf.fmt != 0);
     if ((size_t)head_k * pl.groups > 65535)
         return fail(DA_ERR_INVALID_ARGUMENT, "head_k * groups exceeds the grid limit 65535");
+    if (kf.fmt == da::kKvInt4 && pl.kind == kKindMfma)
+        return fail(DA_ERR_UNSUPPORTED,
+                    "an int4 K/V cache at (576, 512) is built for up to 32 query heads per KV head (the grouped kernel); "
+                    "%zu heads would need the latent kernel", head_q / head_k);
 
     void* ws = nullptr;
     if (pl.ws_bytes > 0) {
@@ -620,6 +624,12 @@ int run_attention(const void* q, const void* k, const void* v, void* o, const in
     // V absent: the values are the leading dim_v columns of each K row, read with K's pitch
     // (reference csrc/ops/decoding_attn.cpp:30-37).
     sp.v = v ? v : k;
+    if (kf.fmt == da::kKvInt4) {
+        // two elements to a byte: the kernels do the int8 cache's address arithmetic on twice the address and halve
+        // it at the load (da::kKvInt4 in da_common.h)
+        sp.k = reinterpret_cast<const void*>(reinterpret_cast<uintptr_t>(sp.k) * 2);
+        sp.v = reinterpret_cast<const void*>(reinterpret_cast<uintptr_t>(sp.v) * 2);
+    }
     sp.o = o;
     sp.cu_seq_k = cu_seq_k;
     sp.ws_o = reinterpret_cast<float*>(ws);
@@ -667,6 +677,8 @@ int run_attention(const void* q, const void* k, const void* v, void* o, const in
             e = da::launch_mla_kv8(sp, kf.fmt, is_bf16 != 0, pl.rt, grid, stream);
         else if (pl.kind == kKindGroup && kf.fmt == da::kKvInt8)
             e = da::launch_gqa_mfma_i8(sp, is_bf16 != 0, (int)dim, pl.rt, pl.wave_per_head, grid, stream);
+        else if (pl.kind == kKindGroup && kf.fmt == da::kKvInt4)
+            e = da::launch_gqa_mfma_i4(sp, is_bf16 != 0, (int)dim, pl.rt, pl.wave_per_head, grid, stream);
         else if (pl.kind == kKindGroup)
             e = da::launch_gqa_mfma_kv8(sp, is_bf16 != 0, (int)dim, pl.rt, pl.wave_per_head, grid, stream);
         else
@@ -845,6 +857,37 @@ int da_decoding_attn_paged_int8kv(const void* q, const void* k_pages, const void
     return run_attention(q, k_pages, v_pages, o, nullptr, pg, kv8_format(da::kKvInt8, k_scale, v_scale), max_seq_k,
                          batch, head_q, head_k, dim, dim_v, is_alibi, is_bf16, softmax_scale, alibi_slopes, total_k,
                          workspace, workspace_bytes, hip_stream);
+}
+
+int da_decoding_attn_int4kv(const void* q, const void* k4, const void* v4, void* o, const int32_t* cu_seq_k,
+                            size_t max_seq_k, size_t batch, size_t head_q, size_t head_k, size_t dim, size_t dim_v,
+                            int is_alibi, int is_bf16, float softmax_scale, const float* alibi_slopes,
+                            const float* k_scale, const float* v_scale, size_t total_k, void* workspace,
+                            size_t workspace_bytes, void* hip_stream) {
+    return run_attention(q, k4, v4, o, cu_seq_k, Paging{}, kv8_format(da::kKvInt4, k_scale, v_scale), max_seq_k, batch,
+                         head_q, head_k, dim, dim_v, is_alibi, is_bf16, softmax_scale, alibi_slopes, total_k,
+                         workspace, workspace_bytes, hip_stream);
+}
+
+int da_decoding_attn_paged_int4kv(const void* q, const void* k_pages, const void* v_pages, void* o,
+                                  const int32_t* block_table, const int32_t* seq_lens, size_t max_seq_k, size_t batch,
+                                  size_t head_q, size_t head_k, size_t dim, size_t dim_v, size_t page_size,
+                                  size_t max_blocks_per_seq, size_t k_page_stride, size_t v_page_stride, int is_alibi,
+                                  int is_bf16, float softmax_scale, const float* alibi_slopes, const float* k_scale,
+                                  const float* v_scale, size_t total_k, void* workspace, size_t workspace_bytes,
+                                  void* hip_stream) {
+    Paging pg;
+    const int rc = check_paging(block_table, seq_lens, max_seq_k, head_k, dim, dim_v, page_size, max_blocks_per_seq,
+                                k_page_stride, v_page_stride, v_pages != nullptr, &pg);
+    if (rc != DA_OK) return rc;
+    return run_attention(q, k_pages, v_pages, o, nullptr, pg, kv8_format(da::kKvInt4, k_scale, v_scale), max_seq_k,
+                         batch, head_q, head_k, dim, dim_v, is_alibi, is_bf16, softmax_scale, alibi_slopes, total_k,
+                         workspace, workspace_bytes, hip_stream);
+}
+
+size_t da_workspace_bytes_int4kv(size_t max_seq_k, size_t batch, size_t head_q, size_t head_k, size_t dim,
+                                 size_t dim_v, size_t total_k, size_t page_size) {
+    return da_workspace_bytes_fp8kv(max_seq_k, batch, head_q, head_k, dim, dim_v, total_k, page_size);
 }
 
 int da_release_workspaces(void) { return release_cached_workspaces(true); }

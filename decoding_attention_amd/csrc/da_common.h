@@ -101,6 +101,12 @@ __device__ __forceinline__ uint4 stream_load16(const void* p) {
 // Formats of an 8-bit K/V cache (template argument KV8 of the kernels; 0 = 16-bit K/V).
 constexpr int kKvFp8 = 1;   // OCP e4m3
 constexpr int kKvInt8 = 2;  // two's-complement integers
+// Four-bit integers (two's complement, -8 .. 7), two to a byte, element 2 i in the low half of byte i.  The kernels
+// address such a cache as if it held one byte per element: the host hands them TWICE the buffer's address
+// (SweepParams::k and ::v), all their row, head and lane arithmetic is the int8 arithmetic on those doubled addresses,
+// and the load halves the address again (kv4_load8 / kv4_load16; every address the kernels form is even).  A load
+// widens the nibbles to sign-extended bytes, from where on the data is an int8 cache's.
+constexpr int kKvInt4 = 3;
 
 // Eight FP8 (OCP e4m3) values -> eight 16-bit elements of the compute type.  Both conversions are exact (e4m3
 // has 3 mantissa bits and |x| <= 448), so an FP8 K/V cache feeds the same arithmetic as a 16-bit one.
@@ -150,10 +156,36 @@ __device__ __forceinline__ uint2 int8x4_to_16(uint32_t w) {
     return r;
 }
 
-// Eight elements of an 8-bit K/V cache of format FMT -> eight 16-bit elements of the compute type.
+// Eight four-bit integers (one 32-bit word, element i in bits 4 i .. 4 i + 3) -> eight sign-extended bytes in element
+// order.  Low and high nibbles are separated, interleaved again with two byte permutes, and each byte is
+// sign-extended from four bits without carries between the bytes: (u ^ 8 | 0x80) - 8 lies in 0x78 .. 0x87, and
+// flipping the top bit again gives u - 8 ... the value of the nibble as a two's-complement byte.
+__device__ __forceinline__ uint2 int4x8_to_int8(uint32_t w) {
+    const uint32_t lo = w & 0x0F0F0F0Fu;         // elements 0, 2, 4, 6
+    const uint32_t hi = (w >> 4) & 0x0F0F0F0Fu;  // elements 1, 3, 5, 7
+    // v_perm_b32 selector: 0 .. 3 = bytes of the second operand, 4 .. 7 = bytes of the first
+    const uint32_t d0 = __builtin_amdgcn_perm(hi, lo, 0x05010400u);  // elements 0, 1, 2, 3
+    const uint32_t d1 = __builtin_amdgcn_perm(hi, lo, 0x07030602u);  // elements 4, 5, 6, 7
+    uint2 r;
+    r.x = ((((d0 ^ 0x08080808u) | 0x80808080u) - 0x08080808u) ^ 0x80808080u);
+    r.y = ((((d1 ^ 0x08080808u) | 0x80808080u) - 0x08080808u) ^ 0x80808080u);
+    return r;
+}
+// Sixteen (eight) elements of an int4 cache at the doubled address `vptr` (see kKvInt4), as sign-extended bytes.
+__device__ __forceinline__ uint4 kv4_load16(const void* vptr) {
+    const uint2 w = *reinterpret_cast<const uint2*>(reinterpret_cast<uintptr_t>(vptr) >> 1);
+    const uint2 a = int4x8_to_int8(w.x), b = int4x8_to_int8(w.y);
+    return make_uint4(a.x, a.y, b.x, b.y);
+}
+__device__ __forceinline__ uint2 kv4_load8(const void* vptr) {
+    return int4x8_to_int8(*reinterpret_cast<const uint32_t*>(reinterpret_cast<uintptr_t>(vptr) >> 1));
+}
+
+// Eight elements of an 8-bit K/V cache of format FMT -> eight 16-bit elements of the compute type (an int4 cache's
+// elements have been widened to int8 by the load).
 template <typename Tag, int FMT>
 __device__ __forceinline__ uint4 kv8x8_to_16(uint2 w) {
-    static_assert(FMT == kKvFp8 || FMT == kKvInt8, "8-bit K/V format");
+    static_assert(FMT == kKvFp8 || FMT == kKvInt8 || FMT == kKvInt4, "8-bit K/V format");
     if constexpr (FMT == kKvFp8) {
         return fp8x8_to_16<Tag>(w);
     } else {

@@ -228,7 +228,9 @@ __device__ __forceinline__ void gqa_segment(const SweepParams& p, uint8_t* const
     // serve several head groups from the caches and which measured slower with the hint (16 heads, batch 64 x 4096
     // tokens: 63.8 -> 67.2 us).
     auto kv_load16 = [](const uint8_t* ptr) __attribute__((always_inline)) {
-        if constexpr (VK)
+        if constexpr (KV8 == kKvInt4)
+            return kv4_load16(ptr);  // (eight bytes from half the address, widened to sixteen int8 elements)
+        else if constexpr (VK)
             return *reinterpret_cast<const uint4*>(ptr);
         else
             return stream_load16(ptr);
@@ -611,6 +613,9 @@ hipError_t launch_gqa_mfma_kv8(const SweepParams& p, bool is_bf16, int dim, int 
                                dim3 grid, hipStream_t stream);
 // the same with int8 K and V; dim must be a multiple of 64
 hipError_t launch_gqa_mfma_i8(const SweepParams& p, bool is_bf16, int dim, int heads_per_group, bool wave_per_head,
+                              dim3 grid, hipStream_t stream);
+// ... and over an int4 one (two elements to a byte, see kKvInt4 in da_common.h)
+hipError_t launch_gqa_mfma_i4(const SweepParams& p, bool is_bf16, int dim, int heads_per_group, bool wave_per_head,
                               dim3 grid, hipStream_t stream);
 
 }  // namespace da

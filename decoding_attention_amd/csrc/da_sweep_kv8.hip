@@ -1,4 +1,4 @@
-// Sweep-kernel instantiations for an 8-bit K/V cache (FP8 e4m3 or int8), all head dimensions.
+// Sweep-kernel instantiations for an 8-bit or 4-bit K/V cache (FP8 e4m3, int8, int4), all head dimensions.
 #include "da_sweep_launch.h"
 namespace da {
 namespace {
@@ -17,6 +17,7 @@ hipError_t launch_fmt(const SweepParams& p, bool is_bf16, int dim, int rt, dim3 
 
 hipError_t launch_sweep_kv8(const SweepParams& p, int fmt, bool is_bf16, int dim, int rt, dim3 grid,
                             hipStream_t stream) {
+    if (fmt == kKvInt4) return launch_fmt<kKvInt4>(p, is_bf16, dim, rt, grid, stream);
     return fmt == kKvInt8 ? launch_fmt<kKvInt8>(p, is_bf16, dim, rt, grid, stream)
                           : launch_fmt<kKvFp8>(p, is_bf16, dim, rt, grid, stream);
 }

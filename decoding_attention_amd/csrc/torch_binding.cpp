@@ -22,20 +22,22 @@ namespace {
     TORCH_CHECK(x.sizes() == torch::IntArrayRef({__VA_ARGS__}), #x " must have shape (" #__VA_ARGS__ ")")
 #define DA_CHECK_CONTIGUOUS(x) TORCH_CHECK(x.is_contiguous(), #x " must be contiguous")
 
-// K/V element format: the 16-bit type of q (0), or FP8 e4m3 (1) or int8 (2) with optional per-KV-head
-// de-quantisation factors.
+// K/V element format: the 16-bit type of q (0), or FP8 e4m3 (1), int8 (2) or int4 (3: a uint8 tensor whose last
+// dimension holds two elements to a byte) with optional per-KV-head de-quantisation factors.
 int kv8_format(const at::Tensor &q, const at::Tensor &k) {
     if (k.dtype() == torch::kFloat8_e4m3fn) return 1;
     if (k.dtype() == torch::kInt8) return 2;
+    if (k.dtype() == torch::kUInt8) return 3;
     TORCH_CHECK(k.dtype() == q.dtype(),
-                "query and key must have the same dtype (or the key cache is float8_e4m3fn or int8)");
+                "query and key must have the same dtype (or the key cache is float8_e4m3fn, int8, or uint8 holding "
+                "int4 pairs)");
     return 0;
 }
 
 const float *scale_ptr(const std::optional<at::Tensor> &t, const at::Tensor &q, int64_t head_k, const char *name,
                        int kv8) {
     if (!t.has_value()) return nullptr;
-    TORCH_CHECK(kv8 != 0, name, " applies to a float8_e4m3fn or int8 K/V cache only");
+    TORCH_CHECK(kv8 != 0, name, " applies to a float8_e4m3fn, int8 or int4 K/V cache only");
     const at::Tensor &s = t.value();
     TORCH_CHECK(s.dtype() == torch::kFloat32 && s.is_cuda() && s.device() == q.device() && s.is_contiguous() &&
                     s.numel() == head_k,
@@ -78,7 +80,9 @@ at::Tensor dmha_fwd(const at::Tensor &q, const at::Tensor &k, const std::optiona
     TORCH_CHECK(head_q % head_k == 0, "number of heads in key/value must divide number of heads in query");
 
     DA_CHECK_SHAPE(q, total_q, head_q, dim);
-    DA_CHECK_SHAPE(k, total_k, head_k, dim);
+    const int64_t pack = kv8 == 3 ? 2 : 1;  // K/V elements per tensor element
+    TORCH_CHECK(dim % pack == 0 && dim_v % pack == 0, "int4 K/V needs even head dims");
+    DA_CHECK_SHAPE(k, total_k, head_k, dim / pack);
     DA_CHECK_SHAPE(cu_seq_k, batch + 1);
     DA_CHECK_CONTIGUOUS(q);
     DA_CHECK_CONTIGUOUS(k);
@@ -93,7 +97,7 @@ at::Tensor dmha_fwd(const at::Tensor &q, const at::Tensor &k, const std::optiona
         DA_CHECK_DEVICE(v);
         TORCH_CHECK(v.device() == q.device(), "v must be on q's device");
         TORCH_CHECK(v.stride(-1) == 1, "value must have contiguous last dimension");
-        DA_CHECK_SHAPE(v, total_k, head_k, dim_v);
+        DA_CHECK_SHAPE(v, total_k, head_k, dim_v / pack);
         DA_CHECK_CONTIGUOUS(v);
         v_ptr = v.data_ptr();
     } else {
@@ -139,7 +143,8 @@ at::Tensor dmha_fwd(const at::Tensor &q, const at::Tensor &k, const std::optiona
     if (ws_bytes > 0) ws = torch::empty({(int64_t)ws_bytes}, q.options().dtype(torch::kUInt8));
 
     const float scale = softmax_scale.has_value() ? (float)softmax_scale.value() : 0.0f;
-    const auto kv8_entry = kv8 == 2 ? da_decoding_attn_int8kv : da_decoding_attn_fp8kv;
+    const auto kv8_entry =
+        kv8 == 3 ? da_decoding_attn_int4kv : (kv8 == 2 ? da_decoding_attn_int8kv : da_decoding_attn_fp8kv);
     const int rc =
         kv8 ? kv8_entry(q.data_ptr(), k.data_ptr(), v_ptr, o.data_ptr(), cu_seq_k.data_ptr<int32_t>(),
                         (size_t)max_seq_k, (size_t)batch, (size_t)head_q, (size_t)head_k, (size_t)dim, (size_t)dim_v,
@@ -186,7 +191,9 @@ at::Tensor dmha_fwd_paged(const at::Tensor &q, const at::Tensor &k_pages, const 
     const int64_t batch = q.size(0), head_q = q.size(1), dim = q.size(2);
     const int64_t page_size = k_pages.size(1), head_k = k_pages.size(2);
     TORCH_CHECK(batch > 0, "batch size must be positive");
-    TORCH_CHECK(k_pages.size(3) == dim, "k_pages must have q's head dim");
+    const int64_t pack = kv8 == 3 ? 2 : 1;  // K/V elements per tensor element
+    TORCH_CHECK(dim % pack == 0 && dim_v % pack == 0, "int4 K/V needs even head dims");
+    TORCH_CHECK(k_pages.size(3) * pack == dim, "k_pages must have q's head dim");
     TORCH_CHECK(head_q % head_k == 0, "number of heads in key/value must divide number of heads in query");
     DA_CHECK_SHAPE(seq_lens, batch);
     TORCH_CHECK(block_table.size(0) == batch, "block_table must have one row per sequence");
@@ -205,11 +212,11 @@ at::Tensor dmha_fwd_paged(const at::Tensor &q, const at::Tensor &k_pages, const 
         DA_CHECK_DEVICE(v);
         TORCH_CHECK(v.device() == q.device(), "v_pages must be on q's device");
         TORCH_CHECK(v.dim() == 4 && v.size(0) == k_pages.size(0) && v.size(1) == page_size && v.size(2) == head_k &&
-                        v.size(3) == dim_v,
+                        v.size(3) * pack == dim_v,
                     "v_pages must have shape (pages, page_size, head_k, dim_v)");
         TORCH_CHECK(page_dense(v), "v_pages must be dense within a page");
         v_ptr = v.data_ptr();
-        v_stride = v.stride(0);
+        v_stride = v.stride(0) * pack;  // (the C-ABI counts page strides in K/V elements)
     } else {
         TORCH_CHECK(dim_v <= dim, "without v the values are the first dim_v columns of k: dim_v must not exceed dim");
     }
@@ -250,14 +257,15 @@ at::Tensor dmha_fwd_paged(const at::Tensor &q, const at::Tensor &k_pages, const 
     if (ws_bytes > 0) ws = torch::empty({(int64_t)ws_bytes}, q.options().dtype(torch::kUInt8));
 
     const float scale = softmax_scale.has_value() ? (float)softmax_scale.value() : 0.0f;
-    const auto kv8_entry = kv8 == 2 ? da_decoding_attn_paged_int8kv : da_decoding_attn_paged_fp8kv;
+    const auto kv8_entry = kv8 == 3 ? da_decoding_attn_paged_int4kv
+                                    : (kv8 == 2 ? da_decoding_attn_paged_int8kv : da_decoding_attn_paged_fp8kv);
     const int rc =
         kv8 ? kv8_entry(
                   q.data_ptr(), k_pages.data_ptr(), v_ptr, o.data_ptr(), block_table.data_ptr<int32_t>(),
                   seq_lens.data_ptr<int32_t>(), (size_t)max_seq_k, (size_t)batch, (size_t)head_q, (size_t)head_k,
                   (size_t)dim, (size_t)dim_v, (size_t)page_size, (size_t)block_table.size(1),
-                  (size_t)k_pages.stride(0), (size_t)v_stride, is_alibi ? 1 : 0, is_bf16 ? 1 : 0, scale, slopes_ptr,
-                  k_scale_ptr, v_scale_ptr, hint, ws_bytes > 0 ? ws.data_ptr() : nullptr, ws_bytes, (void *)stream)
+                  (size_t)(k_pages.stride(0) * pack), (size_t)v_stride, is_alibi ? 1 : 0, is_bf16 ? 1 : 0, scale,
+                  slopes_ptr, k_scale_ptr, v_scale_ptr, hint, ws_bytes > 0 ? ws.data_ptr() : nullptr, ws_bytes, (void *)stream)
             : da_decoding_attn_paged(
                   q.data_ptr(), k_pages.data_ptr(), v_ptr, o.data_ptr(), block_table.data_ptr<int32_t>(),
                   seq_lens.data_ptr<int32_t>(), (size_t)max_seq_k, (size_t)batch, (size_t)head_q, (size_t)head_k,

@@ -58,6 +58,15 @@ def fwd(q: torch.Tensor, k: torch.Tensor, v_: Optional[torch.Tensor], o_: Option
                             None if softmax_scale is None else float(softmax_scale), alibi_slopes, k_scale, v_scale)
 
 
+def pack_int4(x: torch.Tensor) -> torch.Tensor:
+    """Integers in -8 .. 7 (any integer dtype, last dimension even) -> the int4 K/V cache layout: torch.uint8 with
+    half the last dimension, element 2 i in the low half of byte i, two's complement."""
+    if x.shape[-1] % 2 != 0:
+        raise ValueError("the last dimension must be even")
+    n = x.to(torch.int16) & 0xF
+    return (n[..., 0::2] | (n[..., 1::2] << 4)).to(torch.uint8)
+
+
 def decoding_attn_fwd(q: torch.Tensor, k: torch.Tensor, v: Optional[torch.Tensor], cu_seq_k: torch.Tensor,
                       max_seq_k: int, dim_v: int, is_alibi: bool, *, softmax_scale: Optional[float] = None,
                       alibi_slopes: Optional[torch.Tensor] = None, k_scale: Optional[torch.Tensor] = None,
@@ -74,7 +83,8 @@ def decoding_attn_fwd(q: torch.Tensor, k: torch.Tensor, v: Optional[torch.Tensor
         softmax_scale (keyword only): defaults to 1/sqrt(dim) as in the reference.
         alibi_slopes (keyword only): float32 [head_q] on the GPU; defaults to 2^(-8(h+1)/head_q).
         k_scale, v_scale (keyword only): k and v may be torch.float8_e4m3fn or torch.int8 (an 8-bit K/V cache; q
-            stays 16-bit); these are then float32 [head_k] GPU tensors of de-quantisation factors (default 1):
+            stays 16-bit), or torch.uint8 holding pairs of int4 values (see pack_int4: last dimensions dim / 2 and
+            dim_v / 2); these are then float32 [head_k] GPU tensors of de-quantisation factors (default 1):
             K = k_scale * k.
     Return:
         o: [total_q, head_q, dim_v], same dtype as q.
@@ -105,7 +115,8 @@ def decoding_attn_paged_fwd(q: torch.Tensor, k_pages: torch.Tensor, v_pages: Opt
         max_seq_k: upper bound of seq_lens (a host integer: nothing here synchronises with the device).
         page_size (from k_pages.shape[1]) must be a power of two.
         total_k (keyword only): sum of seq_lens if the host knows it; only a hint for sizing sequence splits.
-        k_scale, v_scale (keyword only): as for decoding_attn_fwd, when the pools are torch.float8_e4m3fn or torch.int8.
+        k_scale, v_scale (keyword only): as for decoding_attn_fwd, when the pools are torch.float8_e4m3fn, torch.int8
+            or torch.uint8 holding pairs of int4 values (last dimensions dim / 2 and dim_v / 2).
     Return:
         o: [batch, head_q, dim_v], same dtype as q.
     """

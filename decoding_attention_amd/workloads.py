@@ -126,12 +126,13 @@ def to_pages(w: Workload, page_size: int, *, seed=0, combined=False, spare_pages
     nan = float("nan") if poison else 0
     if combined:
         assert w.v is not None and w.dim == w.dim_v
-        pool = torch.full((n_pages, 2, page_size, w.head_k, w.dim), nan, dtype=w.k.dtype)
+        pool = torch.full((n_pages, 2, page_size, w.head_k, w.k.shape[-1]), nan, dtype=w.k.dtype)
         k_pages, v_pages = pool[:, 0], pool[:, 1]
     else:
         pool = None
-        k_pages = torch.full((n_pages, page_size, w.head_k, w.dim), nan, dtype=w.k.dtype)
-        v_pages = None if w.v is None else torch.full((n_pages, page_size, w.head_k, w.dim_v), nan, dtype=w.k.dtype)
+        # (row widths from the tensors themselves: an int4 cache holds two elements to a byte)
+        k_pages = torch.full((n_pages, page_size, w.head_k, w.k.shape[-1]), nan, dtype=w.k.dtype)
+        v_pages = None if w.v is None else torch.full((n_pages, page_size, w.head_k, w.v.shape[-1]), nan, dtype=w.k.dtype)
     # unused table entries point at a spare (all-NaN) page
     table = torch.full((w.batch, max_blocks), order[-1], dtype=torch.int32)
     cu = w.cu_seq_k.tolist()

@@ -176,6 +176,34 @@ size_t da_workspace_bytes_int8kv(size_t max_seq_k, size_t batch, size_t head_q, 
                                  size_t dim_v, size_t total_k, size_t page_size);
 
 /*
+ * The same attention over an int4 K/V cache (the third format of the reference's quantisation to-do,
+ * README.md:154-156; it has no such path).  k4 and v4 hold two's-complement four-bit integers (-8 .. 7), two to a
+ * byte, element 2 i of a row in the low half of byte i: k4 [total_k, head_k, dim / 2] bytes, v4 [total_k, head_k,
+ * dim_v / 2] bytes or NULL at (576, 512) (V = the leading 512 elements of each K row), 16-byte aligned; page pools
+ * likewise, with page strides counted in ELEMENTS as for the other formats.  Symmetric quantisation with one factor
+ * per KV head: K = k_scale[hk] * int4 value, V likewise (NULL for 1).  Other arguments as for the FP8 entry points.
+ * The values convert exactly to fp16 and bf16, so the only error added is the cache's own quantisation.
+ * (576, 512) with more than 32 query heads per KV head returns DA_ERR_UNSUPPORTED (the latent kernel has no int4
+ * form).
+ */
+int da_decoding_attn_int4kv(const void *q, const void *k4, const void *v4, void *o, const int32_t *cu_seq_k,
+                            size_t max_seq_k, size_t batch, size_t head_q, size_t head_k, size_t dim, size_t dim_v,
+                            int is_alibi, int is_bf16, float softmax_scale, const float *alibi_slopes,
+                            const float *k_scale, const float *v_scale, size_t total_k, void *workspace,
+                            size_t workspace_bytes, void *hip_stream);
+
+int da_decoding_attn_paged_int4kv(const void *q, const void *k_pages, const void *v_pages, void *o,
+                                  const int32_t *block_table, const int32_t *seq_lens, size_t max_seq_k,
+                                  size_t batch, size_t head_q, size_t head_k, size_t dim, size_t dim_v,
+                                  size_t page_size, size_t max_blocks_per_seq, size_t k_page_stride,
+                                  size_t v_page_stride, int is_alibi, int is_bf16, float softmax_scale,
+                                  const float *alibi_slopes, const float *k_scale, const float *v_scale,
+                                  size_t total_k, void *workspace, size_t workspace_bytes, void *hip_stream);
+
+size_t da_workspace_bytes_int4kv(size_t max_seq_k, size_t batch, size_t head_q, size_t head_k, size_t dim,
+                                 size_t dim_v, size_t total_k, size_t page_size);
+
+/*
  * Launch plan the library would use for this shape, for tests and benchmarks:
  *   kernel_kind 1 = VALU sweep, 2 = latent (MLA) MFMA sweep, 3 = grouped-head MFMA sweep (also the latent form with
  *   16 query heads or fewer); nsplit = sequence splits;

@@ -10,7 +10,7 @@ import random
 import pytest
 import torch
 
-from decoding_attention_amd import decoding_attn_fwd, decoding_attn_paged_fwd
+from decoding_attention_amd import decoding_attn_fwd, decoding_attn_paged_fwd, pack_int4
 from decoding_attention_amd import workloads as wl
 from oracle import oracle
 from tests.gpu_util import TOL, run_hip_ex, sub_workload
@@ -23,7 +23,9 @@ HEADS = [(32, 8), (32, 32), (32, 1), (8, 2), (28, 4), (16, 16), (64, 8), (12, 4)
 CASES_PER_CHUNK = 12
 
 
-def _one_case(rng, seed, case):
+def _one_case(rng, seed, case, int4=False):
+    """int4: the case runs over an int4 cache (whatever format the draws below pick; the stream of draws is the same
+    either way, so the other cases do not move)."""
     latent = rng.random() < 0.3
     dtype = rng.choice([torch.float16, torch.bfloat16])
     if latent:
@@ -55,6 +57,11 @@ def _one_case(rng, seed, case):
     page = rng.choice([1, 8, 16, 32, 64, 128])
     int8 = fp8 and rng.random() < 0.4  # the 8-bit cache holds int8 instead of FP8
     kv8_dtype = torch.int8 if int8 else FP8
+    if int4:
+        fp8, int8, kv8_dtype = True, True, torch.uint8
+        if latent and hq > 32:  # (the latent kernel has no int4 form)
+            hq = 32
+            q = q[:, :32].contiguous()
     desc = (f"seed {seed} case {case}: latent={latent} {hq}/{hk} d{d} {dtype} b{batch} max{maxlen} {mode} "
             f"alibi={alibi} fp8={fp8} int8={int8} {layout} page={page} total={total}")
     kw, k8, v8 = {}, None, None
@@ -62,16 +69,23 @@ def _one_case(rng, seed, case):
     if fp8:
         def quantise(x, scale):
             y = x.float() / scale.view(1, -1, 1)
+            if int4:
+                return torch.round(y).clamp(-8, 7).to(torch.int8)
             return torch.round(y).clamp(-128, 127).to(torch.int8) if int8 else y.to(FP8)
 
         ks = 0.015 + 0.015 * torch.rand(hk, generator=g)
         vs = ks if latent else 0.015 + 0.015 * torch.rand(hk, generator=g)
+        if int4:
+            ks, vs = ks * 20, vs * 20  # sixteen levels over about three standard deviations
         k8 = quantise(k, ks)
         k_true = k8.float() * ks.view(1, -1, 1)
         if v is not None:
             v8 = quantise(v, vs)
             v_true = v8.float() * vs.view(1, -1, 1)
         kw = dict(k_scale=ks.to(DEV), v_scale=vs.to(DEV))
+        if int4:  # from here on the cache is its packed bytes
+            k8 = pack_int4(k8)
+            v8 = None if v8 is None else pack_int4(v8)
     cu = wl.get_cu_seq(lens)
     max_seq_k = int(lens.max())
     if layout == "paged":
@@ -99,6 +113,14 @@ def _one_case(rng, seed, case):
     for b in range(batch):
         if int(lens[b]) == 0:
             assert torch.count_nonzero(o[b]) == 0, desc
+
+
+@pytest.mark.parametrize("chunk", range(3))
+def test_random_cases_over_an_int4_cache(chunk):
+    seed = 11
+    rng = random.Random(seed * 1000 + chunk)
+    for i in range(CASES_PER_CHUNK):
+        _one_case(rng, seed, chunk * CASES_PER_CHUNK + i, int4=True)
 
 
 @pytest.mark.parametrize("chunk", range(8))

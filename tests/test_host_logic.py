@@ -124,6 +124,17 @@ def test_workspace_sizes_of_the_paged_and_fp8_variants():
     assert lib.da_workspace_bytes_int8kv(*shape, 0, 0) == lib.da_workspace_bytes_fp8kv(*shape, 0, 0) and lib.da_workspace_bytes_int8kv(*mla, 0, 0) > 0
 
 
+def test_int4_entry_points_check_their_arguments_without_a_gpu():
+    lib = _lib.load()
+    shape = (4096, 64, 32, 8, 128, 128)
+    assert lib.da_workspace_bytes_int4kv(*shape, 0, 0) == lib.da_workspace_bytes_int8kv(*shape, 0, 0)
+    args = (16, 16, 16, 16, 16, 8, 1, 4, 4, 64, 64, 0, 0, 0.0, None, None, None, 0, None, 0, None)
+    assert lib.da_decoding_attn_int4kv(None, *args[1:]) == _lib.DA_ERR_INVALID_ARGUMENT and "q is null" in _lib.last_error()
+    bad = list(args)
+    bad[1] = 24  # k4 not 16-byte aligned
+    assert lib.da_decoding_attn_int4kv(*bad) == _lib.DA_ERR_INVALID_ARGUMENT and "aligned" in _lib.last_error()
+
+
 def test_plan_rejects_bad_shapes():
     with pytest.raises(RuntimeError):
         _lib.plan(128, 1, 6, 4, 64, 64)
