@@ -130,9 +130,12 @@ int rows_per_trip(size_t dim) {
 // shorter splits so that the work-groups, whose number is sized for max_seq_k, balance.
 // page_size: 0 for the packed layout, else tokens per page of paged K/V (any power of two: the MFMA kernels fetch a
 // tile whole from pages of 32 tokens and more, as two runs from 16-token pages, row by row below that).
-// kv_8bit: K/V are FP8 or int8; the grouped kernel then needs dim % 64 == 0.
+// kv_8bit: K/V are FP8, int8 or int4; the grouped kernel then needs dim % 64 == 0.
+// no_latent_kernel: the cache format has no form of the latent kernel (int4): the latent form then runs on the grouped
+// kernel whatever its size, as ceil(heads / 16) groups per sequence that read the same rows.
 Plan make_plan(size_t max_seq_k, size_t batch, size_t head_q, size_t head_k, size_t dim, size_t dim_v,
-               bool v_distinct, size_t total_k, size_t page_size = 0, bool kv_8bit = false) {
+               bool v_distinct, size_t total_k, size_t page_size = 0, bool kv_8bit = false,
+               bool no_latent_kernel = false) {
     const bool packed = page_size == 0;
     Plan pl;
     const int ratio = (int)(head_q / head_k);
@@ -161,7 +164,8 @@ Plan make_plan(size_t max_seq_k, size_t batch, size_t head_q, size_t head_k, siz
         pipe_kernel ? (long long)tun().mla_group_small / 4 : (groups16 <= 2 ? 2 : 1) * (long long)tun().mla_group_small;
     const bool latent_small = tun().mla_group_heads > 0 && group_rows <= small_bound;
     const bool latent_group = latent && !force_sweep &&
-                              (ratio <= (kv_8bit ? 2 * tun().mla_group_heads : tun().mla_group_heads) || latent_small);
+                              (ratio <= (kv_8bit ? 2 * tun().mla_group_heads : tun().mla_group_heads) || latent_small ||
+                               no_latent_kernel);
     const bool mfma = (latent && !force_sweep && !latent_group) || latent_vd;
     if (latent_group) {
         pl.kind = kKindGroup;
@@ -597,13 +601,11 @@ int run_attention(const void* q, const void* k, const void* v, void* o, const in
 
     hipStream_t stream = reinterpret_cast<hipStream_t>(hip_stream);
     const Plan pl = make_plan(max_seq_k, batch, head_q, head_k, dim, dim_v, v != nullptr, total_k,
-                              pg.table ? pg.page_size : 0, kf.fmt != 0);
+                              pg.table ? pg.page_size : 0, kf.fmt != 0, kf.fmt == da::kKvInt4);
     if ((size_t)head_k * pl.groups > 65535)
         return fail(DA_ERR_INVALID_ARGUMENT, "head_k * groups exceeds the grid limit 65535");
-    if (kf.fmt == da::kKvInt4 && pl.kind == kKindMfma)
-        return fail(DA_ERR_UNSUPPORTED,
-                    "an int4 K/V cache at (576, 512) is built for up to 32 query heads per KV head (the grouped kernel); "
-                    "%zu heads would need the latent kernel", head_q / head_k);
+    if (kf.fmt == da::kKvInt4 && pl.kind == kKindMfma)  // (DA_MLA_GROUP_HEADS=0 takes the grouped kernel away)
+        return fail(DA_ERR_UNSUPPORTED, "an int4 K/V cache at (576, 512) needs the grouped kernel's latent form");
 
     void* ws = nullptr;
     if (pl.ws_bytes > 0) {
@@ -887,7 +889,11 @@ int da_decoding_attn_paged_int4kv(const void* q, const void* k_pages, const void
 
 size_t da_workspace_bytes_int4kv(size_t max_seq_k, size_t batch, size_t head_q, size_t head_k, size_t dim,
                                  size_t dim_v, size_t total_k, size_t page_size) {
-    return da_workspace_bytes_fp8kv(max_seq_k, batch, head_q, head_k, dim, dim_v, total_k, page_size);
+    if (head_k == 0 || head_q % head_k != 0 || !supported_dims(dim, dim_v)) return 0;
+    // (as the FP8 cache's plans, but the latent form always on the grouped kernel)
+    const size_t a = make_plan(max_seq_k, batch, head_q, head_k, dim, dim_v, false, total_k, page_size, true, true).ws_bytes;
+    const size_t b = make_plan(max_seq_k, batch, head_q, head_k, dim, dim_v, true, total_k, page_size, true, true).ws_bytes;
+    return a > b ? a : b;
 }
 
 int da_release_workspaces(void) { return release_cached_workspaces(true); }

@@ -135,8 +135,9 @@ at::Tensor dmha_fwd(const at::Tensor &q, const at::Tensor &k, const std::optiona
 
     // k.size(0) is the sum of the key lengths: a free host-side hint for sizing the sequence splits
     const size_t ws_bytes =
-        kv8 ? da_workspace_bytes_fp8kv((size_t)max_seq_k, (size_t)batch, (size_t)head_q, (size_t)head_k, (size_t)dim,
-                                       (size_t)dim_v, (size_t)total_k, 0)
+        kv8 ? (kv8 == 3 ? da_workspace_bytes_int4kv : da_workspace_bytes_fp8kv)(
+                  (size_t)max_seq_k, (size_t)batch, (size_t)head_q, (size_t)head_k, (size_t)dim, (size_t)dim_v,
+                  (size_t)total_k, 0)
             : da_workspace_bytes((size_t)max_seq_k, (size_t)batch, (size_t)head_q, (size_t)head_k, (size_t)dim,
                                  (size_t)dim_v, (size_t)total_k);
     at::Tensor ws;  // from torch's stream-aware caching allocator
@@ -249,8 +250,9 @@ at::Tensor dmha_fwd_paged(const at::Tensor &q, const at::Tensor &k_pages, const 
     const float *v_scale_ptr = scale_ptr(v_scale, q, head_k, "v_scale", kv8);
     const size_t hint = total_k > 0 ? (size_t)total_k : 0;
     const size_t ws_bytes =
-        kv8 ? da_workspace_bytes_fp8kv((size_t)max_seq_k, (size_t)batch, (size_t)head_q, (size_t)head_k, (size_t)dim,
-                                       (size_t)dim_v, hint, (size_t)page_size)
+        kv8 ? (kv8 == 3 ? da_workspace_bytes_int4kv : da_workspace_bytes_fp8kv)(
+                  (size_t)max_seq_k, (size_t)batch, (size_t)head_q, (size_t)head_k, (size_t)dim, (size_t)dim_v, hint,
+                  (size_t)page_size)
             : da_workspace_bytes_paged((size_t)max_seq_k, (size_t)batch, (size_t)head_q, (size_t)head_k, (size_t)dim,
                                        (size_t)dim_v, hint, (size_t)page_size);
     at::Tensor ws;

@@ -183,8 +183,8 @@ size_t da_workspace_bytes_int8kv(size_t max_seq_k, size_t batch, size_t head_q, 
  * likewise, with page strides counted in ELEMENTS as for the other formats.  Symmetric quantisation with one factor
  * per KV head: K = k_scale[hk] * int4 value, V likewise (NULL for 1).  Other arguments as for the FP8 entry points.
  * The values convert exactly to fp16 and bf16, so the only error added is the cache's own quantisation.
- * (576, 512) with more than 32 query heads per KV head returns DA_ERR_UNSUPPORTED (the latent kernel has no int4
- * form).
+ * (576, 512) always runs on the grouped-head kernel, as ceil(heads / 16) groups per sequence that read the same rows
+ * (the latent kernel has no int4 form): correct at any head count, but slower than the 8-bit formats from 64 heads up.
  */
 int da_decoding_attn_int4kv(const void *q, const void *k4, const void *v4, void *o, const int32_t *cu_seq_k,
                             size_t max_seq_k, size_t batch, size_t head_q, size_t head_k, size_t dim, size_t dim_v,

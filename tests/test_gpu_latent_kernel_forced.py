@@ -17,7 +17,7 @@ FILES = ["tests/test_gpu_parity.py", "tests/test_gpu_fp8kv.py", "tests/test_gpu_
 def test_latent_cases_on_the_latent_kernel():
     root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
     env = dict(os.environ, DA_MLA_GROUP_HEADS="0", DA_MLA_GROUP_SMALL="0")
-    cmd = [sys.executable, "-m", "pytest", *FILES, "-q", "-x", "-m", "gpu", "-k", "(mla or latent or random) and not int4",  # (the latent kernel has no int4 form)
+    cmd = [sys.executable, "-m", "pytest", *FILES, "-q", "-x", "-m", "gpu", "-k", "mla or latent or random",
            "-p", "no:cacheprovider"]
     r = subprocess.run(cmd, env=env, cwd=root, capture_output=True, text=True, timeout=900)
     tail = r.stdout[-3000:] + r.stderr[-2000:]

@@ -59,9 +59,6 @@ def _one_case(rng, seed, case, int4=False):
     kv8_dtype = torch.int8 if int8 else FP8
     if int4:
         fp8, int8, kv8_dtype = True, True, torch.uint8
-        if latent and hq > 32:  # (the latent kernel has no int4 form)
-            hq = 32
-            q = q[:, :32].contiguous()
     desc = (f"seed {seed} case {case}: latent={latent} {hq}/{hk} d{d} {dtype} b{batch} max{maxlen} {mode} "
             f"alibi={alibi} fp8={fp8} int8={int8} {layout} page={page} total={total}")
     kw, k8, v8 = {}, None, None
