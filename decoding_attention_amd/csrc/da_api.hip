@@ -224,6 +224,10 @@ Plan make_plan(size_t max_seq_k, size_t batch, size_t head_q, size_t head_k, siz
         // (16-bit K/V in whole tiles or 16-token runs only: the 8-bit forms and the per-row page lookups keep fewer
         // bytes in flight per work-group and need the 512; FP8, batch 64 x 4096 tokens: 96 us against 110)
         if (dim == 128 && !kv_8bit && (packed || page_size >= 16) && !pl.wave_per_head) target_wgs = tun().group_target_wgs_d128;
+        // d = 96 (rows of 192 bytes, the slowest stream of the four head dims): 256 work-groups, half the merge
+        // (measured, 32/8 heads: batch 64 x 4096 tokens 156.6 -> 149.9 us, batch 32 x 8192 156.4 -> 150.4, batch 128 x
+        // 2048 152.6 -> 143.0; 16/4 heads, batch 64 x 4096 79.6 -> 77.2)
+        if (dim == 96 && !kv_8bit && (packed || page_size >= 16)) target_wgs = tun().group_target_wgs_d128;
     } else {
         pl.kind = kKindSweep;
         const int max_rt = dim > 256 ? 2 : 4;
@@ -319,10 +323,11 @@ Plan make_plan(size_t max_seq_k, size_t batch, size_t head_q, size_t head_k, siz
     // longer split loses again, batch 32 x 16384 tokens 360 -> 377 us with 4096-token splits)
     if (pl.kind == kKindGroup && !latent_group && total_k > 0 && !ragged && !kv_8bit && (packed || page_size >= 16))
         by_cap = base >= 512 ? 1 : ((long long)max_seq_k + 2047) / 2048;
-    // ... and without a token count (the reference-signature entry point) the same kernel at d = 128 caps at 2048
-    // tokens: as good as the counted plan on a uniform batch and better than the 1024 cap on a ragged one (measured,
-    // 32/8 heads, batch 64: 4096 tokens each 184.6 -> 181.6 us, 181.4 with the count; 1..8192 tokens 264.7 -> 246.1 us)
-    if (pl.kind == kKindGroup && !latent_group && total_k == 0 && dim == 128 && !kv_8bit && (packed || page_size >= 16))
+    // ... and without a token count (the reference-signature entry point) the same kernel caps at 2048 tokens: as
+    // good as the counted plan on a uniform batch and better than the 1024 cap on a ragged one (measured, 32/8 heads,
+    // batch 64, d 128: 4096 tokens each 184.6 -> 181.6 us, 181.4 with the count; 1..8192 tokens 264.7 -> 246.1 us; d 96:
+    // 152.0 -> 147.0 and 255.8 -> 242.8; d 256: a tie and 540.2 -> 519.9; d 64: a tie and 151.2 -> 146.8)
+    if (pl.kind == kKindGroup && !latent_group && total_k == 0 && !kv_8bit && (packed || page_size >= 16))
         by_cap = ((long long)max_seq_k + 2047) / 2048;
     // (one round of long splits beats two rounds with the second nearly empty)
     if (latent_group && base <= target_wgs && base * by_cap > target_wgs) by_cap = 1;
@@ -334,14 +339,16 @@ Plan make_plan(size_t max_seq_k, size_t batch, size_t head_q, size_t head_k, siz
     // 256 poorly, take the split count that fills it best instead (fewer splits on a tie).  Measured, 32/8 heads d
     // 128, 4096 tokens: batch 40, 7 splits (560 work-groups) 138.6 us, 3 splits (240) 117.9; batch 48, 6 splits (576)
     // 158.8, 5 splits (480) 142.4; batch 100, 4 splits (800) 320.5, 1 split (200) 284.8.
-    // (not at d = 96, where the re-planning loses as often as it wins)
+    // (d = 96 counts as long rows, 256 work-groups a round, like its target above: 32/8 heads, 4096 tokens, batch 40
+    // 117.6 -> 93.3 us, batch 48 135.1 -> 116.8, batch 72 199.6 -> 174.7, batch 100 259.9 -> 246.5; batch 24 x 8192
+    // 143.2 -> 111.7; 32/4 heads, batch 80 x 4096 119.4 -> 90.4)
     // (measured on 16-bit K/V in whole tiles or 16-token runs, and applied there only)
     // (... and on 8-bit K/V at d = 128, whose rows are as short as 16-bit rows at d = 64: FP8, 32/8 heads, batch 100
     // x 4096 tokens 184 -> 154 us, batch 72 131 -> 116, batch 40 74 -> 66)
     const bool whole_tiles = packed || page_size >= 16;
     const bool plain16 = !kv_8bit && whole_tiles;
-    const bool short_rows = dim < 128 || kv_8bit;
-    if (pl.kind == kKindGroup && (plain16 || (kv_8bit && dim == 128 && whole_tiles)) && dim != 96 && dim <= 256 &&
+    const bool short_rows = dim < 96 || kv_8bit;
+    if (pl.kind == kKindGroup && (plain16 || (kv_8bit && dim == 128 && whole_tiles)) && dim <= 256 &&
         tun().fill_rounds) {
         // (at d = 64 a work-group streams too few bytes for one per CU to saturate HBM: rounds of two per CU there;
         // 32/8 heads, batch 56 x 4096 tokens 100.1 -> 84.9 us, 32/4 heads, batch 150 x 4096 127.2 -> 112.3)
