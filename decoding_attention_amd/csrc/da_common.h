@@ -40,6 +40,12 @@ struct Elem<f16_tag> {
         _Float16 h = (_Float16)f;
         return __builtin_bit_cast(uint16_t, h);
     }
+    // two values rounded and packed (lo in bits 0 .. 15) by one instruction, v_cvt_pk_f16_f32
+    static __device__ __forceinline__ uint32_t pack2(float lo, float hi) {
+        typedef float f32x2 __attribute__((ext_vector_type(2)));
+        const f32x2 v = {lo, hi};
+        return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, f16x2));
+    }
 };
 
 template <>
@@ -50,12 +56,14 @@ struct Elem<bf16_tag> {
     }
     static __device__ __forceinline__ float lo(uint32_t a) { return __uint_as_float(a << 16); }
     static __device__ __forceinline__ float hi(uint32_t a) { return __uint_as_float(a & 0xffff0000u); }
-    // round-to-nearest-even, the reference's __float2bfloat16
-    static __device__ __forceinline__ uint16_t from_f32(float f) {
-        uint32_t x = __float_as_uint(f);
-        if ((x & 0x7fffffffu) > 0x7f800000u) return (uint16_t)((x >> 16) | 0x40u);
-        x += 0x7fffu + ((x >> 16) & 1u);
-        return (uint16_t)(x >> 16);
+    // round-to-nearest-even, the reference's __float2bfloat16 (gfx950 converts in hardware, v_cvt_pk_bf16_f32; a NaN
+    // stays a NaN)
+    static __device__ __forceinline__ uint16_t from_f32(float f) { return __builtin_bit_cast(uint16_t, (__bf16)f); }
+    // two values rounded and packed (lo in bits 0 .. 15) by one instruction
+    static __device__ __forceinline__ uint32_t pack2(float lo, float hi) {
+        typedef float f32x2 __attribute__((ext_vector_type(2)));
+        const f32x2 v = {lo, hi};
+        return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, bf16x2));
     }
 };
 

@@ -809,10 +809,10 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_num_vgpr(kScV))) void la
             constexpr int c = decltype(ic)::value / 4, r4 = decltype(ic)::value % 4;
             const int col = c * 32 + r4 * 8 + half * 4;
             u32x2 w;
-            w.x = (uint32_t)EL::from_f32(acc_at(std::integral_constant<int, c * 16 + r4 * 4 + 0>{}) * inv) |
-                  ((uint32_t)EL::from_f32(acc_at(std::integral_constant<int, c * 16 + r4 * 4 + 1>{}) * inv) << 16);
-            w.y = (uint32_t)EL::from_f32(acc_at(std::integral_constant<int, c * 16 + r4 * 4 + 2>{}) * inv) |
-                  ((uint32_t)EL::from_f32(acc_at(std::integral_constant<int, c * 16 + r4 * 4 + 3>{}) * inv) << 16);
+            w.x = EL::pack2(acc_at(std::integral_constant<int, c * 16 + r4 * 4 + 0>{}) * inv,
+                            acc_at(std::integral_constant<int, c * 16 + r4 * 4 + 1>{}) * inv);
+            w.y = EL::pack2(acc_at(std::integral_constant<int, c * 16 + r4 * 4 + 2>{}) * inv,
+                            acc_at(std::integral_constant<int, c * 16 + r4 * 4 + 3>{}) * inv);
             *reinterpret_cast<__attribute__((address_space(3))) u32x2*>(wbuf + n * PITCH + col * 2) = w;
         });
         // (LDS operations of one wave complete in order: the wave reads its own rows back)
