@@ -677,6 +677,13 @@ int run_attention(const void* q, const void* k, const void* v, void* o, const in
         sp.flat_cu = flat_cu;
     }
 
+    if (pl.nsplit > 1 && da::mla_half_partials(pl.kind == kKindMfma && !pl.v_distinct, pl.rt, kf.fmt)) {
+        // the pipelined kernel's 16-bit partials take whole blocks of 32 heads: they must fit the area sized for
+        // fp32 partials of head_q rows (they do from 65 heads per KV head up, where that kernel runs)
+        const size_t need = (size_t)batch * pl.nsplit * da::nat_split_bytes(da::nat_blocks((int)head_k, pl.groups));
+        if (need > (size_t)batch * head_q * pl.nsplit * dim_v * sizeof(float))
+            return fail(DA_ERR_WORKSPACE, "16-bit partials of %zu bytes do not fit the workspace's partial area", need);
+    }
     const dim3 grid((unsigned)(pl.flat_tokens ? pl.flat_wgs : pl.nsplit),
                     (unsigned)((pl.wave_per_head ? head_k / 4 : head_k) * pl.groups),
                     (unsigned)(pl.flat_tokens ? 1 : batch));
@@ -725,6 +732,9 @@ int run_attention(const void* q, const void* k, const void* v, void* o, const in
         rp.flat_cu = sp.flat_cu;
         rp.early = pl.ws_bytes <= ((size_t)8 << 20) ? 1 : 0;
         rp.half_partials = da::mla_half_partials(pl.kind == kKindMfma && !pl.v_distinct, pl.rt, kf.fmt) ? 1 : 0;
+        rp.ratio = sp.ratio;
+        rp.groups = pl.groups;
+        rp.nat_blocks = da::nat_blocks((int)head_k, pl.groups);
         e = da::launch_reduce(rp, is_bf16 != 0, (int)(batch * head_q), stream);
         if (e != hipSuccess) return fail(DA_ERR_HIP, "merge kernel launch: %s", hipGetErrorString(e));
     }

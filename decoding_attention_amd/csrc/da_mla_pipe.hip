@@ -790,18 +790,41 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_num_vgpr(kScV))) void la
     // (the last matrix instructions' results must have landed before the accumulation registers are read)
     asm volatile("s_nop 15\n\ts_nop 15" ::: "memory");
     auto acc_at = [&](auto ic) { return read_acc_n<decltype(ic)::value>(); };
-    // The wave's 32 output rows (its heads) leave through LDS: a lane holds groups of four columns of its head's row,
-    // so storing from registers would scatter 8-byte pieces over 32 rows per instruction; instead the rows are
-    // written to the wave's own tile buffer (pitch 1040 bytes: lanes of one write fall on different banks) and read
-    // back a whole row (1 KiB, 16 bytes a lane) per instruction.  Normalised by the denominator, as 16-bit values:
-    // the final output, or (sequence split) the split's partial (ReduceParams::half_partials) beside the running
-    // maximum and the denominator as fp32.
-    __syncthreads();  // every wave is done with the tile buffers
-    {
+    typedef unsigned int u32x2 __attribute__((ext_vector_type(2)));
+    // Normalised by the denominator, as 16-bit values: the final output, or (sequence split) the split's partial
+    // (ReduceParams::half_partials) beside the running maximum and the denominator as fp32.
+    if (p.nsplit > 1) {
+        // A split's partial leaves as it lies in the registers (nat_piece in da_common.h): lane (n, half) holds four
+        // columns of head n per 32 x 32 tile quarter, the wave stores 512 contiguous bytes per quarter, and the merge
+        // kernel reads in that order.  No trip through LDS and no barrier in the tail every work-group of a
+        // one-round grid runs at the same moment.
+        const float inv = 1.0f / l_tot;
+        const int blk = (hk * p.groups + grp) * NWV + wave;
+        uint8_t* const dst = reinterpret_cast<uint8_t*>(p.ws_o) +
+                             nat_piece((size_t)b, p.nsplit, split, nat_blocks(p.head_k, p.groups), blk, 0, 0) * 8 + lane * 8;
+        static_for<0, CT * 4>([&](auto ic) {
+            constexpr int q = decltype(ic)::value, c = q / 4, r4 = q % 4;
+            u32x2 w;
+            w.x = EL::pack2(acc_at(std::integral_constant<int, c * 16 + r4 * 4 + 0>{}) * inv,
+                            acc_at(std::integral_constant<int, c * 16 + r4 * 4 + 1>{}) * inv);
+            w.y = EL::pack2(acc_at(std::integral_constant<int, c * 16 + r4 * 4 + 2>{}) * inv,
+                            acc_at(std::integral_constant<int, c * 16 + r4 * 4 + 3>{}) * inv);
+            *reinterpret_cast<u32x2*>(dst + q * 512) = w;
+        });
+        if (n < nh && half == 0) {
+            const size_t part = ((size_t)b * p.head_q + h_base + n) * p.nsplit + split;
+            p.ws_ml[part * 2 + 0] = m;
+            p.ws_ml[part * 2 + 1] = l_tot;
+        }
+    } else {
+        // The wave's 32 output rows (its heads) leave through LDS: a lane holds groups of four columns of its head's
+        // row, so storing from registers would scatter 8-byte pieces over 32 rows per instruction; instead the rows
+        // are written to the wave's own tile buffer (pitch 1040 bytes: lanes of one write fall on different banks)
+        // and read back a whole row (1 KiB, 16 bytes a lane) per instruction.
+        __syncthreads();  // every wave is done with the tile buffers
         constexpr int PITCH = DV * 2 + 16;  // (a multiple of 16: the rows are read back 16 bytes a lane)
         static_assert(32 * PITCH <= BUF, "a wave's rows fit its tile buffer");
         typedef __attribute__((address_space(3))) uint8_t* lds_ptr;
-        typedef unsigned int u32x2 __attribute__((ext_vector_type(2)));
         typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
         const lds_ptr wbuf = (lds_ptr)(uintptr_t)(smem_off + (uint32_t)(wave * BUF));
         const float inv = 1.0f / l_tot;
@@ -816,15 +839,8 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_num_vgpr(kScV))) void la
             *reinterpret_cast<__attribute__((address_space(3))) u32x2*>(wbuf + n * PITCH + col * 2) = w;
         });
         // (LDS operations of one wave complete in order: the wave reads its own rows back)
-        uint16_t* dst;
-        size_t row_elems;  // elements between consecutive heads' rows
-        if (p.nsplit == 1) {
-            dst = o16 + ((size_t)b * p.head_q + h_base) * DV;
-            row_elems = DV;
-        } else {
-            dst = reinterpret_cast<uint16_t*>(p.ws_o) + (((size_t)b * p.head_q + h_base) * p.nsplit + split) * DV;
-            row_elems = (size_t)p.nsplit * DV;
-        }
+        uint16_t* const dst = o16 + ((size_t)b * p.head_q + h_base) * DV;
+        constexpr size_t row_elems = DV;  // elements between consecutive heads' rows
         typedef const __attribute__((address_space(3))) u32x4* lds_row;
         if (nh == 32) {
             // eight rows read, then eight rows stored
@@ -842,15 +858,11 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_num_vgpr(kScV))) void la
                 *reinterpret_cast<u32x4*>(dst + (size_t)r * row_elems + lane * 8) = v;
             }
         }
-        if (p.nsplit > 1 && n < nh && half == 0) {
-            const size_t part = ((size_t)b * p.head_q + h_base + n) * p.nsplit + split;
-            p.ws_ml[part * 2 + 0] = m;
-            p.ws_ml[part * 2 + 1] = l_tot;
-        }
     }
 #ifdef DA_PIPE_PROBE
-    if (p.nsplit > 1) {
+    if (p.nsplit > 1 && nat_blocks(p.head_k, p.groups) * 32 <= p.head_q) {
         // stamps into the unused upper half of the fp32-sized partial area, 16 floats per work-group
+        const long long pr_w3 = wall_clock64();  // stores issued
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
         const long long pr_w2 = wall_clock64();
         if (threadIdx.x == 0) {
@@ -868,6 +880,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_num_vgpr(kScV))) void la
             pa[10] = (float)(pr_wq & 0xffffff);
             pa[11] = (float)pr_x1;
             pa[12] = (float)pr_x2;
+            pa[13] = (float)(pr_w3 & 0xffffff);
         }
     }
 #endif

@@ -261,7 +261,28 @@ __global__ __launch_bounds__(256) void reduce_kernel(const ReduceParams p, int r
     using EL = Elem<Tag>;
     const int nc4 = p.dim_v >> 2;
     int row, c4, sgi = 0;
-    if constexpr (SG == 1) {
+    size_t nat_b = 0;     // (H16) sequence,
+    int nat_blk = 0, nat_n = 0;  // block and row within it
+    if constexpr (H16) {
+        // (SG > 1 only) the CW = 64 / SG elements of a wave are CW consecutive rows of one block at one column group:
+        // consecutive 8-byte pieces of the partials
+        static_assert(SG > 1 && 32 % (64 / SG) == 0, "the one-lane-per-element form is reduce16_kernel");
+        constexpr int CW = 64 / SG;
+        const int wave_id = blockIdx.x * 4 + (threadIdx.x >> 6), lane = threadIdx.x & 63;
+        const long long id = (long long)wave_id * CW + (lane % CW);
+        sgi = lane / CW;
+        nat_n = (int)(id & 31);
+        const long long rest = id >> 5;
+        c4 = (int)(rest % nc4);
+        const long long bg = rest / nc4;  // sequence * blocks + block
+        if (bg >= (long long)(rows / p.head_q) * p.nat_blocks) return;  // (a whole wave: its elements share bg)
+        nat_b = (size_t)(bg / p.nat_blocks);
+        nat_blk = (int)(bg % p.nat_blocks);
+        const int per_kv = p.groups * 4;
+        const int r = (nat_blk % per_kv) * 32 + nat_n;  // head within its KV head's group of `ratio`
+        if (r >= p.ratio) return;                       // (the SG lanes of an element leave together)
+        row = (int)nat_b * p.head_q + (nat_blk / per_kv) * p.ratio + r;
+    } else if constexpr (SG == 1) {
         const int gid = blockIdx.x * 256 + threadIdx.x;
         row = gid / nc4;  // (sequence, head) index
         c4 = gid - row * nc4;
@@ -277,7 +298,7 @@ __global__ __launch_bounds__(256) void reduce_kernel(const ReduceParams p, int r
     const size_t part0 = (size_t)row * p.nsplit;
     const float2* const ml = reinterpret_cast<const float2*>(p.ws_ml) + part0;
     const float4* const src = reinterpret_cast<const float4*>(p.ws_o + part0 * p.dim_v) + c4;
-    const uint2* const src16 = reinterpret_cast<const uint2*>(reinterpret_cast<const uint16_t*>(p.ws_o) + part0 * p.dim_v) + c4;
+    const uint2* const src16 = reinterpret_cast<const uint2*>(p.ws_o);
     // This lane's next four partials: slots s0, s0 + SG, ... (clamped to `last`; the caller masks the rest).
     float2 e[4];
     float4 x[4];
@@ -287,7 +308,7 @@ __global__ __launch_bounds__(256) void reduce_kernel(const ReduceParams p, int r
             const int s = min(s0 + u * SG, last);
             e[u] = ml[s];
             if constexpr (H16) {
-                const uint2 h = src16[(size_t)s * nc4];
+                const uint2 h = src16[nat_piece(nat_b, p.nsplit, s, p.nat_blocks, nat_blk, c4, nat_n)];
                 x[u] = make_float4(EL::lo(h.x), EL::hi(h.x), EL::lo(h.y), EL::hi(h.y));
             } else {
                 x[u] = src[(size_t)s * nc4];
@@ -373,20 +394,27 @@ __global__ __launch_bounds__(256) void reduce_kernel(const ReduceParams p, int r
     *reinterpret_cast<ushort4*>(reinterpret_cast<uint16_t*>(p.o) + (size_t)row * p.dim_v + c4 * 4) = r;
 }
 
-// The merge for normalised 16-bit partials (ReduceParams::half_partials) in its one-lane-per-element form: one thread
-// per (sequence, query head, eight output columns), 16-byte loads; the partials of four splits are fetched together.
-// A partial's weight is 2^(m_i - m) times its denominator l_i.
+// The merge for normalised 16-bit partials (ReduceParams::half_partials, laid out as nat_piece says) in its
+// one-lane-per-element form: one thread per (sequence, query head, eight output columns), consecutive threads taking
+// consecutive heads of a block, so that a wave's loads are runs of 256 bytes; the partials of four splits are fetched
+// together.  A partial's weight is 2^(m_i - m) times its denominator l_i.
 template <typename Tag>
 __global__ __launch_bounds__(256) void reduce16_kernel(const ReduceParams p, int rows) {
     using EL = Elem<Tag>;
-    const int nc8 = p.dim_v >> 3;
-    const int gid = blockIdx.x * 256 + threadIdx.x;
-    const int row = gid / nc8;  // (sequence, head) index
-    const int c8 = gid - row * nc8;
-    if (row >= rows) return;
+    const long long gid = (long long)blockIdx.x * 256 + threadIdx.x;
+    const int n = (int)(gid & 31);        // row of the block
+    const int c8 = (int)(gid >> 5) & 63;  // eight columns
+    const long long bg = gid >> 11;       // sequence * blocks + block
+    if (bg >= (long long)(rows / p.head_q) * p.nat_blocks) return;
+    const size_t b = (size_t)(bg / p.nat_blocks);
+    const int blk = (int)(bg % p.nat_blocks);
+    const int per_kv = p.groups * 4;
+    const int hr = (blk % per_kv) * 32 + n;  // head within its KV head's group of `ratio`
+    if (hr >= p.ratio) return;               // a dead row of the group's last block
+    const int row = (int)b * p.head_q + (blk / per_kv) * p.ratio + hr;
     const size_t part0 = (size_t)row * p.nsplit;
     const float2* const ml = reinterpret_cast<const float2*>(p.ws_ml) + part0;
-    const uint4* const src = reinterpret_cast<const uint4*>(reinterpret_cast<const uint16_t*>(p.ws_o) + part0 * p.dim_v) + c8;
+    const uint2* const src = reinterpret_cast<const uint2*>(p.ws_o);
     float2 e[4];
     uint4 x[4];
     auto fetch = [&](int s0, int last) {
@@ -394,11 +422,13 @@ __global__ __launch_bounds__(256) void reduce16_kernel(const ReduceParams p, int
         for (int u = 0; u < 4; ++u) {
             const int s = min(s0 + u, last);
             e[u] = ml[s];
-            x[u] = src[(size_t)s * nc8];
+            // columns 8 c8 .. + 3 lie with lane n of the storing wave, + 4 .. + 7 with lane 32 + n
+            const size_t at = nat_piece(b, p.nsplit, s, p.nat_blocks, blk, 2 * c8, n);
+            const uint2 lo = src[at], hi = src[at + 32];
+            x[u] = make_uint4(lo.x, lo.y, hi.x, hi.y);
         }
     };
     if (p.early) fetch(0, p.nsplit - 1);
-    const int b = row / p.head_q;
     const int len = p.cu_seq_k ? p.cu_seq_k[b + 1] - p.cu_seq_k[b] : p.seq_lens[b];
     const int ns = len > 0 ? min(p.nsplit, (len + p.chunk - 1) / p.chunk) : 0;
     float mm = kNegBig, den = 0.0f;
@@ -431,10 +461,10 @@ __global__ __launch_bounds__(256) void reduce16_kernel(const ReduceParams p, int
     }
     const float inv = ns > 0 ? 1.0f / den : 0.0f;  // an empty sequence yields a zero row
     uint4 r;
-    r.x = (uint32_t)EL::from_f32(num[0] * inv) | ((uint32_t)EL::from_f32(num[1] * inv) << 16);
-    r.y = (uint32_t)EL::from_f32(num[2] * inv) | ((uint32_t)EL::from_f32(num[3] * inv) << 16);
-    r.z = (uint32_t)EL::from_f32(num[4] * inv) | ((uint32_t)EL::from_f32(num[5] * inv) << 16);
-    r.w = (uint32_t)EL::from_f32(num[6] * inv) | ((uint32_t)EL::from_f32(num[7] * inv) << 16);
+    r.x = EL::pack2(num[0] * inv, num[1] * inv);
+    r.y = EL::pack2(num[2] * inv, num[3] * inv);
+    r.z = EL::pack2(num[4] * inv, num[5] * inv);
+    r.w = EL::pack2(num[6] * inv, num[7] * inv);
     *reinterpret_cast<uint4*>(reinterpret_cast<uint16_t*>(p.o) + (size_t)row * p.dim_v + c8 * 8) = r;
 }
 

@@ -8,13 +8,19 @@ hipError_t launch_sweep_d576(const SweepParams& p, bool is_bf16, int rt, dim3 gr
 template <typename Tag, int SG>
 static void launch_reduce_sg(const ReduceParams& p, int blocks, hipStream_t stream) {
     const long long nc4 = p.dim_v / 4;
+    if constexpr (SG > 1) {
+        if (p.half_partials) {
+            // SG lanes per (row of a block, four columns), dead rows of the blocks included
+            const long long lanes = (long long)(blocks / p.head_q) * p.nat_blocks * 32 * nc4 * SG;
+            hipLaunchKernelGGL((reduce_kernel<Tag, SG, true>), dim3((unsigned)((lanes + 255) / 256)), dim3(256), 0, stream, p,
+                               blocks);
+            return;
+        }
+    }
     // SG = 1: one thread per (row, four columns); SG > 1: one wave per (row, 64 / SG column groups), four waves a block
     const long long units = SG == 1 ? (long long)blocks * nc4 : (long long)blocks * (nc4 / (64 / SG)) * 64;
     const dim3 grid((unsigned)((units + 255) / 256));
-    if (p.half_partials)
-        hipLaunchKernelGGL((reduce_kernel<Tag, SG, true>), grid, dim3(256), 0, stream, p, blocks);
-    else
-        hipLaunchKernelGGL((reduce_kernel<Tag, SG, false>), grid, dim3(256), 0, stream, p, blocks);
+    hipLaunchKernelGGL((reduce_kernel<Tag, SG, false>), grid, dim3(256), 0, stream, p, blocks);
 }
 
 hipError_t launch_reduce(const ReduceParams& p, bool is_bf16, int blocks, hipStream_t stream) {
@@ -24,9 +30,12 @@ hipError_t launch_reduce(const ReduceParams& p, bool is_bf16, int blocks, hipStr
     int sg = 1;
     while (sg < 8 && p.nsplit >= 8 * sg && threads * sg < (1ll << 18)) sg *= 2;
     while (sg > 1 && (p.dim_v / 4) % (64 / sg) != 0) sg /= 2;
-    // normalised 16-bit partials, one lane per element: eight columns a thread (the balanced grid never has them)
-    if (p.half_partials && sg == 1 && p.flat_tokens == 0 && p.dim_v % 8 == 0) {
-        const long long units = (long long)blocks * (p.dim_v / 8);
+    // normalised 16-bit partials (the pipelined latent kernel's: dim_v = 512, never the balanced grid), one lane per
+    // element: eight columns a thread, dead rows of the blocks included
+    if (p.half_partials && (p.dim_v != 512 || p.flat_tokens != 0 || p.nat_blocks <= 0 || p.head_q <= 0))
+        return hipErrorInvalidValue;
+    if (p.half_partials && sg == 1) {
+        const long long units = (long long)(blocks / p.head_q) * p.nat_blocks * 32 * (p.dim_v / 8);
         const dim3 grid((unsigned)((units + 255) / 256));
         if (is_bf16)
             hipLaunchKernelGGL((reduce16_kernel<bf16_tag>), grid, dim3(256), 0, stream, p, blocks);

@@ -18,9 +18,10 @@ def run_hip(w, **kw):
     return o.cpu()
 
 
-def run_hip_ex(w, total_k_hint):
+def run_hip_ex(w, total_k_hint, fill=None):
     """The packed call through da_decoding_attn_ex with a caller-owned workspace and the given token-count hint
-    (the Python face always passes k.shape[0]; 0 here selects the plan of a caller who does not know it)."""
+    (the Python face always passes k.shape[0]; 0 here selects the plan of a caller who does not know it).  `fill`: a
+    byte value the workspace holds before the call (default: whatever the allocator hands out)."""
     from decoding_attention_amd import _lib
     lib = _lib.load()
     dev = torch.device("cuda:0")
@@ -29,6 +30,8 @@ def run_hip_ex(w, total_k_hint):
     hk = w.k.shape[1]
     n = lib.da_workspace_bytes(w.max_seq_k, b, hq, hk, d, w.dim_v, total_k_hint)
     ws = torch.empty(max(n, 16), dtype=torch.uint8, device=dev)
+    if fill is not None:
+        ws.fill_(fill)
     o = torch.full((b, hq, w.dim_v), float("nan"), dtype=w.q.dtype, device=dev)
     rc = lib.da_decoding_attn_ex(wd.q.data_ptr(), wd.k.data_ptr(), None if wd.v is None else wd.v.data_ptr(),
                                  o.data_ptr(), wd.cu_seq_k.data_ptr(), w.max_seq_k, b, hq, hk, d, w.dim_v,
