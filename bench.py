@@ -35,7 +35,7 @@ MFMA_PEAK_TFLOPS = 2500.0   # MI355X dense fp16/bf16 MFMA, published
 # it was measured under; when the library plans the workload differently, the bench line carries null instead.
 MEASURED_TRAFFIC = {
     "gqa": {"bytes": 1092312678, "plan": {"kind": 3, "nsplit": 4, "chunk": 1024, "heads_per_group": 16}},
-    "mla": {"bytes": 388134502, "plan": {"kind": 2, "nsplit": 4, "chunk": 1024, "heads_per_group": 128},
+    "mla": {"bytes": 389949440, "plan": {"kind": 2, "nsplit": 4, "chunk": 1024, "heads_per_group": 128},
             "partials": "16-bit"},
 }
 
@@ -500,7 +500,9 @@ def run_sweep(args, measure_fn=None, workload_fn=None, out=None):
 # tokens, length at batch 16) and the reference's lists around them.
 LATENT_PLAN_SHAPES = ([(b, 4096) for b in (1, 2, 4, 8, 16, 32, 64, 128, 256)] +
                       [(16, sk) for sk in (512, 1024, 2048, 8192, 16384)] + [(1, sk) for sk in (512, 2048, 8192)] +
-                      [(4, 16384), (8, 8192), (32, 1024), (64, 1024), (100, 4096)])
+                      [(4, 16384), (8, 8192), (32, 1024), (64, 1024), (100, 4096)] +
+                      # short sequences of small batches, where a work-group's fixed cost decides the split count
+                      [(8, 512), (8, 1024), (24, 1024), (16, 768), (16, 1536), (4, 2048), (8, 2048), (24, 2048), (8, 3072)])
 
 
 def run_latent_plan_sweep(args):

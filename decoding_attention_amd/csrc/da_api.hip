@@ -47,7 +47,7 @@ int env_int(const char* name, int dflt) {
 struct Tunables {
     int target_wgs, mfma_target_wgs, max_chunk, min_chunk, ragged_chunk, force_kind, group_min_ratio, wave_per_head,
         mla_heads, gqa_heads, flat_wgs, flat_min_tokens, flat_paged_min_mb, nsplit, mfma_small_wgs, group_small_wgs,
-        group_small_chunk, mla_group_heads, mla_group_small, fill_rounds, group_target_wgs_d128, mla_distinct_v;
+        group_small_chunk, mla_group_heads, mla_group_small, fill_rounds, group_target_wgs_d128, mla_distinct_v, pipe_small_wgs;
     Tunables() {
         target_wgs = env_int("DA_TARGET_WGS", 512);
         mfma_target_wgs = env_int("DA_MFMA_TARGET_WGS", 256);
@@ -61,6 +61,7 @@ struct Tunables {
         flat_min_tokens = env_int("DA_FLAT_MIN_TOKENS", 256);
         flat_paged_min_mb = env_int("DA_FLAT_PAGED_MIN_MB", 512);  // paged K/V takes the balanced grid from this many MB of K/V
         mfma_small_wgs = env_int("DA_MFMA_SMALL_WGS", 256);  // latent kernel: below this many 256-token splits, split finer
+        pipe_small_wgs = env_int("DA_PIPE_SMALL_WGS", 33);   // the same for its pipelined form (128 heads a work-group)
         // latent form: up to this many query heads take the grouped kernel (0 = never)
         mla_group_heads = env_int("DA_MLA_GROUP_HEADS", 16);
         mla_distinct_v = env_int("DA_MLA_DISTINCT_V", 1);  // (576, 512) with V in its own buffer on the latent kernel (0 = VALU sweep)
@@ -270,7 +271,15 @@ Plan make_plan(size_t max_seq_k, size_t batch, size_t head_q, size_t head_k, siz
         // too few work-groups for the chip even so: 128-token splits, as long as that keeps the merge at 32
         // partials or fewer (measured: batch 1 x 512 tokens 26.8 -> 20.5 us, batch 16 x 512 33.1 -> 29.4 us,
         // batch 4 x 2048 32.9 -> 28.3 us; batch 1 x 8192 with 64 partials loses, 36.0 -> 38.5 us)
-        if (wgs_at_min < tun().mfma_small_wgs && max_seq_k <= 32 * 128) min_chunk = std::max(std::min(min_chunk, 128), trip);
+        // The pipelined kernel's work-groups carry a larger fixed cost (147 KB of Q in, 131 KB of partials out and in
+        // again at the merge: about 0.1 us per work-group once more than 64 of them share the chip), so it goes below
+        // 256 tokens only while that leaves at most 64 work-groups.  Measured, 128 heads, old -> new plan: batch 16 x
+        // 1024 tokens, 8 -> 4 splits, 31.7 -> 25.8 us; batch 24 x 1024 35.6 -> 28.9; batch 8 x 2048, 16 -> 8 splits, 30.7
+        // -> 27.0; batch 16 x 1536 33.6 -> 31.1; batch 8 x 3072 32.2 -> 30.2; batch 16 x 768 26.5 -> 25.1.  Up to 32
+        // splits of 256 tokens the finer ones still win: batch 16 x 512, 4 splits 21.2 us, 2 splits 23.5; batch 8 x
+        // 1024, 8 splits 22.2, 4 splits 23.3; batch 4 x 2048, 16 splits 23.1, 8 splits 24.5.
+        const int small_wgs = pipe_kernel ? tun().pipe_small_wgs : tun().mfma_small_wgs;
+        if (wgs_at_min < small_wgs && max_seq_k <= 32 * 128) min_chunk = std::max(std::min(min_chunk, 128), trip);
     } else {
         // 512-token splits run best; go down to 256 only when that is needed to give every CU a work-group (the
         // VALU sweep: two, measured batch 4 x 1024 tokens 21.4 -> 18.6 us; the grouped kernel loses there)
@@ -806,6 +815,7 @@ int da_probe_set_tunable(const char* name, int value) {
     else if (n == "DA_MLA_GROUP_HEADS") t.mla_group_heads = value;
     else if (n == "DA_MFMA_TARGET_WGS") t.mfma_target_wgs = value;
     else if (n == "DA_MFMA_SMALL_WGS") t.mfma_small_wgs = value;
+    else if (n == "DA_PIPE_SMALL_WGS") t.pipe_small_wgs = value;
     else return fail(DA_ERR_INVALID_ARGUMENT, "unknown tunable %s", name);
     return DA_OK;
 }

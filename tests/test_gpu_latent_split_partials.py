@@ -21,7 +21,9 @@ SHAPES = [
     (20, 129, 1, 1500, 1),
     (32, 128, 1, 1024, 1),
     (16, 100, 1, 2048, 2),
-    (4, 192, 2, 3000, 4),
+    (4, 192, 2, 3000, 2),
+    (2, 192, 2, 4096, 4),
+    (3, 100, 1, 4096, 4),
     (1, 200, 2, 8192, 8),
     (2, 65, 1, 4096, 8),
 ]
