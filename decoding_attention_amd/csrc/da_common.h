@@ -287,9 +287,10 @@ struct ReduceParams {
     // the workspace is small (cache-resident): request the first partials before the sequence's length is known
     int early;
     // the partial outputs are normalised (divided by their denominators) and stored as 16-bit values of the output
-    // type from the start of ws_o, in the order the matrix instruction leaves them in registers (nat_piece below),
-    // instead of un-normalised fp32 by rows (the pipelined latent kernel: its partials, 128 heads x 512 columns per
-    // split, are most of the traffic that splitting adds)
+    // type from the start of ws_o, in the order the matrix instruction leaves them in registers and with their
+    // (m, l) pairs beside them (nat_block below; ws_ml is not used), instead of un-normalised fp32 by rows (the
+    // pipelined latent kernel: its partials, 128 heads x 512 columns per split, are most of the traffic that
+    // splitting adds)
     int half_partials;
     int ratio, groups, nat_blocks;  // (half_partials) query heads per KV head, work-groups per KV head, nat_blocks()
 };
@@ -297,15 +298,21 @@ struct ReduceParams {
 // Normalised 16-bit partials of the pipelined latent kernel (dim_v = 512).  A wave of that kernel owns 32 query heads
 // (a block; block id = (KV head * groups + group) * 4 + wave, rows past the group's last head are dead), and after
 // the last matrix step lane (n, half) holds, for each q = 0 .. 63, the four columns 8 q + 4 half .. + 3 of head n.
-// The wave stores them as they lie, 8 bytes a lane: one split's partial of one block is 64 runs of 512 bytes, run q
-// holding lane after lane.  Index, in 8-byte pieces, of columns 4 c4 .. 4 c4 + 3 of row n of block blk, split s of
-// sequence b:
+// The wave stores them as they lie, 8 bytes a lane: one split's partial of one block is a record of 64 runs of 512
+// bytes, run q holding lane after lane, followed by the 32 rows' (running maximum, denominator) pairs, so that
+// everything the merge reads of 32 rows and one split lies together.  In 8-byte units:
+constexpr int kNatBlockUnits = 64 * 64 + 32;  // a block record: 32 KiB of partial outputs + 32 float2
 __host__ __device__ inline int nat_blocks(int head_k, int groups) { return head_k * groups * 4; }
-__device__ __forceinline__ size_t nat_piece(size_t b, int nsplit, int s, int nblk, int blk, int c4, int n) {
-    return ((((b * nsplit + s) * nblk + blk) * 64 + (size_t)(c4 >> 1)) * 64) + (size_t)((c4 & 1) * 32 + n);
+// start of the record of block blk, split s of sequence b
+__device__ __forceinline__ size_t nat_block(size_t b, int nsplit, int s, int nblk, int blk) {
+    return ((b * nsplit + s) * nblk + blk) * (size_t)kNatBlockUnits;
 }
-// bytes of one sequence split's partials in that order (32 rows x 512 columns x 2 bytes a block)
-__host__ __device__ inline size_t nat_split_bytes(int nblk) { return (size_t)nblk * 32 * 1024; }
+// columns 4 c4 .. 4 c4 + 3 of row n, relative to the record's start
+__device__ __forceinline__ int nat_piece(int c4, int n) { return (c4 >> 1) * 64 + (c4 & 1) * 32 + n; }
+// (m, l) of row n, relative to the record's start
+__device__ __forceinline__ int nat_ml(int n) { return 64 * 64 + n; }
+// bytes of one sequence split's records
+__host__ __device__ inline size_t nat_split_bytes(int nblk) { return (size_t)nblk * kNatBlockUnits * 8; }
 
 // First token (row of the packed K/V buffers) and length of sequence b; paged sequences start at row 0 of their
 // own pages.

@@ -800,8 +800,9 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_num_vgpr(kScV))) void la
         // one-round grid runs at the same moment.
         const float inv = 1.0f / l_tot;
         const int blk = (hk * p.groups + grp) * NWV + wave;
-        uint8_t* const dst = reinterpret_cast<uint8_t*>(p.ws_o) +
-                             nat_piece((size_t)b, p.nsplit, split, nat_blocks(p.head_k, p.groups), blk, 0, 0) * 8 + lane * 8;
+        uint8_t* const rec = reinterpret_cast<uint8_t*>(p.ws_o) +
+                             nat_block((size_t)b, p.nsplit, split, nat_blocks(p.head_k, p.groups), blk) * 8;
+        uint8_t* const dst = rec + lane * 8;
         static_for<0, CT * 4>([&](auto ic) {
             constexpr int q = decltype(ic)::value, c = q / 4, r4 = q % 4;
             u32x2 w;
@@ -811,11 +812,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_num_vgpr(kScV))) void la
                             acc_at(std::integral_constant<int, c * 16 + r4 * 4 + 3>{}) * inv);
             *reinterpret_cast<u32x2*>(dst + q * 512) = w;
         });
-        if (n < nh && half == 0) {
-            const size_t part = ((size_t)b * p.head_q + h_base + n) * p.nsplit + split;
-            p.ws_ml[part * 2 + 0] = m;
-            p.ws_ml[part * 2 + 1] = l_tot;
-        }
+        if (n < nh && half == 0) reinterpret_cast<float2*>(rec)[nat_ml(n)] = make_float2(m, l_tot);
     } else {
         // The wave's 32 output rows (its heads) leave through LDS: a lane holds groups of four columns of its head's
         // row, so storing from registers would scatter 8-byte pieces over 32 rows per instruction; instead the rows
@@ -860,13 +857,13 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_num_vgpr(kScV))) void la
         }
     }
 #ifdef DA_PIPE_PROBE
-    if (p.nsplit > 1 && nat_blocks(p.head_k, p.groups) * 32 <= p.head_q) {
-        // stamps into the unused upper half of the fp32-sized partial area, 16 floats per work-group
+    if (p.nsplit > 1) {
+        // stamps into the unused last quarter of the fp32-sized partial area, 16 floats per work-group
         const long long pr_w3 = wall_clock64();  // stores issued
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
         const long long pr_w2 = wall_clock64();
         if (threadIdx.x == 0) {
-            float* pa = p.ws_o + (size_t)p.batch * p.head_q * p.nsplit * (DV / 2) + ((size_t)b * p.nsplit + split) * 16;
+            float* pa = p.ws_o + (size_t)p.batch * p.head_q * p.nsplit * (DV / 4 * 3) + ((size_t)b * p.nsplit + split) * 16;
             pa[0] = (float)(pr_t1 - pr_t0);
             pa[1] = (float)(pr_w1 - pr_w0);
             pa[2] = (float)pr_top;

@@ -298,7 +298,7 @@ __global__ __launch_bounds__(256) void reduce_kernel(const ReduceParams p, int r
     const size_t part0 = (size_t)row * p.nsplit;
     const float2* const ml = reinterpret_cast<const float2*>(p.ws_ml) + part0;
     const float4* const src = reinterpret_cast<const float4*>(p.ws_o + part0 * p.dim_v) + c4;
-    const uint2* const src16 = reinterpret_cast<const uint2*>(p.ws_o);
+    const uint2* const src16 = reinterpret_cast<const uint2*>(p.ws_o);  // (H16) the block records
     // This lane's next four partials: slots s0, s0 + SG, ... (clamped to `last`; the caller masks the rest).
     float2 e[4];
     float4 x[4];
@@ -306,11 +306,13 @@ __global__ __launch_bounds__(256) void reduce_kernel(const ReduceParams p, int r
 #pragma unroll
         for (int u = 0; u < 4; ++u) {
             const int s = min(s0 + u * SG, last);
-            e[u] = ml[s];
             if constexpr (H16) {
-                const uint2 h = src16[nat_piece(nat_b, p.nsplit, s, p.nat_blocks, nat_blk, c4, nat_n)];
+                const uint2* const rec = src16 + nat_block(nat_b, p.nsplit, s, p.nat_blocks, nat_blk);
+                e[u] = reinterpret_cast<const float2*>(rec)[nat_ml(nat_n)];
+                const uint2 h = rec[nat_piece(c4, nat_n)];
                 x[u] = make_float4(EL::lo(h.x), EL::hi(h.x), EL::lo(h.y), EL::hi(h.y));
             } else {
+                e[u] = ml[s];
                 x[u] = src[(size_t)s * nc4];
             }
         }
@@ -397,75 +399,85 @@ __global__ __launch_bounds__(256) void reduce_kernel(const ReduceParams p, int r
 // The merge for normalised 16-bit partials (ReduceParams::half_partials, laid out as nat_piece says) in its
 // one-lane-per-element form: one thread per (sequence, query head, eight output columns), consecutive threads taking
 // consecutive heads of a block, so that a wave's loads are runs of 256 bytes; the partials of four splits are fetched
-// together.  A partial's weight is 2^(m_i - m) times its denominator l_i.
+// together.  A partial's weight is 2^(m_i - m) times its denominator l_i.  A work-group's 256 results are 32 rows x 128
+// bytes of the output: they change hands through LDS so that each row's 128 bytes leave as one run.
 template <typename Tag>
 __global__ __launch_bounds__(256) void reduce16_kernel(const ReduceParams p, int rows) {
     using EL = Elem<Tag>;
+    __shared__ uint4 out_tile[32][9];  // (a pitch of nine 16-byte units: the rows' writes spread over the banks)
     const long long gid = (long long)blockIdx.x * 256 + threadIdx.x;
     const int n = (int)(gid & 31);        // row of the block
     const int c8 = (int)(gid >> 5) & 63;  // eight columns
-    const long long bg = gid >> 11;       // sequence * blocks + block
+    const long long bg = gid >> 11;       // sequence * blocks + block (the same for the whole work-group)
     if (bg >= (long long)(rows / p.head_q) * p.nat_blocks) return;
     const size_t b = (size_t)(bg / p.nat_blocks);
     const int blk = (int)(bg % p.nat_blocks);
     const int per_kv = p.groups * 4;
-    const int hr = (blk % per_kv) * 32 + n;  // head within its KV head's group of `ratio`
-    if (hr >= p.ratio) return;               // a dead row of the group's last block
-    const int row = (int)b * p.head_q + (blk / per_kv) * p.ratio + hr;
-    const size_t part0 = (size_t)row * p.nsplit;
-    const float2* const ml = reinterpret_cast<const float2*>(p.ws_ml) + part0;
-    const uint2* const src = reinterpret_cast<const uint2*>(p.ws_o);
-    float2 e[4];
-    uint4 x[4];
-    auto fetch = [&](int s0, int last) {
+    const int hr0 = (blk % per_kv) * 32;  // first head of the block within its KV head's group of `ratio`
+    const int row0 = (int)b * p.head_q + (blk / per_kv) * p.ratio + hr0;
+    uint4 r = make_uint4(0u, 0u, 0u, 0u);
+    if (hr0 + n < p.ratio) {  // (else a dead row of the group's last block)
+        const uint2* const src = reinterpret_cast<const uint2*>(p.ws_o);
+        float2 e[4];
+        uint4 x[4];
+        auto fetch = [&](int s0, int last) {
 #pragma unroll
-        for (int u = 0; u < 4; ++u) {
-            const int s = min(s0 + u, last);
-            e[u] = ml[s];
-            // columns 8 c8 .. + 3 lie with lane n of the storing wave, + 4 .. + 7 with lane 32 + n
-            const size_t at = nat_piece(b, p.nsplit, s, p.nat_blocks, blk, 2 * c8, n);
-            const uint2 lo = src[at], hi = src[at + 32];
-            x[u] = make_uint4(lo.x, lo.y, hi.x, hi.y);
-        }
-    };
-    if (p.early) fetch(0, p.nsplit - 1);
-    const int len = p.cu_seq_k ? p.cu_seq_k[b + 1] - p.cu_seq_k[b] : p.seq_lens[b];
-    const int ns = len > 0 ? min(p.nsplit, (len + p.chunk - 1) / p.chunk) : 0;
-    float mm = kNegBig, den = 0.0f;
-    float num[8];
+            for (int u = 0; u < 4; ++u) {
+                const int s = min(s0 + u, last);
+                const uint2* const rec = src + nat_block(b, p.nsplit, s, p.nat_blocks, blk);
+                e[u] = reinterpret_cast<const float2*>(rec)[nat_ml(n)];
+                // columns 8 c8 .. + 3 lie with lane n of the storing wave, + 4 .. + 7 with lane 32 + n
+                const uint2 lo = rec[nat_piece(2 * c8, n)], hi = rec[nat_piece(2 * c8, n) + 32];
+                x[u] = make_uint4(lo.x, lo.y, hi.x, hi.y);
+            }
+        };
+        if (p.early) fetch(0, p.nsplit - 1);
+        const int len = p.cu_seq_k ? p.cu_seq_k[b + 1] - p.cu_seq_k[b] : p.seq_lens[b];
+        const int ns = len > 0 ? min(p.nsplit, (len + p.chunk - 1) / p.chunk) : 0;
+        float mm = kNegBig, den = 0.0f;
+        float num[8];
 #pragma unroll
-    for (int j = 0; j < 8; ++j) num[j] = 0.0f;
-    for (int s0 = 0; s0 < ns; s0 += 4) {
-        if (!p.early || s0 != 0) fetch(s0, ns - 1);
-        float m_new = mm;
+        for (int j = 0; j < 8; ++j) num[j] = 0.0f;
+        for (int s0 = 0; s0 < ns; s0 += 4) {
+            if (!p.early || s0 != 0) fetch(s0, ns - 1);
+            float m_new = mm;
 #pragma unroll
-        for (int u = 0; u < 4; ++u)
-            if (s0 + u < ns) m_new = fmaxf(m_new, e[u].x);
-        const float keep = fast_exp2(mm - m_new);  // 0 on the first round
-        mm = m_new;
-        den *= keep;
+            for (int u = 0; u < 4; ++u)
+                if (s0 + u < ns) m_new = fmaxf(m_new, e[u].x);
+            const float keep = fast_exp2(mm - m_new);  // 0 on the first round
+            mm = m_new;
+            den *= keep;
 #pragma unroll
-        for (int j = 0; j < 8; ++j) num[j] *= keep;
+            for (int j = 0; j < 8; ++j) num[j] *= keep;
 #pragma unroll
-        for (int u = 0; u < 4; ++u) {
-            const float w = s0 + u < ns ? fast_exp2(e[u].x - mm) * e[u].y : 0.0f;
-            den += w;
-            const uint32_t h[4] = {x[u].x, x[u].y, x[u].z, x[u].w};
+            for (int u = 0; u < 4; ++u) {
+                const float w = s0 + u < ns ? fast_exp2(e[u].x - mm) * e[u].y : 0.0f;
+                den += w;
+                const uint32_t h[4] = {x[u].x, x[u].y, x[u].z, x[u].w};
 #pragma unroll
-            for (int j = 0; j < 4; ++j) {
-                // (a slot past the sequence's last split holds stale data, possibly NaN: select, do not multiply by 0)
-                num[2 * j] += s0 + u < ns ? w * EL::lo(h[j]) : 0.0f;
-                num[2 * j + 1] += s0 + u < ns ? w * EL::hi(h[j]) : 0.0f;
+                for (int j = 0; j < 4; ++j) {
+                    // (a slot past the sequence's last split holds stale data, possibly NaN: select, do not multiply by 0)
+                    num[2 * j] += s0 + u < ns ? w * EL::lo(h[j]) : 0.0f;
+                    num[2 * j + 1] += s0 + u < ns ? w * EL::hi(h[j]) : 0.0f;
+                }
             }
         }
+        const float inv = ns > 0 ? 1.0f / den : 0.0f;  // an empty sequence yields a zero row
+        r.x = EL::pack2(num[0] * inv, num[1] * inv);
+        r.y = EL::pack2(num[2] * inv, num[3] * inv);
+        r.z = EL::pack2(num[4] * inv, num[5] * inv);
+        r.w = EL::pack2(num[6] * inv, num[7] * inv);
     }
-    const float inv = ns > 0 ? 1.0f / den : 0.0f;  // an empty sequence yields a zero row
-    uint4 r;
-    r.x = EL::pack2(num[0] * inv, num[1] * inv);
-    r.y = EL::pack2(num[2] * inv, num[3] * inv);
-    r.z = EL::pack2(num[4] * inv, num[5] * inv);
-    r.w = EL::pack2(num[6] * inv, num[7] * inv);
-    *reinterpret_cast<uint4*>(reinterpret_cast<uint16_t*>(p.o) + (size_t)row * p.dim_v + c8 * 8) = r;
+    // thread (n, j) holds columns 8 (c0 + j) .. + 7 of row n, c0 the work-group's first column group; thread t sends off
+    // piece t % 8 of row t / 8
+    out_tile[n][threadIdx.x >> 5] = r;
+    __syncthreads();
+    const int n2 = threadIdx.x >> 3, seg = threadIdx.x & 7;
+    if (hr0 + n2 < p.ratio) {
+        const int c0 = (int)((gid - threadIdx.x) >> 5) & 63;
+        *reinterpret_cast<uint4*>(reinterpret_cast<uint16_t*>(p.o) + (size_t)(row0 + n2) * p.dim_v + (c0 + seg) * 8) =
+            out_tile[n2][seg];
+    }
 }
 
 }  // namespace da
