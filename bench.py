@@ -35,7 +35,7 @@ MFMA_PEAK_TFLOPS = 2500.0   # MI355X dense fp16/bf16 MFMA, published
 # it was measured under; when the library plans the workload differently, the bench line carries null instead.
 MEASURED_TRAFFIC = {
     "gqa": {"bytes": 1092312678, "plan": {"kind": 3, "nsplit": 4, "chunk": 1024, "heads_per_group": 16}},
-    "mla": {"bytes": 389949440, "plan": {"kind": 2, "nsplit": 4, "chunk": 1024, "heads_per_group": 128},
+    "mla": {"bytes": 389967872, "plan": {"kind": 2, "nsplit": 4, "chunk": 1024, "heads_per_group": 128},
             "partials": "16-bit"},
 }
 
