@@ -46,6 +46,14 @@ struct Elem<f16_tag> {
         const f32x2 v = {lo, hi};
         return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, f16x2));
     }
+    // (lo * s, hi * s) rounded and packed: the mixed-precision multiply-adds write the two halves of the result, one
+    // instruction a value, each product rounded once
+    static __device__ __forceinline__ uint32_t pack2_scaled(float lo, float hi, float s) {
+        uint32_t r;
+        asm("v_fma_mixlo_f16 %0, %1, %2, 0" : "=v"(r) : "v"(lo), "v"(s));
+        asm("v_fma_mixhi_f16 %0, %1, %2, 0" : "+v"(r) : "v"(hi), "v"(s));
+        return r;
+    }
 };
 
 template <>
@@ -65,6 +73,8 @@ struct Elem<bf16_tag> {
         const f32x2 v = {lo, hi};
         return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, bf16x2));
     }
+    // (lo * s, hi * s) rounded and packed
+    static __device__ __forceinline__ uint32_t pack2_scaled(float lo, float hi, float s) { return pack2(lo * s, hi * s); }
 };
 
 __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }

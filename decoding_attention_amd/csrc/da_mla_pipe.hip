@@ -806,10 +806,10 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_num_vgpr(kScV))) void la
         static_for<0, CT * 4>([&](auto ic) {
             constexpr int q = decltype(ic)::value, c = q / 4, r4 = q % 4;
             u32x2 w;
-            w.x = EL::pack2(acc_at(std::integral_constant<int, c * 16 + r4 * 4 + 0>{}) * inv,
-                            acc_at(std::integral_constant<int, c * 16 + r4 * 4 + 1>{}) * inv);
-            w.y = EL::pack2(acc_at(std::integral_constant<int, c * 16 + r4 * 4 + 2>{}) * inv,
-                            acc_at(std::integral_constant<int, c * 16 + r4 * 4 + 3>{}) * inv);
+            w.x = EL::pack2_scaled(acc_at(std::integral_constant<int, c * 16 + r4 * 4 + 0>{}),
+                                   acc_at(std::integral_constant<int, c * 16 + r4 * 4 + 1>{}), inv);
+            w.y = EL::pack2_scaled(acc_at(std::integral_constant<int, c * 16 + r4 * 4 + 2>{}),
+                                   acc_at(std::integral_constant<int, c * 16 + r4 * 4 + 3>{}), inv);
             *reinterpret_cast<u32x2*>(dst + q * 512) = w;
         });
         if (n < nh && half == 0) reinterpret_cast<float2*>(rec)[nat_ml(n)] = make_float2(m, l_tot);
@@ -829,10 +829,10 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_num_vgpr(kScV))) void la
             constexpr int c = decltype(ic)::value / 4, r4 = decltype(ic)::value % 4;
             const int col = c * 32 + r4 * 8 + half * 4;
             u32x2 w;
-            w.x = EL::pack2(acc_at(std::integral_constant<int, c * 16 + r4 * 4 + 0>{}) * inv,
-                            acc_at(std::integral_constant<int, c * 16 + r4 * 4 + 1>{}) * inv);
-            w.y = EL::pack2(acc_at(std::integral_constant<int, c * 16 + r4 * 4 + 2>{}) * inv,
-                            acc_at(std::integral_constant<int, c * 16 + r4 * 4 + 3>{}) * inv);
+            w.x = EL::pack2_scaled(acc_at(std::integral_constant<int, c * 16 + r4 * 4 + 0>{}),
+                                   acc_at(std::integral_constant<int, c * 16 + r4 * 4 + 1>{}), inv);
+            w.y = EL::pack2_scaled(acc_at(std::integral_constant<int, c * 16 + r4 * 4 + 2>{}),
+                                   acc_at(std::integral_constant<int, c * 16 + r4 * 4 + 3>{}), inv);
             *reinterpret_cast<__attribute__((address_space(3))) u32x2*>(wbuf + n * PITCH + col * 2) = w;
         });
         // (LDS operations of one wave complete in order: the wave reads its own rows back)
