@@ -303,10 +303,10 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_num_vgpr(kScV))) void la
         else
             issue_tile(c0 + i * kTile, i);
     };
-    // Tile 0 goes out at once (buffer 0), tile 1 behind the second round of Q, tile 2 when Q is through, tile t + 3
-    // in trip t: the first trip needs Q and tile 0 only, and every work-group of the grid asks for them at the same
-    // moment, so nothing else competes with them.
-    if (0 < ntiles) issue_any(0);
+    // Tile 0 goes out behind the first round of Q (buffer 0), tile 1 behind the second, tile 2 when Q is through, tile
+    // t + 3 in trip t: the first trip needs Q and tile 0 only, and every work-group of the grid asks for them at the
+    // same moment, so nothing else competes with them.  Loads complete in order, so a round's wait leaves the tile
+    // issued behind its Q blocks outstanding: the tile arrives while the blocks are read into registers.
 
     // Q rows of this wave's heads as B-operands: lane (n, half) holds Q[head n][ks*16 + half*8 .. +8).  The wave's
     // 32 x 576 block of Q is staged like a K tile (whole-row direct-to-LDS loads, same swizzle) and read back with
@@ -352,10 +352,11 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_num_vgpr(kScV))) void la
     };
     issue_q_share(0);
     issue_q_share(1);
+    issue_any(0);  // (c0 < c1: there is a tile 0)
     // (while the loads are on their way) the output tiles start at zero
     static_for<0, CT * 16>([&](auto ic) { asm volatile("v_accvgpr_write_b32 a[%0], 0" ::"n"(decltype(ic)::value)); });
-    wait_vmcnt<0>();
-    __syncthreads();  // the Q blocks of waves 0 and 1 (and tile 0) are in LDS
+    wait_vmcnt<NLW>();  // (all but tile 0's)
+    __syncthreads();    // the Q blocks of waves 0 and 1 are in LDS
     if ((wave >> 1) == 0) read_q();
     __syncthreads();  // ... and in registers: buffers 2 and 3 take the blocks of waves 2 and 3
     issue_q_share(2);
@@ -803,14 +804,19 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_num_vgpr(kScV))) void la
         uint8_t* const rec = reinterpret_cast<uint8_t*>(p.ws_o) +
                              nat_block((size_t)b, p.nsplit, split, nat_blocks(p.head_k, p.groups), blk) * 8;
         uint8_t* const dst = rec + lane * 8;
-        static_for<0, CT * 4>([&](auto ic) {
-            constexpr int q = decltype(ic)::value, c = q / 4, r4 = q % 4;
-            u32x2 w;
-            w.x = EL::pack2_scaled(acc_at(std::integral_constant<int, c * 16 + r4 * 4 + 0>{}),
-                                   acc_at(std::integral_constant<int, c * 16 + r4 * 4 + 1>{}), inv);
-            w.y = EL::pack2_scaled(acc_at(std::integral_constant<int, c * 16 + r4 * 4 + 2>{}),
-                                   acc_at(std::integral_constant<int, c * 16 + r4 * 4 + 3>{}), inv);
-            *reinterpret_cast<u32x2*>(dst + q * 512) = w;
+        // (a whole 32 x 32 tile's sixteen values are read before any is converted: the reads are independent, and a
+        // lone wave per SIMD has nothing else to cover the wait between a read and its use)
+        static_for<0, CT>([&](auto cc) {
+            constexpr int c = decltype(cc)::value;
+            float a[16];
+            static_for<0, 16>([&](auto ic) { a[decltype(ic)::value] = acc_at(std::integral_constant<int, c * 16 + decltype(ic)::value>{}); });
+#pragma unroll
+            for (int r4 = 0; r4 < 4; ++r4) {
+                u32x2 w;
+                w.x = EL::pack2_scaled(a[r4 * 4 + 0], a[r4 * 4 + 1], inv);
+                w.y = EL::pack2_scaled(a[r4 * 4 + 2], a[r4 * 4 + 3], inv);
+                *reinterpret_cast<u32x2*>(dst + (c * 4 + r4) * 512) = w;
+            }
         });
         if (n < nh && half == 0) reinterpret_cast<float2*>(rec)[nat_ml(n)] = make_float2(m, l_tot);
     } else {
