@@ -353,11 +353,23 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_num_vgpr(kScV))) void la
     issue_q_share(0);
     issue_q_share(1);
     issue_any(0);  // (c0 < c1: there is a tile 0)
-    // (while the loads are on their way) the output tiles start at zero
-    static_for<0, CT * 16>([&](auto ic) { asm volatile("v_accvgpr_write_b32 a[%0], 0" ::"n"(decltype(ic)::value)); });
+    // The output tiles start at zero: 512 register writes, 2048 clocks of a wave alone on its SIMD.  Half of them while
+    // the first loads are on their way (all of them would outlast the loads), the other half while the other pair of
+    // waves reads its Q blocks.
+    auto zero_acc = [&](auto from_c, auto to_c) __attribute__((always_inline)) {
+        static_for<decltype(from_c)::value, decltype(to_c)::value>(
+            [&](auto ic) { asm volatile("v_accvgpr_write_b32 a[%0], 0" ::"n"(decltype(ic)::value)); });
+    };
+    constexpr std::integral_constant<int, 0> acc_lo{};
+    constexpr std::integral_constant<int, CT * 8> acc_mid{};
+    constexpr std::integral_constant<int, CT * 16> acc_hi{};
+    zero_acc(acc_lo, acc_mid);
     wait_vmcnt<NLW>();  // (all but tile 0's)
     __syncthreads();    // the Q blocks of waves 0 and 1 are in LDS
-    if ((wave >> 1) == 0) read_q();
+    if ((wave >> 1) == 0)
+        read_q();
+    else
+        zero_acc(acc_mid, acc_hi);
     __syncthreads();  // ... and in registers: buffers 2 and 3 take the blocks of waves 2 and 3
     issue_q_share(2);
     issue_q_share(3);
@@ -368,7 +380,10 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_num_vgpr(kScV))) void la
         wait_vmcnt<0>();
     }
     __syncthreads();
-    if ((wave >> 1) == 1) read_q();
+    if ((wave >> 1) == 1)
+        read_q();
+    else
+        zero_acc(acc_mid, acc_hi);
     __syncthreads();  // buffers 2 and 3 are free for K
     if (2 < ntiles) issue_any(2);
 
