@@ -421,8 +421,8 @@ def reference_log_line(batch, seq_k, ms, tflops, gbps):
 def sweep_sections(kind):
     """The shapes `--sweep kind` measures, as (section marker or None, tag, workload arguments) in print order.
     `mha` and `mla` are the reference's two sections with its full lists; `baseline` holds the benchmark shapes
-    those lists leave out (the ragged and fixed GQA batches, MQA with ALiBi, sequence length 1536, and the latent
-    form's length sweep at batch 16)."""
+    those lists leave out (the ragged and fixed GQA batches, MQA with ALiBi, sequence length 1536, the latent
+    form's length sweep at batch 16, and the latent shape with V passed as its own buffer)."""
     out = []
     for fam in ("mha", "mla"):
         if kind in (fam, "all"):
@@ -435,6 +435,8 @@ def sweep_sections(kind):
         out += [(title, "gqa-varlen", ("gqa-varlen",)), (None, "gqa-fixed", ("gqa-fixed",)),
                 (None, "mqa-alibi", ("mqa-alibi",)), (None, "mha-seq", ("mha", 1, 1536))]
         out += [(None, "mla-seq-b16", ("mla", 16, sk)) for sk in (512, 1024, 2048, 4096, 8192, 16384)]
+        # (576, 512) with V in a buffer of its own, as the reference's binding accepts it: K and V are both read
+        out += [(None, "mla-distinct-v", ("mla-distinct-v", b, 4096)) for b in (16, 64)]
     return out
 
 
@@ -445,6 +447,9 @@ def _sweep_workload(torch, wl, spec, device):
     if spec[0] == "mla":
         hq, hk, d, dv = REF_SWEEPS["mla"]["heads"]
         return wl.make_workload(spec[1], hq, hk, d, dv, spec[2], torch.float16, device=device)
+    if spec[0] == "mla-distinct-v":
+        hq, hk, d, dv = REF_SWEEPS["mla"]["heads"]
+        return wl.make_workload(spec[1], hq, hk, d, dv, spec[2], torch.float16, device=device, latent=False)
     return {"gqa-varlen": wl.config_gqa_varlen, "gqa-fixed": wl.config_gqa_fixed, "mqa-alibi": wl.config_mqa_alibi}[spec[0]]()
 
 
