@@ -686,13 +686,12 @@ int run_attention(const void* q, const void* k, const void* v, void* o, const in
         sp.flat_cu = flat_cu;
     }
 
-    if (pl.nsplit > 1 && da::mla_half_partials(pl.kind == kKindMfma && !pl.v_distinct, pl.rt, kf.fmt)) {
-        // the pipelined kernel's 16-bit partials take whole blocks of 32 heads: they must fit the area sized for
-        // fp32 partials of head_q rows (they do from 65 heads per KV head up, where that kernel runs)
-        const size_t need = (size_t)batch * pl.nsplit * da::nat_split_bytes(da::nat_blocks((int)head_k, pl.groups));
-        if (need > (size_t)batch * head_q * pl.nsplit * dim_v * sizeof(float))
-            return fail(DA_ERR_WORKSPACE, "16-bit partials of %zu bytes do not fit the workspace's partial area", need);
-    }
+    // the latent kernels' split partials: 16-bit block records where whole blocks of 32 heads fit the area sized for
+    // fp32 partials of head_q rows (mla_half_partials), un-normalised fp32 rows otherwise
+    const bool half_partials = pl.nsplit > 1 && da::mla_half_partials(pl.kind == kKindMfma, pl.rt, head_q, head_k, pl.groups);
+    sp.nat_partials = half_partials ? 1 : 0;
+    if (pl.kind == kKindMfma && pl.rt == 128 && kf.fmt == 0 && !pl.v_distinct && pl.nsplit > 1 && !half_partials)
+        return fail(DA_ERR_WORKSPACE, "the pipelined kernel's 16-bit partials do not fit the workspace's partial area");
     const dim3 grid((unsigned)(pl.flat_tokens ? pl.flat_wgs : pl.nsplit),
                     (unsigned)((pl.wave_per_head ? head_k / 4 : head_k) * pl.groups),
                     (unsigned)(pl.flat_tokens ? 1 : batch));
@@ -740,10 +739,11 @@ int run_attention(const void* q, const void* k, const void* v, void* o, const in
         rp.flat_wgs = pl.flat_wgs;
         rp.flat_cu = sp.flat_cu;
         rp.early = pl.ws_bytes <= ((size_t)8 << 20) ? 1 : 0;
-        rp.half_partials = da::mla_half_partials(pl.kind == kKindMfma && !pl.v_distinct, pl.rt, kf.fmt) ? 1 : 0;
+        rp.half_partials = half_partials ? 1 : 0;
         rp.ratio = sp.ratio;
         rp.groups = pl.groups;
-        rp.nat_blocks = da::nat_blocks((int)head_k, pl.groups);
+        rp.nat_waves = half_partials ? pl.rt / 32 : 0;
+        rp.nat_blocks = half_partials ? da::nat_blocks((int)head_k, pl.groups, pl.rt / 32) : 0;
         e = da::launch_reduce(rp, is_bf16 != 0, (int)(batch * head_q), stream);
         if (e != hipSuccess) return fail(DA_ERR_HIP, "merge kernel launch: %s", hipGetErrorString(e));
     }

@@ -257,6 +257,7 @@ struct SweepParams {
     int head_q, head_k, ratio;
     int groups;               // work-groups per KV head (ceil(ratio / heads per work-group))
     int nsplit, chunk;        // sequence splits and tokens per split
+    int nat_partials;         // latent kernels: split partials as normalised 16-bit block records (nat_block below)
     float scale_log2;         // softmax scale * log2(e)
     int is_alibi;
     // Paged K/V (block_table != null): k and v are page pools [pages, page_size, head_k, dim(_v)], token j of
@@ -303,16 +304,18 @@ struct ReduceParams {
     // splitting adds)
     int half_partials;
     int ratio, groups, nat_blocks;  // (half_partials) query heads per KV head, work-groups per KV head, nat_blocks()
+    int nat_waves;                  // (half_partials) waves, i.e. blocks of 32 heads, per work-group of the sweep
 };
 
-// Normalised 16-bit partials of the pipelined latent kernel (dim_v = 512).  A wave of that kernel owns 32 query heads
-// (a block; block id = (KV head * groups + group) * 4 + wave, rows past the group's last head are dead), and after
+// Normalised 16-bit partials of the latent kernels (dim_v = 512).  A wave of those kernels owns 32 query heads (a
+// block; block id = (KV head * groups + group) * waves per work-group + wave, rows past the group's last head are
+// dead), and after
 // the last matrix step lane (n, half) holds, for each q = 0 .. 63, the four columns 8 q + 4 half .. + 3 of head n.
 // The wave stores them as they lie, 8 bytes a lane: one split's partial of one block is a record of 64 runs of 512
 // bytes, run q holding lane after lane, followed by the 32 rows' (running maximum, denominator) pairs, so that
 // everything the merge reads of 32 rows and one split lies together.  In 8-byte units:
 constexpr int kNatBlockUnits = 64 * 64 + 32;  // a block record: 32 KiB of partial outputs + 32 float2
-__host__ __device__ inline int nat_blocks(int head_k, int groups) { return head_k * groups * 4; }
+__host__ __device__ inline int nat_blocks(int head_k, int groups, int waves) { return head_k * groups * waves; }
 // start of the record of block blk, split s of sequence b
 __device__ __forceinline__ size_t nat_block(size_t b, int nsplit, int s, int nblk, int blk) {
     return ((b * nsplit + s) * nblk + blk) * (size_t)kNatBlockUnits;

@@ -10,9 +10,13 @@ int mla_rows_per_trip();
 // work-groups than this (DA_MLA_TWO_PER_CU_FROM, default 256)
 int mla_two_per_cu_from();
 hipError_t launch_mla(const SweepParams& p, bool is_bf16, int rt, dim3 grid, hipStream_t stream);
-// whether a latent-kernel launch (heads per work-group rt, K format kv_fmt: 0 = 16-bit) leaves its split partials as
-// normalised 16-bit values (ReduceParams::half_partials): the pipelined kernel does
-inline bool mla_half_partials(bool latent_kernel, int rt, int kv_fmt) { return latent_kernel && rt == 128 && kv_fmt == 0; }
+// Whether a latent-kernel launch with rt heads per work-group (rt / 32 waves) leaves its split partials as normalised
+// 16-bit block records (ReduceParams::half_partials, nat_block in da_common.h): whenever the records of whole blocks
+// of 32 heads fit the workspace area sized for fp32 partials of head_q rows, i.e. from 17 heads per KV head up.
+inline bool mla_half_partials(bool latent_kernel, int rt, size_t head_q, size_t head_k, int groups) {
+    return latent_kernel && rt % 32 == 0 &&
+           nat_split_bytes(nat_blocks((int)head_k, groups, rt / 32)) <= head_q * 512 * sizeof(float);
+}
 // the software-pipelined kernel for work-groups of 128 heads over 16-bit K (da_mla_pipe.hip); launch_mla routes to it
 hipError_t launch_mla_pipe(const SweepParams& p, bool is_bf16, dim3 grid, hipStream_t stream);
 // the (576, 512) shape with V in a buffer of its own (16-bit K/V; packed, or pages of 16 tokens and more)

@@ -593,6 +593,23 @@ __global__ __launch_bounds__(64 * NWV) void mfma_latent_kernel(const SweepParams
                     w.w = EL::from_f32(acc[c][r4 * 4 + 3] * inv);
                     *reinterpret_cast<ushort4*>(orow + col) = w;
                 }
+        } else if (p.nat_partials) {
+            // normalised 16-bit values in the order the lanes hold them, the row's (m, l) behind them (nat_block)
+            const float inv = vs / l_tot;
+            uint8_t* const rec = reinterpret_cast<uint8_t*>(p.ws_o) +
+                                 nat_block((size_t)b, p.nsplit, split, nat_blocks(p.head_k, p.groups, NWV),
+                                           (hk * p.groups + grp) * NWV + wave) * 8;
+            typedef unsigned int u32x2 __attribute__((ext_vector_type(2)));
+#pragma unroll
+            for (int c = 0; c < CT; ++c)
+#pragma unroll
+                for (int r4 = 0; r4 < 4; ++r4) {
+                    u32x2 w;
+                    w.x = EL::pack2(acc[c][r4 * 4 + 0] * inv, acc[c][r4 * 4 + 1] * inv);
+                    w.y = EL::pack2(acc[c][r4 * 4 + 2] * inv, acc[c][r4 * 4 + 3] * inv);
+                    *reinterpret_cast<u32x2*>(rec + (c * 4 + r4) * 512 + lane * 8) = w;
+                }
+            if (half == 0) reinterpret_cast<float2*>(rec)[nat_ml(n)] = make_float2(m, l_tot);
         } else {
             const size_t part = ((size_t)b * p.head_q + h) * p.nsplit + split;
             float* wrow = p.ws_o + part * DV;

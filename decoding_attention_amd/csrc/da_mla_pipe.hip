@@ -817,7 +817,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_num_vgpr(kScV))) void la
         const float inv = 1.0f / l_tot;
         const int blk = (hk * p.groups + grp) * NWV + wave;
         uint8_t* const rec = reinterpret_cast<uint8_t*>(p.ws_o) +
-                             nat_block((size_t)b, p.nsplit, split, nat_blocks(p.head_k, p.groups), blk) * 8;
+                             nat_block((size_t)b, p.nsplit, split, nat_blocks(p.head_k, p.groups, NWV), blk) * 8;
         uint8_t* const dst = rec + lane * 8;
         // (a whole 32 x 32 tile's sixteen values are read before any is converted: the reads are independent, and a
         // lone wave per SIMD has nothing else to cover the wait between a read and its use)

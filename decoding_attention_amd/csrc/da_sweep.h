@@ -278,7 +278,7 @@ __global__ __launch_bounds__(256) void reduce_kernel(const ReduceParams p, int r
         if (bg >= (long long)(rows / p.head_q) * p.nat_blocks) return;  // (a whole wave: its elements share bg)
         nat_b = (size_t)(bg / p.nat_blocks);
         nat_blk = (int)(bg % p.nat_blocks);
-        const int per_kv = p.groups * 4;
+        const int per_kv = p.groups * p.nat_waves;
         const int r = (nat_blk % per_kv) * 32 + nat_n;  // head within its KV head's group of `ratio`
         if (r >= p.ratio) return;                       // (the SG lanes of an element leave together)
         row = (int)nat_b * p.head_q + (nat_blk / per_kv) * p.ratio + r;
@@ -412,7 +412,7 @@ __global__ __launch_bounds__(256) void reduce16_kernel(const ReduceParams p, int
     if (bg >= (long long)(rows / p.head_q) * p.nat_blocks) return;
     const size_t b = (size_t)(bg / p.nat_blocks);
     const int blk = (int)(bg % p.nat_blocks);
-    const int per_kv = p.groups * 4;
+    const int per_kv = p.groups * p.nat_waves;
     const int hr0 = (blk % per_kv) * 32;  // first head of the block within its KV head's group of `ratio`
     const int row0 = (int)b * p.head_q + (blk / per_kv) * p.ratio + hr0;
     uint4 r = make_uint4(0u, 0u, 0u, 0u);

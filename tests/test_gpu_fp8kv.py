@@ -115,20 +115,24 @@ def test_latent_form_with_fp8_cache(batch, head_q, seq_k, dtype, is_alibi):
     assert (o.float() - ref).abs().max().item() <= TOL[dtype]
 
 
-@pytest.mark.parametrize("head_q", [64, 128])
-def test_latent_fp8_unit_scales_equal_the_16_bit_call(head_q):
+@pytest.mark.parametrize("batch,head_q,seq_k", [(300, 64, 600), (6, 64, 3000), (6, 128, 3000)])
+def test_latent_fp8_unit_scales_equal_the_16_bit_call(batch, head_q, seq_k):
     """FP8 values convert exactly and the tiles are converted before any arithmetic: with unit scales the FP8 call
-    is the 16-bit call on the same values.  Up to 64 heads both run the same kernel in the same order of operations:
-    same bits.  With 128 heads the 16-bit call runs on the software-pipelined kernel (other rounding of the split
-    partials): equal within the output tolerance."""
+    is the 16-bit call on the same values.  Up to 64 heads both run the same kernel, and where neither call splits
+    its sequences (300 sequences of 600 tokens) in the same order of operations: same bits.  Where they split, the
+    two plans cut the sequences differently (the 16-bit form runs two work-groups to a CU) and the partials are
+    rounded to 16 bits, and with 128 heads the 16-bit call runs on the software-pipelined kernel: equal within the
+    output tolerance."""
     # (large enough for the planner to pick the latent kernel, whose property this is)
-    w, k8, _, ks, _ = _case(6, head_q, 1, 576, 512, 3000, torch.float16, latent=True, unit=True, seed=9)
-    assert _lib.plan(w.max_seq_k, 6, head_q, 1, 576, 512)["kind"] == 2
+    w, k8, _, ks, _ = _case(batch, head_q, 1, 576, 512, seq_k, torch.float16, latent=True, unit=True, seed=9)
+    plan = _lib.plan(w.max_seq_k, batch, head_q, 1, 576, 512, total_k=w.k.shape[0])
+    assert plan["kind"] == 2
     k16 = k8.to(torch.float16).to(DEV)
     args = (w.cu_seq_k.to(DEV), w.max_seq_k, 512, False)
     o8 = decoding_attn_fwd(w.q.to(DEV), k8.to(DEV), None, *args, k_scale=ks.to(DEV), v_scale=ks.to(DEV))
     o16 = decoding_attn_fwd(w.q.to(DEV), k16, None, *args)
-    if head_q <= 64:
+    if batch == 300:
+        assert plan["nsplit"] == 1
         assert torch.equal(o8.view(torch.int16), o16.view(torch.int16))
     else:
         assert (o8.float() - o16.float()).abs().max().item() <= TOL[torch.float16]

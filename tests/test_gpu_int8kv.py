@@ -121,16 +121,18 @@ def test_latent_form_with_int8_cache(batch, head_q, seq_k, dtype, is_alibi):
     assert (o.float() - _reference(w, k8, None, ks, ks)).abs().max().item() <= TOL[dtype]
 
 
-@pytest.mark.parametrize("head_q", [64, 128])
+@pytest.mark.parametrize("batch,head_q,seq_k", [(300, 64, 600), (6, 64, 3000), (6, 128, 3000)])
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
-def test_latent_int8_unit_scales_equal_the_16_bit_call(dtype, head_q):
+def test_latent_int8_unit_scales_equal_the_16_bit_call(dtype, batch, head_q, seq_k):
     """The tiles are converted, exactly, before any arithmetic: with unit scales the int8 call is the 16-bit call on
-    the same integers.  Up to 64 heads both run the same kernel in the same order of operations: same bits.  With 128
-    heads the 16-bit call runs on the software-pipelined kernel (other rounding of the split partials): equal within
-    the output tolerance.  All 256 byte values occur."""
+    the same integers.  Up to 64 heads both run the same kernel, and where neither call splits its sequences (300
+    sequences of up to 600 tokens) in the same order of operations: same bits.  Where they split, the two plans cut
+    the sequences differently and the partials are rounded to 16 bits, and with 128 heads the 16-bit call runs on the
+    software-pipelined kernel: equal within the output tolerance.  All 256 byte values occur."""
     # (large enough for the planner to pick the latent kernel, whose property this is)
-    w = wl.make_workload(6, head_q, 1, 576, 512, 3000, dtype, seed=9, varlen=True, latent=True)
-    assert _lib.plan(w.max_seq_k, 6, head_q, 1, 576, 512)["kind"] == 2
+    w = wl.make_workload(batch, head_q, 1, 576, 512, seq_k, dtype, seed=9, varlen=True, latent=True)
+    plan = _lib.plan(w.max_seq_k, batch, head_q, 1, 576, 512, total_k=w.k.shape[0])
+    assert plan["kind"] == 2
     g = torch.Generator().manual_seed(10)
     k8 = torch.round(torch.randn(w.k.shape, generator=g) * 0.7).to(torch.int8)
     k8.view(-1)[::211] = torch.arange(-128, 128, dtype=torch.int8).repeat(k8.numel() // 211 // 256 + 1)[
@@ -140,7 +142,8 @@ def test_latent_int8_unit_scales_equal_the_16_bit_call(dtype, head_q):
     o8 = decoding_attn_fwd(w.q.to(DEV), k8.to(DEV), None, *args)
     o16 = decoding_attn_fwd(w.q.to(DEV), k8.to(dtype).to(DEV), None, *args)
     assert torch.isfinite(o8.float()).all()
-    if head_q <= 64:
+    if batch == 300:
+        assert plan["nsplit"] == 1
         assert torch.equal(o8.view(torch.int16), o16.view(torch.int16))
     else:
         # (integer values up to 128 in magnitude: outputs of order 1, so the tolerance is relative)
