@@ -226,11 +226,14 @@ __device__ __forceinline__ void gqa_segment(const SweepParams& p, uint8_t* const
     };
     // K/V rows are read once per call: non-temporal loads (see stream_load16).  Not in the latent form, whose rows
     // serve several head groups from the caches and which measured slower with the hint (16 heads, batch 64 x 4096
-    // tokens: 63.8 -> 67.2 us).
+    // tokens: 63.8 -> 67.2 us), and not where a head's row is no whole number of 128-byte lines (d = 96: 192 bytes;
+    // 8-bit K/V at d = 64): the line two neighbouring heads share would be dropped after the first one's read and
+    // fetched again for the second (32/8 heads d 96, batch 256 x 4096 tokens: 594.5 us with the hint, 544.6 without;
+    // batch 16 x 4096: 39.9 and 32.9).
     auto kv_load16 = [](const uint8_t* ptr) __attribute__((always_inline)) {
         if constexpr (KV8 == kKvInt4)
             return kv4_load16(ptr);  // (eight bytes from half the address, widened to sixteen int8 elements)
-        else if constexpr (VK)
+        else if constexpr (VK || (D * KB) % 128 != 0)
             return *reinterpret_cast<const uint4*>(ptr);
         else
             return stream_load16(ptr);
