@@ -225,9 +225,9 @@ Plan make_plan(size_t max_seq_k, size_t batch, size_t head_q, size_t head_k, siz
         // (16-bit K/V in whole tiles or 16-token runs only: the 8-bit forms and the per-row page lookups keep fewer
         // bytes in flight per work-group and need the 512; FP8, batch 64 x 4096 tokens: 96 us against 110)
         if (dim == 128 && !kv_8bit && (packed || page_size >= 16) && !pl.wave_per_head) target_wgs = tun().group_target_wgs_d128;
-        // d = 96 (rows of 192 bytes, the slowest stream of the four head dims): 256 work-groups, half the merge
-        // (measured, 32/8 heads: batch 64 x 4096 tokens 156.6 -> 149.9 us, batch 32 x 8192 156.4 -> 150.4, batch 128 x
-        // 2048 152.6 -> 143.0; 16/4 heads, batch 64 x 4096 79.6 -> 77.2)
+        // d = 96 (rows of 192 bytes, ordinary loads, the slowest stream of the four head dims): 256 work-groups, half
+        // the merge (measured, 32/8 heads: batch 64 x 4096 tokens 144.1 -> 142.0 us, batch 32 x 8192 145.6 -> 142.6,
+        // batch 128 x 2048 142.5 -> 138.1; 16/4 heads, batch 64 x 4096 75.6 -> 74.3)
         if (dim == 96 && !kv_8bit && (packed || page_size >= 16)) target_wgs = tun().group_target_wgs_d128;
     } else {
         pl.kind = kKindSweep;
@@ -349,8 +349,8 @@ Plan make_plan(size_t max_seq_k, size_t batch, size_t head_q, size_t head_k, siz
     // 128, 4096 tokens: batch 40, 7 splits (560 work-groups) 138.6 us, 3 splits (240) 117.9; batch 48, 6 splits (576)
     // 158.8, 5 splits (480) 142.4; batch 100, 4 splits (800) 320.5, 1 split (200) 284.8.
     // (d = 96 counts as long rows, 256 work-groups a round, like its target above: 32/8 heads, 4096 tokens, batch 40
-    // 117.6 -> 93.3 us, batch 48 135.1 -> 116.8, batch 72 199.6 -> 174.7, batch 100 259.9 -> 246.5; batch 24 x 8192
-    // 143.2 -> 111.7; 32/4 heads, batch 80 x 4096 119.4 -> 90.4)
+    // 118.0 -> 92.2 us, batch 48 148.3 -> 113.1, batch 72 225.6 -> 166.0, batch 100 243.8 -> 223.1; batch 24 x 8192
+    // 151.1 -> 109.4; 32/4 heads, batch 80 x 4096 117.4 -> 90.2)
     // (measured on 16-bit K/V in whole tiles or 16-token runs, and applied there only)
     // (... and on 8-bit K/V at d = 128, whose rows are as short as 16-bit rows at d = 64: FP8, 32/8 heads, batch 100
     // x 4096 tokens 184 -> 154 us, batch 72 131 -> 116, batch 40 74 -> 66)
