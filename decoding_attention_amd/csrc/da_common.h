@@ -309,19 +309,22 @@ struct ReduceParams {
 
 // Normalised 16-bit partials of the latent kernels (dim_v = 512).  A wave of those kernels owns 32 query heads (a
 // block; block id = (KV head * groups + group) * waves per work-group + wave, rows past the group's last head are
-// dead), and after
-// the last matrix step lane (n, half) holds, for each q = 0 .. 63, the four columns 8 q + 4 half .. + 3 of head n.
-// The wave stores them as they lie, 8 bytes a lane: one split's partial of one block is a record of 64 runs of 512
-// bytes, run q holding lane after lane, followed by the 32 rows' (running maximum, denominator) pairs, so that
-// everything the merge reads of 32 rows and one split lies together.  In 8-byte units:
+// dead), and after the last matrix step lane (n, half) holds, for each 32-column tile c = 0 .. 15 and r4 = 0 .. 3, the
+// four columns 32 c + 8 r4 + 4 half .. + 3 of head n.  The wave stores them as they lie, 16 bytes a lane (the pieces
+// r4 = 2 rp and 2 rp + 1 together): one split's partial of one block is a record of 32 runs of 1 KiB, run 2 c + rp
+// holding lane after lane, followed by the 32 rows' (running maximum, denominator) pairs, so that everything the
+// merge reads of 32 rows and one split lies together and both sides move 16 bytes a lane.  In 8-byte units:
 constexpr int kNatBlockUnits = 64 * 64 + 32;  // a block record: 32 KiB of partial outputs + 32 float2
 __host__ __device__ inline int nat_blocks(int head_k, int groups, int waves) { return head_k * groups * waves; }
 // start of the record of block blk, split s of sequence b
 __device__ __forceinline__ size_t nat_block(size_t b, int nsplit, int s, int nblk, int blk) {
     return ((b * nsplit + s) * nblk + blk) * (size_t)kNatBlockUnits;
 }
-// columns 4 c4 .. 4 c4 + 3 of row n, relative to the record's start
-__device__ __forceinline__ int nat_piece(int c4, int n) { return (c4 >> 1) * 64 + (c4 & 1) * 32 + n; }
+// columns 4 c4 .. 4 c4 + 3 of row n, relative to the record's start: column bits 5.. = c, 4 = rp, 3 = which half of
+// the lane's 16 bytes, 2 = half-wave
+__device__ __forceinline__ int nat_piece(int c4, int n) {
+    return ((c4 >> 2) * 64 + (c4 & 1) * 32 + n) * 2 + ((c4 >> 1) & 1);
+}
 // (m, l) of row n, relative to the record's start
 __device__ __forceinline__ int nat_ml(int n) { return 64 * 64 + n; }
 // bytes of one sequence split's records

@@ -599,15 +599,17 @@ __global__ __launch_bounds__(64 * NWV) void mfma_latent_kernel(const SweepParams
             uint8_t* const rec = reinterpret_cast<uint8_t*>(p.ws_o) +
                                  nat_block((size_t)b, p.nsplit, split, nat_blocks(p.head_k, p.groups, NWV),
                                            (hk * p.groups + grp) * NWV + wave) * 8;
-            typedef unsigned int u32x2 __attribute__((ext_vector_type(2)));
+            typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
 #pragma unroll
             for (int c = 0; c < CT; ++c)
 #pragma unroll
-                for (int r4 = 0; r4 < 4; ++r4) {
-                    u32x2 w;
-                    w.x = EL::pack2(acc[c][r4 * 4 + 0] * inv, acc[c][r4 * 4 + 1] * inv);
-                    w.y = EL::pack2(acc[c][r4 * 4 + 2] * inv, acc[c][r4 * 4 + 3] * inv);
-                    *reinterpret_cast<u32x2*>(rec + (c * 4 + r4) * 512 + lane * 8) = w;
+                for (int rp = 0; rp < 2; ++rp) {
+                    u32x4 w;
+                    w.x = EL::pack2(acc[c][rp * 8 + 0] * inv, acc[c][rp * 8 + 1] * inv);
+                    w.y = EL::pack2(acc[c][rp * 8 + 2] * inv, acc[c][rp * 8 + 3] * inv);
+                    w.z = EL::pack2(acc[c][rp * 8 + 4] * inv, acc[c][rp * 8 + 5] * inv);
+                    w.w = EL::pack2(acc[c][rp * 8 + 6] * inv, acc[c][rp * 8 + 7] * inv);
+                    *reinterpret_cast<u32x4*>(rec + (c * 2 + rp) * 1024 + lane * 16) = w;
                 }
             if (half == 0) reinterpret_cast<float2*>(rec)[nat_ml(n)] = make_float2(m, l_tot);
         } else {

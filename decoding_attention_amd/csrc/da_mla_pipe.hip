@@ -811,14 +811,15 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_num_vgpr(kScV))) void la
     // (ReduceParams::half_partials) beside the running maximum and the denominator as fp32.
     if (p.nsplit > 1) {
         // A split's partial leaves as it lies in the registers (nat_piece in da_common.h): lane (n, half) holds four
-        // columns of head n per 32 x 32 tile quarter, the wave stores 512 contiguous bytes per quarter, and the merge
-        // kernel reads in that order.  No trip through LDS and no barrier in the tail every work-group of a
+        // columns of head n per 32 x 32 tile quarter, the wave stores 1 KiB (two quarters, 16 bytes a lane) per
+        // instruction, and the merge kernel reads in that order.  No trip through LDS and no barrier in the tail every work-group of a
         // one-round grid runs at the same moment.
         const float inv = 1.0f / l_tot;
         const int blk = (hk * p.groups + grp) * NWV + wave;
         uint8_t* const rec = reinterpret_cast<uint8_t*>(p.ws_o) +
                              nat_block((size_t)b, p.nsplit, split, nat_blocks(p.head_k, p.groups, NWV), blk) * 8;
-        uint8_t* const dst = rec + lane * 8;
+        uint8_t* const dst = rec + lane * 16;
+        typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
         // (a whole 32 x 32 tile's sixteen values are read before any is converted: the reads are independent, and a
         // lone wave per SIMD has nothing else to cover the wait between a read and its use)
         static_for<0, CT>([&](auto cc) {
@@ -826,11 +827,13 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_num_vgpr(kScV))) void la
             float a[16];
             static_for<0, 16>([&](auto ic) { a[decltype(ic)::value] = acc_at(std::integral_constant<int, c * 16 + decltype(ic)::value>{}); });
 #pragma unroll
-            for (int r4 = 0; r4 < 4; ++r4) {
-                u32x2 w;
-                w.x = EL::pack2_scaled(a[r4 * 4 + 0], a[r4 * 4 + 1], inv);
-                w.y = EL::pack2_scaled(a[r4 * 4 + 2], a[r4 * 4 + 3], inv);
-                *reinterpret_cast<u32x2*>(dst + (c * 4 + r4) * 512) = w;
+            for (int rp = 0; rp < 2; ++rp) {
+                u32x4 w;
+                w.x = EL::pack2_scaled(a[rp * 8 + 0], a[rp * 8 + 1], inv);
+                w.y = EL::pack2_scaled(a[rp * 8 + 2], a[rp * 8 + 3], inv);
+                w.z = EL::pack2_scaled(a[rp * 8 + 4], a[rp * 8 + 5], inv);
+                w.w = EL::pack2_scaled(a[rp * 8 + 6], a[rp * 8 + 7], inv);
+                *reinterpret_cast<u32x4*>(dst + (c * 2 + rp) * 1024) = w;
             }
         });
         if (n < nh && half == 0) reinterpret_cast<float2*>(rec)[nat_ml(n)] = make_float2(m, l_tot);

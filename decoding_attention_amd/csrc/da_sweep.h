@@ -399,86 +399,98 @@ __global__ __launch_bounds__(256) void reduce_kernel(const ReduceParams p, int r
 }
 
 // The merge for normalised 16-bit partials (ReduceParams::half_partials, laid out as nat_piece says) in its
-// one-lane-per-element form: one thread per (sequence, query head, eight output columns), consecutive threads taking
-// consecutive heads of a block, so that a wave's loads are runs of 256 bytes; the partials of four splits are fetched
-// together.  A partial's weight is 2^(m_i - m) times its denominator l_i.  A work-group's 256 results are 32 rows x 128
-// bytes of the output: they change hands through LDS so that each row's 128 bytes leave as one run.
+// one-lane-per-element form.  Grid: x = sequence, y = 8 * (block of 32 heads within its KV head) + group of four runs,
+// z = KV head; thread (run, lane) takes the 16 bytes that lane of the sweep stored in that run of the block's record --
+// two groups of four columns of one head -- so a wave's loads are the run's contiguous KiB, one load per split.  With
+// eight waves to a SIMD at the benchmark's latent shape the kernel's time is its vector-instruction count (the first
+// version, with 600 of them, mostly index arithmetic, took 11 us for 44 MB): everything the work-group shares (record
+// addresses, the sequence's length, which splits exist) is scalar, and a value costs one mixed-precision multiply-add.
+// The first four splits are requested before the sequence's length is known (slots past the last split hold stale
+// data and are skipped).  A partial's weight is 2^(m_i - m) times its denominator l_i.  A work-group covers four runs,
+// i.e. 64 columns of the block's 32 rows: its results change hands through LDS so that each row's 128 bytes leave as
+// one run.
 template <typename Tag>
-__global__ __launch_bounds__(256) void reduce16_kernel(const ReduceParams p, int rows) {
+__global__ __launch_bounds__(256) void reduce16_kernel(const ReduceParams p) {
     using EL = Elem<Tag>;
-    __shared__ uint4 out_tile[32][9];  // (a pitch of nine 16-byte units: the rows' writes spread over the banks)
-    const long long gid = (long long)blockIdx.x * 256 + threadIdx.x;
-    const int n = (int)(gid & 31);        // row of the block
-    const int c8 = (int)(gid >> 5) & 63;  // eight columns
-    const long long bg = gid >> 11;       // sequence * blocks + block (the same for the whole work-group)
-    if (bg >= (long long)(rows / p.head_q) * p.nat_blocks) return;
-    const size_t b = (size_t)(bg / p.nat_blocks);
-    const int blk = (int)(bg % p.nat_blocks);
+    typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
+    __shared__ uint2 out_tile[32][18];  // (a pitch of nine 16-byte units: the rows' writes spread over the banks)
+    const int b = (int)blockIdx.x, bpk = (int)blockIdx.y >> 3, rg = (int)blockIdx.y & 7, hk = (int)blockIdx.z;
     const int per_kv = p.groups * p.nat_waves;
-    const int hr0 = (blk % per_kv) * 32;  // first head of the block within its KV head's group of `ratio`
-    const int row0 = (int)b * p.head_q + (blk / per_kv) * p.ratio + hr0;
-    uint4 r = make_uint4(0u, 0u, 0u, 0u);
-    if (hr0 + n < p.ratio) {  // (else a dead row of the group's last block)
-        const uint2* const src = reinterpret_cast<const uint2*>(p.ws_o);
+    const int hr0 = bpk * 32;                   // first head of the block within its KV head's group of `ratio`
+    const int live = min(32, p.ratio - hr0);    // live rows of the block
+    const size_t row0 = (size_t)b * p.head_q + (size_t)hk * p.ratio + hr0;
+    const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
+    const int n = lane & 31, half = lane >> 5;  // row of the block, half-wave of the storing lane
+    constexpr size_t kRec = (size_t)kNatBlockUnits * 8;
+    const uint8_t* const rec0 =
+        reinterpret_cast<const uint8_t*>(p.ws_o) + ((size_t)b * p.nsplit * p.nat_blocks + (size_t)(hk * per_kv + bpk)) * kRec;
+    const size_t sstride = (size_t)p.nat_blocks * kRec;  // from one split's record to the next
+    const uint32_t xoff = (uint32_t)rg * 4096u + threadIdx.x * 16u;
+    const uint32_t eoff = (uint32_t)(64 * 64 * 8) + (uint32_t)n * 8u;
+    uint2 r0 = make_uint2(0u, 0u), r1 = make_uint2(0u, 0u);
+    if (n < live) {  // (else a dead row of the group's last block)
         float2 e[4];
-        uint4 x[4];
-        auto fetch = [&](int s0, int last) {
+        u32x4 x[4];
+        auto fetch = [&](int s0) {
 #pragma unroll
             for (int u = 0; u < 4; ++u) {
-                const int s = min(s0 + u, last);
-                const uint2* const rec = src + nat_block(b, p.nsplit, s, p.nat_blocks, blk);
-                e[u] = reinterpret_cast<const float2*>(rec)[nat_ml(n)];
-                // columns 8 c8 .. + 3 lie with lane n of the storing wave, + 4 .. + 7 with lane 32 + n
-                const uint2 lo = rec[nat_piece(2 * c8, n)], hi = rec[nat_piece(2 * c8, n) + 32];
-                x[u] = make_uint4(lo.x, lo.y, hi.x, hi.y);
+                const uint8_t* const rec = rec0 + (size_t)min(s0 + u, p.nsplit - 1) * sstride;
+                e[u] = *reinterpret_cast<const float2*>(rec + eoff);
+                // (read once: non-temporal, like the K/V streams)
+                x[u] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(rec + xoff));
             }
         };
-        if (p.early) fetch(0, p.nsplit - 1);
+        fetch(0);
         const int len = p.cu_seq_k ? p.cu_seq_k[b + 1] - p.cu_seq_k[b] : p.seq_lens[b];
-        const int ns = len > 0 ? min(p.nsplit, (len + p.chunk - 1) / p.chunk) : 0;
         float mm = kNegBig, den = 0.0f;
         float num[8];
 #pragma unroll
         for (int j = 0; j < 8; ++j) num[j] = 0.0f;
-        for (int s0 = 0; s0 < ns; s0 += 4) {
-            if (!p.early || s0 != 0) fetch(s0, ns - 1);
+        // split s exists when s < nsplit and s * chunk < len (all scalar)
+        for (int s0 = 0; s0 < p.nsplit && (long long)s0 * p.chunk < len; s0 += 4) {
+            if (s0 != 0) fetch(s0);
+            bool valid[4];
+#pragma unroll
+            for (int u = 0; u < 4; ++u) valid[u] = s0 + u < p.nsplit && (long long)(s0 + u) * p.chunk < len;
             float m_new = mm;
 #pragma unroll
             for (int u = 0; u < 4; ++u)
-                if (s0 + u < ns) m_new = fmaxf(m_new, e[u].x);
-            const float keep = fast_exp2(mm - m_new);  // 0 on the first round
-            mm = m_new;
-            den *= keep;
+                if (valid[u]) m_new = fmaxf(m_new, e[u].x);
+            if (s0 != 0) {
+                const float keep = fast_exp2(mm - m_new);
+                den *= keep;
 #pragma unroll
-            for (int j = 0; j < 8; ++j) num[j] *= keep;
+                for (int j = 0; j < 8; ++j) num[j] *= keep;
+            }
+            mm = m_new;
 #pragma unroll
             for (int u = 0; u < 4; ++u) {
-                const float w = s0 + u < ns ? fast_exp2(e[u].x - mm) * e[u].y : 0.0f;
+                if (!valid[u]) continue;  // (a slot past the sequence's last split holds stale data, possibly NaN)
+                const float w = fast_exp2(e[u].x - mm) * e[u].y;
                 den += w;
                 const uint32_t h[4] = {x[u].x, x[u].y, x[u].z, x[u].w};
 #pragma unroll
                 for (int j = 0; j < 4; ++j) {
-                    // (a slot past the sequence's last split holds stale data, possibly NaN: select, do not multiply by 0)
-                    num[2 * j] += s0 + u < ns ? w * EL::lo(h[j]) : 0.0f;
-                    num[2 * j + 1] += s0 + u < ns ? w * EL::hi(h[j]) : 0.0f;
+                    num[2 * j] = __builtin_fmaf(w, EL::lo(h[j]), num[2 * j]);
+                    num[2 * j + 1] = __builtin_fmaf(w, EL::hi(h[j]), num[2 * j + 1]);
                 }
             }
         }
-        const float inv = ns > 0 ? 1.0f / den : 0.0f;  // an empty sequence yields a zero row
-        r.x = EL::pack2(num[0] * inv, num[1] * inv);
-        r.y = EL::pack2(num[2] * inv, num[3] * inv);
-        r.z = EL::pack2(num[4] * inv, num[5] * inv);
-        r.w = EL::pack2(num[6] * inv, num[7] * inv);
+        // (the hardware reciprocal, 1 ulp: far below the 16-bit rounding that follows)
+        const float inv = len > 0 ? __builtin_amdgcn_rcpf(den) : 0.0f;  // an empty sequence yields a zero row
+        r0 = make_uint2(EL::pack2(num[0] * inv, num[1] * inv), EL::pack2(num[2] * inv, num[3] * inv));
+        r1 = make_uint2(EL::pack2(num[4] * inv, num[5] * inv), EL::pack2(num[6] * inv, num[7] * inv));
     }
-    // thread (n, j) holds columns 8 (c0 + j) .. + 7 of row n, c0 the work-group's first column group; thread t sends off
-    // piece t % 8 of row t / 8
-    out_tile[n][threadIdx.x >> 5] = r;
+    // thread (wave wv, lane (n, half)) holds columns 32 (wv / 2) + 16 (wv % 2) + 4 half .. + 3 and the same + 8 of row n,
+    // relative to the work-group's first column; thread t sends off 16-byte piece t % 8 of row t / 8
+    const int u0 = (wv >> 1) * 4 + (wv & 1) * 2;
+    out_tile[n][u0 * 2 + half] = r0;
+    out_tile[n][u0 * 2 + 2 + half] = r1;
     __syncthreads();
     const int n2 = threadIdx.x >> 3, seg = threadIdx.x & 7;
-    if (hr0 + n2 < p.ratio) {
-        const int c0 = (int)((gid - threadIdx.x) >> 5) & 63;
-        *reinterpret_cast<uint4*>(reinterpret_cast<uint16_t*>(p.o) + (size_t)(row0 + n2) * p.dim_v + (c0 + seg) * 8) =
-            out_tile[n2][seg];
+    if (n2 < live) {
+        const uint4 v = *reinterpret_cast<const uint4*>(&out_tile[n2][seg * 2]);
+        *reinterpret_cast<uint4*>(reinterpret_cast<uint16_t*>(p.o) + (row0 + n2) * p.dim_v + rg * 64 + seg * 8) = v;
     }
 }
 

@@ -35,12 +35,13 @@ hipError_t launch_reduce(const ReduceParams& p, bool is_bf16, int blocks, hipStr
     if (p.half_partials && (p.dim_v != 512 || p.flat_tokens != 0 || p.nat_blocks <= 0 || p.head_q <= 0))
         return hipErrorInvalidValue;
     if (p.half_partials && sg == 1) {
-        const long long units = (long long)(blocks / p.head_q) * p.nat_blocks * 32 * (p.dim_v / 8);
-        const dim3 grid((unsigned)((units + 255) / 256));
+        const int per_kv = p.groups * p.nat_waves, head_k = p.nat_blocks / per_kv;
+        if (8 * per_kv > 65535 || head_k > 65535) return hipErrorInvalidValue;
+        const dim3 grid((unsigned)(blocks / p.head_q), (unsigned)(8 * per_kv), (unsigned)head_k);
         if (is_bf16)
-            hipLaunchKernelGGL((reduce16_kernel<bf16_tag>), grid, dim3(256), 0, stream, p, blocks);
+            hipLaunchKernelGGL((reduce16_kernel<bf16_tag>), grid, dim3(256), 0, stream, p);
         else
-            hipLaunchKernelGGL((reduce16_kernel<f16_tag>), grid, dim3(256), 0, stream, p, blocks);
+            hipLaunchKernelGGL((reduce16_kernel<f16_tag>), grid, dim3(256), 0, stream, p);
         return hipGetLastError();
     }
     switch (sg) {
