@@ -141,7 +141,16 @@ def measure(torch, w, steps, warmup, page_size=0, kv_fp8=False, kv_int8=False, k
         nbytes = wl.algorithmic_bytes(w.batch, w.head_q, w.head_k, w.dim, w.dim_v, int(w.k.shape[0]), w.v is not None,
                                       elem_bytes=2) - (kv_elems * 3 // 2 if kv_int4 else kv_elems)
     flops = wl.workload_flops(w)
-    plan = _lib.plan(w.max_seq_k, w.batch, w.head_q, w.head_k, w.dim, w.dim_v, total_k=int(w.k.shape[0]))
+    # the plan of the call that was timed: a V buffer of its own and the page size change it; the 8-bit and 4-bit
+    # formats are planned by rules of their own that the library has no query for (None)
+    plan = None
+    if not (kv_fp8 or kv_int8 or kv_int4):
+        distinct = w.v is not None and w.dim != w.dim_v
+        if distinct or page_size:
+            plan = _lib.plan(w.max_seq_k, w.batch, w.head_q, w.head_k, w.dim, w.dim_v, total_k=int(w.k.shape[0]),
+                             distinct_v=True, page_size=page_size) if distinct else None
+        else:
+            plan = _lib.plan(w.max_seq_k, w.batch, w.head_q, w.head_k, w.dim, w.dim_v, total_k=int(w.k.shape[0]))
     return {
         "workload": w.name,
         "us_per_call": mean_ms * 1e3,

@@ -87,6 +87,9 @@ constexpr int kKindSweep = 1;
 constexpr int kKindMfma = 2;
 constexpr int kKindGroup = 3;
 constexpr int kMaxSplits = 256;
+// most sequences of one launch (a grid axis ends at 65535; a multiple of eight, so that the kernels' renumbering of
+// work-groups over the eight XCDs stays on); larger batches run as several launches
+constexpr size_t kMaxGridBatch = 65528;
 
 struct Plan {
     int kind = 0;
@@ -391,6 +394,21 @@ Plan make_plan(size_t max_seq_k, size_t batch, size_t head_q, size_t head_k, siz
     return pl;
 }
 
+// Workspace bytes of a call: the plan's, or, for a batch beyond one launch (kMaxGridBatch), the largest of its runs'.
+size_t plan_ws_bytes(size_t max_seq_k, size_t batch, size_t head_q, size_t head_k, size_t dim, size_t dim_v,
+                     bool v_distinct, size_t total_k, size_t page_size = 0, bool kv_8bit = false,
+                     bool no_latent_kernel = false) {
+    if (batch <= kMaxGridBatch)
+        return make_plan(max_seq_k, batch, head_q, head_k, dim, dim_v, v_distinct, total_k, page_size, kv_8bit,
+                         no_latent_kernel).ws_bytes;
+    size_t need = make_plan(max_seq_k, kMaxGridBatch, head_q, head_k, dim, dim_v, v_distinct, 0, page_size, kv_8bit,
+                            no_latent_kernel).ws_bytes;
+    if (batch % kMaxGridBatch != 0)
+        need = std::max(need, make_plan(max_seq_k, batch % kMaxGridBatch, head_q, head_k, dim, dim_v, v_distinct, 0,
+                                        page_size, kv_8bit, no_latent_kernel).ws_bytes);
+    return need;
+}
+
 struct CachedWs {
     void* ptr = nullptr;
     size_t bytes = 0;
@@ -533,24 +551,24 @@ int da_plan_distinct_v(size_t max_seq_k, size_t batch, size_t head_q, size_t hea
 size_t da_workspace_bytes(size_t max_seq_k, size_t batch, size_t head_q, size_t head_k, size_t dim, size_t dim_v,
                           size_t total_k) {
     if (head_k == 0 || head_q % head_k != 0 || !supported_dims(dim, dim_v)) return 0;
-    const size_t a = make_plan(max_seq_k, batch, head_q, head_k, dim, dim_v, false, total_k).ws_bytes;
-    const size_t b = make_plan(max_seq_k, batch, head_q, head_k, dim, dim_v, true, total_k).ws_bytes;
+    const size_t a = plan_ws_bytes(max_seq_k, batch, head_q, head_k, dim, dim_v, false, total_k);
+    const size_t b = plan_ws_bytes(max_seq_k, batch, head_q, head_k, dim, dim_v, true, total_k);
     return a > b ? a : b;
 }
 
 size_t da_workspace_bytes_paged(size_t max_seq_k, size_t batch, size_t head_q, size_t head_k, size_t dim, size_t dim_v,
                                 size_t total_k, size_t page_size) {
     if (head_k == 0 || head_q % head_k != 0 || !supported_dims(dim, dim_v)) return 0;
-    const size_t a = make_plan(max_seq_k, batch, head_q, head_k, dim, dim_v, false, total_k, page_size, false).ws_bytes;
-    const size_t b = make_plan(max_seq_k, batch, head_q, head_k, dim, dim_v, true, total_k, page_size, false).ws_bytes;
+    const size_t a = plan_ws_bytes(max_seq_k, batch, head_q, head_k, dim, dim_v, false, total_k, page_size, false);
+    const size_t b = plan_ws_bytes(max_seq_k, batch, head_q, head_k, dim, dim_v, true, total_k, page_size, false);
     return a > b ? a : b;
 }
 
 size_t da_workspace_bytes_fp8kv(size_t max_seq_k, size_t batch, size_t head_q, size_t head_k, size_t dim,
                                 size_t dim_v, size_t total_k, size_t page_size) {
     if (head_k == 0 || head_q % head_k != 0 || !supported_dims(dim, dim_v)) return 0;
-    const size_t a = make_plan(max_seq_k, batch, head_q, head_k, dim, dim_v, false, total_k, page_size, true).ws_bytes;
-    const size_t b = make_plan(max_seq_k, batch, head_q, head_k, dim, dim_v, true, total_k, page_size, true).ws_bytes;
+    const size_t a = plan_ws_bytes(max_seq_k, batch, head_q, head_k, dim, dim_v, false, total_k, page_size, true);
+    const size_t b = plan_ws_bytes(max_seq_k, batch, head_q, head_k, dim, dim_v, true, total_k, page_size, true);
     return a > b ? a : b;
 }
 
@@ -610,10 +628,32 @@ int run_attention(const void* q, const void* k, const void* v, void* o, const in
         return fail(DA_ERR_INVALID_ARGUMENT, "q, k and v must be 16-byte aligned");
     // (every finishing path stores 8 or 16 bytes of a row at a time; rows are multiples of 128 bytes)
     if (!aligned16(o)) return fail(DA_ERR_INVALID_ARGUMENT, "o must be 16-byte aligned");
-    if (max_seq_k > (size_t)INT32_MAX || batch > 65535 || head_q > 65535)
-        return fail(DA_ERR_INVALID_ARGUMENT, "shape out of range (max_seq_k %zu, batch %zu, head_q %zu; grid limit 65535)",
-                    max_seq_k, batch, head_q);
+    if (max_seq_k > (size_t)INT32_MAX || batch > (size_t)INT32_MAX || head_q > 65535)
+        return fail(DA_ERR_INVALID_ARGUMENT, "shape out of range (max_seq_k %zu, batch %zu, head_q %zu)", max_seq_k, batch,
+                    head_q);
     if (batch == 0) return DA_OK;
+    if (batch > kMaxGridBatch) {
+        // The kernels number the sequences along a grid axis that ends at 65535 (the reference numbers them along
+        // grid.x, csrc/kernel/decoding_attn/decoding_fwd_launch_template.h:18, and has no such limit): a larger batch
+        // runs as consecutive launches over runs of sequences.  q, o, cu_seq_k and the block table move on with the
+        // run; packed K/V stay, cu_seq_k holds absolute rows.  The runs share the workspace: they follow each other
+        // on the stream.  (total_k is the whole batch's: the runs are planned without it.)
+        for (size_t b0 = 0; b0 < batch; b0 += kMaxGridBatch) {
+            const size_t nb = std::min(kMaxGridBatch, batch - b0);
+            Paging pgr = pg;
+            if (pg.table) {
+                pgr.table = pg.table + b0 * pg.max_blocks;
+                pgr.seq_lens = pg.seq_lens + b0;
+            }
+            const int rc = run_attention(static_cast<const uint8_t*>(q) + b0 * head_q * dim * 2, k, v,
+                                         static_cast<uint8_t*>(o) + b0 * head_q * dim_v * 2,
+                                         cu_seq_k ? cu_seq_k + b0 : nullptr, pgr, kf, max_seq_k, nb, head_q, head_k, dim,
+                                         dim_v, is_alibi, is_bf16, softmax_scale, alibi_slopes, 0, workspace,
+                                         workspace_bytes, hip_stream);
+            if (rc != DA_OK) return rc;
+        }
+        return DA_OK;
+    }
 
     hipStream_t stream = reinterpret_cast<hipStream_t>(hip_stream);
     const Plan pl = make_plan(max_seq_k, batch, head_q, head_k, dim, dim_v, v != nullptr, total_k,
@@ -918,8 +958,8 @@ size_t da_workspace_bytes_int4kv(size_t max_seq_k, size_t batch, size_t head_q, 
                                  size_t dim_v, size_t total_k, size_t page_size) {
     if (head_k == 0 || head_q % head_k != 0 || !supported_dims(dim, dim_v)) return 0;
     // (as the FP8 cache's plans, but the latent form always on the grouped kernel)
-    const size_t a = make_plan(max_seq_k, batch, head_q, head_k, dim, dim_v, false, total_k, page_size, true, true).ws_bytes;
-    const size_t b = make_plan(max_seq_k, batch, head_q, head_k, dim, dim_v, true, total_k, page_size, true, true).ws_bytes;
+    const size_t a = plan_ws_bytes(max_seq_k, batch, head_q, head_k, dim, dim_v, false, total_k, page_size, true, true);
+    const size_t b = plan_ws_bytes(max_seq_k, batch, head_q, head_k, dim, dim_v, true, total_k, page_size, true, true);
     return a > b ? a : b;
 }
 
@@ -934,12 +974,12 @@ int da_decoding_attn_noalloc(const void* q, const void* k, const void* v, void* 
     // the split partials go to the static device array; a plan that needs more than it holds is refused here, with
     // the numbers, before anything is enqueued (the remaining argument checks are run_attention's)
     if (head_k != 0 && head_q % head_k == 0 && supported_dims(dim, dim_v) && batch > 0) {
-        const Plan pl = make_plan(max_seq_k, batch, head_q, head_k, dim, dim_v, v != nullptr, total_k);
-        if (pl.ws_bytes > kScratchBytes)
+        const size_t need = plan_ws_bytes(max_seq_k, batch, head_q, head_k, dim, dim_v, v != nullptr, total_k);
+        if (need > kScratchBytes)
             return fail(DA_ERR_WORKSPACE,
                         "this shape needs %zu bytes of split workspace, more than the %zu bytes of the static array "
                         "da_decoding_attn_noalloc works in; use da_decoding_attn_ex with a workspace of your own",
-                        pl.ws_bytes, kScratchBytes);
+                        need, kScratchBytes);
     }
     void* ws = nullptr;
     const int rc = scratch_on_current_device(&ws);

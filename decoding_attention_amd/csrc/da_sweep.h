@@ -409,12 +409,14 @@ __global__ __launch_bounds__(256) void reduce_kernel(const ReduceParams p, int r
 // data and are skipped).  A partial's weight is 2^(m_i - m) times its denominator l_i.  A work-group covers four runs,
 // i.e. 64 columns of the block's 32 rows: its results change hands through LDS so that each row's 128 bytes leave as
 // one run.
+constexpr int kReduce16Runs = 1;  // runs of a block record per thread (two: no faster, measured)
 template <typename Tag>
 __global__ __launch_bounds__(256) void reduce16_kernel(const ReduceParams p) {
     using EL = Elem<Tag>;
     typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
-    __shared__ uint2 out_tile[32][18];  // (a pitch of nine 16-byte units: the rows' writes spread over the banks)
-    const int b = (int)blockIdx.x, bpk = (int)blockIdx.y >> 3, rg = (int)blockIdx.y & 7, hk = (int)blockIdx.z;
+    constexpr int NR = kReduce16Runs, NG = 8 / NR;  // NG: groups of four runs along grid y
+    __shared__ uint2 out_tile[NR][32][18];  // (a pitch of nine 16-byte units: the rows' writes spread over the banks)
+    const int b = (int)blockIdx.x, bpk = (int)blockIdx.y / NG, rg = (int)blockIdx.y % NG, hk = (int)blockIdx.z;
     const int per_kv = p.groups * p.nat_waves;
     const int hr0 = bpk * 32;                   // first head of the block within its KV head's group of `ratio`
     const int live = min(32, p.ratio - hr0);    // live rows of the block
@@ -425,27 +427,34 @@ __global__ __launch_bounds__(256) void reduce16_kernel(const ReduceParams p) {
     const uint8_t* const rec0 =
         reinterpret_cast<const uint8_t*>(p.ws_o) + ((size_t)b * p.nsplit * p.nat_blocks + (size_t)(hk * per_kv + bpk)) * kRec;
     const size_t sstride = (size_t)p.nat_blocks * kRec;  // from one split's record to the next
+    // this thread's runs: 4 (rg + NG i) + wv, i < NR (the work-group's i-th four runs: columns 64 (rg + NG i) .. + 63)
     const uint32_t xoff = (uint32_t)rg * 4096u + threadIdx.x * 16u;
     const uint32_t eoff = (uint32_t)(64 * 64 * 8) + (uint32_t)n * 8u;
-    uint2 r0 = make_uint2(0u, 0u), r1 = make_uint2(0u, 0u);
+    uint2 r[NR][2];
+#pragma unroll
+    for (int i = 0; i < NR; ++i) r[i][0] = r[i][1] = make_uint2(0u, 0u);
     if (n < live) {  // (else a dead row of the group's last block)
         float2 e[4];
-        u32x4 x[4];
+        u32x4 x[NR][4];
         auto fetch = [&](int s0) {
 #pragma unroll
             for (int u = 0; u < 4; ++u) {
                 const uint8_t* const rec = rec0 + (size_t)min(s0 + u, p.nsplit - 1) * sstride;
                 e[u] = *reinterpret_cast<const float2*>(rec + eoff);
                 // (read once: non-temporal, like the K/V streams)
-                x[u] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(rec + xoff));
+#pragma unroll
+                for (int i = 0; i < NR; ++i)
+                    x[i][u] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(rec + xoff + i * NG * 4096));
             }
         };
         fetch(0);
         const int len = p.cu_seq_k ? p.cu_seq_k[b + 1] - p.cu_seq_k[b] : p.seq_lens[b];
         float mm = kNegBig, den = 0.0f;
-        float num[8];
+        float num[NR][8];
 #pragma unroll
-        for (int j = 0; j < 8; ++j) num[j] = 0.0f;
+        for (int i = 0; i < NR; ++i)
+#pragma unroll
+            for (int j = 0; j < 8; ++j) num[i][j] = 0.0f;
         // split s exists when s < nsplit and s * chunk < len (all scalar)
         for (int s0 = 0; s0 < p.nsplit && (long long)s0 * p.chunk < len; s0 += 4) {
             if (s0 != 0) fetch(s0);
@@ -460,7 +469,9 @@ __global__ __launch_bounds__(256) void reduce16_kernel(const ReduceParams p) {
                 const float keep = fast_exp2(mm - m_new);
                 den *= keep;
 #pragma unroll
-                for (int j = 0; j < 8; ++j) num[j] *= keep;
+                for (int i = 0; i < NR; ++i)
+#pragma unroll
+                    for (int j = 0; j < 8; ++j) num[i][j] *= keep;
             }
             mm = m_new;
 #pragma unroll
@@ -468,29 +479,40 @@ __global__ __launch_bounds__(256) void reduce16_kernel(const ReduceParams p) {
                 if (!valid[u]) continue;  // (a slot past the sequence's last split holds stale data, possibly NaN)
                 const float w = fast_exp2(e[u].x - mm) * e[u].y;
                 den += w;
-                const uint32_t h[4] = {x[u].x, x[u].y, x[u].z, x[u].w};
 #pragma unroll
-                for (int j = 0; j < 4; ++j) {
-                    num[2 * j] = __builtin_fmaf(w, EL::lo(h[j]), num[2 * j]);
-                    num[2 * j + 1] = __builtin_fmaf(w, EL::hi(h[j]), num[2 * j + 1]);
+                for (int i = 0; i < NR; ++i) {
+                    const uint32_t h[4] = {x[i][u].x, x[i][u].y, x[i][u].z, x[i][u].w};
+#pragma unroll
+                    for (int j = 0; j < 4; ++j) {
+                        num[i][2 * j] = __builtin_fmaf(w, EL::lo(h[j]), num[i][2 * j]);
+                        num[i][2 * j + 1] = __builtin_fmaf(w, EL::hi(h[j]), num[i][2 * j + 1]);
+                    }
                 }
             }
         }
         // (the hardware reciprocal, 1 ulp: far below the 16-bit rounding that follows)
         const float inv = len > 0 ? __builtin_amdgcn_rcpf(den) : 0.0f;  // an empty sequence yields a zero row
-        r0 = make_uint2(EL::pack2(num[0] * inv, num[1] * inv), EL::pack2(num[2] * inv, num[3] * inv));
-        r1 = make_uint2(EL::pack2(num[4] * inv, num[5] * inv), EL::pack2(num[6] * inv, num[7] * inv));
+#pragma unroll
+        for (int i = 0; i < NR; ++i) {
+            r[i][0] = make_uint2(EL::pack2(num[i][0] * inv, num[i][1] * inv), EL::pack2(num[i][2] * inv, num[i][3] * inv));
+            r[i][1] = make_uint2(EL::pack2(num[i][4] * inv, num[i][5] * inv), EL::pack2(num[i][6] * inv, num[i][7] * inv));
+        }
     }
     // thread (wave wv, lane (n, half)) holds columns 32 (wv / 2) + 16 (wv % 2) + 4 half .. + 3 and the same + 8 of row n,
-    // relative to the work-group's first column; thread t sends off 16-byte piece t % 8 of row t / 8
+    // relative to the first column of its four runs; thread t sends off 16-byte piece t % 8 of row t / 8
     const int u0 = (wv >> 1) * 4 + (wv & 1) * 2;
-    out_tile[n][u0 * 2 + half] = r0;
-    out_tile[n][u0 * 2 + 2 + half] = r1;
+#pragma unroll
+    for (int i = 0; i < NR; ++i) {
+        out_tile[i][n][u0 * 2 + half] = r[i][0];
+        out_tile[i][n][u0 * 2 + 2 + half] = r[i][1];
+    }
     __syncthreads();
     const int n2 = threadIdx.x >> 3, seg = threadIdx.x & 7;
     if (n2 < live) {
-        const uint4 v = *reinterpret_cast<const uint4*>(&out_tile[n2][seg * 2]);
-        *reinterpret_cast<uint4*>(reinterpret_cast<uint16_t*>(p.o) + (row0 + n2) * p.dim_v + rg * 64 + seg * 8) = v;
+        uint16_t* const orow = reinterpret_cast<uint16_t*>(p.o) + (row0 + n2) * p.dim_v + rg * 64 + seg * 8;
+#pragma unroll
+        for (int i = 0; i < NR; ++i)
+            *reinterpret_cast<uint4*>(orow + i * NG * 64) = *reinterpret_cast<const uint4*>(&out_tile[i][n2][seg * 2]);
     }
 }
 

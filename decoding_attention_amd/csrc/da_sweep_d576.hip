@@ -36,8 +36,9 @@ hipError_t launch_reduce(const ReduceParams& p, bool is_bf16, int blocks, hipStr
         return hipErrorInvalidValue;
     if (p.half_partials && sg == 1) {
         const int per_kv = p.groups * p.nat_waves, head_k = p.nat_blocks / per_kv;
-        if (8 * per_kv > 65535 || head_k > 65535) return hipErrorInvalidValue;
-        const dim3 grid((unsigned)(blocks / p.head_q), (unsigned)(8 * per_kv), (unsigned)head_k);
+        constexpr int ny = 8 / kReduce16Runs;  // work-groups per block of 32 heads
+        if (ny * per_kv > 65535 || head_k > 65535) return hipErrorInvalidValue;
+        const dim3 grid((unsigned)(blocks / p.head_q), (unsigned)(ny * per_kv), (unsigned)head_k);
         if (is_bf16)
             hipLaunchKernelGGL((reduce16_kernel<bf16_tag>), grid, dim3(256), 0, stream, p);
         else

@@ -76,7 +76,9 @@ int da_release_workspaces(void);
  * da_noalloc_workspace_limit() bytes (80 MiB) that every GPU the library is loaded on holds until the process ends;
  * the call allocates nothing, on the device or through any library, and returns DA_ERR_WORKSPACE (nothing enqueued)
  * for a shape whose plan needs more.  All calls on one GPU share that array: calls that overlap on one GPU (two
- * streams, two threads) race on it; calls on one stream do not.
+ * streams, two threads) race on it; calls on one stream do not.  The first call for a shape on a device looks up the
+ * array's address there and raises the chosen kernel's LDS limit: make one warm-up call per shape and device outside
+ * any graph capture; every later call only enqueues kernels.
  */
 int da_decoding_attn_noalloc(const void *q, const void *k, const void *v, void *o, const int32_t *cu_seq_k,
                              size_t max_seq_k, size_t batch, size_t head_q, size_t head_k, size_t dim, size_t dim_v,

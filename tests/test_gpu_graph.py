@@ -90,3 +90,62 @@ def test_fp8_latent_and_16_token_pages_replay_from_a_graph():
         return decoding_attn_paged_fwd(q2, pk.k_pages, pk.v_pages, pk.block_table, pk.seq_lens, w2.max_seq_k, 128, False)
 
     _replay_matches_eager(run_paged, [q2, pk.k_pages, pk.v_pages], lambda o: o)
+
+
+def test_noalloc_entry_point_under_capture_and_without_allocation():
+    """da_decoding_attn_noalloc, the entry point for callers that cannot allocate: after one warm-up call per shape (the
+    first call on a device looks up the static array's address and raises the kernels' LDS limits, neither of which
+    belongs inside a capture) it is captured, replayed on changed inputs and compared with da_decoding_attn_ex bit for
+    bit; and steady-state calls leave the device's free memory where it was."""
+    from decoding_attention_amd import _lib
+
+    lib = _lib.load()
+    for w in (wl.make_workload(8, 32, 8, 128, 128, 2048, torch.bfloat16, seed=11), wl.config_mla(4, 700, seed=12)):
+        wd = w.to(DEV)
+        b, hq, d = w.q.shape
+        hk, total_k = w.k.shape[1], w.k.shape[0]
+        bf16 = int(w.q.dtype == torch.bfloat16)
+        v_ptr = None if wd.v is None else wd.v.data_ptr()
+        o = torch.zeros((b, hq, w.dim_v), dtype=w.q.dtype, device=DEV)
+        o_ex = torch.zeros_like(o)
+        n = lib.da_workspace_bytes(w.max_seq_k, b, hq, hk, d, w.dim_v, total_k)
+        ws = torch.empty(max(n, 16), dtype=torch.uint8, device=DEV)
+
+        def noalloc():
+            rc = lib.da_decoding_attn_noalloc(wd.q.data_ptr(), wd.k.data_ptr(), v_ptr, o.data_ptr(),
+                                              wd.cu_seq_k.data_ptr(), w.max_seq_k, b, hq, hk, d, w.dim_v,
+                                              int(w.is_alibi), bf16, 0.0, None, total_k,
+                                              torch.cuda.current_stream().cuda_stream)
+            assert rc == 0, _lib.last_error()
+
+        def ex():
+            rc = lib.da_decoding_attn_ex(wd.q.data_ptr(), wd.k.data_ptr(), v_ptr, o_ex.data_ptr(),
+                                         wd.cu_seq_k.data_ptr(), w.max_seq_k, b, hq, hk, d, w.dim_v, int(w.is_alibi),
+                                         bf16, 0.0, None, total_k, ws.data_ptr(), n,
+                                         torch.cuda.current_stream().cuda_stream)
+            assert rc == 0, _lib.last_error()
+
+        s = torch.cuda.Stream()
+        s.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(s):
+            noalloc()  # the warm-up call, outside the capture
+        torch.cuda.current_stream().wait_stream(s)
+        torch.cuda.synchronize()
+        free0 = torch.cuda.mem_get_info()[0]
+        for _ in range(5):
+            noalloc()
+        torch.cuda.synchronize()
+        assert torch.cuda.mem_get_info()[0] == free0, "steady-state calls changed the device's free memory"
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            noalloc()
+        torch.cuda.synchronize()
+        g = torch.Generator(device="cpu").manual_seed(2)
+        for step in range(3):
+            for t in [wd.q, wd.k] + ([] if wd.v is None else [wd.v]):
+                t.copy_(torch.randn(t.shape, generator=g).to(t.dtype))
+            o.zero_()
+            graph.replay()
+            ex()
+            torch.cuda.synchronize()
+            assert torch.equal(o.view(torch.int16), o_ex.view(torch.int16)), f"{w.name} replay {step}"

@@ -47,3 +47,55 @@ def test_offsets_beyond_4_gib(kind):
     # first, last, and the sequences on either side of the 4 GiB byte offset
     edge = (1 << 32) // (sk * hk * d * 2)
     _check_rows(q, k, v, cu, o, [0, edge - 1, edge, edge + 1, batch - 1], dv, "large_" + kind)
+
+
+@pytest.mark.parametrize("kind", ["mha_ragged", "gqa_paged"])
+def test_batch_beyond_one_grid_axis(kind):
+    """70 000 sequences, more than a grid axis numbers (65 535; the reference numbers sequences along grid.x and has no
+    such limit, csrc/kernel/decoding_attn/decoding_fwd_launch_template.h:18): the call runs as two launches.  Every row
+    finite, rows on both sides of the seam and at both ends against the oracle; packed ragged MHA and paged GQA."""
+    from decoding_attention_amd import decoding_attn_paged_fwd
+
+    g = torch.Generator(device="cpu").manual_seed(9)
+    batch = 70000
+    seam = 65528
+    rows = [0, 1, seam - 1, seam, seam + 1, batch - 1]
+    if kind == "mha_ragged":
+        hq, hk, d, sk, dtype = 8, 8, 64, 24, torch.float16
+        lens = torch.randint(0, sk + 1, (batch,), generator=g, dtype=torch.int32)
+        lens[seam] = sk
+        cu = wl.get_cu_seq(lens)
+        total = int(cu[-1])
+        gd = torch.Generator(device=DEV).manual_seed(9)
+        q = torch.randn(batch, hq, d, generator=gd, device=DEV, dtype=dtype)
+        k = torch.randn(total, hk, d, generator=gd, device=DEV, dtype=dtype)
+        v = torch.randn(total, hk, d, generator=gd, device=DEV, dtype=dtype)
+        o = decoding_attn_fwd(q, k, v, cu.to(DEV), sk, d, False)
+        torch.cuda.synchronize()
+        assert torch.isfinite(o.float()).all()
+        assert (o[lens.to(DEV) == 0] == 0).all()  # empty sequences: zero rows
+        rows = [b for b in rows if lens[b] > 0]
+        _check_rows(q, k, v, cu, o, rows, d, "batch70000_mha")
+    else:
+        hq, hk, d, sk, dtype, page = 16, 4, 128, 40, torch.bfloat16, 16
+        lens = torch.randint(1, sk + 1, (batch,), generator=g, dtype=torch.int32)
+        max_blocks = (sk + page - 1) // page
+        npages = batch * max_blocks
+        gd = torch.Generator(device=DEV).manual_seed(10)
+        q = torch.randn(batch, hq, d, generator=gd, device=DEV, dtype=dtype)
+        k_pages = torch.randn(npages, page, hk, d, generator=gd, device=DEV, dtype=dtype)
+        v_pages = torch.randn(npages, page, hk, d, generator=gd, device=DEV, dtype=dtype)
+        table = torch.randperm(npages, generator=g).to(torch.int32).reshape(batch, max_blocks)
+        o = decoding_attn_paged_fwd(q, k_pages, v_pages, table.to(DEV), lens.to(DEV), sk, d, False)
+        torch.cuda.synchronize()
+        assert torch.isfinite(o.float()).all()
+        ks, vs = [], []
+        for b in rows:
+            n = int(lens[b])
+            pages = table[b, : (n + page - 1) // page].long().to(DEV)
+            ks.append(k_pages[pages].reshape(-1, hk, d)[:n].cpu())
+            vs.append(v_pages[pages].reshape(-1, hk, d)[:n].cpu())
+        sub = torch.tensor([int(lens[b]) for b in rows], dtype=torch.int32)
+        w = wl.Workload("batch70000_paged", q[rows].cpu(), torch.cat(ks), torch.cat(vs), wl.get_cu_seq(sub), int(sub.max()),
+                        d, False, sub.tolist())
+        check_against_oracle(w, o[rows].cpu())

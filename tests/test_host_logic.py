@@ -201,3 +201,22 @@ def test_torch_extension_module_exports_fwd():
     doc = ext.fwd.__doc__
     for name in ("q", "k", "v_", "o_", "cu_seq_k", "max_seq_k", "dim_v", "is_alibi"):
         assert name + ":" in doc
+
+
+def test_pipelined_latent_kernel_leaves_the_named_registers_alone():
+    """da_mla_pipe.hip names most of the register file in its instruction text; the build checks the compiler's own
+    code for strays (check_isa).  The same check on the tree's source with the build's flags, and the checker itself on
+    three lines it must flag."""
+    import shutil
+
+    from decoding_attention_amd import build as da_build
+    from decoding_attention_amd import check_isa
+
+    bad = check_isa.check_text("\tv_mov_b32_e32 v64, v1\n\tv_accvgpr_read_b32 v3, a7\n\tscratch_load_dword v1, off, s0\n"
+                               "#ASMSTART\n\tv_mov_b32 v200, v1\n#ASMEND\n\tv_add_u32_e32 v63, v1, v2\n")
+    assert [i for i, _ in bad] == [1, 2, 3]
+    hipcc = da_build._hipcc()
+    if shutil.which(hipcc) is None and not os.path.exists(hipcc):
+        pytest.skip("no hipcc here")
+    src = os.path.join(da_build.CSRC, "da_mla_pipe.hip")
+    assert check_isa.check_source(hipcc, da_build.HIPCC_FLAGS + da_build.EXTRA_FLAGS["da_mla_pipe.hip"], src)
