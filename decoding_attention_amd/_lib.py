@@ -30,6 +30,7 @@ EXPORTED_SYMBOLS = (
     "da_workspace_bytes_int4kv",
     "da_plan",
     "da_plan_distinct_v",
+    "da_plan_is_balanced",
     "da_supported_head_dims",
     "da_last_error",
     "da_version",
@@ -109,6 +110,8 @@ def _declare(lib):
     lib.da_plan.argtypes = [sz, sz, sz, sz, sz, sz, ci, sz, ip, ip, ip, ip]
     lib.da_plan_distinct_v.restype = ci
     lib.da_plan_distinct_v.argtypes = [sz, sz, sz, sz, sz, sz, sz, sz, ip, ip, ip, ip]
+    lib.da_plan_is_balanced.restype = ci
+    lib.da_plan_is_balanced.argtypes = [sz, sz, sz, sz, sz, sz, sz, sz]
     lib.da_supported_head_dims.restype = ci
     lib.da_supported_head_dims.argtypes = [sz, sz]
     lib.da_last_error.restype = ctypes.c_char_p
@@ -165,4 +168,8 @@ def plan(max_seq_k, batch, head_q, head_k, dim, dim_v, is_bf16=False, total_k=0,
                          ctypes.byref(ns), ctypes.byref(ch), ctypes.byref(rt))
     if rc != DA_OK:
         raise RuntimeError(f"da_plan failed ({rc}): {last_error()}")
-    return {"kind": kind.value, "nsplit": ns.value, "chunk": ch.value, "heads_per_group": rt.value}
+    out = {"kind": kind.value, "nsplit": ns.value, "chunk": ch.value, "heads_per_group": rt.value}
+    if not distinct_v or dim == dim_v:
+        out["balanced"] = bool(lib.da_plan_is_balanced(max_seq_k, batch, head_q, head_k, dim, dim_v, int(total_k),
+                                                       int(page_size)) > 0)
+    return out

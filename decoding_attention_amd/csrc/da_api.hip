@@ -46,7 +46,7 @@ int env_int(const char* name, int dflt) {
 // stops being split further; DA_MAX_CHUNK / DA_MIN_CHUNK: bounds on tokens per split.
 struct Tunables {
     int target_wgs, mfma_target_wgs, max_chunk, min_chunk, ragged_chunk, force_kind, group_min_ratio, wave_per_head,
-        mla_heads, gqa_heads, flat_wgs, flat_min_tokens, flat_paged_min_mb, nsplit, mfma_small_wgs, group_small_wgs,
+        mla_heads, gqa_heads, flat_wgs, flat_min_tokens, flat_uncounted, flat_uncounted_min, flat_paged_min_mb, nsplit, mfma_small_wgs, group_small_wgs,
         group_small_chunk, mla_group_heads, mla_group_small, fill_rounds, group_target_wgs_d128, mla_distinct_v, pipe_small_wgs;
     Tunables() {
         target_wgs = env_int("DA_TARGET_WGS", 512);
@@ -59,6 +59,10 @@ struct Tunables {
         // balanced grid of the grouped kernel for ragged batches: work-groups in all (0 = off), fewest tokens each
         flat_wgs = env_int("DA_FLAT_WGS", 512);
         flat_min_tokens = env_int("DA_FLAT_MIN_TOKENS", 256);
+        // ... also for a batch whose token count the caller did not give (0 = fixed splits then), from this many
+        // tokens per share at full length
+        flat_uncounted = env_int("DA_FLAT_UNCOUNTED", 1);
+        flat_uncounted_min = env_int("DA_FLAT_UNCOUNTED_MIN", 512);
         flat_paged_min_mb = env_int("DA_FLAT_PAGED_MIN_MB", 512);  // paged K/V takes the balanced grid from this many MB of K/V
         mfma_small_wgs = env_int("DA_MFMA_SMALL_WGS", 256);  // latent kernel: below this many 256-token splits, split finer
         pipe_small_wgs = env_int("DA_PIPE_SMALL_WGS", 33);   // the same for its pipelined form (128 heads a work-group)
@@ -100,10 +104,13 @@ struct Plan {
     size_t ws_bytes = 0;
     bool wave_per_head = false;  // grouped kernel: the four waves of a work-group take four KV heads
     bool v_distinct = false;     // latent kernel: the form that fetches V from a buffer of its own
-    // Balanced grid (grouped kernel, ragged batch whose total length the caller gave): flat_wgs work-groups
-    // per (KV heads, head group), each over flat_tokens consecutive tokens of the concatenated sequences; nsplit
-    // is then the most partials one sequence can have, chunk == flat_tokens.
-    int flat_tokens = 0, flat_wgs = 0;
+    // Balanced grid (grouped kernel; a batch known to be ragged, or one whose token count the caller did not give):
+    // flat_wgs work-groups per (KV heads, head group), each over an equal share of the concatenated sequences, which
+    // the kernels derive from the line's length on the device (da::flat_share; a multiple of flat_step units, at
+    // least flat_min).  nsplit then reports the shares along the line and chunk the share in tokens (0 when the
+    // host does not know it).
+    int flat_wgs = 0, flat_step = 1, flat_min = 1;
+    int flat_partials = 0;  // most partials the planner expects one sequence to have
     // paged K/V: the line is measured in units of flat_unit = 32 tokens, every sequence rounded up to whole units
     // (shares then start on tile boundaries), and its positions are computed on the device by a small kernel in
     // front of the sweep, into flat_cu_bytes at the end of the workspace
@@ -242,31 +249,54 @@ Plan make_plan(size_t max_seq_k, size_t batch, size_t head_q, size_t head_k, siz
     pl.groups = (ratio + pl.rt - 1) / pl.rt;
     const long long base = (long long)batch * (long long)(pl.wave_per_head ? head_k / 4 : head_k) * pl.groups;
     const bool ragged = total_k > 0 && (long long)total_k * 10 < (long long)batch * (long long)max_seq_k * 9;
-    // Ragged batch of known total length on the grouped kernel: equal shares of the concatenated tokens instead of
-    // fixed splits of every sequence.  Paged K/V pays one more (tiny) kernel for the sequences' positions, so it
-    // takes this form only when the sweep is long enough to win that back.
+    // The grouped kernel's balanced grid: equal shares of the concatenated tokens instead of fixed splits of every
+    // sequence.  Taken for a batch whose token count shows it to be ragged, and for a packed batch whose count the
+    // caller did not give (the reference's signature carries none, csrc/ops/decoding_attn.h:29-30) when it is large
+    // enough for whole shares: a uniform batch is then cut exactly as fixed splits cut it (batch 64 x 4096 tokens:
+    // 256 shares of 1024), and a ragged one is balanced.  The kernels read the line's length from cu_seq_k[batch]
+    // themselves.  Paged K/V pays one more (tiny) kernel for the sequences' positions, so it takes this form only
+    // when the count is given and the sweep is long enough to win that back.
     const double kv_bytes = (double)total_k * (double)head_k * (double)(dim + dim_v) * (kv_8bit ? 1.0 : 2.0);
-    if (pl.kind == kKindGroup && ragged && tun().flat_wgs > 0 && total_k < ((size_t)1 << 30) && total_k >= 64 * batch &&
-        (packed || kv_bytes >= (double)tun().flat_paged_min_mb * 1e6)) {
+    if (pl.kind == kKindGroup && tun().flat_wgs > 0 && batch >= 2) {
         const long long ygrid = base / (long long)batch;
-        long long w = std::max<long long>(1, tun().flat_wgs / ygrid);
+        // (without a count: the work-groups the fixed-split plan of this shape aims at, so that a uniform batch is cut
+        // the same way -- MQA at d = 128, 256 instead of 512: batch 64 x 4096 tokens 42.1 -> 29.5 us)
+        long long w = std::max<long long>(1, (total_k == 0 ? std::min(target_wgs, tun().flat_wgs) : tun().flat_wgs) / ygrid);
         const long long unit = packed ? 1 : da::kGqaTile;
-        const long long line = packed ? (long long)total_k : (long long)total_k / unit + (long long)batch;
         const long long step = std::max<long long>(1, trip / unit);  // a work-group's waves advance `trip` tokens together
-        long long t = (line + w - 1) / w;
-        t = std::max<long long>((t + step - 1) / step * step, std::max<long long>(tun().flat_min_tokens / unit, step));
-        w = std::min<long long>(65535, (line + t - 1) / t);
-        pl.flat_tokens = (int)t;
-        pl.flat_wgs = (int)w;
-        pl.flat_unit = (int)unit;
-        pl.chunk = (int)(t * unit);
-        pl.nsplit = (int)std::min<long long>(w, (((long long)max_seq_k + unit - 1) / unit + t - 1) / t + 1);
-        pl.ws_bytes = (size_t)batch * head_q * pl.nsplit * (dim_v + 2) * sizeof(float);
-        if (!packed) {
-            pl.flat_cu_bytes = ((batch + 1) * sizeof(int32_t) + 15) & ~(size_t)15;
-            pl.ws_bytes += pl.flat_cu_bytes;
+        const long long mn = std::max<long long>(tun().flat_min_tokens / unit, step);
+        const bool counted = ragged && total_k < ((size_t)1 << 30) && total_k >= 64 * batch &&
+                             (packed || kv_bytes >= (double)tun().flat_paged_min_mb * 1e6);
+        const bool uncounted = total_k == 0 && packed && !latent_group && tun().flat_uncounted &&
+                               (long long)batch * (long long)max_seq_k >= w * (long long)tun().flat_uncounted_min &&
+                               (long long)batch * (long long)max_seq_k < (1ll << 30);
+        if (counted || uncounted) {
+            pl.flat_step = (int)step;
+            pl.flat_min = (int)mn;
+            pl.flat_unit = (int)unit;
+            if (counted) {
+                const long long line = packed ? (long long)total_k : (long long)total_k / unit + (long long)batch;
+                const long long t = da::flat_share(line, (int)w, (int)step, (int)mn);
+                w = std::min<long long>(w, (line + t - 1) / t);  // (shares past the line's end would only exit)
+                pl.chunk = (int)(da::flat_share(line, (int)w, (int)step, (int)mn) * unit);
+            } else {
+                pl.chunk = 0;
+            }
+            pl.flat_wgs = (int)w;
+            pl.nsplit = (int)w;
+            // partials a sequence of max_seq_k tokens has when the batch is as long as the host knows it can be (the
+            // merge picks its form by it; a batch that turns out shorter has more, and is merged correctly all the same)
+            const long long line_max = counted ? (packed ? (long long)total_k : (long long)total_k / unit + (long long)batch)
+                                               : (long long)batch * (((long long)max_seq_k + unit - 1) / unit);
+            const long long t_est = da::flat_share(line_max, (int)w, (int)step, (int)mn);
+            pl.flat_partials = (int)std::min<long long>(w, (((long long)max_seq_k + unit - 1) / unit + t_est - 1) / t_est + 1);
+            pl.ws_bytes = da::flat_slots((int)w, batch) * head_q * (dim_v + 2) * sizeof(float);
+            if (!packed) {
+                pl.flat_cu_bytes = ((batch + 1) * sizeof(int32_t) + 15) & ~(size_t)15;
+                pl.ws_bytes += pl.flat_cu_bytes;
+            }
+            return pl;
         }
-        return pl;
     }
     int min_chunk = std::max(mfma ? 256 : tun().min_chunk, trip);
     const long long wgs_at_min = base * std::max<long long>(1, (long long)max_seq_k / min_chunk);
@@ -548,6 +578,12 @@ int da_plan_distinct_v(size_t max_seq_k, size_t batch, size_t head_q, size_t hea
     return DA_OK;
 }
 
+int da_plan_is_balanced(size_t max_seq_k, size_t batch, size_t head_q, size_t head_k, size_t dim, size_t dim_v,
+                        size_t total_k, size_t page_size) {
+    if (head_k == 0 || head_q % head_k != 0 || !supported_dims(dim, dim_v)) return -1;
+    return make_plan(max_seq_k, batch, head_q, head_k, dim, dim_v, false, total_k, page_size).flat_wgs > 0 ? 1 : 0;
+}
+
 size_t da_workspace_bytes(size_t max_seq_k, size_t batch, size_t head_q, size_t head_k, size_t dim, size_t dim_v,
                           size_t total_k) {
     if (head_k == 0 || head_q % head_k != 0 || !supported_dims(dim, dim_v)) return 0;
@@ -691,7 +727,10 @@ int run_attention(const void* q, const void* k, const void* v, void* o, const in
     sp.o = o;
     sp.cu_seq_k = cu_seq_k;
     sp.ws_o = reinterpret_cast<float*>(ws);
-    sp.ws_ml = ws ? reinterpret_cast<float*>(ws) + (size_t)batch * head_q * pl.nsplit * dim_v : nullptr;
+    // rows of partials: a slot per (sequence, share) on the balanced grid, nsplit per sequence otherwise
+    const size_t partial_rows =
+        (pl.flat_wgs ? da::flat_slots(pl.flat_wgs, batch) : (size_t)batch * pl.nsplit) * head_q;
+    sp.ws_ml = ws ? reinterpret_cast<float*>(ws) + partial_rows * dim_v : nullptr;
     sp.slopes = is_alibi ? alibi_slopes : nullptr;
     sp.k_row = (int64_t)(head_k * dim);
     sp.v_row = v ? (int64_t)(head_k * dim_v) : (int64_t)(head_k * dim);
@@ -714,7 +753,9 @@ int run_attention(const void* q, const void* k, const void* v, void* o, const in
     sp.max_blocks = (int)pg.max_blocks;
     sp.k_page = (int64_t)pg.k_page;
     sp.v_page = v ? (int64_t)pg.v_page : (int64_t)pg.k_page;
-    sp.flat_tokens = pl.flat_tokens;
+    sp.flat_wgs = pl.flat_wgs;
+    sp.flat_step = pl.flat_step;
+    sp.flat_min = pl.flat_min;
     sp.flat_unit = pl.flat_unit;
     sp.flat_cu = cu_seq_k;
     sp.batch = (int)batch;
@@ -732,9 +773,9 @@ int run_attention(const void* q, const void* k, const void* v, void* o, const in
     sp.nat_partials = half_partials ? 1 : 0;
     if (pl.kind == kKindMfma && pl.rt == 128 && kf.fmt == 0 && !pl.v_distinct && pl.nsplit > 1 && !half_partials)
         return fail(DA_ERR_WORKSPACE, "the pipelined kernel's 16-bit partials do not fit the workspace's partial area");
-    const dim3 grid((unsigned)(pl.flat_tokens ? pl.flat_wgs : pl.nsplit),
+    const dim3 grid((unsigned)(pl.flat_wgs ? pl.flat_wgs : pl.nsplit),
                     (unsigned)((pl.wave_per_head ? head_k / 4 : head_k) * pl.groups),
-                    (unsigned)(pl.flat_tokens ? 1 : batch));
+                    (unsigned)(pl.flat_wgs ? 1 : batch));
     hipError_t e;
     if (kf.fmt != 0) {
         if (pl.kind == kKindMfma)
@@ -764,7 +805,7 @@ int run_attention(const void* q, const void* k, const void* v, void* o, const in
     }
     if (e != hipSuccess) return fail(DA_ERR_HIP, "sweep kernel launch: %s", hipGetErrorString(e));
 
-    if ((pl.nsplit > 1 || pl.flat_tokens) && !kf.sweep_only) {
+    if ((pl.nsplit > 1 || pl.flat_wgs) && !kf.sweep_only) {
         da::ReduceParams rp;
         rp.o = o;
         rp.cu_seq_k = cu_seq_k;
@@ -773,12 +814,15 @@ int run_attention(const void* q, const void* k, const void* v, void* o, const in
         rp.ws_ml = sp.ws_ml;
         rp.head_q = (int)head_q;
         rp.dim_v = (int)dim_v;
-        rp.nsplit = pl.nsplit;
+        rp.nsplit = pl.flat_wgs ? pl.flat_partials : pl.nsplit;
         rp.chunk = pl.chunk;
-        rp.flat_tokens = pl.flat_tokens;
         rp.flat_wgs = pl.flat_wgs;
+        rp.flat_step = pl.flat_step;
+        rp.flat_min = pl.flat_min;
         rp.flat_cu = sp.flat_cu;
-        rp.early = pl.ws_bytes <= ((size_t)8 << 20) ? 1 : 0;
+        rp.batch = (int)batch;
+        // (the balanced grid's partial slots are known only once the sequences' positions have been read)
+        rp.early = pl.ws_bytes <= ((size_t)8 << 20) && !pl.flat_wgs ? 1 : 0;
         rp.half_partials = half_partials ? 1 : 0;
         rp.ratio = sp.ratio;
         rp.groups = pl.groups;

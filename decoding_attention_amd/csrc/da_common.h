@@ -271,12 +271,14 @@ struct SweepParams {
     // The kernels fold k_scale into the softmax scale and v_scale into the final normalisation.
     const float* k_scale;
     const float* v_scale;
-    // Balanced form of the grouped-head kernel's grid (flat_tokens == 0: off).  The sequences lie end to end on
-    // one line measured in units of flat_unit tokens (1 for packed K/V, where the line is cu_seq_k itself; 32 for
-    // paged K/V, where every sequence is rounded up to whole units so that shares start on tile boundaries);
-    // flat_cu[b] is the position of sequence b on the line ([batch + 1] entries), flat_tokens the units per
-    // work-group.
-    int flat_tokens;
+    // Balanced form of the grouped-head kernel's grid (flat_wgs == 0: off).  The sequences lie end to end on one line
+    // measured in units of flat_unit tokens (1 for packed K/V, where the line is cu_seq_k itself; 32 for paged K/V,
+    // where every sequence is rounded up to whole units so that shares start on tile boundaries); flat_cu[b] is the
+    // position of sequence b on the line ([batch + 1] entries).  Each of flat_wgs work-groups takes an equal share of
+    // the line, flat_share() units, which the kernels derive from the line's length flat_cu[batch] themselves: the
+    // host never needs the token count.
+    int flat_wgs;
+    int flat_step, flat_min;  // a share is a multiple of flat_step units and at least flat_min
     int flat_unit;
     const int32_t* flat_cu;
     int batch;
@@ -291,10 +293,11 @@ struct ReduceParams {
     const float* ws_o;
     const float* ws_ml;
     int head_q, dim_v, nsplit, chunk;
-    // balanced form of the sweep's grid (flat_tokens > 0): units per work-group, work-groups, the sequences'
-    // positions on the line (see SweepParams)
-    int flat_tokens, flat_wgs;
+    // balanced form of the sweep's grid (flat_wgs > 0): work-groups along the line, share granularity and minimum, the
+    // sequences' positions on the line (see SweepParams)
+    int flat_wgs, flat_step, flat_min;
     const int32_t* flat_cu;
+    int batch;
     // the workspace is small (cache-resident): request the first partials before the sequence's length is known
     int early;
     // the partial outputs are normalised (divided by their denominators) and stored as 16-bit values of the output
@@ -329,6 +332,18 @@ __device__ __forceinline__ int nat_piece(int c4, int n) {
 __device__ __forceinline__ int nat_ml(int n) { return 64 * 64 + n; }
 // bytes of one sequence split's records
 __host__ __device__ inline size_t nat_split_bytes(int nblk) { return (size_t)nblk * kNatBlockUnits * 8; }
+
+// Balanced grid: units per work-group for a line of `total` units cut into `wgs` shares.
+__host__ __device__ inline int flat_share(long long total, int wgs, int step, int mn) {
+    long long t = (total + wgs - 1) / wgs;
+    t = (t + step - 1) / step * step;
+    const long long floor_t = mn > step ? mn : step;
+    return (int)(t > floor_t ? t : floor_t);
+}
+// Partial slot of (sequence b, share i): consecutive sequences may meet in one share, so the slots of a batch are
+// numbered share + sequence -- strictly increasing along the line, below wgs + batch -- which needs no knowledge of the
+// share length when the workspace is sized.
+__host__ __device__ inline size_t flat_slots(int wgs, size_t batch) { return (size_t)wgs + batch; }
 
 // First token (row of the packed K/V buffers) and length of sequence b; paged sequences start at row 0 of their
 // own pages.

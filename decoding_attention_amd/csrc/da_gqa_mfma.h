@@ -111,14 +111,14 @@ constexpr size_t gqa_lds_bytes(int nt) {
 // (K) or the LDS tile (V).
 // One segment of work: tokens [c0, c1) of sequence b (first row `start`, `len` tokens) for the KV heads and head
 // group `by` selects (blockIdx.y, or its renumbered stand-in).  `direct`: the segment is the whole sequence, so the result goes to o; otherwise the
-// un-normalised partial goes to workspace slot `split` of the sequence.
+// un-normalised partial of head h goes to workspace row part0 + h * part_stride.
 // PGM: how paged K/V is addressed.  0: one page lookup per tile (pages hold a multiple of 32 tokens; also the packed
 // layout); 1: 16-token pages, a tile is fetched as two runs of 16 tokens, each from one page; 2: smaller pages, every
 // lane looks up the page of the row it loads.
 template <typename Tag, int D, int DV, int NT, bool PREFETCH, bool WH, int KV8, int PGM>
 __device__ __forceinline__ void gqa_segment(const SweepParams& p, uint8_t* const smem, const int by, const int b,
                                             const int start, const int len, const int c0, const int c1,
-                                            const int split, const bool direct) {
+                                            const size_t part0, const int part_stride, const bool direct) {
     using MM = Mma16<Tag>;
     using vec8 = typename MM::vec8;
     using EL = Elem<Tag>;
@@ -470,7 +470,7 @@ __device__ __forceinline__ void gqa_segment(const SweepParams& p, uint8_t* const
                         *reinterpret_cast<ushort4*>(orow + ct * 16) = w;
                     }
                 } else {
-                    const size_t part = ((size_t)b * p.head_q + h) * p.nsplit + split;
+                    const size_t part = part0 + (size_t)h * part_stride;
                     float* wrow = p.ws_o + part * DV + g * 4;
 #pragma unroll
                     for (int ct = 0; ct < CT; ++ct) *reinterpret_cast<f32x4*>(wrow + ct * 16) = acc[nt][ct] * vs;
@@ -530,7 +530,7 @@ __device__ __forceinline__ void gqa_segment(const SweepParams& p, uint8_t* const
             w16.w = EL::from_f32(num[3] * inv);
             *reinterpret_cast<ushort4*>(o16 + ((size_t)b * p.head_q + h) * DV + col) = w16;
         } else {
-            const size_t part = ((size_t)b * p.head_q + h) * p.nsplit + split;
+            const size_t part = part0 + (size_t)h * part_stride;
             *reinterpret_cast<f32x4*>(p.ws_o + part * DV + col) = num * vs;
             if (col == 0) {
                 p.ws_ml[part * 2 + 0] = mm;
@@ -541,17 +541,17 @@ __device__ __forceinline__ void gqa_segment(const SweepParams& p, uint8_t* const
 }
 
 // Grid, packed or paged K/V with a fixed split length: (split, KV heads x head groups, sequence).
-// Grid, balanced form (p.flat_tokens > 0): (work-group i of W, KV heads x head groups, 1).  The tokens of all
-// sequences form one line (positions p.flat_cu, in units of p.flat_unit tokens); work-group i takes positions
-// [i T, (i+1) T) of it (the last one to the end), whatever sequences they belong to, one segment per sequence it
-// touches.  Every work-group then streams the same number of bytes, which a ragged batch cut into fixed splits
+// Grid, balanced form (p.flat_wgs > 0): (work-group i of W, KV heads x head groups, 1).  The tokens of all
+// sequences form one line (positions p.flat_cu, in units of p.flat_unit tokens) whose length the kernel reads from
+// p.flat_cu[batch]; work-group i takes positions [i T, (i+1) T) of it, T = flat_share() (the last one to the end),
+// whatever sequences they belong to, one segment per sequence it touches.  Every work-group then streams the same number of bytes, which a ragged batch cut into fixed splits
 // does not give.  Sequence b spans work-groups first(b) = cu[b] / T ... last(b) = (cu[b+1] - 1) / T (both capped
-// at W - 1); its segment in work-group i is partial number i - first(b), and goes straight to o when
+// at W - 1); its segment in work-group i is the partial in slot i + b (flat_slots), and goes straight to o when
 // first(b) == last(b).
 template <typename Tag, int D, int DV, int NT, bool PREFETCH, bool WH, int MINW, int KV8 = 0, int PGM = 0>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(MINW))) void gqa_mfma_kernel(const SweepParams p) {
     extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
-    if (p.flat_tokens == 0) {
+    if (p.flat_wgs == 0) {
         int split = blockIdx.x, by = blockIdx.y, b = blockIdx.z;
         // Several head groups per KV head read the same K/V rows.  Work-groups go to the eight XCDs round-robin by
         // linear id, and each XCD has its own L2: renumber so that the groups of one (sequence, KV heads, split) are
@@ -572,12 +572,14 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(MINW))) voi
         seq_range(p, b, start, len);
         const int c0 = split * p.chunk;
         const int c1 = (split == p.nsplit - 1) ? len : min(len, c0 + p.chunk);
-        gqa_segment<Tag, D, DV, NT, PREFETCH, WH, KV8, PGM>(p, smem, by, b, start, len, c0, c1, split, p.nsplit == 1);
+        gqa_segment<Tag, D, DV, NT, PREFETCH, WH, KV8, PGM>(p, smem, by, b, start, len, c0, c1,
+                                                            (size_t)b * p.head_q * p.nsplit + split, p.nsplit, p.nsplit == 1);
         return;
     }
-    const int T = p.flat_tokens, W = (int)gridDim.x, i = (int)blockIdx.x, unit = p.flat_unit;
+    const int W = (int)gridDim.x, i = (int)blockIdx.x, fby = (int)blockIdx.y, unit = p.flat_unit;
     const int32_t* const cu = p.flat_cu;
     const int total = cu[p.batch];
+    const int T = flat_share(total, W, p.flat_step, p.flat_min);
     const int r0 = (int)min((long long)i * T, (long long)total);
     const int r1 = (i == W - 1) ? total : (int)min((long long)r0 + T, (long long)total);
     if (r0 >= r1) return;
@@ -602,8 +604,8 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(MINW))) voi
         seq_range(p, b, start, len);
         const int first = min(s / T, W - 1), last = min((e - 1) / T, W - 1);
         const int c0 = (max(r0, s) - s) * unit, c1 = min((min(r1, e) - s) * unit, len);
-        gqa_segment<Tag, D, DV, NT, PREFETCH, WH, KV8, PGM>(p, smem, (int)blockIdx.y, b, start, len, c0, c1, i - first,
-                                                            first == last);
+        gqa_segment<Tag, D, DV, NT, PREFETCH, WH, KV8, PGM>(p, smem, fby, b, start, len, c0, c1,
+                                                            (size_t)(i + b) * p.head_q, 1, first == last);
         if (!WH) __syncthreads();  // the merge area of this segment is the V tile area of the next
     }
 }

@@ -925,7 +925,7 @@ hipError_t launch_mla_pipe(const SweepParams& p_in, bool is_bf16, dim3 grid, hip
 #ifdef DA_PIPE_PROBE
     {
         const char* s = getenv("DA_PIPE_FLAGS");
-        p.flat_tokens = s ? atoi(s) : 0;
+        p.flat_min = s ? atoi(s) : 0;
     }
 #endif
     const bool pg = p.block_table != nullptr && p.page_shift < 4;

@@ -297,9 +297,12 @@ __global__ __launch_bounds__(256) void reduce_kernel(const ReduceParams p, int r
         sgi = lane / CW;
     }
     if (row >= rows) return;  // (whole waves leave together when SG > 1)
-    const size_t part0 = (size_t)row * p.nsplit;
-    const float2* const ml = reinterpret_cast<const float2*>(p.ws_ml) + part0;
-    const float4* const src = reinterpret_cast<const float4*>(p.ws_o + part0 * p.dim_v) + c4;
+    // partial s of this row sits in workspace row part0 + s * pstride (fixed splits: the row's own nsplit slots;
+    // balanced grid: slot first share + sequence + s of the batch, see flat_slots, known once the positions are read)
+    size_t part0 = (size_t)row * p.nsplit;
+    size_t pstride = 1;
+    const float2* ml = reinterpret_cast<const float2*>(p.ws_ml) + part0;
+    const float4* src = reinterpret_cast<const float4*>(p.ws_o + part0 * p.dim_v) + c4;
     const uint2* const src16 = reinterpret_cast<const uint2*>(p.ws_o);  // (H16) the block records
     // This lane's next four partials: slots s0, s0 + SG, ... (clamped to `last`; the caller masks the rest).
     float2 e[4];
@@ -314,8 +317,8 @@ __global__ __launch_bounds__(256) void reduce_kernel(const ReduceParams p, int r
                 const uint2 h = rec[nat_piece(c4, nat_n)];
                 x[u] = make_float4(EL::lo(h.x), EL::hi(h.x), EL::lo(h.y), EL::hi(h.y));
             } else {
-                e[u] = ml[s];
-                x[u] = src[(size_t)s * nc4];
+                e[u] = ml[(size_t)s * pstride];
+                x[u] = src[(size_t)s * pstride * nc4];
             }
         }
     };
@@ -326,13 +329,19 @@ __global__ __launch_bounds__(256) void reduce_kernel(const ReduceParams p, int r
     const int b = row / p.head_q;
     const int len = p.cu_seq_k ? p.cu_seq_k[b + 1] - p.cu_seq_k[b] : p.seq_lens[b];
     int ns = 0;
-    if (p.flat_tokens > 0) {
+    if (p.flat_wgs > 0) {
         // balanced sweep grid: the sequence's partials come from the work-groups its tokens fall into; a sequence
         // inside one work-group was written to o by the sweep itself
         if (len > 0) {
             const int lo = p.flat_cu[b], hi = p.flat_cu[b + 1];
-            ns = min((hi - 1) / p.flat_tokens, p.flat_wgs - 1) - min(lo / p.flat_tokens, p.flat_wgs - 1) + 1;
+            const int T = flat_share(p.flat_cu[p.batch], p.flat_wgs, p.flat_step, p.flat_min);
+            const int first = min(lo / T, p.flat_wgs - 1);
+            ns = min((hi - 1) / T, p.flat_wgs - 1) - first + 1;
             if (ns == 1) return;
+            part0 = (size_t)(first + b) * p.head_q + (size_t)(row - b * p.head_q);
+            pstride = (size_t)p.head_q;
+            ml = reinterpret_cast<const float2*>(p.ws_ml) + part0;
+            src = reinterpret_cast<const float4*>(p.ws_o + part0 * p.dim_v) + c4;
         }
     } else if (len > 0) {
         ns = min(p.nsplit, (len + p.chunk - 1) / p.chunk);

@@ -32,7 +32,7 @@ hipError_t launch_reduce(const ReduceParams& p, bool is_bf16, int blocks, hipStr
     while (sg > 1 && (p.dim_v / 4) % (64 / sg) != 0) sg /= 2;
     // normalised 16-bit partials (the pipelined latent kernel's: dim_v = 512, never the balanced grid), one lane per
     // element: eight columns a thread, dead rows of the blocks included
-    if (p.half_partials && (p.dim_v != 512 || p.flat_tokens != 0 || p.nat_blocks <= 0 || p.head_q <= 0))
+    if (p.half_partials && (p.dim_v != 512 || p.flat_wgs != 0 || p.nat_blocks <= 0 || p.head_q <= 0))
         return hipErrorInvalidValue;
     if (p.half_partials && sg == 1) {
         const int per_kv = p.groups * p.nat_waves, head_k = p.nat_blocks / per_kv;

@@ -229,6 +229,16 @@ int da_plan_distinct_v(size_t max_seq_k, size_t batch, size_t head_q, size_t hea
                        size_t total_k, size_t page_size, int *kernel_kind, int *nsplit, int *chunk,
                        int *heads_per_group);
 
+/*
+ * 1 when the 16-bit call (packed: page_size 0; else pages of page_size tokens) takes the grouped kernel's balanced
+ * grid -- equal shares of the concatenated sequences per work-group instead of fixed splits of every sequence, the
+ * share derived on the device from cu_seq_k[batch] -- 0 when not, negative on an error.  da_plan then reports the
+ * shares along the line as nsplit and the share as chunk (0 when no token count was given).  No counterpart in the
+ * reference, whose kernel never splits a sequence.
+ */
+int da_plan_is_balanced(size_t max_seq_k, size_t batch, size_t head_q, size_t head_k, size_t dim, size_t dim_v,
+                        size_t total_k, size_t page_size);
+
 /* 1 when (dim, dim_v) is a supported pair: the reference's DA_HEADDIM_SWITCH set (csrc/common/common.h:73-96). */
 int da_supported_head_dims(size_t dim, size_t dim_v);
 

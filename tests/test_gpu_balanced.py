@@ -1,5 +1,6 @@
-"""Balanced grid of the grouped-head kernel: when the caller gives the total token count of a ragged packed batch,
-every work-group takes an equal share of the concatenated tokens, across sequence boundaries.  The results must
+"""Balanced grid of the grouped-head kernel: for a packed batch that the token count shows to be ragged, and for a
+large batch given without a count, every work-group takes an equal share of the concatenated tokens (derived on the
+device from cu_seq_k[batch]), across sequence boundaries.  The results must
 match the oracle exactly as the fixed-split grid's do, whatever the lengths are: empty sequences anywhere, many
 short sequences inside one share, one sequence over many shares, and a hint that is too small or too large.
 """
@@ -34,11 +35,10 @@ def _run_ex(w, hint):
 
 
 def _is_balanced(w, hint):
-    """The planner chose equal token shares: its split length is the share, not a divisor of max_seq_k."""
+    """The planner chose equal token shares of the concatenated sequences."""
     b, hq, d = w.q.shape
     hk = w.k.shape[1]
-    with_hint = _lib.plan(w.max_seq_k, b, hq, hk, d, w.dim_v, True, hint)
-    return with_hint["kind"] == 3 and with_hint["nsplit"] * with_hint["chunk"] >= w.max_seq_k + with_hint["chunk"]
+    return _lib.plan(w.max_seq_k, b, hq, hk, d, w.dim_v, True, hint)["balanced"]
 
 
 MIXED = [0, 0, 1, 5000, 0, 37, 2048, 1, 8191, 64, 0, 3000, 333, 4096, 31, 33, 0]
@@ -138,7 +138,10 @@ def test_paged_large_ragged_batch_takes_the_balanced_grid():
     assert total * 8 * 256 * 2 >= 512e6
     lib = _lib.load()
     flat = lib.da_workspace_bytes_paged(w.max_seq_k, b, 32, 8, 128, 128, total, 64)
-    assert (flat - ((b + 1) * 4 + 15) // 16 * 16) % (b * 32 * (128 + 2) * 4) == 0  # partials, then the positions
+    assert _lib.plan(w.max_seq_k, b, 32, 8, 128, 128, total_k=total, page_size=64)["balanced"]
+    # a partial slot per (share, sequence) pair that can occur, then the sequences' positions
+    slots, rest = divmod(flat - ((b + 1) * 4 + 15) // 16 * 16, 32 * (128 + 2) * 4)
+    assert rest == 0 and b < slots <= 256 + b
     pk = wl.to_pages(w, 64, seed=3).to(DEV)
     wd = w.to(DEV)
     o = decoding_attn_paged_fwd(wd.q, pk.k_pages, pk.v_pages, pk.block_table, pk.seq_lens, w.max_seq_k, w.dim_v,

@@ -60,10 +60,16 @@ def test_plan_is_consistent(d, dv, batch, sk):
     hq, hk = (128, 1) if d == 576 else (32, 8)
     p = _lib.plan(sk, batch, hq, hk, d, dv)
     assert p["kind"] in (1, 2, 3)
+    ws = _lib.load().da_workspace_bytes(sk, batch, hq, hk, d, dv, 0)
+    if p["balanced"]:
+        # no token count given: equal shares of the concatenated tokens, the share derived on the device; a partial
+        # slot per (share, sequence) pair that can occur
+        assert p["kind"] == 3 and p["chunk"] == 0 and batch >= 2 and 1 <= p["nsplit"] <= 512
+        assert ws == (p["nsplit"] + batch) * hq * (dv + 2) * 4
+        return
     assert 1 <= p["nsplit"] <= 256
     assert p["nsplit"] * p["chunk"] >= sk
     assert (p["nsplit"] - 1) * p["chunk"] < max(sk, 1)
-    ws = _lib.load().da_workspace_bytes(sk, batch, hq, hk, d, dv, 0)
     need = 0 if p["nsplit"] == 1 else batch * hq * p["nsplit"] * (dv + 2) * 4
     # (576, 512) also covers the plan used when V is passed as its own buffer
     assert ws >= need if d == 576 else ws == need
@@ -78,12 +84,13 @@ def test_plan_total_k_hint_changes_the_splits_and_never_the_kernel():
     ragged = _lib.plan(sk, batch, 32, 8, 128, 128, total_k=batch * sk // 2)
     assert full["kind"] == base["kind"] and full["chunk"] >= base["chunk"] and full["nsplit"] <= base["nsplit"]
     # grouped kernel: equal shares of the concatenated tokens, 512 work-groups over the 2 groups of 4 KV heads
-    assert ragged["kind"] == base["kind"] == 3
-    assert ragged["chunk"] == batch * sk // 2 // 256
-    # a sequence of max_seq_k tokens can straddle one more share than its length fills
-    assert ragged["nsplit"] == sk // ragged["chunk"] + 1
+    assert ragged["kind"] == base["kind"] == 3 and ragged["balanced"] and not full["balanced"]
+    assert ragged["nsplit"] == 256 and ragged["chunk"] == batch * sk // 2 // 256
+    # a partial slot per (share, sequence) pair that can occur: shares + sequences
     ws = _lib.load().da_workspace_bytes(sk, batch, 32, 8, 128, 128, batch * sk // 2)
-    assert ws == batch * 32 * ragged["nsplit"] * (128 + 2) * 4
+    assert ws == (ragged["nsplit"] + batch) * 32 * (128 + 2) * 4
+    # without a count the same grid, the share left to the device
+    assert base["balanced"] and base["nsplit"] == 256 and base["chunk"] == 0
     # VALU sweep (one query head per KV head, short sequences): shorter fixed splits
     sk, batch = 2048, 16
     base = _lib.plan(sk, batch, 32, 32, 256, 256)
@@ -93,14 +100,17 @@ def test_plan_total_k_hint_changes_the_splits_and_never_the_kernel():
 
 
 def test_plan_without_a_token_count_at_d128():
-    """The reference-signature entry point passes no token count: the grouped kernel at d = 128 then cuts a sequence
-    into splits of up to 2048 tokens, on a uniform batch the same cut as the plan that knows the count."""
+    """The reference-signature entry point passes no token count: a batch large enough for whole shares then takes the
+    balanced grid, which cuts a uniform batch exactly as the counted plan's fixed splits do (256 shares of 64 x 4096 /
+    256 = 1024 tokens, the share derived on the device); smaller problems keep fixed splits of up to 2048 tokens."""
     blind = _lib.plan(4096, 64, 32, 8, 128, 128)
     counted = _lib.plan(4096, 64, 32, 8, 128, 128, total_k=64 * 4096)
     assert blind["kind"] == counted["kind"] == 3
-    assert (blind["nsplit"], blind["chunk"]) == (counted["nsplit"], counted["chunk"]) == (4, 1024)
-    # a long sequence of a small batch: the cap, not the work-group target, sets the cut
-    assert _lib.plan(16384, 64, 32, 8, 128, 128)["chunk"] == 2048
+    assert (counted["nsplit"], counted["chunk"], counted["balanced"]) == (4, 1024, False)
+    assert (blind["nsplit"], blind["chunk"], blind["balanced"]) == (256, 0, True)
+    # a single long sequence: nothing to balance, the cap sets the cut
+    one = _lib.plan(16384, 1, 32, 8, 128, 128)
+    assert not one["balanced"] and one["chunk"] <= 2048
     # MQA (four waves share the one KV head's tokens): 256 work-groups
     assert _lib.plan(4096, 64, 32, 1, 128, 128, total_k=64 * 4096)["nsplit"] == 4
     assert _lib.load().da_release_workspaces() == _lib.DA_OK  # nothing cached, nothing to free, no GPU needed
@@ -109,14 +119,16 @@ def test_plan_without_a_token_count_at_d128():
 def test_workspace_sizes_of_the_paged_and_fp8_variants():
     lib = _lib.load()
     shape = (4096, 64, 32, 8, 128, 128)
-    packed = lib.da_workspace_bytes(*shape, 0)
+    # (with the token count: without one the packed layout takes the balanced grid, which paged K/V only takes with it)
+    shape_total = 64 * 4096
+    packed = lib.da_workspace_bytes(*shape, shape_total)
     # pages of 16 tokens and more take the packed layout's kernels and plan; shorter pages keep the shorter splits
     for page in (16, 64, 256):
-        assert lib.da_workspace_bytes_paged(*shape, 0, page) == packed
+        assert lib.da_workspace_bytes_paged(*shape, shape_total, page) == packed
     for page in (1, 8):
-        assert lib.da_workspace_bytes_paged(*shape, 0, page) >= packed
+        assert lib.da_workspace_bytes_paged(*shape, shape_total, page) >= packed
     # 8-bit K/V: the same kernel kind, with the shorter splits its half-length rows were measured on
-    assert lib.da_workspace_bytes_fp8kv(*shape, 0, 0) >= packed
+    assert lib.da_workspace_bytes_fp8kv(*shape, shape_total, 0) >= packed
     # the latent form: the larger of the MFMA kernel's plan (V inside K) and the VALU sweep's (a distinct V buffer)
     mla = (4096, 16, 128, 1, 576, 512)
     assert lib.da_workspace_bytes_fp8kv(*mla, 0, 0) > 0

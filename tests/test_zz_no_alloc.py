@@ -57,18 +57,18 @@ def test_noalloc_matches_ex_on_two_calls_in_a_row():
 def test_noalloc_refuses_a_plan_beyond_the_static_array():
     lib = _lib.load()
     dev = torch.device("cuda:0")
-    # a pathologically ragged batch on the balanced grid: one sequence of 262144 tokens among 255 of one token; its
-    # plan keeps a partial slot per (sequence, share) -- gigabytes.  The call must fail before anything is enqueued,
-    # so the tensors only need to exist.
-    b, hq, hk, d = 256, 32, 8, 128
+    # 60 sequences of 131072 tokens each, known to be uniform, 32/8 heads at d = 256: 64 fixed splits of 2048 tokens
+    # with fp32 partials, 127 MB.  The call must fail before anything is enqueued, so the tensors only need to exist.
+    b, hq, hk, d = 60, 32, 8, 256
     q = torch.zeros((b, hq, d), dtype=torch.bfloat16, device=dev)
     k = torch.zeros((16, hk, d), dtype=torch.bfloat16, device=dev)
     o = torch.zeros((b, hq, d), dtype=torch.bfloat16, device=dev)
     cu = torch.zeros((b + 1,), dtype=torch.int32, device=dev)
-    total_k = 262144 + 255
-    need = lib.da_workspace_bytes(262144, b, hq, hk, d, d, total_k)
+    max_seq = 131072
+    total_k = b * max_seq
+    need = lib.da_workspace_bytes(max_seq, b, hq, hk, d, d, total_k)
     assert need > lib.da_noalloc_workspace_limit()
-    rc = lib.da_decoding_attn_noalloc(q.data_ptr(), k.data_ptr(), k.data_ptr(), o.data_ptr(), cu.data_ptr(), 262144, b, hq,
+    rc = lib.da_decoding_attn_noalloc(q.data_ptr(), k.data_ptr(), k.data_ptr(), o.data_ptr(), cu.data_ptr(), max_seq, b, hq,
                                       hk, d, d, 0, 1, 0.0, None, total_k, torch.cuda.current_stream().cuda_stream)
     assert rc == _lib.DA_ERR_WORKSPACE
     assert "static array" in _lib.last_error()
