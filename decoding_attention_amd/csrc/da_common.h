@@ -122,8 +122,8 @@ constexpr int kKvInt8 = 2;  // two's-complement integers
 // Four-bit integers (two's complement, -8 .. 7), two to a byte, element 2 i in the low half of byte i.  The kernels
 // address such a cache as if it held one byte per element: the host hands them TWICE the buffer's address
 // (SweepParams::k and ::v), all their row, head and lane arithmetic is the int8 arithmetic on those doubled addresses,
-// and the load halves the address again (kv4_load8 / kv4_load16; every address the kernels form is even).  A load
-// widens the nibbles to sign-extended bytes, from where on the data is an int8 cache's.
+// and the load halves the address again (kv4_load8 / kv4_load16; every address the kernels form is even); the
+// conversion to the compute type takes the nibbles straight to 16-bit values (int4x8_to_16).
 constexpr int kKvInt4 = 3;
 
 // Eight FP8 (OCP e4m3) values -> eight 16-bit elements of the compute type.  Both conversions are exact (e4m3
@@ -146,70 +146,91 @@ __device__ __forceinline__ uint4 fp8x8_to_16(uint2 w) {
 }
 
 // Four int8 values -> four 16-bit elements of the compute type, exactly (|x| <= 128 fits the 8 significant bits
-// of bf16).  The bytes are biased to 0..255 and planted in the mantissa of a constant whose unit in the last place
-// is one, and the constant and the bias are subtracted again: for fp16 two elements at a time (0x6400 | u is
-// 1024 + u), for bf16 through fp32 (0x4B000000 | u is 2^23 + u), whose upper half is the bf16 value.
-// v_perm_b32 picks result bytes from {first operand, second operand}: selector 0..3 = bytes of the second,
-// 4..7 = bytes of the first, 0x0c = zero.
+// of bf16).  One conversion instruction per element: the sub-dword addressing of the vector ALU picks byte k of the
+// word, sign-extends it, and (fp16) writes the result into one half of the destination register; bf16 goes through
+// fp32, whose upper half is the bf16 value, and one byte permute packs a pair.
 template <typename Tag>
 __device__ __forceinline__ uint2 int8x4_to_16(uint32_t w) {
-    const uint32_t u = w ^ 0x80808080u;
     uint2 r;
     if constexpr (std::is_same<Tag, f16_tag>::value) {
-        typedef _Float16 half2_t __attribute__((ext_vector_type(2)));
-        const half2_t bias = {(_Float16)-1152.0f, (_Float16)-1152.0f};
-        const uint32_t lo = __builtin_amdgcn_perm(0x64646464u, u, 0x04010400u);  // {0x64, u1, 0x64, u0}
-        const uint32_t hi = __builtin_amdgcn_perm(0x64646464u, u, 0x04030402u);  // {0x64, u3, 0x64, u2}
-        r.x = __builtin_bit_cast(uint32_t, __builtin_bit_cast(half2_t, lo) + bias);
-        r.y = __builtin_bit_cast(uint32_t, __builtin_bit_cast(half2_t, hi) + bias);
+        asm("v_cvt_f16_i16_sdwa %0, sext(%1) dst_sel:WORD_0 dst_unused:UNUSED_PAD src0_sel:BYTE_0" : "=v"(r.x) : "v"(w));
+        asm("v_cvt_f16_i16_sdwa %0, sext(%1) dst_sel:WORD_1 dst_unused:UNUSED_PRESERVE src0_sel:BYTE_1" : "+v"(r.x) : "v"(w));
+        asm("v_cvt_f16_i16_sdwa %0, sext(%1) dst_sel:WORD_0 dst_unused:UNUSED_PAD src0_sel:BYTE_2" : "=v"(r.y) : "v"(w));
+        asm("v_cvt_f16_i16_sdwa %0, sext(%1) dst_sel:WORD_1 dst_unused:UNUSED_PRESERVE src0_sel:BYTE_3" : "+v"(r.y) : "v"(w));
     } else {
-        constexpr float kBias = 8388608.0f + 128.0f;
-        const float f0 = __builtin_bit_cast(float, __builtin_amdgcn_perm(0x4B000000u, u, 0x070c0c00u)) - kBias;
-        const float f1 = __builtin_bit_cast(float, __builtin_amdgcn_perm(0x4B000000u, u, 0x070c0c01u)) - kBias;
-        const float f2 = __builtin_bit_cast(float, __builtin_amdgcn_perm(0x4B000000u, u, 0x070c0c02u)) - kBias;
-        const float f3 = __builtin_bit_cast(float, __builtin_amdgcn_perm(0x4B000000u, u, 0x070c0c03u)) - kBias;
+        // (the compiler turns each cast into v_cvt_f32_i32 with a sign-extended byte operand)
+        const float f0 = (float)(int8_t)(w), f1 = (float)(int8_t)(w >> 8);
+        const float f2 = (float)(int8_t)(w >> 16), f3 = (float)(int8_t)(w >> 24);
+        // v_perm_b32 picks result bytes from {first operand, second operand}: selector 0..3 = bytes of the second,
+        // 4..7 = bytes of the first
         r.x = __builtin_amdgcn_perm(__builtin_bit_cast(uint32_t, f1), __builtin_bit_cast(uint32_t, f0), 0x07060302u);
         r.y = __builtin_amdgcn_perm(__builtin_bit_cast(uint32_t, f3), __builtin_bit_cast(uint32_t, f2), 0x07060302u);
     }
     return r;
 }
 
-// Eight four-bit integers (one 32-bit word, element i in bits 4 i .. 4 i + 3) -> eight sign-extended bytes in element
-// order.  Low and high nibbles are separated, interleaved again with two byte permutes, and each byte is
-// sign-extended from four bits without carries between the bytes: (u ^ 8 | 0x80) - 8 lies in 0x78 .. 0x87, and
-// flipping the top bit again gives u - 8 ... the value of the nibble as a two's-complement byte.
-__device__ __forceinline__ uint2 int4x8_to_int8(uint32_t w) {
-    const uint32_t lo = w & 0x0F0F0F0Fu;         // elements 0, 2, 4, 6
-    const uint32_t hi = (w >> 4) & 0x0F0F0F0Fu;  // elements 1, 3, 5, 7
-    // v_perm_b32 selector: 0 .. 3 = bytes of the second operand, 4 .. 7 = bytes of the first
-    const uint32_t d0 = __builtin_amdgcn_perm(hi, lo, 0x05010400u);  // elements 0, 1, 2, 3
-    const uint32_t d1 = __builtin_amdgcn_perm(hi, lo, 0x07030602u);  // elements 4, 5, 6, 7
-    uint2 r;
-    r.x = ((((d0 ^ 0x08080808u) | 0x80808080u) - 0x08080808u) ^ 0x80808080u);
-    r.y = ((((d1 ^ 0x08080808u) | 0x80808080u) - 0x08080808u) ^ 0x80808080u);
+// Factor by which int4x8_to_16 scales its values (the kernels divide it out of the per-head factors, exactly).
+constexpr float kInt4Widening = 16.0f;
+// Eight four-bit integers (one 32-bit word, element i in bits 4 i .. 4 i + 3, two's complement) -> eight 16-bit
+// elements of the compute type holding SIXTEEN TIMES their values, in element order.  A nibble moved to the upper half
+// of a byte whose lower half is zero is the signed byte 16 n, so two masks (and one shift) turn the word into the even
+// elements' bytes and the odd elements' bytes, and from there on it is the int8 conversion: about 1.4 (fp16) and 1.9
+// (bf16) vector instructions per element.  The factor 16 is a power of two: every product and sum downstream is the
+// exact multiple, and dividing the per-head factors by it gives the int8 cache's results bit for bit.
+template <typename Tag>
+__device__ __forceinline__ uint4 int4x8_to_16(uint32_t w) {
+    const uint32_t odd = w & 0xF0F0F0F0u;          // byte j: 16 x element 2 j + 1
+    const uint32_t even = (w << 4) & 0xF0F0F0F0u;  // byte j: 16 x element 2 j
+    uint4 r;
+    if constexpr (std::is_same<Tag, f16_tag>::value) {
+#define DA_CVT_PAIR(dst, B)                                                                                               \
+    asm("v_cvt_f16_i16_sdwa %0, sext(%1) dst_sel:WORD_0 dst_unused:UNUSED_PAD src0_sel:BYTE_" #B : "=v"(dst) : "v"(even)); \
+    asm("v_cvt_f16_i16_sdwa %0, sext(%1) dst_sel:WORD_1 dst_unused:UNUSED_PRESERVE src0_sel:BYTE_" #B : "+v"(dst) : "v"(odd));
+        DA_CVT_PAIR(r.x, 0)
+        DA_CVT_PAIR(r.y, 1)
+        DA_CVT_PAIR(r.z, 2)
+        DA_CVT_PAIR(r.w, 3)
+#undef DA_CVT_PAIR
+    } else {
+        auto pair = [&](int sh) {
+            const float lo = (float)(int8_t)(even >> sh), hi = (float)(int8_t)(odd >> sh);
+            return __builtin_amdgcn_perm(__builtin_bit_cast(uint32_t, hi), __builtin_bit_cast(uint32_t, lo), 0x07060302u);
+        };
+        r.x = pair(0);
+        r.y = pair(8);
+        r.z = pair(16);
+        r.w = pair(24);
+    }
     return r;
 }
-// Sixteen (eight) elements of an int4 cache at the doubled address `vptr` (see kKvInt4), as sign-extended bytes.
+// Sixteen (eight) elements of an int4 cache at the doubled address `vptr` (see kKvInt4): the packed words, each in
+// the slot where the 8-bit formats keep the eight bytes of the same elements (the other word of the pair is unused).
 __device__ __forceinline__ uint4 kv4_load16(const void* vptr) {
     const uint2 w = *reinterpret_cast<const uint2*>(reinterpret_cast<uintptr_t>(vptr) >> 1);
-    const uint2 a = int4x8_to_int8(w.x), b = int4x8_to_int8(w.y);
-    return make_uint4(a.x, a.y, b.x, b.y);
+    return make_uint4(w.x, 0u, w.y, 0u);
 }
 __device__ __forceinline__ uint2 kv4_load8(const void* vptr) {
-    return int4x8_to_int8(*reinterpret_cast<const uint32_t*>(reinterpret_cast<uintptr_t>(vptr) >> 1));
+    return make_uint2(*reinterpret_cast<const uint32_t*>(reinterpret_cast<uintptr_t>(vptr) >> 1), 0u);
 }
 
 // Eight elements of an 8-bit K/V cache of format FMT -> eight 16-bit elements of the compute type (an int4 cache's
-// elements have been widened to int8 by the load).
+// eight elements are the nibbles of w.x, and come out scaled by kInt4Widening).
 template <typename Tag, int FMT>
 __device__ __forceinline__ uint4 kv8x8_to_16(uint2 w) {
     static_assert(FMT == kKvFp8 || FMT == kKvInt8 || FMT == kKvInt4, "8-bit K/V format");
     if constexpr (FMT == kKvFp8) {
         return fp8x8_to_16<Tag>(w);
+    } else if constexpr (FMT == kKvInt4) {
+        return int4x8_to_16<Tag>(w.x);
     } else {
         const uint2 a = int8x4_to_16<Tag>(w.x), b = int8x4_to_16<Tag>(w.y);
         return make_uint4(a.x, a.y, b.x, b.y);
     }
+}
+// What the conversion multiplied the elements by, inverted (divided out of the per-head factors).
+template <int FMT>
+__device__ __forceinline__ float kv_widening_inverse() {
+    return FMT == kKvInt4 ? 1.0f / kInt4Widening : 1.0f;
 }
 
 // f(integral_constant<int, B>), ..., f(integral_constant<int, E-1>): a loop whose index is a constant

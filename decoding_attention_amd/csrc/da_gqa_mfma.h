@@ -194,8 +194,9 @@ __device__ __forceinline__ void gqa_segment(const SweepParams& p, uint8_t* const
     const uint8_t* const kbytes = reinterpret_cast<const uint8_t*>(p.k) + (size_t)hk * D * KB;
     const uint8_t* const vbytes = reinterpret_cast<const uint8_t*>(p.v) + (size_t)hk * p.v_head * KB;
     const uint32_t k_row_b = (uint32_t)p.k_row * KB, v_row_b = (uint32_t)p.v_row * KB;
-    const float sl = p.scale_log2 * head_scale(p.k_scale, hk);  // score scale, log2 units
-    const float vs = head_scale(p.v_scale, hk);
+    // (an int4 cache's elements come out of the conversion times a power of two, divided out here)
+    const float sl = p.scale_log2 * head_scale(p.k_scale, hk) * kv_widening_inverse<KV8>();  // score scale, log2 units
+    const float vs = head_scale(p.v_scale, hk) * kv_widening_inverse<KV8>();
 
     // wave-private V tile in LDS
     uint8_t* const vt = smem + wave * (kGqaTile * VP);

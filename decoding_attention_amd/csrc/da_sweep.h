@@ -90,8 +90,9 @@ __global__ __launch_bounds__(256) void sweep_kernel(const SweepParams p) {
     // rows are addressed one by one (row_ref), so paged K/V of any page size costs one table lookup per row
     const uint8_t* kbase = reinterpret_cast<const uint8_t*>(p.k) + ((size_t)hk * D + g * 8) * KB;
     const uint8_t* vbase = reinterpret_cast<const uint8_t*>(p.v) + ((size_t)hk * p.v_head + g * 8) * KB;
-    const float sl = p.scale_log2 * head_scale(p.k_scale, hk);  // score scale, log2 units
-    const float vs = head_scale(p.v_scale, hk);
+    // (an int4 cache's elements come out of the conversion times a power of two, divided out here)
+    const float sl = p.scale_log2 * head_scale(p.k_scale, hk) * kv_widening_inverse<KV8>();  // score scale, log2 units
+    const float vs = head_scale(p.v_scale, hk) * kv_widening_inverse<KV8>();
     auto load8 = [](const uint8_t* ptr) __attribute__((always_inline)) {  // eight elements as 16-bit pairs
         if constexpr (KV8 == kKvInt4)
             return kv8x8_to_16<Tag, KV8>(kv4_load8(ptr));  // (four bytes from half the address)

@@ -151,3 +151,30 @@ def test_paged_large_ragged_batch_takes_the_balanced_grid():
     rows = [0, 1, 7, 17]
     sub = sub_workload(w, rows)
     check_against_oracle(sub, o[rows])
+
+
+@pytest.mark.parametrize("hq,hk,dim,dtype", [(32, 8, 128, torch.bfloat16), (32, 1, 128, torch.float16),
+                                             (16, 4, 64, torch.float16)])
+def test_large_batch_without_a_token_count_takes_the_balanced_grid(hq, hk, dim, dtype):
+    """The reference's signature carries no token count (csrc/ops/decoding_attn.h:29-30): a batch large enough for
+    whole shares takes the balanced grid all the same, the share derived on the device.  Ragged lengths with empty
+    sequences, every row against the oracle, through da_decoding_attn itself; and a workspace poisoned with NaN
+    (stale slots must never be read) through da_decoding_attn_ex with hint 0."""
+    g = torch.Generator().manual_seed(31)
+    lens = torch.randint(1, 8193, (40,), generator=g).tolist()
+    lens[3], lens[17], lens[39] = 0, 8192, 1
+    w = _workload(lens, hq, hk, dim, dtype, seed=32)
+    b = len(lens)
+    assert _lib.plan(w.max_seq_k, b, hq, hk, dim, dim)["balanced"]
+    lib = _lib.load()
+    wd = w.to(DEV)
+    o = torch.full((b, hq, dim), float("nan"), dtype=dtype, device=DEV)
+    rc = lib.da_decoding_attn(wd.q.data_ptr(), wd.k.data_ptr(), wd.v.data_ptr(), o.data_ptr(), wd.cu_seq_k.data_ptr(),
+                              w.max_seq_k, b, hq, hk, dim, dim, 0, int(dtype == torch.bfloat16),
+                              torch.cuda.current_stream().cuda_stream)
+    assert rc == 0, _lib.last_error()
+    torch.cuda.synchronize()
+    check_against_oracle(w, o.cpu())
+    assert torch.count_nonzero(o[3]) == 0
+    o2 = run_hip_ex(w, 0, fill=0xFF)
+    assert torch.equal(o2.view(torch.int16), o.cpu().view(torch.int16))
