@@ -168,7 +168,9 @@ Plan make_plan(size_t max_seq_k, size_t batch, size_t head_q, size_t head_k, siz
     // (65 heads and more over 16-bit K run on the software-pipelined latent kernel, which wins from a quarter of that
     // bound on: 128 heads, batch 1 x 4096 tokens 21.6 -> 19.8 us, batch 2 x 4096 26.2 -> 24.3, batch 16 x 512 27.1 ->
     // 24.6; batch 1 x 512 stays, 16.5 against 17.7, batch 1 x 2048 is a tie)
-    const bool pipe_kernel = latent && ratio > 64 && !kv_8bit;
+    // (its 8-bit form serves rows of one KV head in runs of 16 tokens: the packed layout and pages of 16 tokens and more)
+    const bool pipe_kernel = latent && ratio > 64 &&
+                             (!kv_8bit || (head_k == 1 && (packed || page_size >= 16) && !no_latent_kernel && !da::mla_pipe_kv8_off()));
     const long long groups16 = (ratio + 15) / 16;
     const long long group_rows = groups16 * (long long)batch * (long long)max_seq_k;
     const long long small_bound =

@@ -19,6 +19,10 @@ inline bool mla_half_partials(bool latent_kernel, int rt, size_t head_q, size_t 
 }
 // the software-pipelined kernel for work-groups of 128 heads over 16-bit K (da_mla_pipe.hip); launch_mla routes to it
 hipError_t launch_mla_pipe(const SweepParams& p, bool is_bf16, dim3 grid, hipStream_t stream);
+// its form over an 8-bit K cache of format fmt (kKvFp8 or kKvInt8), for the layouts mla_pipe_kv8_supported names
+bool mla_pipe_kv8_supported(const SweepParams& p);
+bool mla_pipe_kv8_off();  // DA_MLA_PIPE_KV8=0: 8-bit K stays on the compiler-scheduled kernel (measurements)
+hipError_t launch_mla_pipe_kv8(const SweepParams& p, int fmt, bool is_bf16, dim3 grid, hipStream_t stream);
 // the (576, 512) shape with V in a buffer of its own (16-bit K/V; packed, or pages of 16 tokens and more)
 hipError_t launch_mla_vd(const SweepParams& p, bool is_bf16, int rt, dim3 grid, hipStream_t stream);
 // the same over an 8-bit K cache of format fmt (kKvFp8 or kKvInt8)

@@ -44,6 +44,7 @@ namespace {
 
 using namespace mla;
 
+
 // PG: paged K/V with pages of fewer than 16 tokens (down to 1): every row of a tile has its own page lookup.
 // NB: tile buffers of the 16-bit form.  Three keep two tiles in flight behind the one being read; two (one in
 // flight) halve the LDS footprint, so that two work-groups of one or two waves share a CU.
@@ -676,15 +677,28 @@ hipError_t launch_tag(const SweepParams& p, int rt, dim3 grid, hipStream_t strea
         case 64: return launch_one<Tag, 576, 512, 2, KV8>(p, grid, stream);
         case 128:
             // 16-bit K: the software-pipelined kernel (da_mla_pipe.hip); this kernel's four-wave form serves 8-bit K
-            if constexpr (KV8 == 0)
+            if constexpr (KV8 == 0) {
                 return launch_mla_pipe(p, std::is_same<Tag, bf16_tag>::value, grid, stream);
-            else
+            } else {
+                // (the pipelined kernel's 8-bit form where the live heads fill a work-group's second pair of waves and
+                // the layout suits it; this kernel's four-wave form otherwise)
+                if (p.ratio > 64 && mla_pipe_kv8_supported(p) && !mla_pipe_kv8_off())
+                    return launch_mla_pipe_kv8(p, KV8, std::is_same<Tag, bf16_tag>::value, grid, stream);
                 return launch_one<Tag, 576, 512, 4, KV8>(p, grid, stream);
+            }
         default: return hipErrorInvalidValue;
     }
 }
 
 }  // namespace
+
+bool mla_pipe_kv8_off() {
+    static const bool v = [] {
+        const char* s = getenv("DA_MLA_PIPE_KV8");
+        return s && *s && atoi(s) == 0;
+    }();
+    return v;
+}
 
 int mla_two_per_cu_from() {
     static const int v = [] {

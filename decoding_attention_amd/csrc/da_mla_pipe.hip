@@ -48,6 +48,22 @@ using namespace mla;
 
 constexpr int kPipeBufs = 4;  // LDS tile buffers
 constexpr int kRing = 8;      // LDS fragments requested ahead of the matrix step that uses them
+constexpr int kDmaRaw = 200;  // phase A's DMA argument: the loads of a raw (8-bit) tile, one every eight steps
+// byte offsets of a thread's conversion slot c: of the source in the stage (rows of 576 bytes), of the destination in
+// its region (value rows of 1024 bytes, 16-byte columns 16 apart; key-tail rows of 128 bytes)
+constexpr int conv_src_off(int c) { return (c / 5) * 16 * 576 + (c % 5) * 128; }
+constexpr int conv_dst_off(int c) { return c % 5 < 4 ? (c / 5) * 16 * 1024 + (c % 5) * 256 : (c / 5) * 16 * 128; }
+constexpr int kConvSlots = 10;  // 8-byte chunks of a raw tile per thread: two rows x (4 value chunks + the tail chunk)
+// LDS operations of the 8-bit form's conversion issued in steps lo .. hi of phase A: a read behind steps 0, 3, ..., 27
+// and `wr` writes behind steps 2, 5, ..., 29
+constexpr int conv_ops_between(int lo, int hi, int wr) {
+    int n = 0;
+    for (int s = lo < 0 ? 0 : lo; s <= hi; ++s) {
+        if (s % 3 == 0 && s / 3 < kConvSlots) ++n;
+        if (s % 3 == 2 && s / 3 < kConvSlots) n += wr;
+    }
+    return n;
+}
 
 typedef short s16x8 __attribute__((__vector_size__(8 * sizeof(short))));
 
@@ -150,7 +166,16 @@ template <int K>
 __device__ __forceinline__ void sc_bf16_hi(float& dst) { asm volatile("v_and_b32 %0, 0xffff0000, v[%1]" : "=v"(dst) : "n"(kScV + K)); }
 
 // PG: paged K/V with pages of fewer than 16 tokens (down to 1): every row of a tile has its own page lookup.
-template <typename Tag, bool PG>
+// KV8: K holds 8-bit elements (kKvFp8 or kKvInt8) in rows of 576 bytes (one KV head).  A tile's bytes then stream into
+// one of three raw stages (18 KiB, row after row), and the work-group converts a staged tile into the 16-bit tile
+// layout two tiles ahead of its use: in the steady-state loop between the matrix steps of phase A (thread (row, j)
+// reads the row's 8-byte chunks j, j + 8, ..., converts each to eight 16-bit values -- exactly -- and writes them to
+// their swizzled place), in the other trips in one go behind the trip's barrier.  Everything downstream of the 16-bit
+// tile is the same instruction sequence, so with unit scales the output equals the 16-bit call's on the widened
+// values bit for bit.  LDS: three value regions (the 512 value columns of a tile: one being written, one read as K,
+// one read as V), two regions for the remaining 64 key columns (needed only while a tile is written or read as K)
+// and the three stages, 158 KiB.
+template <typename Tag, bool PG, int KV8 = 0>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_num_vgpr(kScV))) void latent_pipe_kernel(const SweepParams p) {
     // the register file as this kernel uses it: v0 .. v255 and a0 .. a255 (the compiler itself stays below v64)
     asm volatile("" ::: "v255", "a255");
@@ -169,6 +194,17 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_num_vgpr(kScV))) void la
     constexpr int NV = CT * 2;              // matrix steps of O += V^T P^T
     constexpr int NB = kPipeBufs;
     static_assert(NLB == 1 && KS == 36 && NV == 32, "schedule below is written for (576, 512), four waves");
+    static_assert(!(KV8 && PG), "the 8-bit form takes whole runs of 16 tokens");
+    // 8-bit K: region A (value columns) of tile i lives at (i % 3) * ABUF, its region B at OFF_BB + (i % 2) * BBUF,
+    // its raw bytes in stage i % 3
+    constexpr int KB = KV8 ? 1 : 2;           // bytes per K element in memory
+    constexpr int ABUF = kTile * ROW_A;       // 32 KiB
+    constexpr int BBUF = kTile * ROW_B;       // 4 KiB
+    constexpr int OFF_BB = 3 * ABUF;
+    constexpr int OFF_STG = OFF_BB + 2 * BBUF;
+    constexpr int STG = kTile * D;            // bytes of a raw tile
+    constexpr int NLW8 = 5;                   // load instructions per raw tile per wave: four of 1 KiB, one of 512 bytes
+    static_assert(STG == 16 * 1024 + 4 * 512 && (16 * D) % 1024 == 0, "raw tile: 16 whole loads + four half loads; a run of 16 rows ends on a load boundary");
 
 #ifdef DA_PIPE_PROBE
     const long long pr_wk = wall_clock64();
@@ -215,16 +251,17 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_num_vgpr(kScV))) void la
     }
 
     const int q_last = max(nh, 1) - 1;
-    const int hq = min(h_base + min(n, q_last), p.head_q - 1);
     const uint32_t lane16 = lane * 16;
     const int rb = lane >> 3;  // region B: row within the group of eight, chunk lane & 7
+    const int hq = min(h_base + min(n, q_last), p.head_q - 1);
     const float slope = p.is_alibi ? alibi_slope_log2(p.slopes, hq, p.head_q) : 0.0f;
 
     float m = kNegBig, l = 0.0f;
 
-    const uint8_t* const kbytes = reinterpret_cast<const uint8_t*>(p.k) + (size_t)hk * D * 2;
-    const size_t k_row_bytes = (size_t)p.k_row * 2;
-    const float sl = p.scale_log2;  // score scale, log2 units
+    const uint8_t* const kbytes = reinterpret_cast<const uint8_t*>(p.k) + (size_t)hk * D * KB;
+    const size_t k_row_bytes = (size_t)p.k_row * KB;
+    // score scale, log2 units (8-bit K: times the KV head's de-quantisation factor)
+    const float sl = KV8 ? p.scale_log2 * head_scale(p.k_scale, hk) : p.scale_log2;
 
     // One direct-to-LDS load of a tile: region-A row wave + 4 q for q < NLA, then the wave's eight region-B rows.
     // `base` / `base1`: addresses of the rows of the tile's tokens 0 and 16 (a tile is fetched as two runs of 16
@@ -260,7 +297,90 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_num_vgpr(kScV))) void la
     auto tile_rows = [&](int tok0) {
         const int64_t r0 = row_ref(p, b, start, tok0).k;
         const int64_t r1 = tok0 + 16 < c1 ? row_ref(p, b, start, tok0 + 16).k : r0;
-        return TileRows{kbytes + r0 * 2, kbytes + r1 * 2, c1 - 1 - tok0};
+        return TileRows{kbytes + r0 * KB, kbytes + r1 * KB, c1 - 1 - tok0};
+    };
+    // ---- 8-bit K: raw tiles and their conversion --------------------------------------------------------------------
+    // A raw tile is the tile's 32 x 576 bytes row after row (rows are 576 bytes apart in memory, so a run of 16 tokens
+    // is 9 KiB of contiguous memory).  Every wave issues five loads per tile: 1 KiB pieces wave, wave + 4, wave + 8,
+    // wave + 12 and the 512-byte piece 16 KiB + 512 wave (lanes 0 .. 31).  base / base1: rows of tokens 0 and 16.
+    auto issue_raw_whole = [&](const uint8_t* base, const uint8_t* base1, uint32_t lds0) __attribute__((always_inline)) {
+        static_for<0, 4>([&](auto qc) {
+            const int j = wave + 4 * decltype(qc)::value;  // wave-uniform
+            const uint8_t* const src = (j >= 9 ? base1 - 9 * 1024 : base) + j * 1024;
+            lds_dma16<true>(src, lane16, lds0 + (uint32_t)(j * 1024));
+        });
+        if (lane < 32) lds_dma16<true>(base1 + (7 * 1024 + 512 * wave), lane16, lds0 + (uint32_t)(16 * 1024 + 512 * wave));
+    };
+    // piece q = 0 .. 4 of a whole raw tile (as issue_raw_whole), one at a time between matrix steps
+    auto issue_raw_piece = [&](auto qc, const uint8_t* base, const uint8_t* base1, uint32_t lds0) __attribute__((always_inline)) {
+        constexpr int q = decltype(qc)::value;
+        if constexpr (q < 4) {
+            const int j = wave + 4 * q;  // wave-uniform
+            lds_dma16<true>((j >= 9 ? base1 - 9 * 1024 : base) + j * 1024, lane16, lds0 + (uint32_t)(j * 1024));
+        } else {
+            if (lane < 32) lds_dma16<true>(base1 + (7 * 1024 + 512 * wave), lane16, lds0 + (uint32_t)(16 * 1024 + 512 * wave));
+        }
+    };
+    auto issue_raw = [&](int tok0, int stg) {
+        const TileRows tr = tile_rows(tok0);
+        const uint32_t lds0 = smem_off + (uint32_t)(OFF_STG + stg * STG);
+        if (tr.last >= kTile - 1) {
+            issue_raw_whole(tr.base, tr.base1, lds0);
+            return;
+        }
+        // the split's last tile: rows past the end re-read the last row (they are masked later), per-lane addresses
+        // (the lane's offset passes through an opaque statement: the row arithmetic is then worked out at each call
+        // instead of once in the prologue and kept in registers across the loop)
+        uint32_t l16 = lane16;
+        asm volatile("" : "+v"(l16));
+        auto piece = [&](uint32_t at) {
+            const uint32_t sb = at + l16, row = sb / (uint32_t)D, within = sb - row * (uint32_t)D;
+            const int rc = min((int)row, tr.last), run = rc >> 4;
+            lds_dma16_v<true>((run ? tr.base1 : tr.base) + (size_t)(rc - 16 * run) * k_row_bytes + within, lds0 + at);
+        };
+        static_for<0, 4>([&](auto qc) { piece((uint32_t)((wave + 4 * decltype(qc)::value) * 1024)); });
+        if (lane < 32) piece((uint32_t)(16 * 1024 + 512 * wave));
+    };
+    // Conversion of a staged tile into value region a_off and key-tail region b_off (byte offsets in LDS).  Thread
+    // (row r = tid / 16, j = tid % 16) converts, for the rows r and r + 16, the 8-element chunks j, j + 16, j + 32, j + 48
+    // of the value columns and, for j < 8, chunk 64 + j (the remaining key columns): ten slots, the last of each row with
+    // half the lanes.  Sixteen lanes of a row write sixteen different 16-byte columns (the swizzle permutes them among
+    // themselves), so the writes are free of bank conflicts, and since the swizzles of rows r and r + 16 are equal every
+    // slot is a constant offset from one source and two destination addresses.
+    // (the thread's three addresses are worked out from its index where they are needed, a dozen instructions, rather
+    // than kept in registers across the loop: the compiler's 64 registers do not have the room)
+    struct ConvAddr {
+        uint32_t src, dst_a, dst_b;
+    };
+    auto conv_addr = [&](uint32_t stg_off, uint32_t a_off, uint32_t b_off) __attribute__((always_inline)) {
+        uint32_t tid = threadIdx.x;
+        asm volatile("" : "+v"(tid));  // (not to be hoisted out of the loop)
+        const int cv_j = (int)tid & 15, cv_r = (int)tid >> 4;
+        ConvAddr ca;
+        ca.src = smem_off + (uint32_t)(OFF_STG + cv_r * D + cv_j * 8) + stg_off;
+        ca.dst_a = smem_off + (uint32_t)(cv_r * ROW_A + ((cv_j ^ swz_a(cv_r)) * 16)) + a_off;
+        ca.dst_b = smem_off + (uint32_t)(OFF_BB + cv_r * ROW_B + (((cv_j & 7) ^ swz_b(cv_r)) * 16)) + b_off;
+        return ca;
+    };
+    // slot c = 0 .. 9 of a thread: rows r + 16 (c / 5); c % 5 < 4: value chunk j + 16 (c % 5), else the tail chunk
+    // (byte offsets of the source in the stage, of the destination in its region)
+    static_assert(D == 576 && ROW_A == 1024 && ROW_B == 128, "conv_src_off / conv_dst_off");
+    auto convert_burst = [&](int stg, uint32_t a_off, uint32_t b_off) {
+        typedef unsigned int u32x2 __attribute__((ext_vector_type(2)));
+        typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
+        typedef const __attribute__((address_space(3))) u32x2* lds_src;
+        typedef __attribute__((address_space(3))) u32x4* lds_dst;
+        const ConvAddr ca = conv_addr((uint32_t)(stg * STG), a_off, b_off);
+        const bool tail_lane = (threadIdx.x & 15) < 8;
+#pragma unroll
+        for (int c = 0; c < kConvSlots; ++c) {
+            if (c % 5 == 4 && !tail_lane) continue;
+            const u32x2 rv = *reinterpret_cast<lds_src>((uintptr_t)(ca.src + conv_src_off(c)));
+            // (this lambda is compiled, and never called, for 16-bit K as well)
+            const uint4 cv = kv8x8_to_16<Tag, KV8 ? KV8 : kKvFp8>(make_uint2(rv.x, rv.y));
+            const uint32_t dst = (c % 5 < 4 ? ca.dst_a : ca.dst_b) + conv_dst_off(c);
+            *reinterpret_cast<lds_dst>((uintptr_t)dst) = u32x4{cv.x, cv.y, cv.z, cv.w};
+        }
     };
     auto issue_tile = [&](int tok0, int buf) {
         const TileRows tr = tile_rows(tok0);
@@ -321,25 +441,29 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_num_vgpr(kScV))) void la
         const uint8_t* const qb = reinterpret_cast<const uint8_t*>(p.q) + (size_t)b * p.head_q * (D * 2);
         const int first = hk * p.ratio + grp * 32 * NWV + blk * 32;  // first head of the block
         const int last_row = max(min(32, wg_heads - blk * 32), 1) - 1;  // rows past the block's live heads repeat one
-        const uint32_t qbuf = smem_off + (uint32_t)((2 + (blk & 1)) * BUF);
+        // (8-bit K: through value regions 0 and 1 and the two key-tail regions, while the first raw tiles land in
+        // the stages)
+        const uint32_t qbuf_a = smem_off + (uint32_t)(KV8 ? (blk & 1) * ABUF : (2 + (blk & 1)) * BUF);
+        const uint32_t qbuf_b = smem_off + (uint32_t)(KV8 ? OFF_BB + (blk & 1) * BBUF : (2 + (blk & 1)) * BUF + OFF_B);
 #pragma unroll
         for (int q = 0; q < NLA; ++q) {
             const int row = wave + NWV * q;  // wave-uniform
             const int head = min(first + min(row, last_row), p.head_q - 1);
             lds_dma16(qb, (uint32_t)head * (uint32_t)(D * 2) + (lane16 ^ (uint32_t)(swz_a(row) * 16)),
-                      qbuf + (uint32_t)(row * ROW_A));
+                      qbuf_a + (uint32_t)(row * ROW_A));
         }
         {
             const int row = wave * 8 + rb;
             const int head = min(first + min(row, last_row), p.head_q - 1);
             lds_dma16(qb, (uint32_t)head * (uint32_t)(D * 2) + (uint32_t)(DV * 2 + (((lane & 7) ^ swz_b(row)) * 16)),
-                      qbuf + (uint32_t)(OFF_B + wave * 1024));
+                      qbuf_b + (uint32_t)(wave * 1024));
         }
     };
     auto read_q = [&]() {
-        const uint32_t qbuf = smem_off + (uint32_t)((2 + (wave & 1)) * BUF);
-        const uint32_t qa = qbuf + n * ROW_A + ((swz_a(n) ^ half) * 16);
-        const uint32_t qbb = qbuf + OFF_B + n * ROW_B + ((swz_b(n) ^ half) * 16);
+        const uint32_t qbuf_a = smem_off + (uint32_t)(KV8 ? (wave & 1) * ABUF : (2 + (wave & 1)) * BUF);
+        const uint32_t qbuf_b = smem_off + (uint32_t)(KV8 ? OFF_BB + (wave & 1) * BBUF : (2 + (wave & 1)) * BUF + OFF_B);
+        const uint32_t qa = qbuf_a + n * ROW_A + ((swz_a(n) ^ half) * 16);
+        const uint32_t qbb = qbuf_b + n * ROW_B + ((swz_b(n) ^ half) * 16);
         static_for<0, KS>([&](auto ic) {
             constexpr int ks = decltype(ic)::value;
             uint32_t tmp;
@@ -352,7 +476,14 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_num_vgpr(kScV))) void la
     };
     issue_q_share(0);
     issue_q_share(1);
-    issue_any(0);  // (c0 < c1: there is a tile 0)
+    if constexpr (KV8) {
+        // the first three raw tiles go out behind the first round of Q (the stages are free from the start)
+        issue_raw(c0, 0);
+        if (1 < ntiles) issue_raw(c0 + kTile, 1);
+        if (2 < ntiles) issue_raw(c0 + 2 * kTile, 2);
+    } else {
+        issue_any(0);  // (c0 < c1: there is a tile 0)
+    }
     // The output tiles start at zero: 512 register writes, 2048 clocks of a wave alone on its SIMD.  Half of them while
     // the first loads are on their way (all of them would outlast the loads), the other half while the other pair of
     // waves reads its Q blocks.
@@ -364,16 +495,28 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_num_vgpr(kScV))) void la
     constexpr std::integral_constant<int, CT * 8> acc_mid{};
     constexpr std::integral_constant<int, CT * 16> acc_hi{};
     zero_acc(acc_lo, acc_mid);
-    wait_vmcnt<NLW>();  // (all but tile 0's)
+    if constexpr (KV8) {
+        // (all but the raw tiles')
+        if (2 < ntiles)
+            wait_vmcnt<3 * NLW8>();
+        else if (1 < ntiles)
+            wait_vmcnt<2 * NLW8>();
+        else
+            wait_vmcnt<NLW8>();
+    } else {
+        wait_vmcnt<NLW>();  // (all but tile 0's)
+    }
     __syncthreads();    // the Q blocks of waves 0 and 1 are in LDS
     if ((wave >> 1) == 0)
         read_q();
     else
         zero_acc(acc_mid, acc_hi);
-    __syncthreads();  // ... and in registers: buffers 2 and 3 take the blocks of waves 2 and 3
+    __syncthreads();  // ... and in registers: their buffers take the blocks of waves 2 and 3
     issue_q_share(2);
     issue_q_share(3);
-    if (1 < ntiles) {
+    if constexpr (KV8) {
+        wait_vmcnt<0>();  // (the raw tiles, issued before, have landed too)
+    } else if (1 < ntiles) {
         issue_any(1);
         wait_vmcnt<NLW>();  // (loads complete in order: tile 1's may stay outstanding)
     } else {
@@ -384,8 +527,16 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_num_vgpr(kScV))) void la
         read_q();
     else
         zero_acc(acc_mid, acc_hi);
-    __syncthreads();  // buffers 2 and 3 are free for K
-    if (2 < ntiles) issue_any(2);
+    __syncthreads();  // the Q buffers are free for K
+    if constexpr (KV8) {
+        // tile 0 into its 16-bit form (tile 1 follows between the matrix steps of S(0) below); then its stage takes raw
+        // tile 3
+        convert_burst(0, 0, 0);
+        __syncthreads();
+        if (3 < ntiles) issue_raw(c0 + 3 * kTile, 0);
+    } else {
+        if (2 < ntiles) issue_any(2);
+    }
 
     // The fast form of a tile's loads, for whole tiles (no row past the end) between the matrix steps of phase A: the
     // row part of the address is added to the tile's base in scalar registers, the lane part is one XOR.
@@ -419,12 +570,16 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_num_vgpr(kScV))) void la
     // K rows: lane (n, half) reads chunk 2 ks + half of row n.
     //   ks < 32: (base_a ^ 32 (ks & 7)) + 256 (ks >> 3)        ks >= 32: base_b ^ 32 (ks - 32)
     const uint32_t base_a = smem_off + n * ROW_A + ((swz_a(n) ^ half) * 16);
-    const uint32_t base_b = smem_off + OFF_B + n * ROW_B + ((swz_b(n) ^ half) * 16);
+    const uint32_t base_b = smem_off + (KV8 ? OFF_BB : OFF_B) + n * ROW_B + ((swz_b(n) ^ half) * 16);
+    // LDS offsets of tile i's value region (added to base_a / base_v) and of its key-tail region (added to base_b)
+    auto a_of = [](int i) { return KV8 ? (uint32_t)((i % 3) * ABUF) : (uint32_t)((i & (NB - 1)) * BUF); };
+    auto b_of = [](int i) { return KV8 ? (uint32_t)((i & 1) * BBUF) : (uint32_t)((i & (NB - 1)) * BUF); };
     // V^T: as a source lane of the transpose read this lane addresses row half*4 + q (+16 s2, +8 for the second
     // read), 8 bytes at chunk 4 c + 2 b1 + b0 of it, q = (lane & 15) >> 2, b1 = lane bit 4, b0 = lane bit 1:
     //   (base_v ^ (64 c | 32 hi)) + 16 KiB s2 + 8 KiB hi
     const uint32_t base_v = smem_off + (half * 4 + ((lane & 15) >> 2)) * ROW_A + 64 * ((lane & 15) >> 2) +
                             16 * ((2 * ((lane >> 4) & 1) + ((lane >> 1) & 1)) ^ half) + 8 * (lane & 1);
+
 
     const float bias0 = slope * (float)(half * 4 - (len - 1));  // ALiBi: slope * (token - (len - 1)), split in lane and tile parts
 
@@ -434,7 +589,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_num_vgpr(kScV))) void la
     // instruction of step g; ring slot g % kRing.
     // Addresses of the K reads of the tile being multiplied (region A: one register per k-step % 8, moved from buffer
     // to buffer once a trip; region B: XOR in front of the read)
-    constexpr int NKA = PG ? 1 : 8;
+    constexpr int NKA = (PG || KV8) ? 1 : 8;  // (the 8-bit form needs the registers for its conversion)
     uint32_t ka[NKA];
     uint32_t xa = 0, xb = 0;  // V^T read addresses of the current column tile
     uint32_t xt = 0;          // scratch for K read addresses
@@ -449,7 +604,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_num_vgpr(kScV))) void la
     auto read_k = [&](auto ksc, uint32_t tb, auto ro_c) __attribute__((always_inline)) {
         constexpr int ks = decltype(ksc)::value;
         constexpr int slot = (ks + decltype(ro_c)::value) % kRing;
-        if constexpr (ks < 32 && PG)
+        if constexpr (ks < 32 && NKA == 1)
             ring_read_b128<kRingV + 4 * slot, 32 * (ks & 7), (ks >> 3) * 256>(ka[0], xt);
         else if constexpr (ks < 32)
             ring_read_b128<kRingV + 4 * slot, 0, (ks >> 3) * 256>(ka[ks & 7], xt);
@@ -508,15 +663,69 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_num_vgpr(kScV))) void la
         if constexpr (j == 10) asm volatile("v_max_f32 %0, %0, %1" : "+v"(mxr) : "v"(tlo));
     };
 
+    // ---- 8-bit K: the conversion of tile t+2 between the matrix steps of phase A ---------------------------------------
+    // Slot c = 0 .. 9 of this thread (see conv_addr) is read from the stage behind step 3 c's ring read and written,
+    // converted, behind step 3 c + 2's; both are LDS operations and count in the waits of the ring (conv_ops_between).
+    typedef unsigned int u32x2_t __attribute__((ext_vector_type(2)));
+    typedef unsigned int u32x4_t __attribute__((ext_vector_type(4)));
+    constexpr int kConvWrites = KV8 == kKvInt8 ? 2 : 1;  // LDS writes per converted chunk
+    uint32_t csrc = 0, cdst_a = 0, cdst_b = 0;  // this trip's source and destinations (thread's row and chunk)
+    u32x2_t craw = {0u, 0u};
+    auto conv_read = [&](auto cc) __attribute__((always_inline)) {
+        constexpr int c = decltype(cc)::value;
+        u32x2_t& raw = craw;  // (named outside the dependent statement, so that the lambda captures them)
+        const uint32_t src = csrc;
+        if constexpr (c % 5 == 4) {
+            if ((threadIdx.x & 15) < 8) asm volatile("ds_read_b64 %0, %1 offset:%2" : "+v"(raw) : "v"(src), "n"(conv_src_off(c)));
+        } else {
+            asm volatile("ds_read_b64 %0, %1 offset:%2" : "=v"(raw) : "v"(src), "n"(conv_src_off(c)));
+        }
+    };
+    // VN: the phase goes on into phase B (the ring reads behind steps 28 and up are then two transpose reads each)
+    auto conv_write = [&](auto cc, auto vn_c) __attribute__((always_inline)) {
+        constexpr int c = decltype(cc)::value;
+        constexpr int g = 3 * c + 2;  // the step this runs behind
+        // the chunk's read has landed: behind it went the ring reads of this step and the one before
+        constexpr int r1 = g - 1 + kRing < KS ? 1 : (decltype(vn_c)::value ? 2 : 0);
+        constexpr int r0 = g + kRing < KS ? 1 : (decltype(vn_c)::value ? 2 : 0);
+        asm volatile("s_waitcnt lgkmcnt(%1)" : "+v"(craw) : "n"(r0 + r1));
+        constexpr bool kTail = c % 5 == 4;  // the row's last chunk: key columns 512 .. 575, lanes j < 8
+        const uint32_t dbase = kTail ? cdst_b : cdst_a;
+        constexpr int OFF = conv_dst_off(c);
+        auto write = [&]() __attribute__((always_inline)) {
+            if constexpr (kConvWrites == 2) {
+                // (int8: four elements at a time, so that two registers of results are live instead of four)
+                const uint2 lo = int8x4_to_16<Tag>(craw.x);
+                const u32x2_t vlo = {lo.x, lo.y};
+                asm volatile("ds_write_b64 %0, %1 offset:%2" ::"v"(dbase), "v"(vlo), "n"(OFF) : "memory");
+                const uint2 hi = int8x4_to_16<Tag>(craw.y);
+                const u32x2_t vhi = {hi.x, hi.y};
+                asm volatile("ds_write_b64 %0, %1 offset:%2" ::"v"(dbase), "v"(vhi), "n"(OFF + 8) : "memory");
+            } else {
+                const uint4 cv = kv8x8_to_16<Tag, KV8 ? KV8 : kKvFp8>(make_uint2(craw.x, craw.y));
+                const u32x4_t v = {cv.x, cv.y, cv.z, cv.w};
+                asm volatile("ds_write_b128 %0, %1 offset:%2" ::"v"(dbase), "v"(v), "n"(OFF) : "memory");
+            }
+        };
+        if constexpr (kTail) {
+            if ((threadIdx.x & 15) < 8) write();
+        } else {
+            write();
+        }
+    };
+
     // ---- phase A: S(t+1) = K(t+1) Q^T beside the softmax of S(t) and the loads of tile t+3 ------------------------
     // QK: the matrix steps (else only the softmax runs: last trip); SM: the softmax (else only the matrix steps:
     // prologue); DMA >= 0: the nine loads of a whole tile go out behind steps DMA, DMA + 4, ..., DMA + 32.  (A
     // direct-to-LDS load blocks its wave until the memory path accepts it, ~100 clocks at this kernel's 4 TB/s; giving
     // each of the four waves another DMA, so that their loads do not come together, measured slower, 2970 against
     // 2800 clocks per tile.)
+    // CONV (8-bit K, steady-state trips): the conversion of tile t+2 and the five loads of raw tile t+4 (DMA == kDmaRaw,
+    // behind steps 1, 9, ..., 33) ride along.
     auto phase_a = [&](auto qk_c, auto sm_c, auto dma_c, uint32_t tb, uint32_t tv, const uint8_t* base,
-                       const uint8_t* base1, uint32_t dma_lds, auto ro_c) __attribute__((always_inline)) {
+                       const uint8_t* base1, uint32_t dma_lds, auto ro_c, auto conv_c) __attribute__((always_inline)) {
         constexpr bool QK = decltype(qk_c)::value, SM = decltype(sm_c)::value;
+        constexpr bool CONV = decltype(conv_c)::value;
         constexpr int DMA = decltype(dma_c)::value;
         constexpr int RO = decltype(ro_c)::value;
         constexpr bool VNEXT = SM;  // a trip with a softmax continues with phase B
@@ -528,17 +737,28 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_num_vgpr(kScV))) void la
                 constexpr int last_issued = VNEXT ? g + kRing - 1 : (g + kRing - 1 < KS ? g + kRing - 1 : KS - 1);
                 constexpr int nk = (last_issued < KS ? last_issued : KS - 1) - g;           // K reads among them
                 constexpr int nv = last_issued >= KS ? last_issued - KS + 1 : 0;            // V steps among them
-                wait_lgkm_n<nk + 2 * nv>();
+                // (the counter of outstanding operations has four bits: waiting for fewer than are behind is safe)
+                constexpr int behind = nk + 2 * nv + (CONV ? conv_ops_between(g - kRing, g - 1, kConvWrites) : 0);
+                wait_lgkm_n<(behind < 15 ? behind : 15)>();
                 mma_s<Tag, kRingV + 4 * ((g + RO) % kRing), kQV + 4 * g, g == 0>(sacc);
                 if constexpr (g + kRing < KS)
                     read_k(std::integral_constant<int, g + kRing>{}, tb, ro_c);
                 else if constexpr (VNEXT)
                     read_v(std::integral_constant<int, g + kRing - KS>{}, tv, ro_c);
+                if constexpr (CONV) {
+                    if constexpr (g % 3 == 0 && g / 3 < kConvSlots) conv_read(std::integral_constant<int, g / 3>{});
+                    if constexpr (g % 3 == 2 && g / 3 < kConvSlots)
+                        conv_write(std::integral_constant<int, g / 3>{}, std::integral_constant<bool, VNEXT>{});
+                }
                 if constexpr (SM) {
                     constexpr int per = (SMN + 27) / 28;  // spread over the first 28 steps (the last 8 carry two reads)
                     static_for<(g * per < SMN ? g * per : SMN), ((g + 1) * per < SMN ? (g + 1) * per : SMN)>(sm_op);
                 }
-                if constexpr (DMA >= 0 && g % 4 == (DMA >= 0 ? DMA : 0)) issue_load_fast(std::integral_constant<int, g / 4>{}, base, base1, dma_lds);
+                if constexpr (DMA == kDmaRaw) {
+                    if constexpr (g % 8 == 1) issue_raw_piece(std::integral_constant<int, g / 8>{}, base, base1, dma_lds);
+                } else if constexpr (DMA >= 0 && g % 4 == (DMA >= 0 ? DMA : 0)) {
+                    issue_load_fast(std::integral_constant<int, g / 4>{}, base, base1, dma_lds);
+                }
             });
         } else {
             static_for<0, SMN>(sm_op);
@@ -570,7 +790,9 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_num_vgpr(kScV))) void la
             wait_lgkm_n<2 * nv + nk>();
             mma_o<Tag, kRingV + 4 * slot, kScV + 4 * (i & 1), 16 * (i >> 1)>();
             if constexpr (NEXTK && i == NV - AHEAD) {
-                wait_vmcnt<NLW>();  // this wave's share of tile t+2 has landed (tile t+3's loads may be outstanding)
+                // this wave's share of tile t+2 has landed (tile t+3's loads may be outstanding); 8-bit K: every wave
+                // has converted its share of tile t+2 (its writes lie behind the ring reads waited for since)
+                if constexpr (!KV8) wait_vmcnt<NLW>();
                 asm volatile("s_barrier" ::: "memory");
             }
             if constexpr (i + AHEAD < NV)
@@ -639,21 +861,33 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_num_vgpr(kScV))) void la
     };
 
     // ---- prologue: S(0) ---------------------------------------------------------------------------------------------
-    if (ntiles > 2)
-        wait_vmcnt<2 * NLW>();
-    else if (ntiles > 1)
-        wait_vmcnt<NLW>();
-    else
-        wait_vmcnt<0>();
-    __syncthreads();
+    if constexpr (!KV8) {  // (8-bit K: tile 0 was converted behind the barrier above)
+        if (ntiles > 2)
+            wait_vmcnt<2 * NLW>();
+        else if (ntiles > 1)
+            wait_vmcnt<NLW>();
+        else
+            wait_vmcnt<0>();
+        __syncthreads();
+    }
 #ifdef DA_PIPE_PROBE
     const long long pr_wq = wall_clock64();
 #endif
     {
         prime_k(base_b);
-        phase_a(std::true_type{}, std::false_type{}, std::integral_constant<int, -1>{}, base_b, base_v, nullptr, nullptr, 0, ro0);
+        if (KV8 != 0 && 1 < ntiles) {
+            const ConvAddr ca = conv_addr((uint32_t)STG, a_of(1), b_of(1));
+            csrc = ca.src;
+            cdst_a = ca.dst_a;
+            cdst_b = ca.dst_b;
+            phase_a(std::true_type{}, std::false_type{}, std::integral_constant<int, -1>{}, base_b, base_v, nullptr, nullptr, 0,
+                    ro0, std::integral_constant<bool, KV8 != 0>{});
+        } else {
+            phase_a(std::true_type{}, std::false_type{}, std::integral_constant<int, -1>{}, base_b, base_v, nullptr, nullptr, 0,
+                    ro0, std::false_type{});
+        }
 #pragma unroll
-        for (int j = 0; j < NKA; ++j) ka[j] += (uint32_t)BUF;  // on to buffer 1
+        for (int j = 0; j < NKA; ++j) ka[j] += a_of(1);  // on to tile 1
         // the compiler does not see the matrix instructions inside the assembly: cover the result latency of the
         // last one before anything reads the scores
         asm volatile("s_nop 15\n\ts_nop 7" : "+v"(sacc));
@@ -683,117 +917,205 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_num_vgpr(kScV))) void la
     // second, plain barrier at the top of a trip keeps the loads of tile t+3 behind every wave's last read of tile
     // t-1, whose buffer they fill.  Trips come in pairs (see RO at read_k).
     bool primed = false;  // the ring holds the first K fragments of tile t+1, which is in LDS for every wave
-    if (!PG && packed && !gen_all && t + NB < nfull) {
-        uint32_t cur = 0, nxt = (uint32_t)BUF, dst = (uint32_t)((NB - 1) * BUF);  // buffers of tiles t, t+1, t+3
-        wait_vmcnt<NLW>();  // tile 1 landed; tile 2 may still be in flight
-        __syncthreads();
-        prime_k(base_b + nxt);
-        auto steady_trip = [&](auto ro_c) __attribute__((always_inline)) {
-#if DA_PIPE_PROBE > 1
-            const long long pr_s0 = clock64();
-#endif
-            softmax_head(t, std::true_type{});
-#if DA_PIPE_PROBE > 1
-            const long long pr_s0b = clock64();
-#endif
-            asm volatile("s_barrier" ::: "memory");  // every wave is done with tile t-1
-#if DA_PIPE_PROBE > 1
-            const long long pr_s1 = clock64();
-            pr_x2 += pr_s1 - pr_s0b;
-            pr_top += pr_s1 - pr_s0;
-#endif
-            phase_a(std::true_type{}, std::true_type{}, std::integral_constant<int, 1>{}, base_b + nxt, base_v + cur, kt3,
-                    kt3 + 16 * k_row_bytes, smem_off + dst, ro_c);
-#if DA_PIPE_PROBE > 1
-            const long long pr_s2 = clock64();
-            pr_a += pr_s2 - pr_s1;
-#endif
-            kt3 += kTile * k_row_bytes;
-            const uint32_t nn = dst == (uint32_t)((NB - 1) * BUF) ? 0u : dst + (uint32_t)BUF;  // buffer after dst = that of tile t+4
-            // (tile t+2 lies in the buffer behind nxt)
-            const uint32_t nx2 = nxt == (uint32_t)((NB - 1) * BUF) ? 0u : nxt + (uint32_t)BUF;
-            phase_b(std::integral_constant<int, kRing>{}, std::true_type{}, base_v + cur, nx2 - nxt, ro_c, std::true_type{},
-                    base_b + nx2);
-#if DA_PIPE_PROBE > 1
-            pr_b += clock64() - pr_s2;
-#endif
-            cur = nxt;
-            nxt = nx2;
-            dst = nn;
-            ++t;
-        };
-        // (both trips of a pair load a whole tile: t + 3 and t + 4 lie below nfull)
-        for (; t + NB < nfull;) {
-            steady_trip(ro0);
-            steady_trip(ro1);
-        }
-        primed = true;
-    }
-    for (; t + 1 < ntiles; ++t) {
-#if DA_PIPE_PROBE > 1
-        const long long pr_s0 = clock64();
-#endif
-        const uint32_t cur = (uint32_t)((t & (NB - 1)) * BUF), nxt = (uint32_t)(((t + 1) & (NB - 1)) * BUF);
-        const bool fast = !PG && t + NB - 1 < nfull;
-        TileRows tr{nullptr, nullptr, 0};
-        if (fast) {
-            if (packed) {  // rows follow each other at the pitch
-                tr.base = kt3;
-                tr.base1 = kt3 + 16 * k_row_bytes;
-                kt3 += kTile * k_row_bytes;
-            } else {
-                tr = tile_rows(c0 + (t + NB - 1) * kTile);
+    if constexpr (KV8 != 0) {
+        // ---- 8-bit K.  Entering trip t, tiles t and t+1 are in LDS in 16-bit form, raw tiles t+2 and t+3 are on their
+        // way or there.  The trip converts tile t+2 and requests raw tile t+4 into the stage tile t+1 came from.
+        if (packed && !gen_all && t + 5 < nfull) {
+            // steady state: conversion and loads between the matrix steps, the ring runs on from trip to trip
+            uint32_t cur_a = a_of(0), nxt_a = a_of(1), nx2_a = a_of(2), nxt_b = b_of(1), nx2_b = b_of(2);
+            uint32_t stg_conv = (uint32_t)(2 * STG), stg_load = (uint32_t)(1 * STG);  // stages of raw tiles t+2, t+4
+            const uint8_t* kt4 = kbytes + (size_t)(start + c0 + 4 * kTile) * k_row_bytes;  // first row of tile t+4
+            __syncthreads();  // (tile 1 was converted on the way through S(0): now it is there for every wave)
+            prime_k(base_b + nxt_b);
+            auto steady_trip = [&](auto ro_c) __attribute__((always_inline)) {
+                softmax_head(t, std::true_type{});
+                wait_vmcnt<NLW8>();  // raw tile t+2 has landed (raw tile t+3's loads may be outstanding)
+                // every wave is done with tile t-1, whose value region tile t+2 is converted into (and with the stage
+                // of tile t+1, which raw tile t+4 is loaded into)
+                asm volatile("s_barrier" ::: "memory");
+                {
+                    const ConvAddr ca = conv_addr(stg_conv, nx2_a, nx2_b);
+                    csrc = ca.src;
+                    cdst_a = ca.dst_a;
+                    cdst_b = ca.dst_b;
+                }
+                phase_a(std::true_type{}, std::true_type{}, std::integral_constant<int, kDmaRaw>{}, base_b + nxt_b,
+                        base_v + cur_a, kt4, kt4 + 16 * k_row_bytes, smem_off + (uint32_t)OFF_STG + stg_load, ro_c,
+                        std::true_type{});
+                kt4 += kTile * k_row_bytes;
+                phase_b(std::integral_constant<int, kRing>{}, std::true_type{}, base_v + cur_a, nx2_a - nxt_a, ro_c,
+                        std::true_type{}, base_b + nx2_b);
+                const uint32_t nx3_a = nx2_a == (uint32_t)(2 * ABUF) ? 0u : nx2_a + (uint32_t)ABUF;
+                cur_a = nxt_a;
+                nxt_a = nx2_a;
+                nx2_a = nx3_a;
+                const uint32_t b_tmp = nxt_b;
+                nxt_b = nx2_b;
+                nx2_b = b_tmp;
+                stg_conv = stg_conv == (uint32_t)(2 * STG) ? 0u : stg_conv + (uint32_t)STG;
+                stg_load = stg_load == (uint32_t)(2 * STG) ? 0u : stg_load + (uint32_t)STG;
+                ++t;
+            };
+            // (both trips of a pair load a whole raw tile: t + 4 and t + 5 lie below nfull)
+            for (; t + 5 < nfull;) {
+                steady_trip(ro0);
+                steady_trip(ro1);
             }
+            primed = true;
         }
-#if DA_PIPE_PROBE > 1
-        const long long pr_s0a = clock64();
-#endif
-        if (primed) {
-            // behind the steady-state loop: tile t+1 is in LDS for every wave and its first K fragments are on their
-            // way; what is left to wait for is every wave's last read of tile t-1
-            __syncthreads();
-            primed = false;
-        } else {
-            if (t + 2 < ntiles)
-                wait_vmcnt<NLW>();  // tile t+1 landed; tile t+2 may still be in flight
+        for (; t + 1 < ntiles; ++t) {
+            const uint32_t cur_a = a_of(t), nxt_a = a_of(t + 1), nxt_b = b_of(t + 1);
+            // raw tile t+2 has landed (raw tile t+3's loads may be outstanding); behind the barrier every wave is done
+            // with tile t-1 and has converted its share of tile t+1
+            if (t + 3 < ntiles)
+                wait_vmcnt<NLW8>();
             else
                 wait_vmcnt<0>();
-            __syncthreads();  // every wave's share of tile t+1 is in LDS, and every wave is done with tile t-1
-            prime_k(base_b + nxt);
-        }
-        if (!fast && t + NB - 1 < ntiles) {
-            if constexpr (PG)
-                issue_tile_pg(c0 + (t + NB - 1) * kTile, (t + NB - 1) & (NB - 1));
+            __syncthreads();
+            // raw tile t+4: a whole one goes out between the matrix steps below, the split's last one here
+            const bool whole4 = t + 4 < nfull;
+            if (!whole4 && t + 4 < ntiles) issue_raw(c0 + (t + 4) * kTile, (t + 4) % 3);
+            if (primed)
+                primed = false;  // (the first K fragments of tile t+1 are on their way already)
             else
-                issue_tile(c0 + (t + NB - 1) * kTile, (t + NB - 1) & (NB - 1));
+                prime_k(base_b + nxt_b);
+            softmax_head(t, std::false_type{});
+            if (t + 2 < ntiles) {
+                // tile t+2 is converted between the matrix steps, as in the steady-state trips
+                const ConvAddr ca = conv_addr((uint32_t)(((t + 2) % 3) * STG), a_of(t + 2), b_of(t + 2));
+                csrc = ca.src;
+                cdst_a = ca.dst_a;
+                cdst_b = ca.dst_b;
+                if (whole4) {
+                    const TileRows tr = tile_rows(c0 + (t + 4) * kTile);
+                    phase_a(std::true_type{}, std::true_type{}, std::integral_constant<int, kDmaRaw>{}, base_b + nxt_b,
+                            base_v + cur_a, tr.base, tr.base1, smem_off + (uint32_t)(OFF_STG + ((t + 4) % 3) * STG), ro0,
+                            std::true_type{});
+                } else {
+                    phase_a(std::true_type{}, std::true_type{}, std::integral_constant<int, -1>{}, base_b + nxt_b,
+                            base_v + cur_a, nullptr, nullptr, 0, ro0, std::true_type{});
+                }
+            } else {
+                phase_a(std::true_type{}, std::true_type{}, std::integral_constant<int, -1>{}, base_b + nxt_b,
+                        base_v + cur_a, nullptr, nullptr, 0, ro0, std::false_type{});
+            }
+            phase_b(std::integral_constant<int, kRing>{}, std::true_type{}, base_v + cur_a, a_of(t + 2) - nxt_a, ro0,
+                    std::false_type{}, 0);
         }
-        softmax_head(t, std::false_type{});
-#if DA_PIPE_PROBE > 1
-        const long long pr_s1 = clock64();
-        pr_top += pr_s1 - pr_s0;
-#endif
-        if (fast)
-            phase_a(std::true_type{}, std::true_type{}, std::integral_constant<int, 1>{}, base_b + nxt, base_v + cur, tr.base,
-                    tr.base1, smem_off + (uint32_t)(((t + NB - 1) & (NB - 1)) * BUF), ro0);
-        else
-            phase_a(std::true_type{}, std::true_type{}, std::integral_constant<int, -1>{}, base_b + nxt, base_v + cur, nullptr,
-                    nullptr, 0, ro0);
-#if DA_PIPE_PROBE > 1
-        const long long pr_s2 = clock64();
-        pr_a += pr_s2 - pr_s1;
-#endif
-        // (tile t+2 lies in buffer (t+2) % NB)
-        phase_b(std::integral_constant<int, kRing>{}, std::true_type{}, base_v + cur,
-                (uint32_t)(((t + 2) & (NB - 1)) * BUF) - nxt, ro0, std::false_type{}, 0);
-#if DA_PIPE_PROBE > 1
-        pr_b += clock64() - pr_s2;
-#endif
+    } else {
+        if (!PG && packed && !gen_all && t + NB < nfull) {
+            uint32_t cur = 0, nxt = (uint32_t)BUF, dst = (uint32_t)((NB - 1) * BUF);  // buffers of tiles t, t+1, t+3
+            wait_vmcnt<NLW>();  // tile 1 landed; tile 2 may still be in flight
+            __syncthreads();
+            prime_k(base_b + nxt);
+            auto steady_trip = [&](auto ro_c) __attribute__((always_inline)) {
+    #if DA_PIPE_PROBE > 1
+                const long long pr_s0 = clock64();
+    #endif
+                softmax_head(t, std::true_type{});
+    #if DA_PIPE_PROBE > 1
+                const long long pr_s0b = clock64();
+    #endif
+                asm volatile("s_barrier" ::: "memory");  // every wave is done with tile t-1
+    #if DA_PIPE_PROBE > 1
+                const long long pr_s1 = clock64();
+                pr_x2 += pr_s1 - pr_s0b;
+                pr_top += pr_s1 - pr_s0;
+    #endif
+                phase_a(std::true_type{}, std::true_type{}, std::integral_constant<int, 1>{}, base_b + nxt, base_v + cur, kt3,
+                        kt3 + 16 * k_row_bytes, smem_off + dst, ro_c, std::false_type{});
+    #if DA_PIPE_PROBE > 1
+                const long long pr_s2 = clock64();
+                pr_a += pr_s2 - pr_s1;
+    #endif
+                kt3 += kTile * k_row_bytes;
+                const uint32_t nn = dst == (uint32_t)((NB - 1) * BUF) ? 0u : dst + (uint32_t)BUF;  // buffer after dst = that of tile t+4
+                // (tile t+2 lies in the buffer behind nxt)
+                const uint32_t nx2 = nxt == (uint32_t)((NB - 1) * BUF) ? 0u : nxt + (uint32_t)BUF;
+                phase_b(std::integral_constant<int, kRing>{}, std::true_type{}, base_v + cur, nx2 - nxt, ro_c, std::true_type{},
+                        base_b + nx2);
+    #if DA_PIPE_PROBE > 1
+                pr_b += clock64() - pr_s2;
+    #endif
+                cur = nxt;
+                nxt = nx2;
+                dst = nn;
+                ++t;
+            };
+            // (both trips of a pair load a whole tile: t + 3 and t + 4 lie below nfull)
+            for (; t + NB < nfull;) {
+                steady_trip(ro0);
+                steady_trip(ro1);
+            }
+            primed = true;
+        }
+        for (; t + 1 < ntiles; ++t) {
+    #if DA_PIPE_PROBE > 1
+            const long long pr_s0 = clock64();
+    #endif
+            const uint32_t cur = (uint32_t)((t & (NB - 1)) * BUF), nxt = (uint32_t)(((t + 1) & (NB - 1)) * BUF);
+            const bool fast = !PG && t + NB - 1 < nfull;
+            TileRows tr{nullptr, nullptr, 0};
+            if (fast) {
+                if (packed) {  // rows follow each other at the pitch
+                    tr.base = kt3;
+                    tr.base1 = kt3 + 16 * k_row_bytes;
+                    kt3 += kTile * k_row_bytes;
+                } else {
+                    tr = tile_rows(c0 + (t + NB - 1) * kTile);
+                }
+            }
+    #if DA_PIPE_PROBE > 1
+            const long long pr_s0a = clock64();
+    #endif
+            if (primed) {
+                // behind the steady-state loop: tile t+1 is in LDS for every wave and its first K fragments are on their
+                // way; what is left to wait for is every wave's last read of tile t-1
+                __syncthreads();
+                primed = false;
+            } else {
+                if (t + 2 < ntiles)
+                    wait_vmcnt<NLW>();  // tile t+1 landed; tile t+2 may still be in flight
+                else
+                    wait_vmcnt<0>();
+                __syncthreads();  // every wave's share of tile t+1 is in LDS, and every wave is done with tile t-1
+                prime_k(base_b + nxt);
+            }
+            if (!fast && t + NB - 1 < ntiles) {
+                if constexpr (PG)
+                    issue_tile_pg(c0 + (t + NB - 1) * kTile, (t + NB - 1) & (NB - 1));
+                else
+                    issue_tile(c0 + (t + NB - 1) * kTile, (t + NB - 1) & (NB - 1));
+            }
+            softmax_head(t, std::false_type{});
+    #if DA_PIPE_PROBE > 1
+            const long long pr_s1 = clock64();
+            pr_top += pr_s1 - pr_s0;
+    #endif
+            if (fast)
+                phase_a(std::true_type{}, std::true_type{}, std::integral_constant<int, 1>{}, base_b + nxt, base_v + cur, tr.base,
+                        tr.base1, smem_off + (uint32_t)(((t + NB - 1) & (NB - 1)) * BUF), ro0, std::false_type{});
+            else
+                phase_a(std::true_type{}, std::true_type{}, std::integral_constant<int, -1>{}, base_b + nxt, base_v + cur, nullptr,
+                        nullptr, 0, ro0, std::false_type{});
+    #if DA_PIPE_PROBE > 1
+            const long long pr_s2 = clock64();
+            pr_a += pr_s2 - pr_s1;
+    #endif
+            // (tile t+2 lies in buffer (t+2) % NB)
+            phase_b(std::integral_constant<int, kRing>{}, std::true_type{}, base_v + cur,
+                    (uint32_t)(((t + 2) & (NB - 1)) * BUF) - nxt, ro0, std::false_type{}, 0);
+    #if DA_PIPE_PROBE > 1
+            pr_b += clock64() - pr_s2;
+    #endif
+        }
     }
     // ---- the last trip: softmax and O += V^T P^T of the last tile -------------------------------------------------------
     {
-        const uint32_t cur = (uint32_t)((t & (NB - 1)) * BUF);
+        const uint32_t cur = a_of(t);
         softmax_head(t, std::false_type{});
-        phase_a(std::false_type{}, std::true_type{}, std::integral_constant<int, -1>{}, 0, base_v + cur, nullptr, nullptr, 0, ro0);
+        phase_a(std::false_type{}, std::true_type{}, std::integral_constant<int, -1>{}, 0, base_v + cur, nullptr, nullptr, 0, ro0,
+                std::false_type{});
         phase_b(std::integral_constant<int, kRing - 1>{}, std::false_type{}, base_v + cur, 0, ro0, std::false_type{}, 0);
     }
 
@@ -814,7 +1136,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_num_vgpr(kScV))) void la
         // columns of head n per 32 x 32 tile quarter, the wave stores 1 KiB (two quarters, 16 bytes a lane) per
         // instruction, and the merge kernel reads in that order.  No trip through LDS and no barrier in the tail every work-group of a
         // one-round grid runs at the same moment.
-        const float inv = 1.0f / l_tot;
+        const float inv = (KV8 ? head_scale(p.v_scale, hk) : 1.0f) / l_tot;  // (8-bit K: times the V factor)
         const int blk = (hk * p.groups + grp) * NWV + wave;
         uint8_t* const rec = reinterpret_cast<uint8_t*>(p.ws_o) +
                              nat_block((size_t)b, p.nsplit, split, nat_blocks(p.head_k, p.groups, NWV), blk) * 8;
@@ -848,7 +1170,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_num_vgpr(kScV))) void la
         typedef __attribute__((address_space(3))) uint8_t* lds_ptr;
         typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
         const lds_ptr wbuf = (lds_ptr)(uintptr_t)(smem_off + (uint32_t)(wave * BUF));
-        const float inv = 1.0f / l_tot;
+        const float inv = (KV8 ? head_scale(p.v_scale, hk) : 1.0f) / l_tot;  // (8-bit K: times the V factor)
         static_for<0, CT * 4>([&](auto ic) {
             constexpr int c = decltype(ic)::value / 4, r4 = decltype(ic)::value % 4;
             const int col = c * 32 + r4 * 8 + half * 4;
@@ -907,10 +1229,13 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_num_vgpr(kScV))) void la
 #endif
 }
 
-template <typename Tag, bool PG>
+template <typename Tag, bool PG, int KV8 = 0>
 hipError_t launch_form(const SweepParams& p, dim3 grid, hipStream_t stream) {
-    auto kern = latent_pipe_kernel<Tag, PG>;
-    constexpr size_t lds = (size_t)kPipeBufs * kTile * 576 * 2;
+    auto kern = latent_pipe_kernel<Tag, PG, KV8>;
+    // four 16-bit tile buffers; 8-bit K: three value regions, two key-tail regions, three raw stages
+    constexpr size_t lds = KV8 ? (size_t)3 * kTile * 512 * 2 + (size_t)2 * kTile * 64 * 2 + (size_t)3 * kTile * 576
+                               : (size_t)kPipeBufs * kTile * 576 * 2;
+    static_assert(lds <= 160 * 1024, "LDS of one CU");
     static std::atomic<uint64_t> devices_done{0};
     const hipError_t attr_err = ensure_lds_limit(reinterpret_cast<const void*>(kern), lds, devices_done);
     if (attr_err != hipSuccess) return attr_err;
@@ -931,6 +1256,18 @@ hipError_t launch_mla_pipe(const SweepParams& p_in, bool is_bf16, dim3 grid, hip
     const bool pg = p.block_table != nullptr && p.page_shift < 4;
     if (is_bf16) return pg ? launch_form<bf16_tag, true>(p, grid, stream) : launch_form<bf16_tag, false>(p, grid, stream);
     return pg ? launch_form<f16_tag, true>(p, grid, stream) : launch_form<f16_tag, false>(p, grid, stream);
+}
+
+bool mla_pipe_kv8_supported(const SweepParams& p) {
+    // rows of 576 bytes (one KV head), fetched in runs of 16 tokens: the packed layout, or pages of 16 tokens and more
+    return p.k_row == 576 && (p.block_table == nullptr || p.page_shift >= 4);
+}
+
+hipError_t launch_mla_pipe_kv8(const SweepParams& p, int fmt, bool is_bf16, dim3 grid, hipStream_t stream) {
+    if (!mla_pipe_kv8_supported(p)) return hipErrorInvalidValue;
+    if (fmt == kKvInt8)
+        return is_bf16 ? launch_form<bf16_tag, false, kKvInt8>(p, grid, stream) : launch_form<f16_tag, false, kKvInt8>(p, grid, stream);
+    return is_bf16 ? launch_form<bf16_tag, false, kKvFp8>(p, grid, stream) : launch_form<f16_tag, false, kKvFp8>(p, grid, stream);
 }
 
 }  // namespace da
