@@ -31,18 +31,21 @@ if ROOT not in sys.path:
 HBM_PEAK_GBPS = 8000.0      # MI355X HBM3E, published
 MFMA_PEAK_TFLOPS = 2500.0   # MI355X dense fp16/bf16 MFMA, published
 # HBM bytes per call from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of `bench.py --only gqa|mla`, each counter
-# scaled by what it reads for a 1 GiB device copy (profiles/*_hbm_traffic.md).  A figure belongs to the launch plan
-# it was measured under; when the library plans the workload differently, the bench line carries null instead.
-MEASURED_TRAFFIC = {
-    "gqa": {"bytes": 1092312678, "plan": {"kind": 3, "nsplit": 4, "chunk": 1024, "heads_per_group": 16}},
-    "mla": {"bytes": 389967872, "plan": {"kind": 2, "nsplit": 4, "chunk": 1024, "heads_per_group": 128},
-            "partials": "16-bit"},
-}
+# scaled by what it reads for a 1 GiB device copy: profiles/hbm_traffic.json, written from the counter runs by
+# `python -m decoding_attention_amd.profile_traffic` (profiles/*_hbm_traffic.md describe the runs).  A figure belongs
+# to the launch plan it was measured under; when the library plans the workload differently, or the file is not there,
+# the bench line carries null instead.
+TRAFFIC_JSON = os.path.join(ROOT, "profiles", "hbm_traffic.json")
 
 
 def measured_traffic(key, plan):
-    rec = MEASURED_TRAFFIC[key]
-    return rec["bytes"] if all(plan.get(k) == v for k, v in rec["plan"].items()) else None
+    try:
+        with open(TRAFFIC_JSON) as f:
+            rec = json.load(f)[key]
+    except (OSError, KeyError, ValueError):
+        return None
+    same = all(plan.get(k) == v for k, v in rec["plan"].items())
+    return rec["bytes"] if same else None
 
 
 def _time_calls(torch, fn_list, steps, warmup):

@@ -125,7 +125,7 @@ _probe = None
 
 
 def load_probe():
-    """The benchmark's measurement aids (include/decoding_attn_probe.h): a second build of the library with the
+    """The benchmark's measurement aids (csrc/decoding_attn_probe.h): a second build of the library with the
     sweep-only entry point and the streaming-read kernel.  Not part of the drop-in ABI; only bench.py loads it."""
     global _probe
     if _probe is not None:

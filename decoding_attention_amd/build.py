@@ -28,7 +28,7 @@ SOURCES = [
     "da_gqa_mfma_i4.hip",
 ]
 
-# libdecoding_attn_probe.so (measurement aids of bench.py, include/decoding_attn_probe.h): the same objects, with
+# libdecoding_attn_probe.so (measurement aids of bench.py, csrc/decoding_attn_probe.h): the same objects, with
 # da_api.hip compiled once more with the sweep-only entry point, plus the streaming-read kernel.
 PROBE_LIB_PATH = os.path.join(PKG_DIR, "libdecoding_attn_probe.so")
 

@@ -16,7 +16,7 @@
 
 #include "../../include/decoding_attn_hip.h"
 #ifdef DA_BUILD_PROBES
-#include "../../include/decoding_attn_probe.h"
+#include "decoding_attn_probe.h"
 #endif
 #include "da_gqa_mfma.h"
 #include "da_mla.h"
@@ -879,7 +879,7 @@ int da_decoding_attn_ex(const void* q, const void* k, const void* v, void* o, co
 }
 
 #ifdef DA_BUILD_PROBES
-// (libdecoding_attn_probe.so only, declared in include/decoding_attn_probe.h)
+// (libdecoding_attn_probe.so only, declared in decoding_attn_probe.h)
 int da_probe_sweep_only(const void* q, const void* k, const void* v, void* o, const int32_t* cu_seq_k, size_t max_seq_k,
                         size_t batch, size_t head_q, size_t head_k, size_t dim, size_t dim_v, int is_alibi, int is_bf16,
                         size_t total_k, void* workspace, size_t workspace_bytes, void* hip_stream) {

@@ -5,7 +5,7 @@
 #include <stdint.h>
 
 #include "../../include/decoding_attn_hip.h"
-#include "../../include/decoding_attn_probe.h"
+#include "decoding_attn_probe.h"
 
 namespace {
 
