@@ -519,7 +519,12 @@ LATENT_PLAN_SHAPES = ([(b, 4096) for b in (1, 2, 4, 8, 16, 32, 64, 128, 256)] +
                       [(16, sk) for sk in (512, 1024, 2048, 8192, 16384)] + [(1, sk) for sk in (512, 2048, 8192)] +
                       [(4, 16384), (8, 8192), (32, 1024), (64, 1024), (100, 4096)] +
                       # short sequences of small batches, where a work-group's fixed cost decides the split count
-                      [(8, 512), (8, 1024), (24, 1024), (16, 768), (16, 1536), (4, 2048), (8, 2048), (24, 2048), (8, 3072)])
+                      [(8, 512), (8, 1024), (24, 1024), (16, 768), (16, 1536), (4, 2048), (8, 2048), (24, 2048), (8, 3072)] +
+                      # batches of 20 to 128 sequences between one and two work-groups a CU
+                      [(20, 4096), (40, 2048), (48, 1024), (48, 2048), (48, 4096), (64, 512), (64, 2048), (96, 1024),
+                       (128, 512), (128, 1024)] +
+                      # the smallest problems, where the grouped kernel's latent form competes
+                      [(1, 128), (1, 256), (1, 1024), (2, 256), (2, 512), (2, 1024), (4, 256), (4, 512), (4, 1024)])
 
 
 def run_latent_plan_sweep(args):
@@ -579,7 +584,7 @@ def run_latent_plan_sweep(args):
         if k2 == 3:
             results[f"g/{rt2}/{ns2}"] = time_us(copies, w)
         for heads in (64, 128):
-            for nsplit in (1, 2, 3, 4, 6, 8, 12, 16, 24, 32):
+            for nsplit in (1, 2, 3, 4, 5, 6, 8, 10, 12, 16, 24, 32):
                 if sk // nsplit < 128 or batch * nsplit * (128 // heads) > 1024:
                     continue
                 set_tunables(DA_MLA_GROUP_SMALL=0, DA_MLA_HEADS=heads, DA_NSPLIT=nsplit)

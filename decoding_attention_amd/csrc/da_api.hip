@@ -47,7 +47,7 @@ int env_int(const char* name, int dflt) {
 struct Tunables {
     int target_wgs, mfma_target_wgs, max_chunk, min_chunk, ragged_chunk, force_kind, group_min_ratio, wave_per_head,
         mla_heads, gqa_heads, flat_wgs, flat_min_tokens, flat_uncounted, flat_uncounted_min, flat_paged_min_mb, nsplit, mfma_small_wgs, group_small_wgs,
-        group_small_chunk, mla_group_heads, mla_group_small, fill_rounds, group_target_wgs_d128, mla_distinct_v, pipe_small_wgs;
+        group_small_chunk, mla_group_heads, mla_group_small, fill_rounds, group_target_wgs_d128, mla_distinct_v;
     Tunables() {
         target_wgs = env_int("DA_TARGET_WGS", 512);
         mfma_target_wgs = env_int("DA_MFMA_TARGET_WGS", 256);
@@ -65,7 +65,6 @@ struct Tunables {
         flat_uncounted_min = env_int("DA_FLAT_UNCOUNTED_MIN", 512);
         flat_paged_min_mb = env_int("DA_FLAT_PAGED_MIN_MB", 512);  // paged K/V takes the balanced grid from this many MB of K/V
         mfma_small_wgs = env_int("DA_MFMA_SMALL_WGS", 256);  // latent kernel: below this many 256-token splits, split finer
-        pipe_small_wgs = env_int("DA_PIPE_SMALL_WGS", 33);   // the same for its pipelined form (128 heads a work-group)
         // latent form: up to this many query heads take the grouped kernel (0 = never)
         mla_group_heads = env_int("DA_MLA_GROUP_HEADS", 16);
         mla_distinct_v = env_int("DA_MLA_DISTINCT_V", 1);  // (576, 512) with V in its own buffer on the latent kernel (0 = VALU sweep)
@@ -165,9 +164,9 @@ Plan make_plan(size_t max_seq_k, size_t batch, size_t head_q, size_t head_k, siz
     // rows: the latent kernel's work-groups pay ~6 us to stage Q before their first tile, which a few tiles do not
     // win back (measured, 128 heads: batch 1 x 8192 tokens 34.4 -> 24.8 us, batch 16 x 512 29.8 -> 23.4; 32 heads:
     // batch 1 x 16384 33.4 -> 23.0; past the bound below the re-read rows cost more than the staging).
-    // (65 heads and more over 16-bit K run on the software-pipelined latent kernel, which wins from a quarter of that
-    // bound on: 128 heads, batch 1 x 4096 tokens 21.6 -> 19.8 us, batch 2 x 4096 26.2 -> 24.3, batch 16 x 512 27.1 ->
-    // 24.6; batch 1 x 512 stays, 16.5 against 17.7, batch 1 x 2048 is a tie)
+    // (65 heads and more run on the software-pipelined latent kernel, which wins wherever the sequences are split:
+    // 128 heads, batch 1 x 4096 tokens 21.4 -> 19.3 us, batch 1 x 512 16.2 -> 15.2, batch 2 x 1024 18.5 -> 16.6, batch
+    // 4 x 512 18.4 -> 15.8, batch 4 x 256 17.1 -> 15.2; a single unsplit launch stays, batch 1 x 128 12.9 against 13.8)
     // (its 8-bit form serves rows of one KV head in runs of 16 tokens: the packed layout and pages of 16 tokens and more)
     const bool pipe_kernel = latent && ratio > 64 &&
                              (!kv_8bit || (head_k == 1 && (packed || page_size >= 16) && !no_latent_kernel && !da::mla_pipe_kv8_off()));
@@ -175,7 +174,7 @@ Plan make_plan(size_t max_seq_k, size_t batch, size_t head_q, size_t head_k, siz
     const long long group_rows = groups16 * (long long)batch * (long long)max_seq_k;
     const long long small_bound =
         pipe_kernel ? (long long)tun().mla_group_small / 4 : (groups16 <= 2 ? 2 : 1) * (long long)tun().mla_group_small;
-    const bool latent_small = tun().mla_group_heads > 0 && group_rows <= small_bound;
+    const bool latent_small = tun().mla_group_heads > 0 && group_rows <= small_bound && (!pipe_kernel || max_seq_k < 256);
     const bool latent_group = latent && !force_sweep &&
                               (ratio <= (kv_8bit ? 2 * tun().mla_group_heads : tun().mla_group_heads) || latent_small ||
                                no_latent_kernel);
@@ -306,15 +305,9 @@ Plan make_plan(size_t max_seq_k, size_t batch, size_t head_q, size_t head_k, siz
         // too few work-groups for the chip even so: 128-token splits, as long as that keeps the merge at 32
         // partials or fewer (measured: batch 1 x 512 tokens 26.8 -> 20.5 us, batch 16 x 512 33.1 -> 29.4 us,
         // batch 4 x 2048 32.9 -> 28.3 us; batch 1 x 8192 with 64 partials loses, 36.0 -> 38.5 us)
-        // The pipelined kernel's work-groups carry a larger fixed cost (147 KB of Q in, 131 KB of partials out and in
-        // again at the merge: about 0.1 us per work-group once more than 64 of them share the chip), so it goes below
-        // 256 tokens only while that leaves at most 64 work-groups.  Measured, 128 heads, old -> new plan: batch 16 x
-        // 1024 tokens, 8 -> 4 splits, 31.7 -> 25.8 us; batch 24 x 1024 35.6 -> 28.9; batch 8 x 2048, 16 -> 8 splits, 30.7
-        // -> 27.0; batch 16 x 1536 33.6 -> 31.1; batch 8 x 3072 32.2 -> 30.2; batch 16 x 768 26.5 -> 25.1.  Up to 32
-        // splits of 256 tokens the finer ones still win: batch 16 x 512, 4 splits 21.2 us, 2 splits 23.5; batch 8 x
-        // 1024, 8 splits 22.2, 4 splits 23.3; batch 4 x 2048, 16 splits 23.1, 8 splits 24.5.
-        const int small_wgs = pipe_kernel ? tun().pipe_small_wgs : tun().mfma_small_wgs;
-        if (wgs_at_min < small_wgs && max_seq_k <= 32 * 128) min_chunk = std::max(std::min(min_chunk, 128), trip);
+        if (wgs_at_min < tun().mfma_small_wgs && max_seq_k <= 32 * 128) min_chunk = std::max(std::min(min_chunk, 128), trip);
+        // (the pipelined kernel takes 128-token splits whenever its work-group count, chosen below, asks for them)
+        if (pipe_kernel && pl.rt == 128 && max_seq_k <= 32 * 128) min_chunk = std::max(std::min(min_chunk, 128), trip);
     } else {
         // 512-token splits run best; go down to 256 only when that is needed to give every CU a work-group (the
         // VALU sweep: two, measured batch 4 x 1024 tokens 21.4 -> 18.6 us; the grouped kernel loses there)
@@ -348,13 +341,21 @@ Plan make_plan(size_t max_seq_k, size_t batch, size_t head_q, size_t head_k, siz
     // 40 x 8192, 280 work-groups 209 us, 240 work-groups 146 us; 16 heads, batch 150 x 4096, 300 work-groups 183 us,
     // 150 work-groups 153 us).
     if ((latent_group || mfma) && base > 0) want = std::max<long long>(1, target_wgs / base);
-    // The pipelined latent kernel with splits under 512 tokens: three quarters of the CUs do better than all of them
-    // (a work-group's fixed cost, Q in and partials out, is then most of its time, and fewer splits mean fewer
-    // partials; the chip also clocks higher).  Measured, 128 heads: batch 16 x 4096 tokens, 16 -> 12 splits, 40.4 ->
-    // 37.3 us; batch 8 x 8192, 32 -> 24, 40.8 -> 37.9; batch 64 x 1024, 4 -> 3, 41.1 -> 38.6; from 512-token splits
-    // up the full grid wins or ties (batch 64 x 4096, 4 splits 87.3 us, 3 splits 91.6; batch 32 x 4096, 8 and 6 tie).
-    if (mfma && pipe_kernel && pl.rt == 128 && base > 0 && want > 1 && (long long)max_seq_k / want < 512)
-        want = std::max<long long>(1, (target_wgs * 3 / 4) / base);
+    // The pipelined latent kernel: every work-group pays a fixed cost (147 KB of Q in, 131 KB of partials out), and the
+    // chip, power-limited under this kernel, runs few active CUs at a higher clock, so the best grid grows with the
+    // work: 128 work-groups up to 64 Ki tokens of (sequence, KV head) rows, one more per Ki tokens from there, all
+    // 256 CUs from 192 Ki.  Split counts are rounded to the nearest (a half down) and kept to one round of the CUs.
+    // Measured, 128 heads, us a call by work-groups: batch 16 x 4096 tokens 128: 33.7, 192: 33.1, 256: 41.8; batch 8 x
+    // 8192 128: 34.3, 192: 37.5, 256: 42.2; batch 16 x 1024 64: 21.3, 128: 18.4; batch 8 x 2048 64: 21.6, 128: 19.2;
+    // batch 40 x 2048 120: 41.9, 160: 39.0, 200: 40.9; batch 32 x 4096 128: 55.9, 192: 52.7, 256: 56.6; batch 64 x 2048
+    // 128: 59.5, 192: 54.5, 256: 59.1; batch 48 x 4096 144: 82.3, 192: 72.7, 240: 71.8; batch 64 x 4096 192: 92.3, 256:
+    // 86.6; batch 96 x 1024 96: 52.7, 192: 48.2; batch 128 x 1024 128: 56.1, 256: 59.9.
+    if (mfma && pipe_kernel && pl.rt == 128 && base > 0) {
+        const long long rows = base * (long long)max_seq_k;
+        const long long w = std::min<long long>(std::max<long long>(64 + rows / 1024, 128), target_wgs);
+        want = std::max<long long>(1, (2 * w + base - 1) / (2 * base));
+        while (want > 1 && base * want > target_wgs) --want;
+    }
     const long long by_len = std::max<long long>(1, (long long)max_seq_k / min_chunk);
     // sweep work-groups are also kept short (shorter still for a ragged batch); the latent MFMA kernel's partials
     // are too large (heads x dim_v floats per split) to split more than occupancy asks for
@@ -901,7 +902,6 @@ int da_probe_set_tunable(const char* name, int value) {
     else if (n == "DA_MLA_GROUP_HEADS") t.mla_group_heads = value;
     else if (n == "DA_MFMA_TARGET_WGS") t.mfma_target_wgs = value;
     else if (n == "DA_MFMA_SMALL_WGS") t.mfma_small_wgs = value;
-    else if (n == "DA_PIPE_SMALL_WGS") t.pipe_small_wgs = value;
     else return fail(DA_ERR_INVALID_ARGUMENT, "unknown tunable %s", name);
     return DA_OK;
 }

@@ -30,6 +30,11 @@ hipError_t launch_reduce(const ReduceParams& p, bool is_bf16, int blocks, hipStr
     int sg = 1;
     while (sg < 8 && p.nsplit >= 8 * sg && threads * sg < (1ll << 18)) sg *= 2;
     while (sg > 1 && (p.dim_v / 4) % (64 / sg) != 0) sg /= 2;
+    // The 16-byte-a-lane merge of the 16-bit records is the faster one as soon as it has a few work-groups a CU: the
+    // several-lanes-a-value form only where there are too few rows for that (measured, 128 heads over one latent head:
+    // batch 8 x 4096 tokens, 16 splits, 30.6 -> 24.4 us a call; batch 4 x 2048, 16 splits, 23.9 -> 19.9; batch 8 x
+    // 1024, 8 splits, 21.6 -> 16.7; batch 2 x 4096 a tie; batch 1 x 4096, 32 splits, loses 19.5 -> 20.6)
+    if (p.half_partials && threads >= (1ll << 15)) sg = 1;
     // normalised 16-bit partials (the pipelined latent kernel's: dim_v = 512, never the balanced grid), one lane per
     // element: eight columns a thread, dead rows of the blocks included
     if (p.half_partials && (p.dim_v != 512 || p.flat_wgs != 0 || p.nat_blocks <= 0 || p.head_q <= 0))

@@ -102,7 +102,8 @@ def test_value_passed_as_a_view_of_the_key_rows(head_q):
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
 def test_small_problems_of_any_head_count_as_groups_of_16(head_q, dtype):
     """Small latent problems run on the grouped kernel whatever the head count, ceil(heads / 16) groups per sequence,
-    the last one partly idle when 16 does not divide the head count."""
-    w = _latent(3, head_q, 600, dtype, seed=head_q, is_alibi=head_q == 40)
+    the last one partly idle when 16 does not divide the head count (65 heads and more: only sequences short enough
+    to stay unsplit, the pipelined latent kernel takes the rest)."""
+    w = _latent(3, head_q, 600 if head_q <= 64 else 200, dtype, seed=head_q, is_alibi=head_q == 40)
     assert _lib.plan(w.max_seq_k, 3, head_q, 1, 576, 512)["kind"] == 3
     check_against_oracle(w, run_hip(w))

@@ -15,23 +15,26 @@ from gpu_util import TOL, check_against_oracle, run_hip, run_hip_ex, run_oracle,
 
 pytestmark = pytest.mark.gpu
 
-# batch, head_q, head_k, seq_k, lanes per element in the merge (the launcher's rule: doubled while the splits number
-# 8 x lanes or more and batch x head_q x 128 x lanes stays under 2^18)
+# batch, head_q, head_k, seq_k, lanes per element in the merge (the launcher's rule: one lane per element from 2^15
+# elements' worth of threads; below that doubled while the splits number 8 x lanes or more)
 SHAPES = [
     (20, 129, 1, 1500, 1),
     (32, 128, 1, 1024, 1),
-    (16, 100, 1, 2048, 2),
-    (4, 192, 2, 3000, 2),
-    (2, 192, 2, 4096, 4),
-    (3, 100, 1, 4096, 4),
+    (16, 100, 1, 2048, 1),
+    (4, 192, 2, 3000, 1),
+    (1, 128, 1, 1536, 2),
+    (1, 192, 2, 1280, 2),
+    (2, 100, 1, 2560, 4),
     (1, 200, 2, 8192, 8),
     (2, 65, 1, 4096, 8),
 ]
 
 
 def _merge_lanes(batch, head_q, nsplit):
+    if batch * head_q * 128 >= (1 << 15):
+        return 1
     sg = 1
-    while sg < 8 and nsplit >= 8 * sg and batch * head_q * 128 * sg < (1 << 18):
+    while sg < 8 and nsplit >= 8 * sg:
         sg *= 2
     return sg
 
