@@ -144,16 +144,11 @@ def measure(torch, w, steps, warmup, page_size=0, kv_fp8=False, kv_int8=False, k
         nbytes = wl.algorithmic_bytes(w.batch, w.head_q, w.head_k, w.dim, w.dim_v, int(w.k.shape[0]), w.v is not None,
                                       elem_bytes=2) - (kv_elems * 3 // 2 if kv_int4 else kv_elems)
     flops = wl.workload_flops(w)
-    # the plan of the call that was timed: a V buffer of its own and the page size change it; the 8-bit and 4-bit
-    # formats are planned by rules of their own that the library has no query for (None)
-    plan = None
-    if not (kv_fp8 or kv_int8 or kv_int4):
-        distinct = w.v is not None and w.dim != w.dim_v
-        if distinct or page_size:
-            plan = _lib.plan(w.max_seq_k, w.batch, w.head_q, w.head_k, w.dim, w.dim_v, total_k=int(w.k.shape[0]),
-                             distinct_v=True, page_size=page_size) if distinct else None
-        else:
-            plan = _lib.plan(w.max_seq_k, w.batch, w.head_q, w.head_k, w.dim, w.dim_v, total_k=int(w.k.shape[0]))
+    # the plan of the call that was timed
+    plan = _lib.plan(w.max_seq_k, w.batch, w.head_q, w.head_k, w.dim, w.dim_v,
+                     total_k=int(w.k.shape[0]),
+                     distinct_v=w.v is not None and w.dim != w.dim_v, page_size=page_size,
+                     kv_bits=4 if kv_int4 else (8 if (kv_fp8 or kv_int8) else 16))
     return {
         "workload": w.name,
         "us_per_call": mean_ms * 1e3,
@@ -548,25 +543,39 @@ def run_latent_plan_sweep(args):
         for name, value in {**defaults, **kw}.items():
             assert probe.da_probe_set_tunable(name.encode(), int(value)) == 0
 
+    kv_bits = 8 if args.kv == "fp8" else 16
+
     def plan_of(w):
         kind, ns, ch, rt = (ctypes.c_int() for _ in range(4))
-        assert probe.da_plan(w.max_seq_k, w.batch, 128, 1, 576, 512, 0, int(w.k.shape[0]), ctypes.byref(kind),
-                             ctypes.byref(ns), ctypes.byref(ch), ctypes.byref(rt)) == 0
+        assert probe.da_plan_call(w.max_seq_k, w.batch, 128, 1, 576, 512, int(w.k.shape[0]), 0, 0, kv_bits,
+                                  ctypes.byref(kind), ctypes.byref(ns), ctypes.byref(ch), ctypes.byref(rt), None) == 0
         return kind.value, rt.value, ns.value, ch.value
 
     def time_us(copies, w):
         total = int(w.k.shape[0])
-        n = probe.da_workspace_bytes(w.max_seq_k, w.batch, 128, 1, 576, 512, total)
+        if kv_bits == 8:
+            n = probe.da_workspace_bytes_fp8kv(w.max_seq_k, w.batch, 128, 1, 576, 512, total, 0)
+        else:
+            n = probe.da_workspace_bytes(w.max_seq_k, w.batch, 128, 1, 576, 512, total)
         ws = torch.empty(max(n, 16), dtype=torch.uint8, device=dev)
         o = torch.empty(w.batch, 128, 512, dtype=torch.float16, device=dev)
+        scale = torch.full((1,), 0.02, device=dev)
+        k8 = [(c.k.float() / 0.02).to(torch.float8_e4m3fn) for c in copies] if kv_bits == 8 else None
 
-        def call(c):
-            rc = probe.da_decoding_attn_ex(c.q.data_ptr(), c.k.data_ptr(), None, o.data_ptr(), c.cu_seq_k.data_ptr(),
-                                           w.max_seq_k, w.batch, 128, 1, 576, 512, 0, 0, 0.0, None, total,
-                                           ws.data_ptr(), n, stream)
+        def call(i):
+            c = copies[i]
+            if kv_bits == 8:
+                rc = probe.da_decoding_attn_fp8kv(c.q.data_ptr(), k8[i].data_ptr(), None, o.data_ptr(),
+                                                  c.cu_seq_k.data_ptr(), w.max_seq_k, w.batch, 128, 1, 576, 512, 0, 0,
+                                                  0.0, None, scale.data_ptr(), scale.data_ptr(), total, ws.data_ptr(),
+                                                  n, stream)
+            else:
+                rc = probe.da_decoding_attn_ex(c.q.data_ptr(), c.k.data_ptr(), None, o.data_ptr(),
+                                               c.cu_seq_k.data_ptr(), w.max_seq_k, w.batch, 128, 1, 576, 512, 0, 0,
+                                               0.0, None, total, ws.data_ptr(), n, stream)
             assert rc == 0, probe.da_last_error().decode("utf-8", "replace")
 
-        mean_ms, _ = _time_calls(torch, [lambda c=c: call(c) for c in copies], args.steps, args.warmup)
+        mean_ms, _ = _time_calls(torch, [lambda i=i: call(i) for i in range(len(copies))], args.steps, args.warmup)
         return mean_ms * 1e3
 
     print("shape: candidates as kernel/heads-per-work-group/splits = us per call; kernel g = grouped (16 heads per "
@@ -608,6 +617,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--kv", choices=["16", "fp8"], default="16", help="--sweep latent-plan: the K cache's format")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU oracle timing")
     ap.add_argument("--no-mla", action="store_true", help="skip the MLA measurement")
     ap.add_argument("--only", choices=["gqa", "mla"], help="measure one workload only and print its record "

@@ -31,6 +31,7 @@ EXPORTED_SYMBOLS = (
     "da_plan",
     "da_plan_distinct_v",
     "da_plan_is_balanced",
+    "da_plan_call",
     "da_supported_head_dims",
     "da_last_error",
     "da_version",
@@ -112,6 +113,9 @@ def _declare(lib):
     lib.da_plan_distinct_v.argtypes = [sz, sz, sz, sz, sz, sz, sz, sz, ip, ip, ip, ip]
     lib.da_plan_is_balanced.restype = ci
     lib.da_plan_is_balanced.argtypes = [sz, sz, sz, sz, sz, sz, sz, sz]
+    ip = ctypes.POINTER(ci)
+    lib.da_plan_call.restype = ci
+    lib.da_plan_call.argtypes = [sz, sz, sz, sz, sz, sz, sz, sz, ci, ci, ip, ip, ip, ip, ip]
     lib.da_supported_head_dims.restype = ci
     lib.da_supported_head_dims.argtypes = [sz, sz]
     lib.da_last_error.restype = ctypes.c_char_p
@@ -155,21 +159,17 @@ def last_error() -> str:
     return load().da_last_error().decode("utf-8", "replace")
 
 
-def plan(max_seq_k, batch, head_q, head_k, dim, dim_v, is_bf16=False, total_k=0, distinct_v=False, page_size=0):
-    """Launch plan for a shape: dict(kind, nsplit, chunk, heads_per_group).  `distinct_v`: the plan of a call that
-    passes V as its own buffer (packed, or pages of `page_size` tokens)."""
+def plan(max_seq_k, batch, head_q, head_k, dim, dim_v, is_bf16=False, total_k=0, distinct_v=False, page_size=0,
+         kv_bits=16):
+    """Launch plan of a call: dict(kind, nsplit, chunk, heads_per_group, balanced).  `distinct_v`: V passed as its own
+    buffer; `page_size`: pages of that many tokens (0 = packed); `kv_bits`: 16, 8 (FP8, int8) or 4 (int4)."""
+    del is_bf16  # (the plan does not depend on it)
     lib = load()
-    kind, ns, ch, rt = ctypes.c_int(), ctypes.c_int(), ctypes.c_int(), ctypes.c_int()
-    if distinct_v:
-        rc = lib.da_plan_distinct_v(max_seq_k, batch, head_q, head_k, dim, dim_v, int(total_k), int(page_size),
-                                    ctypes.byref(kind), ctypes.byref(ns), ctypes.byref(ch), ctypes.byref(rt))
-    else:
-        rc = lib.da_plan(max_seq_k, batch, head_q, head_k, dim, dim_v, int(is_bf16), int(total_k), ctypes.byref(kind),
-                         ctypes.byref(ns), ctypes.byref(ch), ctypes.byref(rt))
+    kind, ns, ch, rt, bal = (ctypes.c_int() for _ in range(5))
+    rc = lib.da_plan_call(max_seq_k, batch, head_q, head_k, dim, dim_v, int(total_k), int(page_size), int(distinct_v),
+                          int(kv_bits), ctypes.byref(kind), ctypes.byref(ns), ctypes.byref(ch), ctypes.byref(rt),
+                          ctypes.byref(bal))
     if rc != DA_OK:
-        raise RuntimeError(f"da_plan failed ({rc}): {last_error()}")
-    out = {"kind": kind.value, "nsplit": ns.value, "chunk": ch.value, "heads_per_group": rt.value}
-    if not distinct_v or dim == dim_v:
-        out["balanced"] = bool(lib.da_plan_is_balanced(max_seq_k, batch, head_q, head_k, dim, dim_v, int(total_k),
-                                                       int(page_size)) > 0)
-    return out
+        raise RuntimeError(f"da_plan_call failed ({rc}): {last_error()}")
+    return {"kind": kind.value, "nsplit": ns.value, "chunk": ch.value, "heads_per_group": rt.value,
+            "balanced": bool(bal.value)}

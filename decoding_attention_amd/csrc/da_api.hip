@@ -350,9 +350,13 @@ Plan make_plan(size_t max_seq_k, size_t batch, size_t head_q, size_t head_k, siz
     // batch 40 x 2048 120: 41.9, 160: 39.0, 200: 40.9; batch 32 x 4096 128: 55.9, 192: 52.7, 256: 56.6; batch 64 x 2048
     // 128: 59.5, 192: 54.5, 256: 59.1; batch 48 x 4096 144: 82.3, 192: 72.7, 240: 71.8; batch 64 x 4096 192: 92.3, 256:
     // 86.6; batch 96 x 1024 96: 52.7, 192: 48.2; batch 128 x 1024 128: 56.1, 256: 59.9.
+    // Over an 8-bit cache a tile takes longer (the conversion) and the chip is less power-bound: 192 work-groups up
+    // to 64 Ki rows, all CUs from 128 Ki (FP8: batch 16 x 4096 128: 41.0, 192: 35.6, 256: 37.0; batch 24 x 2048 120:
+    // 36.9, 192: 30.6; batch 64 x 1024 128: 44.2, 192: 38.2; batch 32 x 4096 192: 54.8, 256: 52.9; batch 128 x 512 128:
+    // 38.4, 256: 42.0).
     if (mfma && pipe_kernel && pl.rt == 128 && base > 0) {
-        const long long rows = base * (long long)max_seq_k;
-        const long long w = std::min<long long>(std::max<long long>(64 + rows / 1024, 128), target_wgs);
+        const long long rows = base * (long long)max_seq_k, least = kv_8bit ? 192 : 128;
+        const long long w = std::min<long long>(std::max<long long>(least - 64 + rows / 1024, least), target_wgs);
         want = std::max<long long>(1, (2 * w + base - 1) / (2 * base));
         while (want > 1 && base * want > target_wgs) --want;
     }
@@ -585,6 +589,29 @@ int da_plan_is_balanced(size_t max_seq_k, size_t batch, size_t head_q, size_t he
                         size_t total_k, size_t page_size) {
     if (head_k == 0 || head_q % head_k != 0 || !supported_dims(dim, dim_v)) return -1;
     return make_plan(max_seq_k, batch, head_q, head_k, dim, dim_v, false, total_k, page_size).flat_wgs > 0 ? 1 : 0;
+}
+
+int da_plan_call(size_t max_seq_k, size_t batch, size_t head_q, size_t head_k, size_t dim, size_t dim_v, size_t total_k,
+                 size_t page_size, int distinct_v, int kv_bits, int* kernel_kind, int* nsplit, int* chunk,
+                 int* heads_per_group, int* balanced) {
+    if (head_k == 0 || head_q % head_k != 0)
+        return fail(DA_ERR_INVALID_ARGUMENT, "head_q (%zu) must be a multiple of head_k (%zu)", head_q, head_k);
+    if (!supported_dims(dim, dim_v))
+        return fail(DA_ERR_UNSUPPORTED, "unsupported head dims (dim %zu, dim_v %zu)", dim, dim_v);
+    if (kv_bits != 16 && kv_bits != 8 && kv_bits != 4)
+        return fail(DA_ERR_INVALID_ARGUMENT, "kv_bits (%d) must be 16, 8 or 4", kv_bits);
+    if (page_size != 0 && (page_size & (page_size - 1)) != 0)
+        return fail(DA_ERR_INVALID_ARGUMENT, "page_size (%zu) must be a power of two", page_size);
+    // (as run_attention plans one launch; a batch beyond one grid axis is planned run by run, without the count)
+    const bool folded = batch > kMaxGridBatch;
+    const Plan pl = make_plan(max_seq_k, folded ? kMaxGridBatch : batch, head_q, head_k, dim, dim_v, distinct_v != 0,
+                              folded ? 0 : total_k, page_size, kv_bits != 16, kv_bits == 4);
+    if (kernel_kind) *kernel_kind = pl.kind;
+    if (nsplit) *nsplit = pl.nsplit;
+    if (chunk) *chunk = pl.chunk;
+    if (heads_per_group) *heads_per_group = pl.rt;
+    if (balanced) *balanced = pl.flat_wgs > 0 ? 1 : 0;
+    return DA_OK;
 }
 
 size_t da_workspace_bytes(size_t max_seq_k, size_t batch, size_t head_q, size_t head_k, size_t dim, size_t dim_v,

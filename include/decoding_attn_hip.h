@@ -239,6 +239,17 @@ int da_plan_distinct_v(size_t max_seq_k, size_t batch, size_t head_q, size_t hea
 int da_plan_is_balanced(size_t max_seq_k, size_t batch, size_t head_q, size_t head_k, size_t dim, size_t dim_v,
                         size_t total_k, size_t page_size);
 
+/*
+ * The plan of any call of this library, for benchmarks that report it beside a measurement: page_size 0 = packed
+ * layout, else pages of page_size tokens; distinct_v != 0 = V passed as a buffer of its own; kv_bits 16 = fp16/bf16
+ * K/V, 8 = the FP8 and int8 caches, 4 = the int4 cache.  Outputs as da_plan's, balanced as da_plan_is_balanced's
+ * result; any output pointer may be NULL.  No counterpart in the reference (one tile shape per head dim,
+ * csrc/kernel/decoding_attn/decoding_fwd_hd*.cu).
+ */
+int da_plan_call(size_t max_seq_k, size_t batch, size_t head_q, size_t head_k, size_t dim, size_t dim_v, size_t total_k,
+                 size_t page_size, int distinct_v, int kv_bits, int *kernel_kind, int *nsplit, int *chunk,
+                 int *heads_per_group, int *balanced);
+
 /* 1 when (dim, dim_v) is a supported pair: the reference's DA_HEADDIM_SWITCH set (csrc/common/common.h:73-96). */
 int da_supported_head_dims(size_t dim, size_t dim_v);
 
