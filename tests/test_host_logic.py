@@ -154,6 +154,32 @@ def test_plan_rejects_bad_shapes():
         _lib.plan(128, 1, 4, 4, 80, 80)
 
 
+def test_plan_of_every_call_form():
+    """da_plan_call: the plan of packed and paged calls, of a V buffer of its own and of the 8- and 4-bit caches, and
+    its agreement with the narrower queries."""
+    import ctypes
+    lib = _lib.load()
+    shape = (4096, 64, 128, 1, 576, 512)
+    base = _lib.plan(*shape, total_k=64 * 4096)
+    assert base == {"kind": 2, "nsplit": 4, "chunk": 1024, "heads_per_group": 128, "balanced": False}
+    kind, ns = ctypes.c_int(), ctypes.c_int()
+    assert lib.da_plan(*shape, 0, 64 * 4096, ctypes.byref(kind), ctypes.byref(ns), None, None) == 0
+    assert (kind.value, ns.value) == (base["kind"], base["nsplit"])
+    assert _lib.plan(*shape, total_k=64 * 4096, kv_bits=8)["kind"] == 2       # FP8 / int8: the latent kernel
+    assert _lib.plan(*shape, total_k=64 * 4096, kv_bits=4)["kind"] == 3       # int4: groups of 16 heads
+    assert _lib.plan(*shape, total_k=64 * 4096, distinct_v=True)["kind"] == 2
+    assert _lib.plan(*shape, total_k=64 * 4096, distinct_v=True, page_size=8)["kind"] == 1  # the remaining cliff
+    assert _lib.plan(*shape, total_k=64 * 4096, distinct_v=True, kv_bits=8)["kind"] == 1
+    # more work-groups over an 8-bit latent cache than over a 16-bit one at a mid-sized batch
+    assert _lib.plan(4096, 16, 128, 1, 576, 512, kv_bits=8)["nsplit"] > _lib.plan(4096, 16, 128, 1, 576, 512)["nsplit"]
+    ragged = _lib.plan(8192, 64, 32, 8, 128, 128, total_k=300000, page_size=64)
+    assert ragged["balanced"] == bool(lib.da_plan_is_balanced(8192, 64, 32, 8, 128, 128, 300000, 64))
+    for bad in (dict(kv_bits=12), dict(page_size=48)):
+        with pytest.raises(RuntimeError):
+            _lib.plan(*shape, **bad)
+    assert lib.da_plan_call(*shape, 0, 0, 0, 16, None, None, None, None, None) == 0  # every output may be null
+
+
 def test_python_face_checks_cpu_inputs():
     w = wl.make_workload(2, 4, 2, 64, 64, 8, torch.float16)
     with pytest.raises(RuntimeError, match="GPU"):
