@@ -32,6 +32,9 @@ EXPORTED_SYMBOLS = (
     "da_plan_distinct_v",
     "da_plan_is_balanced",
     "da_plan_call",
+    "da_decoding_attn_int4kv_tok",
+    "da_decoding_attn_paged_int4kv_tok",
+    "da_workspace_bytes_int4kv_tok",
     "da_supported_head_dims",
     "da_last_error",
     "da_version",
@@ -106,6 +109,13 @@ def _declare(lib):
     lib.da_decoding_attn_paged_int4kv.argtypes = lib.da_decoding_attn_paged_fp8kv.argtypes
     lib.da_workspace_bytes_int4kv.restype = sz
     lib.da_workspace_bytes_int4kv.argtypes = lib.da_workspace_bytes_fp8kv.argtypes
+    # ... and so do the int4 entry points with per-token (scale, zero) pairs (k_params, v_params in the scales' places)
+    lib.da_decoding_attn_int4kv_tok.restype = ci
+    lib.da_decoding_attn_int4kv_tok.argtypes = lib.da_decoding_attn_fp8kv.argtypes
+    lib.da_decoding_attn_paged_int4kv_tok.restype = ci
+    lib.da_decoding_attn_paged_int4kv_tok.argtypes = lib.da_decoding_attn_paged_fp8kv.argtypes
+    lib.da_workspace_bytes_int4kv_tok.restype = sz
+    lib.da_workspace_bytes_int4kv_tok.argtypes = lib.da_workspace_bytes_fp8kv.argtypes
     ip = ctypes.POINTER(ci)
     lib.da_plan.restype = ci
     lib.da_plan.argtypes = [sz, sz, sz, sz, sz, sz, ci, sz, ip, ip, ip, ip]
@@ -159,10 +169,16 @@ def last_error() -> str:
     return load().da_last_error().decode("utf-8", "replace")
 
 
+KV_BITS_INT4_PER_TOKEN = 5  # DA_KV_BITS_INT4_PER_TOKEN of include/decoding_attn_hip.h
+
+
 def plan(max_seq_k, batch, head_q, head_k, dim, dim_v, is_bf16=False, total_k=0, distinct_v=False, page_size=0,
          kv_bits=16):
     """Launch plan of a call: dict(kind, nsplit, chunk, heads_per_group, balanced).  `distinct_v`: V passed as its own
-    buffer; `page_size`: pages of that many tokens (0 = packed); `kv_bits`: 16, 8 (FP8, int8) or 4 (int4)."""
+    buffer; `page_size`: pages of that many tokens (0 = packed); `kv_bits`: 16, 8 (FP8, int8), 4 (int4) or KV_BITS_INT4_PER_TOKEN
+    (int4 with per-token pairs; distinct_v is implied)."""
+    if kv_bits == KV_BITS_INT4_PER_TOKEN:
+        distinct_v = True
     del is_bf16  # (the plan does not depend on it)
     lib = load()
     kind, ns, ch, rt, bal = (ctypes.c_int() for _ in range(5))

@@ -143,9 +143,10 @@ int rows_per_trip(size_t dim) {
 // kv_8bit: K/V are FP8, int8 or int4; the grouped kernel then needs dim % 64 == 0.
 // no_latent_kernel: the cache format has no form of the latent kernel (int4): the latent form then runs on the grouped
 // kernel whatever its size, as ceil(heads / 16) groups per sequence that read the same rows.
+// group_only: the call has a form on the grouped kernel only (per-token quantisation factors): every shape takes it.
 Plan make_plan(size_t max_seq_k, size_t batch, size_t head_q, size_t head_k, size_t dim, size_t dim_v,
                bool v_distinct, size_t total_k, size_t page_size = 0, bool kv_8bit = false,
-               bool no_latent_kernel = false) {
+               bool no_latent_kernel = false, bool group_only = false) {
     const bool packed = page_size == 0;
     Plan pl;
     const int ratio = (int)(head_q / head_k);
@@ -214,7 +215,7 @@ Plan make_plan(size_t max_seq_k, size_t batch, size_t head_q, size_t head_k, siz
         // of them than CUs, and then run two to a CU (not with a distinct V, whose two buffers fill the LDS)
         if (pl.rt <= 64 && !kv_8bit && !latent_vd) target_wgs *= 2;
     } else if (dim <= 256 && !force_sweep && (!kv_8bit || dim % 64 == 0) &&
-               (ratio >= tun().group_min_ratio ||
+               (ratio >= tun().group_min_ratio || group_only ||
                 (tun().group_min_ratio > 1 && (max_seq_k >= 1024 || dim <= 96) &&
                  (long long)batch * (long long)head_k * (long long)max_seq_k >= (1ll << 21)))) {
         // Two or more query heads per KV head, or a single one over long sequences of a large batch: the MFMA sweep streams K/V
@@ -434,15 +435,15 @@ Plan make_plan(size_t max_seq_k, size_t batch, size_t head_q, size_t head_k, siz
 // Workspace bytes of a call: the plan's, or, for a batch beyond one launch (kMaxGridBatch), the largest of its runs'.
 size_t plan_ws_bytes(size_t max_seq_k, size_t batch, size_t head_q, size_t head_k, size_t dim, size_t dim_v,
                      bool v_distinct, size_t total_k, size_t page_size = 0, bool kv_8bit = false,
-                     bool no_latent_kernel = false) {
+                     bool no_latent_kernel = false, bool group_only = false) {
     if (batch <= kMaxGridBatch)
         return make_plan(max_seq_k, batch, head_q, head_k, dim, dim_v, v_distinct, total_k, page_size, kv_8bit,
-                         no_latent_kernel).ws_bytes;
+                         no_latent_kernel, group_only).ws_bytes;
     size_t need = make_plan(max_seq_k, kMaxGridBatch, head_q, head_k, dim, dim_v, v_distinct, 0, page_size, kv_8bit,
-                            no_latent_kernel).ws_bytes;
+                            no_latent_kernel, group_only).ws_bytes;
     if (batch % kMaxGridBatch != 0)
         need = std::max(need, make_plan(max_seq_k, batch % kMaxGridBatch, head_q, head_k, dim, dim_v, v_distinct, 0,
-                                        page_size, kv_8bit, no_latent_kernel).ws_bytes);
+                                        page_size, kv_8bit, no_latent_kernel, group_only).ws_bytes);
     return need;
 }
 
@@ -598,14 +599,17 @@ int da_plan_call(size_t max_seq_k, size_t batch, size_t head_q, size_t head_k, s
         return fail(DA_ERR_INVALID_ARGUMENT, "head_q (%zu) must be a multiple of head_k (%zu)", head_q, head_k);
     if (!supported_dims(dim, dim_v))
         return fail(DA_ERR_UNSUPPORTED, "unsupported head dims (dim %zu, dim_v %zu)", dim, dim_v);
-    if (kv_bits != 16 && kv_bits != 8 && kv_bits != 4)
-        return fail(DA_ERR_INVALID_ARGUMENT, "kv_bits (%d) must be 16, 8 or 4", kv_bits);
+    const bool per_token = kv_bits == DA_KV_BITS_INT4_PER_TOKEN;
+    if (kv_bits != 16 && kv_bits != 8 && kv_bits != 4 && !per_token)
+        return fail(DA_ERR_INVALID_ARGUMENT, "kv_bits (%d) must be 16, 8, 4 or DA_KV_BITS_INT4_PER_TOKEN", kv_bits);
+    if (per_token && (dim != dim_v || (dim != 64 && dim != 128 && dim != 256) || !distinct_v))
+        return fail(DA_ERR_UNSUPPORTED, "per-token factors: head dims (64,64), (128,128) and (256,256), V of its own");
     if (page_size != 0 && (page_size & (page_size - 1)) != 0)
         return fail(DA_ERR_INVALID_ARGUMENT, "page_size (%zu) must be a power of two", page_size);
     // (as run_attention plans one launch; a batch beyond one grid axis is planned run by run, without the count)
     const bool folded = batch > kMaxGridBatch;
     const Plan pl = make_plan(max_seq_k, folded ? kMaxGridBatch : batch, head_q, head_k, dim, dim_v, distinct_v != 0,
-                              folded ? 0 : total_k, page_size, kv_bits != 16, kv_bits == 4);
+                              folded ? 0 : total_k, page_size, kv_bits != 16, kv_bits == 4 || per_token, per_token);
     if (kernel_kind) *kernel_kind = pl.kind;
     if (nsplit) *nsplit = pl.nsplit;
     if (chunk) *chunk = pl.chunk;
@@ -661,6 +665,9 @@ struct KvFormat {
     int fmt = 0;
     const float* k_scale = nullptr;
     const float* v_scale = nullptr;
+    // (int4) a (scale, zero) pair per (token, KV head) instead of the per-head factors
+    const float* k_tok = nullptr;
+    const float* v_tok = nullptr;
 };
 
 KvFormat kv8_format(int fmt, const float* k_scale, const float* v_scale) {
@@ -722,8 +729,19 @@ int run_attention(const void* q, const void* k, const void* v, void* o, const in
     }
 
     hipStream_t stream = reinterpret_cast<hipStream_t>(hip_stream);
+    const bool per_token = kf.k_tok != nullptr || kf.v_tok != nullptr;
+    if (per_token) {
+        if (kf.fmt != da::kKvInt4 || !kf.k_tok || !kf.v_tok || !v)
+            return fail(DA_ERR_INVALID_ARGUMENT, "per-token factors need an int4 cache, both k_params and v_params, and v");
+        if (dim != dim_v || (dim != 64 && dim != 128 && dim != 256))
+            return fail(DA_ERR_UNSUPPORTED, "per-token factors: head dims (64,64), (128,128) and (256,256) only");
+        if ((reinterpret_cast<uintptr_t>(kf.k_tok) | reinterpret_cast<uintptr_t>(kf.v_tok)) & 7u)
+            return fail(DA_ERR_INVALID_ARGUMENT, "k_params and v_params must be 8-byte aligned");
+    }
     const Plan pl = make_plan(max_seq_k, batch, head_q, head_k, dim, dim_v, v != nullptr, total_k,
-                              pg.table ? pg.page_size : 0, kf.fmt != 0, kf.fmt == da::kKvInt4);
+                              pg.table ? pg.page_size : 0, kf.fmt != 0, kf.fmt == da::kKvInt4, per_token);
+    if (per_token && pl.kind != kKindGroup)  // (DA_FORCE_KIND=1 takes the grouped kernel away)
+        return fail(DA_ERR_UNSUPPORTED, "per-token factors need the grouped kernel");
     if ((size_t)head_k * pl.groups > 65535)
         return fail(DA_ERR_INVALID_ARGUMENT, "head_k * groups exceeds the grid limit 65535");
     if (kf.fmt == da::kKvInt4 && pl.kind == kKindMfma)  // (DA_MLA_GROUP_HEADS=0 takes the grouped kernel away)
@@ -776,6 +794,8 @@ int run_attention(const void* q, const void* k, const void* v, void* o, const in
     sp.is_alibi = is_alibi ? 1 : 0;
     sp.k_scale = kf.k_scale;
     sp.v_scale = kf.v_scale;
+    sp.k_tok = kf.k_tok;
+    sp.v_tok = kf.v_tok;
     sp.block_table = pg.table;
     sp.seq_lens = pg.seq_lens;
     sp.page_shift = 0;
@@ -812,6 +832,8 @@ int run_attention(const void* q, const void* k, const void* v, void* o, const in
             e = da::launch_mla_kv8(sp, kf.fmt, is_bf16 != 0, pl.rt, grid, stream);
         else if (pl.kind == kKindGroup && kf.fmt == da::kKvInt8)
             e = da::launch_gqa_mfma_i8(sp, is_bf16 != 0, (int)dim, pl.rt, pl.wave_per_head, grid, stream);
+        else if (pl.kind == kKindGroup && per_token)
+            e = da::launch_gqa_mfma_i4t(sp, is_bf16 != 0, (int)dim, pl.rt, pl.wave_per_head, grid, stream);
         else if (pl.kind == kKindGroup && kf.fmt == da::kKvInt4)
             e = da::launch_gqa_mfma_i4(sp, is_bf16 != 0, (int)dim, pl.rt, pl.wave_per_head, grid, stream);
         else if (pl.kind == kKindGroup)
@@ -1034,6 +1056,45 @@ size_t da_workspace_bytes_int4kv(size_t max_seq_k, size_t batch, size_t head_q, 
     const size_t a = plan_ws_bytes(max_seq_k, batch, head_q, head_k, dim, dim_v, false, total_k, page_size, true, true);
     const size_t b = plan_ws_bytes(max_seq_k, batch, head_q, head_k, dim, dim_v, true, total_k, page_size, true, true);
     return a > b ? a : b;
+}
+
+int da_decoding_attn_int4kv_tok(const void* q, const void* k4, const void* v4, void* o, const int32_t* cu_seq_k,
+                                size_t max_seq_k, size_t batch, size_t head_q, size_t head_k, size_t dim, size_t dim_v,
+                                int is_alibi, int is_bf16, float softmax_scale, const float* alibi_slopes,
+                                const float* k_params, const float* v_params, size_t total_k, void* workspace,
+                                size_t workspace_bytes, void* hip_stream) {
+    if (!k_params || !v_params) return fail(DA_ERR_INVALID_ARGUMENT, "k_params or v_params is null");
+    KvFormat kf = kv8_format(da::kKvInt4, nullptr, nullptr);
+    kf.k_tok = k_params;
+    kf.v_tok = v_params;
+    return run_attention(q, k4, v4, o, cu_seq_k, Paging{}, kf, max_seq_k, batch, head_q, head_k, dim, dim_v, is_alibi,
+                         is_bf16, softmax_scale, alibi_slopes, total_k, workspace, workspace_bytes, hip_stream);
+}
+
+int da_decoding_attn_paged_int4kv_tok(const void* q, const void* k_pages, const void* v_pages, void* o,
+                                      const int32_t* block_table, const int32_t* seq_lens, size_t max_seq_k,
+                                      size_t batch, size_t head_q, size_t head_k, size_t dim, size_t dim_v,
+                                      size_t page_size, size_t max_blocks_per_seq, size_t k_page_stride,
+                                      size_t v_page_stride, int is_alibi, int is_bf16, float softmax_scale,
+                                      const float* alibi_slopes, const float* k_params, const float* v_params,
+                                      size_t total_k, void* workspace, size_t workspace_bytes, void* hip_stream) {
+    if (!k_params || !v_params) return fail(DA_ERR_INVALID_ARGUMENT, "k_params or v_params is null");
+    Paging pg;
+    const int rc = check_paging(block_table, seq_lens, max_seq_k, head_k, dim, dim_v, page_size, max_blocks_per_seq,
+                                k_page_stride, v_page_stride, v_pages != nullptr, &pg);
+    if (rc != DA_OK) return rc;
+    KvFormat kf = kv8_format(da::kKvInt4, nullptr, nullptr);
+    kf.k_tok = k_params;
+    kf.v_tok = v_params;
+    return run_attention(q, k_pages, v_pages, o, nullptr, pg, kf, max_seq_k, batch, head_q, head_k, dim, dim_v,
+                         is_alibi, is_bf16, softmax_scale, alibi_slopes, total_k, workspace, workspace_bytes,
+                         hip_stream);
+}
+
+size_t da_workspace_bytes_int4kv_tok(size_t max_seq_k, size_t batch, size_t head_q, size_t head_k, size_t dim,
+                                     size_t dim_v, size_t total_k, size_t page_size) {
+    if (head_k == 0 || head_q % head_k != 0 || dim != dim_v || (dim != 64 && dim != 128 && dim != 256)) return 0;
+    return plan_ws_bytes(max_seq_k, batch, head_q, head_k, dim, dim_v, true, total_k, page_size, true, true, true);
 }
 
 int da_release_workspaces(void) { return release_cached_workspaces(true); }

@@ -125,6 +125,9 @@ constexpr int kKvInt8 = 2;  // two's-complement integers
 // and the load halves the address again (kv4_load8 / kv4_load16; every address the kernels form is even); the
 // conversion to the compute type takes the nibbles straight to 16-bit values (int4x8_to_16).
 constexpr int kKvInt4 = 3;
+// Flag on top of a format (grouped kernel's template argument only): every (token, KV head) row carries its own
+// (scale, zero) pair, element = scale * (integer - zero), instead of one factor per KV head (SweepParams::k_tok).
+constexpr int kKvPerToken = 8;
 
 // Eight FP8 (OCP e4m3) values -> eight 16-bit elements of the compute type.  Both conversions are exact (e4m3
 // has 3 mantissa bits and |x| <= 448), so an FP8 K/V cache feeds the same arithmetic as a 16-bit one.
@@ -292,6 +295,11 @@ struct SweepParams {
     // The kernels fold k_scale into the softmax scale and v_scale into the final normalisation.
     const float* k_scale;
     const float* v_scale;
+    // Per-token asymmetric quantisation (grouped kernel, int4): (scale, zero) float pairs per (token, KV head), laid
+    // out like the rows they belong to ([total_k, head_k, 2], or [pages, page_size, head_k, 2] dense);
+    // K[t, hk, c] = k_tok[t, hk].scale * (integer - k_tok[t, hk].zero), V likewise.  Null: per-head factors above.
+    const float* k_tok;
+    const float* v_tok;
     // Balanced form of the grouped-head kernel's grid (flat_wgs == 0: off).  The sequences lie end to end on one line
     // measured in units of flat_unit tokens (1 for packed K/V, where the line is cu_seq_k itself; 32 for paged K/V,
     // where every sequence is rounded up to whole units so that shares start on tile boundaries); flat_cu[b] is the

@@ -79,6 +79,15 @@ struct Mma16<bf16_tag> {
     }
 };
 
+// x rounded to the 16-bit compute type and widened again
+template <typename Tag>
+__device__ __forceinline__ float round16(float x) {
+    if constexpr (std::is_same<Tag, bf16_tag>::value)
+        return (float)(__bf16)x;
+    else
+        return (float)(_Float16)x;
+}
+
 // Wait states between the last matrix instruction issued from assembly and the first ordinary read of its result
 // (the compiler cannot see into the assembly to place them).
 __device__ __forceinline__ void settle(f32x4& c) { asm volatile("s_nop 15\n\ts_nop 3" : "+v"(c)); }
@@ -91,10 +100,13 @@ constexpr int gqa_v_pitch() { return DV * 2 + 32; }  // LDS row pitch of the V t
 template <int DV>
 constexpr int gqa_merge_pitch() { return DV + 4; }  // floats per row of the merge area: conflict-free row writes
 
+constexpr int kGqaTokBytes = 512;  // per wave: the (scale, zero) pairs of a tile's tokens, K and V (per-token factors)
+
 template <int DV>
-constexpr size_t gqa_lds_bytes(int nt) {
-    // V tiles of the four waves, reused for the final merge ([4][heads][pitch] floats + (m, l))
-    const size_t vt = 4 * (size_t)kGqaTile * gqa_v_pitch<DV>();
+constexpr size_t gqa_lds_bytes(int nt, bool per_token = false) {
+    // V tiles of the four waves (and, behind them, their tiles' per-token pairs), reused for the final merge
+    // ([4][heads][pitch] floats + (m, l))
+    const size_t vt = 4 * (size_t)kGqaTile * gqa_v_pitch<DV>() + (per_token ? 4 * kGqaTokBytes : 0);
     const size_t mg = 4 * (size_t)(16 * nt) * (gqa_merge_pitch<DV>() + 2) * sizeof(float);
     return vt > mg ? vt : mg;
 }
@@ -129,6 +141,13 @@ __device__ __forceinline__ void gqa_segment(const SweepParams& p, uint8_t* const
     constexpr int NW = WH ? 1 : 4;  // wavefronts that share the tokens of one KV head
     constexpr int HG = 16 * NT;     // query heads per KV head and work-group
     constexpr float kLazy = 8.0f;   // the running maximum moves only when exceeded by this much (log2 units)
+    constexpr int FMT = KV8 & 7;                    // element format (kKvFp8, kKvInt8, kKvInt4; 0 = 16-bit)
+    // TOK: every (token, KV head) row has its own (scale, zero) pair (p.k_tok, p.v_tok): with integers n,
+    // K[t][c] = a_k[t] (n[t][c] - z_k[t]), so q . K[t] = a_k[t] (q . n[t] - z_k[t] sum_c q[c]): the matrix
+    // instruction works on the integers, and the score tile takes one multiply-add per element with the sum of the
+    // head's q row.  V[t][c] = a_v[t] (n[t][c] - z_v[t]) likewise: the probabilities are multiplied by a_v[t] on
+    // their way into the second product, and sum_t p'[t] z_v[t], one number per head, comes off every column at the end.
+    constexpr bool TOK = (KV8 & kKvPerToken) != 0;
     constexpr int KB = KV8 ? 1 : 2;                 // bytes per K/V element
     constexpr int KSR = KV8 ? KS / 2 : KS;          // K registers (16 bytes) per 16-token tile
     constexpr int CPRL = KV8 ? DV / 16 : CPR;       // 16-byte chunks per V row as loaded
@@ -139,6 +158,7 @@ __device__ __forceinline__ void gqa_segment(const SweepParams& p, uint8_t* const
     static_assert(!VK || (DV < D && DV % 64 == 0), "value columns inside the key rows");
     static_assert(D % 32 == 0 && DV % 16 == 0 && (kGqaTile * CPR) % 64 == 0, "shape");
     static_assert(!KV8 || (D % 64 == 0 && (kGqaTile * CPRL) % 64 == 0), "8-bit K/V: two k-steps per 16-byte load");
+    static_assert(!TOK || (!VK && (FMT == kKvInt8 || FMT == kKvInt4)), "per-token factors: integer K/V, V of its own");
 
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
@@ -177,13 +197,30 @@ __device__ __forceinline__ void gqa_segment(const SweepParams& p, uint8_t* const
         }
         slope[nt] = p.is_alibi ? alibi_slope_log2(p.slopes, h, p.head_q) : 0.0f;
     }
+    // (TOK) sum of each head's q row: the four 16-lane groups hold different elements of the same rows
+    float qsum[NT];
+    if constexpr (TOK) {
+#pragma unroll
+        for (int nt = 0; nt < NT; ++nt) {
+            float acc_q = 0.0f;
+#pragma unroll
+            for (int ks = 0; ks < KS; ++ks)
+#pragma unroll
+                for (int j = 0; j < 8; ++j) acc_q += (float)qf[nt][ks][j];
+            acc_q += __shfl_xor(acc_q, 16);
+            acc_q += __shfl_xor(acc_q, 32);
+            qsum[nt] = acc_q;
+        }
+    }
 
     f32x4 acc[NT][CT];
     float m[NT], l[NT];
+    float corr[NT];  // (TOK) sum over tokens of p'[t] z_v[t], in the accumulators' units
 #pragma unroll
     for (int nt = 0; nt < NT; ++nt) {
         m[nt] = kNegBig;
         l[nt] = 0.0f;
+        corr[nt] = 0.0f;
 #pragma unroll
         for (int ct = 0; ct < CT; ++ct) acc[nt][ct] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
     }
@@ -195,8 +232,8 @@ __device__ __forceinline__ void gqa_segment(const SweepParams& p, uint8_t* const
     const uint8_t* const vbytes = reinterpret_cast<const uint8_t*>(p.v) + (size_t)hk * p.v_head * KB;
     const uint32_t k_row_b = (uint32_t)p.k_row * KB, v_row_b = (uint32_t)p.v_row * KB;
     // (an int4 cache's elements come out of the conversion times a power of two, divided out here)
-    const float sl = p.scale_log2 * head_scale(p.k_scale, hk) * kv_widening_inverse<KV8>();  // score scale, log2 units
-    const float vs = head_scale(p.v_scale, hk) * kv_widening_inverse<KV8>();
+    const float sl = p.scale_log2 * head_scale(p.k_scale, hk) * kv_widening_inverse<FMT>();  // score scale, log2 units
+    const float vs = head_scale(p.v_scale, hk) * kv_widening_inverse<FMT>();
 
     // wave-private V tile in LDS
     uint8_t* const vt = smem + wave * (kGqaTile * VP);
@@ -211,6 +248,7 @@ __device__ __forceinline__ void gqa_segment(const SweepParams& p, uint8_t* const
     struct TileRegs {
         uint4 k[2][KSR];
         uint4 v[NVR];
+        float2 tokp;  // (TOK) lanes 0 .. 31: the K pair of the tile's token `lane`; 32 .. 63: the V pair of lane - 32
     };
     TileRegs tr;
 
@@ -232,7 +270,7 @@ __device__ __forceinline__ void gqa_segment(const SweepParams& p, uint8_t* const
     // fetched again for the second (32/8 heads d 96, batch 256 x 4096 tokens: 594.5 us with the hint, 544.6 without;
     // batch 16 x 4096: 39.9 and 32.9).
     auto kv_load16 = [](const uint8_t* ptr) __attribute__((always_inline)) {
-        if constexpr (KV8 == kKvInt4)
+        if constexpr (FMT == kKvInt4)
             return kv4_load16(ptr);  // (eight bytes from half the address, widened to sixteen int8 elements)
         else if constexpr (VK || (D * KB) % 128 != 0)
             return *reinterpret_cast<const uint4*>(ptr);
@@ -261,6 +299,26 @@ __device__ __forceinline__ void gqa_segment(const SweepParams& p, uint8_t* const
             const uint32_t off = (uint32_t)(min(mt * 16 + n, last) - (second ? 16 : 0)) * k_row_b + g * 16;
 #pragma unroll
             for (int ks = 0; ks < KSR; ++ks) r.k[mt][ks] = kv_load16(base + off + ks * 64);
+        }
+    };
+    // (TOK) one pair per lane and tile, rows past the end as the last valid one; the wave passes them through its
+    // corner of LDS (tokbuf: K scales, K zeros, V scales, V zeros, 32 floats each) to the lanes that need them
+    float* const tokbuf = reinterpret_cast<float*>(smem + 4 * kGqaTile * VP + wave * kGqaTokBytes);
+    auto load_tok = [&](int tok0, TileRegs& r) __attribute__((always_inline)) {
+        if constexpr (TOK) {
+            const int row = min(lane & 31, c1 - 1 - tok0);
+            int64_t at;  // the row's number in the pools' row numbering (a page holds 2^page_shift rows)
+            if (p.block_table == nullptr) {
+                at = (int64_t)start + tok0 + row;
+            } else if constexpr (PGM == 0) {
+                at = ((int64_t)page_of(p, b, tok0) << p.page_shift) + ((tok0 & ((1 << p.page_shift) - 1)) + row);
+            } else {
+                const int tok = tok0 + row;
+                at = ((int64_t)p.block_table[(int64_t)b * p.max_blocks + (tok >> p.page_shift)] << p.page_shift) +
+                     (tok & ((1 << p.page_shift) - 1));
+            }
+            const float2* const pool = reinterpret_cast<const float2*>(lane < 32 ? p.k_tok : p.v_tok);
+            r.tokp = pool[at * p.head_k + hk];
         }
     };
     auto load_v = [&](int tok0, TileRegs& r) __attribute__((always_inline)) {
@@ -294,6 +352,7 @@ __device__ __forceinline__ void gqa_segment(const SweepParams& p, uint8_t* const
     if (tw < ntiles) {
         if constexpr (!VK) load_v(c0 + tw * kGqaTile, tr);
         load_k(c0 + tw * kGqaTile, tr);
+        load_tok(c0 + tw * kGqaTile, tr);
     }
 
     for (int t = tw; t < ntiles; t += NW) {
@@ -309,9 +368,9 @@ __device__ __forceinline__ void gqa_segment(const SweepParams& p, uint8_t* const
             const int row = slot / CPRL, ch = slot % CPRL;
             if constexpr (KV8) {  // sixteen 8-bit elements become 32 bytes of the 16-bit tile
                 *reinterpret_cast<uint4*>(vt + row * VP + ch * 32) =
-                    kv8x8_to_16<Tag, KV8>(make_uint2(tr.v[i].x, tr.v[i].y));
+                    kv8x8_to_16<Tag, FMT>(make_uint2(tr.v[i].x, tr.v[i].y));
                 *reinterpret_cast<uint4*>(vt + row * VP + ch * 32 + 16) =
-                    kv8x8_to_16<Tag, KV8>(make_uint2(tr.v[i].z, tr.v[i].w));
+                    kv8x8_to_16<Tag, FMT>(make_uint2(tr.v[i].z, tr.v[i].w));
             } else {
                 *reinterpret_cast<uint4*>(vt + row * VP + ch * 16) = tr.v[i];
             }
@@ -331,7 +390,7 @@ __device__ __forceinline__ void gqa_segment(const SweepParams& p, uint8_t* const
                     uint4 kfrag;
                     if constexpr (KV8) {
                         const uint4 w = tr.k[mt][ks >> 1];
-                        kfrag = kv8x8_to_16<Tag, KV8>((ks & 1) ? make_uint2(w.z, w.w) : make_uint2(w.x, w.y));
+                        kfrag = kv8x8_to_16<Tag, FMT>((ks & 1) ? make_uint2(w.z, w.w) : make_uint2(w.x, w.y));
                     } else {
                         kfrag = tr.k[mt][ks];
                     }
@@ -356,9 +415,9 @@ __device__ __forceinline__ void gqa_segment(const SweepParams& p, uint8_t* const
 #pragma unroll
                     for (int j = 0; j < DV / 64; ++j) {
                         const uint4 w = tr.k[mt][j];
-                        *reinterpret_cast<uint4*>(row + j * 128 + g * 32) = kv8x8_to_16<Tag, KV8>(make_uint2(w.x, w.y));
+                        *reinterpret_cast<uint4*>(row + j * 128 + g * 32) = kv8x8_to_16<Tag, FMT>(make_uint2(w.x, w.y));
                         *reinterpret_cast<uint4*>(row + j * 128 + g * 32 + 16) =
-                            kv8x8_to_16<Tag, KV8>(make_uint2(w.z, w.w));
+                            kv8x8_to_16<Tag, FMT>(make_uint2(w.z, w.w));
                     }
                 } else {
 #pragma unroll
@@ -373,10 +432,57 @@ __device__ __forceinline__ void gqa_segment(const SweepParams& p, uint8_t* const
         vec8 pf[NT];
         const bool tail = tok0 + kGqaTile > c1;
         float x[NT][8], mx[NT];
+        // (TOK) per token: A = score scale x a_k, Z = z_k in the score tile's units (the integers come out of the
+        // conversion times kv_widening_inverse()^-1); x = A (s - Z qsum)
+        float tokA[TOK ? 8 : 1], tokZ[TOK ? 8 : 1], tokV[TOK ? 8 : 1], tokW[TOK ? 8 : 1], tokVinv[TOK ? 8 : 1];
+        if constexpr (TOK) {
+            float* const mine = tokbuf + (lane >> 5) * 64 + (lane & 31);
+            mine[0] = tr.tokp.x;
+            mine[32] = tr.tokp.y;
+            if (PREFETCH && more) load_tok(tok_next, tr);
+#pragma unroll
+            for (int mt = 0; mt < 2; ++mt) {
+                const f32x4 ak = *reinterpret_cast<const f32x4*>(tokbuf + mt * 16 + g * 4);
+                const f32x4 zk = *reinterpret_cast<const f32x4*>(tokbuf + 32 + mt * 16 + g * 4);
+                const f32x4 av = *reinterpret_cast<const f32x4*>(tokbuf + 64 + mt * 16 + g * 4);
+                const f32x4 zv = *reinterpret_cast<const f32x4*>(tokbuf + 96 + mt * 16 + g * 4);
+#pragma unroll
+                for (int r = 0; r < 4; ++r) {
+                    tokA[mt * 4 + r] = sl * ak[r];
+                    tokZ[mt * 4 + r] = zk[r] * (1.0f / kv_widening_inverse<FMT>());
+                    tokV[mt * 4 + r] = av[r];
+                    tokW[mt * 4 + r] = zv[r] * (1.0f / kv_widening_inverse<FMT>());
+                    if constexpr (std::is_same<Tag, bf16_tag>::value)
+                        tokVinv[mt * 4 + r] = __builtin_amdgcn_rcpf(av[r]);
+                }
+            }
+        }
 #pragma unroll
         for (int nt = 0; nt < NT; ++nt) {
             mx[nt] = -INFINITY;
-            if (p.is_alibi || tail) {
+            if constexpr (TOK) {
+                if (p.is_alibi || tail) {
+#pragma unroll
+                    for (int mt = 0; mt < 2; ++mt)
+#pragma unroll
+                        for (int r = 0; r < 4; ++r) {
+                            const int tok = tok0 + mt * 16 + g * 4 + r;
+                            float v = (s[mt][nt][r] - tokZ[mt * 4 + r] * qsum[nt]) * tokA[mt * 4 + r] +
+                                      slope[nt] * (float)(tok - (len - 1));
+                            if (tok >= c1) v = -INFINITY;
+                            x[nt][mt * 4 + r] = v;
+                            mx[nt] = fmaxf(mx[nt], v);
+                        }
+                } else {
+#pragma unroll
+                    for (int mt = 0; mt < 2; ++mt)
+#pragma unroll
+                        for (int r = 0; r < 4; ++r) {
+                            x[nt][mt * 4 + r] = (s[mt][nt][r] - tokZ[mt * 4 + r] * qsum[nt]) * tokA[mt * 4 + r];
+                            mx[nt] = fmaxf(mx[nt], x[nt][mt * 4 + r]);
+                        }
+                }
+            } else if (p.is_alibi || tail) {
 #pragma unroll
                 for (int mt = 0; mt < 2; ++mt)
 #pragma unroll
@@ -412,6 +518,7 @@ __device__ __forceinline__ void gqa_segment(const SweepParams& p, uint8_t* const
                 const float alpha = fast_exp2(m[nt] - mn);
                 m[nt] = mn;
                 l[nt] *= alpha;
+                if constexpr (TOK) corr[nt] *= alpha;
 #pragma unroll
                 for (int ct = 0; ct < CT; ++ct) acc[nt][ct] *= alpha;
             }
@@ -420,8 +527,21 @@ __device__ __forceinline__ void gqa_segment(const SweepParams& p, uint8_t* const
         for (int nt = 0; nt < NT; ++nt) {
 #pragma unroll
             for (int j = 0; j < 8; ++j) {
-                x[nt][j] = as_second_operand<Tag>(fast_exp2(x[nt][j] - m[nt]));
-                l[nt] += x[nt][j];
+                if constexpr (TOK) {
+                    // the second product's operand is p a_v[t], rounded to 16 bits; the zero-point sum uses the
+                    // rounded value, and so does the denominator where the rounding is coarse (bf16)
+                    const float pe = fast_exp2(x[nt][j] - m[nt]);
+                    const float pv = round16<Tag>(pe * tokV[j]);
+                    if constexpr (std::is_same<Tag, bf16_tag>::value)
+                        l[nt] += pv * tokVinv[j];
+                    else
+                        l[nt] += pe;
+                    corr[nt] = __builtin_fmaf(pv, tokW[j], corr[nt]);
+                    x[nt][j] = pv;
+                } else {
+                    x[nt][j] = as_second_operand<Tag>(fast_exp2(x[nt][j] - m[nt]));
+                    l[nt] += x[nt][j];
+                }
             }
             pf[nt] = MM::pack8(x[nt]);  // k index j <-> token g*4+j (j<4), 16+g*4+(j-4) (j>=4)
         }
@@ -440,6 +560,7 @@ __device__ __forceinline__ void gqa_segment(const SweepParams& p, uint8_t* const
         if (!PREFETCH && more) {
             if constexpr (!VK) load_v(tok_next, tr);
             load_k(tok_next, tr);
+            load_tok(tok_next, tr);
         }
     }
 
@@ -448,6 +569,12 @@ __device__ __forceinline__ void gqa_segment(const SweepParams& p, uint8_t* const
     for (int nt = 0; nt < NT; ++nt) {
         l[nt] += __shfl_xor(l[nt], 16);
         l[nt] += __shfl_xor(l[nt], 32);
+        if constexpr (TOK) {  // the zero points' share comes off every column of the head
+            corr[nt] += __shfl_xor(corr[nt], 16);
+            corr[nt] += __shfl_xor(corr[nt], 32);
+#pragma unroll
+            for (int ct = 0; ct < CT; ++ct) acc[nt][ct] -= corr[nt];
+        }
     }
 
     if constexpr (WH) {
@@ -623,5 +750,8 @@ hipError_t launch_gqa_mfma_i8(const SweepParams& p, bool is_bf16, int dim, int h
 // ... and over an int4 one (two elements to a byte, see kKvInt4 in da_common.h)
 hipError_t launch_gqa_mfma_i4(const SweepParams& p, bool is_bf16, int dim, int heads_per_group, bool wave_per_head,
                               dim3 grid, hipStream_t stream);
+// ... and over an int4 one whose rows carry their own (scale, zero) pairs (SweepParams::k_tok, v_tok); dim 64, 128, 256
+hipError_t launch_gqa_mfma_i4t(const SweepParams& p, bool is_bf16, int dim, int heads_per_group, bool wave_per_head,
+                               dim3 grid, hipStream_t stream);
 
 }  // namespace da

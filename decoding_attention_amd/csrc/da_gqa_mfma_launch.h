@@ -1,5 +1,5 @@
 // Launch helpers of the grouped-head MFMA sweep, shared by the translation units that instantiate it (16-bit
-// K/V in da_gqa_mfma.hip, FP8 in da_gqa_mfma_kv8.hip, int8 in da_gqa_mfma_i8.hip; separate units so that the sets
+// K/V in da_gqa_mfma.hip, FP8 in da_gqa_mfma_kv8.hip, int8 in da_gqa_mfma_i8.hip, int4 in da_gqa_mfma_i4.hip and da_gqa_mfma_i4t.hip; separate units so that the sets
 // compile in parallel).
 #pragma once
 #include "da_gqa_mfma.h"
@@ -15,7 +15,7 @@ hipError_t launch_form(const SweepParams& p, dim3 grid, hipStream_t stream) {
     constexpr bool kPrefetch = D <= 128 || D == 576;
     constexpr int kMinWaves = (D <= 128 && (NT == 1 || D <= 64)) ? 2 : 1;
     auto kern = gqa_mfma_kernel<Tag, D, DV, NT, kPrefetch, WH, kMinWaves, KV8, PGM>;
-    const size_t lds = gqa_lds_bytes<DV>(NT);
+    const size_t lds = gqa_lds_bytes<DV>(NT, (KV8 & kKvPerToken) != 0);
     if (lds > 48 * 1024) {
         static std::atomic<uint64_t> devices_done{0};
         const hipError_t attr_err = ensure_lds_limit(reinterpret_cast<const void*>(kern), lds, devices_done);
@@ -53,7 +53,8 @@ hipError_t launch_tag(const SweepParams& p, int dim, int heads_per_group, bool w
         case 128: return launch_dim<Tag, 128, KV8>(p, heads_per_group, wh, grid, stream);
         case 256: return launch_dim<Tag, 256, KV8>(p, heads_per_group, wh, grid, stream);
         case 576:  // the latent form with up to 16 query heads: one KV head, its tokens shared by the four waves
-            if (heads_per_group == 16 && !wh) return launch_one<Tag, 576, 1, false, KV8>(p, grid, stream);
+            if constexpr ((KV8 & kKvPerToken) == 0)
+                if (heads_per_group == 16 && !wh) return launch_one<Tag, 576, 1, false, KV8>(p, grid, stream);
             return hipErrorInvalidValue;
         default: return hipErrorInvalidValue;
     }

@@ -67,6 +67,18 @@ def pack_int4(x: torch.Tensor) -> torch.Tensor:
     return (n[..., 0::2] | (n[..., 1::2] << 4)).to(torch.uint8)
 
 
+def quantize_int4_per_token(x: torch.Tensor):
+    """Asymmetric int4 quantisation with one (scale, zero) pair per row of the last dimension (per token and KV head):
+    returns (packed, pairs) with x ~= pairs[..., 0] * (n - pairs[..., 1]), n the integers -8 .. 7 stored in `packed`
+    (pack_int4's layout), pairs float32 [..., 2].  The row's minimum maps to -8 and its maximum to 7."""
+    xf = x.float()
+    lo, hi = xf.amin(dim=-1, keepdim=True), xf.amax(dim=-1, keepdim=True)
+    scale = ((hi - lo) / 15.0).clamp_min(1e-8)
+    zero = -8.0 - lo / scale
+    n = torch.round(xf / scale + zero).clamp(-8, 7).to(torch.int8)
+    return pack_int4(n), torch.cat([scale, zero], dim=-1).contiguous()
+
+
 def decoding_attn_fwd(q: torch.Tensor, k: torch.Tensor, v: Optional[torch.Tensor], cu_seq_k: torch.Tensor,
                       max_seq_k: int, dim_v: int, is_alibi: bool, *, softmax_scale: Optional[float] = None,
                       alibi_slopes: Optional[torch.Tensor] = None, k_scale: Optional[torch.Tensor] = None,
@@ -85,7 +97,9 @@ def decoding_attn_fwd(q: torch.Tensor, k: torch.Tensor, v: Optional[torch.Tensor
         k_scale, v_scale (keyword only): k and v may be torch.float8_e4m3fn or torch.int8 (an 8-bit K/V cache; q
             stays 16-bit), or torch.uint8 holding pairs of int4 values (see pack_int4: last dimensions dim / 2 and
             dim_v / 2); these are then float32 [head_k] GPU tensors of de-quantisation factors (default 1):
-            K = k_scale * k.
+            K = k_scale * k.  For an int4 cache they may instead be float32 [total_k, head_k, 2] tensors of
+            (scale, zero) pairs, one per token and KV head (quantize_int4_per_token builds them):
+            K[t, h] = k_scale[t, h, 0] * (k[t, h] - k_scale[t, h, 1]); head dims 64, 128 and 256, v required.
     Return:
         o: [total_q, head_q, dim_v], same dtype as q.
     """
@@ -116,7 +130,8 @@ def decoding_attn_paged_fwd(q: torch.Tensor, k_pages: torch.Tensor, v_pages: Opt
         page_size (from k_pages.shape[1]) must be a power of two.
         total_k (keyword only): sum of seq_lens if the host knows it; only a hint for sizing sequence splits.
         k_scale, v_scale (keyword only): as for decoding_attn_fwd, when the pools are torch.float8_e4m3fn, torch.int8
-            or torch.uint8 holding pairs of int4 values (last dimensions dim / 2 and dim_v / 2).
+            or torch.uint8 holding pairs of int4 values (last dimensions dim / 2 and dim_v / 2); per-token
+            (scale, zero) pairs of an int4 cache are float32 [pages, page_size, head_k, 2].
     Return:
         o: [batch, head_q, dim_v], same dtype as q.
     """

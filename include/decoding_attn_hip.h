@@ -206,6 +206,37 @@ size_t da_workspace_bytes_int4kv(size_t max_seq_k, size_t batch, size_t head_q, 
                                  size_t dim_v, size_t total_k, size_t page_size);
 
 /*
+ * int4 K/V with a (scale, zero) pair per (token, KV head) -- asymmetric per-token quantisation, the group-wise scheme
+ * with the head dimension as the group (the reference's quantisation to-do, README.md:154-156, names no scheme; it
+ * has no such path).  k4 and v4 as for da_decoding_attn_int4kv, both required; k_params and v_params hold float pairs
+ * laid out like the rows they belong to: [total_k, head_k, 2] for the packed layout, [pages, page_size, head_k, 2]
+ * (dense, indexed through the same block table) for page pools, 8-byte aligned:
+ *   K[t, hk, c] = k_params[t, hk, 0] * (int4 value - k_params[t, hk, 1]),   V likewise with v_params.
+ * Head dims (64,64), (128,128) and (256,256), any head grouping, every page size, ALiBi; all shapes run on the
+ * grouped-head kernel, whose matrix instructions work on the integers: the score tile takes one multiply-add per
+ * element with the sum of the head's q row (q . K[t] = scale (q . n[t] - zero sum(q))), the probabilities are
+ * multiplied by the V scale of their token on the way into the second product, and the zero points' share, one number
+ * per head, comes off every output column at the end.  V scales must keep p * scale inside the compute type's range
+ * (fp16: below 2^7 is always safe).  Returns DA_ERR_UNSUPPORTED for other head dims.
+ */
+int da_decoding_attn_int4kv_tok(const void *q, const void *k4, const void *v4, void *o, const int32_t *cu_seq_k,
+                                size_t max_seq_k, size_t batch, size_t head_q, size_t head_k, size_t dim, size_t dim_v,
+                                int is_alibi, int is_bf16, float softmax_scale, const float *alibi_slopes,
+                                const float *k_params, const float *v_params, size_t total_k, void *workspace,
+                                size_t workspace_bytes, void *hip_stream);
+
+int da_decoding_attn_paged_int4kv_tok(const void *q, const void *k_pages, const void *v_pages, void *o,
+                                      const int32_t *block_table, const int32_t *seq_lens, size_t max_seq_k,
+                                      size_t batch, size_t head_q, size_t head_k, size_t dim, size_t dim_v,
+                                      size_t page_size, size_t max_blocks_per_seq, size_t k_page_stride,
+                                      size_t v_page_stride, int is_alibi, int is_bf16, float softmax_scale,
+                                      const float *alibi_slopes, const float *k_params, const float *v_params,
+                                      size_t total_k, void *workspace, size_t workspace_bytes, void *hip_stream);
+
+size_t da_workspace_bytes_int4kv_tok(size_t max_seq_k, size_t batch, size_t head_q, size_t head_k, size_t dim,
+                                     size_t dim_v, size_t total_k, size_t page_size);
+
+/*
  * Launch plan the library would use for this shape, for tests and benchmarks:
  *   kernel_kind 1 = VALU sweep, 2 = latent (MLA) MFMA sweep, 3 = grouped-head MFMA sweep (also the latent form with
  *   16 query heads or fewer); nsplit = sequence splits;
@@ -242,10 +273,12 @@ int da_plan_is_balanced(size_t max_seq_k, size_t batch, size_t head_q, size_t he
 /*
  * The plan of any call of this library, for benchmarks that report it beside a measurement: page_size 0 = packed
  * layout, else pages of page_size tokens; distinct_v != 0 = V passed as a buffer of its own; kv_bits 16 = fp16/bf16
- * K/V, 8 = the FP8 and int8 caches, 4 = the int4 cache.  Outputs as da_plan's, balanced as da_plan_is_balanced's
+ * K/V, 8 = the FP8 and int8 caches, 4 = the int4 cache, DA_KV_BITS_INT4_PER_TOKEN = the int4 cache with per-token
+ * (scale, zero) pairs (distinct_v must be set).  Outputs as da_plan's, balanced as da_plan_is_balanced's
  * result; any output pointer may be NULL.  No counterpart in the reference (one tile shape per head dim,
  * csrc/kernel/decoding_attn/decoding_fwd_hd*.cu).
  */
+#define DA_KV_BITS_INT4_PER_TOKEN 5
 int da_plan_call(size_t max_seq_k, size_t batch, size_t head_q, size_t head_k, size_t dim, size_t dim_v, size_t total_k,
                  size_t page_size, int distinct_v, int kv_bits, int *kernel_kind, int *nsplit, int *chunk,
                  int *heads_per_group, int *balanced);
