@@ -217,7 +217,14 @@ Plan make_plan(size_t max_seq_k, size_t batch, size_t head_q, size_t head_k, siz
     } else if (dim <= 256 && !force_sweep && (!kv_8bit || dim % 64 == 0) &&
                (ratio >= tun().group_min_ratio || group_only ||
                 (tun().group_min_ratio > 1 && (max_seq_k >= 1024 || dim <= 96) &&
-                 (long long)batch * (long long)head_k * (long long)max_seq_k >= (1ll << 21)))) {
+                 (long long)batch * (long long)head_k * (long long)max_seq_k >= (1ll << 21)) ||
+                // an int4 cache (the format without a latent kernel): the VALU sweep pays more per nibble than the
+                // matrix kernel's word-wise conversion does (measured, MHA 32 heads d 128: batch 512 x 128 tokens 92.0
+                // -> 54.8 us, batch 2048 x 128 397 -> 254, batch 32 x 1024 50.5 -> 30.8, batch 32 x 128 8.7 -> 6.8,
+                // batch 1 x 4096 16.0 -> 10.2; d 64, batch 16 x 512 14.4 -> 11.0; below 2^17 rows of tokens the sweep's
+                // single small launch wins, batch 16 x 128 5.9 against 7.5, and at d 256 it ties or wins)
+                (tun().group_min_ratio > 1 && no_latent_kernel && dim <= 128 &&
+                 (long long)batch * (long long)head_k * (long long)max_seq_k >= (1ll << 17)))) {
         // Two or more query heads per KV head, or a single one over long sequences of a large batch: the MFMA sweep streams K/V
         // a few percent faster than the VALU sweep even though most of its matrix columns are idle (measured:
         // ratio 2, 2048 tokens: 201 -> 185 us; ratio 1, batch 64 x 2048 tokens: 375 -> 364 us; at batch 1 the VALU sweep wins, and
@@ -951,6 +958,8 @@ int da_probe_set_tunable(const char* name, int value) {
     else if (n == "DA_MLA_GROUP_HEADS") t.mla_group_heads = value;
     else if (n == "DA_MFMA_TARGET_WGS") t.mfma_target_wgs = value;
     else if (n == "DA_MFMA_SMALL_WGS") t.mfma_small_wgs = value;
+    else if (n == "DA_GROUP_MIN_RATIO") t.group_min_ratio = value;
+    else if (n == "DA_FORCE_KIND") t.force_kind = value;
     else return fail(DA_ERR_INVALID_ARGUMENT, "unknown tunable %s", name);
     return DA_OK;
 }

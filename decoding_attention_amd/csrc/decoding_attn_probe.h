@@ -46,7 +46,7 @@ int da_probe_sweep_only(const void *q, const void *k, const void *v, void *o, co
 
 /*
  * Overrides one planner tunable (by the name of its environment variable: DA_NSPLIT, DA_MLA_HEADS,
- * DA_MLA_GROUP_SMALL, DA_MLA_GROUP_HEADS, DA_MFMA_TARGET_WGS, DA_MFMA_SMALL_WGS) for later calls into this library in
+ * DA_MLA_GROUP_SMALL, DA_MLA_GROUP_HEADS, DA_MFMA_TARGET_WGS, DA_MFMA_SMALL_WGS, DA_GROUP_MIN_RATIO, DA_FORCE_KIND) for later calls into this library in
  * this process, so that one process can time a shape under several launch plans (bench.py --sweep latent-plan).
  */
 int da_probe_set_tunable(const char *name, int value);

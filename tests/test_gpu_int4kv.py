@@ -110,6 +110,24 @@ def test_int4_equals_int8_on_the_same_integers(shape, dtype):
 
 
 @pytest.mark.gpu
+@pytest.mark.parametrize("dim", [64, 128])
+def test_mha_over_int4_takes_the_grouped_kernel_from_2_17_rows(dim):
+    """One query head per KV head: the matrix kernel (one live head in sixteen) still beats the VALU sweep's
+    nibble conversion once the problem is large enough for its launch to pay."""
+    assert _lib.plan(256, 40, 32, 32, dim, dim, total_k=40 * 256, kv_bits=4)["kind"] == 3
+    assert _lib.plan(256, 8, 32, 32, dim, dim, total_k=8 * 256, kv_bits=4)["kind"] == 1
+    assert _lib.plan(256, 40, 32, 32, dim, dim, total_k=40 * 256, kv_bits=8)["kind"] == 1
+    w, k4, v4, ks, vs = _case(40, 32, 32, dim, dim, 256, torch.float16, seed=31)
+    o = _run(w, k4, v4, ks, vs)
+    rows = [0, 13, 39]
+    cu = w.cu_seq_k.tolist()
+    k4s = torch.cat([k4[cu[b]:cu[b + 1]] for b in rows])
+    v4s = torch.cat([v4[cu[b]:cu[b + 1]] for b in rows])
+    err = (o[rows].float() - _reference(sub_workload(w, rows), k4s, v4s, ks, vs)).abs().max().item()
+    assert torch.isfinite(o.float()).all() and err <= TOL[torch.float16]
+
+
+@pytest.mark.gpu
 def test_alibi_and_softmax_scale_with_int4_kv():
     w, k4, v4, ks, vs = _case(4, 32, 1, 128, 128, 800, torch.float16, is_alibi=True)
     o = _run(w, k4, v4, ks, vs, softmax_scale=0.05)
