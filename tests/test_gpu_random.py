@@ -10,7 +10,7 @@ import random
 import pytest
 import torch
 
-from decoding_attention_amd import decoding_attn_fwd, decoding_attn_paged_fwd, pack_int4
+from decoding_attention_amd import decoding_attn_fwd, decoding_attn_paged_fwd, pack_int4, quantize_int4_per_token
 from decoding_attention_amd import workloads as wl
 from oracle import oracle
 from tests.gpu_util import TOL, run_hip_ex, sub_workload
@@ -23,16 +23,19 @@ HEADS = [(32, 8), (32, 32), (32, 1), (8, 2), (28, 4), (16, 16), (64, 8), (12, 4)
 CASES_PER_CHUNK = 12
 
 
-def _one_case(rng, seed, case, int4=False):
+def _one_case(rng, seed, case, int4=False, per_token=False):
     """int4: the case runs over an int4 cache (whatever format the draws below pick; the stream of draws is the same
-    either way, so the other cases do not move)."""
-    latent = rng.random() < 0.3
+    either way, so the other cases do not move).  per_token: an int4 cache with a (scale, zero) pair per token and KV
+    head (never the latent form, never d = 96, which that entry point does not serve)."""
+    latent = rng.random() < 0.3 and not per_token
     dtype = rng.choice([torch.float16, torch.bfloat16])
     if latent:
         hq, hk, d, dv = rng.choice([16, 32, 64, 128, 96, 8]), 1, 576, 512
     else:
         hq, hk = rng.choice(HEADS)
         d = dv = rng.choice([64, 96, 128, 256])
+        if per_token and d == 96:
+            d = dv = 128
     batch = rng.choice([1, 2, 3, 5, 8, 17, 40, 90])
     maxlen = rng.choice([5, 33, 100, 300, 777, 1500, 3000, 6000])
     if batch * maxlen * hk * d > 1.5e8:
@@ -57,13 +60,27 @@ def _one_case(rng, seed, case, int4=False):
     page = rng.choice([1, 8, 16, 32, 64, 128])
     int8 = fp8 and rng.random() < 0.4  # the 8-bit cache holds int8 instead of FP8
     kv8_dtype = torch.int8 if int8 else FP8
-    if int4:
+    if int4 or per_token:
         fp8, int8, kv8_dtype = True, True, torch.uint8
     desc = (f"seed {seed} case {case}: latent={latent} {hq}/{hk} d{d} {dtype} b{batch} max{maxlen} {mode} "
             f"alibi={alibi} fp8={fp8} int8={int8} {layout} page={page} total={total}")
     kw, k8, v8 = {}, None, None
     k_true, v_true = k.float(), None if v is None else v.float()
-    if fp8:
+    if per_token:
+        # rows of different spread and offset: the pairs differ from token to token and head to head
+        k = k.float() * (0.5 + torch.rand(total, hk, 1, generator=g)) + torch.randn(total, hk, 1, generator=g)
+        v = v.float() * (0.5 + torch.rand(total, hk, 1, generator=g)) + 0.5 * torch.randn(total, hk, 1, generator=g)
+        k8, kpairs = quantize_int4_per_token(k)
+        v8, vpairs = quantize_int4_per_token(v)
+
+        def unpack(p4):
+            n = torch.stack([(p4 & 15).to(torch.int16), (p4 >> 4).to(torch.int16)], dim=-1).flatten(-2)
+            return torch.where(n >= 8, n - 16, n).double()
+
+        k_true = kpairs[..., :1].double() * (unpack(k8) - kpairs[..., 1:].double())
+        v_true = vpairs[..., :1].double() * (unpack(v8) - vpairs[..., 1:].double())
+        kw = dict(k_scale=kpairs.to(DEV), v_scale=vpairs.to(DEV))
+    elif fp8:
         def quantise(x, scale):
             y = x.float() / scale.view(1, -1, 1)
             if int4:
@@ -90,6 +107,10 @@ def _one_case(rng, seed, case, int4=False):
                           None if v is None else (v8.view(torch.uint8) if fp8 else v), cu, max_seq_k, dv, alibi,
                           lens.tolist())
         pk = wl.to_pages(src, page, seed=case, poison=not fp8).to(DEV)
+        if per_token:  # the pairs in pools of their own, numbered like the pages (same seed)
+            pp = wl.to_pages(wl.Workload("pp", q, kpairs, vpairs, cu, max_seq_k, dv, alibi, lens.tolist()), page,
+                             seed=case).to(DEV)
+            kw = dict(k_scale=pp.k_pages, v_scale=pp.v_pages)
         kp = pk.k_pages.view(kv8_dtype) if fp8 else pk.k_pages
         vp = None if pk.v_pages is None else (pk.v_pages.view(kv8_dtype) if fp8 else pk.v_pages)
         o = decoding_attn_paged_fwd(q.to(DEV), kp, vp, pk.block_table, pk.seq_lens, max_seq_k, dv, alibi,
@@ -118,6 +139,14 @@ def test_random_cases_over_an_int4_cache(chunk):
     rng = random.Random(seed * 1000 + chunk)
     for i in range(CASES_PER_CHUNK):
         _one_case(rng, seed, chunk * CASES_PER_CHUNK + i, int4=True)
+
+
+@pytest.mark.parametrize("chunk", range(3))
+def test_random_cases_over_an_int4_cache_with_per_token_pairs(chunk):
+    seed = 13
+    rng = random.Random(seed * 1000 + chunk)
+    for i in range(CASES_PER_CHUNK):
+        _one_case(rng, seed, chunk * CASES_PER_CHUNK + i, per_token=True)
 
 
 @pytest.mark.parametrize("chunk", range(8))
