@@ -206,6 +206,43 @@ __device__ __forceinline__ uint4 int4x8_to_16(uint32_t w) {
     }
     return r;
 }
+// The matrix kernel's conversion of the same word: eight 16-bit elements holding kInt4Bias + n, in the order
+// kInt4Order (slot s holds element kInt4Order[s]: the low halves of the four result words are nibbles 0 .. 3, the
+// high halves nibbles 4 .. 7).  With the top bit of every nibble flipped, n + 8 = 0 .. 15 placed in the four leading
+// mantissa bits of 16.0 is the number 16 + (n + 8) exactly, in fp16 and in bf16: one XOR per word, then a shift and an
+// AND-OR (one instruction) per pair, 1.1 vector instructions per element.  The kernel takes the bias back out of its sums (q . (24 + n)
+// = q . n + 24 sum(q); sum_t p (24 + n) = sum_t p n + 24 sum_t p) and undoes the order where it matters.
+constexpr float kInt4Bias = 24.0f;
+template <typename Tag>
+__device__ __forceinline__ uint32_t int4_biased_one() {
+    uint32_t one = std::is_same<Tag, f16_tag>::value ? 0x4C004C00u : 0x41804180u;  // 16.0 in both halves
+    asm("" : "+v"(one));  // (kept in a vector register: see int4x8_biased)
+    return one;
+}
+template <typename Tag>
+__device__ __forceinline__ uint4 int4x8_biased(uint32_t w, uint32_t one) {
+    constexpr bool kHalf = std::is_same<Tag, f16_tag>::value;
+    // the four leading mantissa bits of both halves, and 16.0 in both halves (fp16 0x4C00: bits 6 .. 9; bf16 0x4180:
+    // bits 3 .. 6)
+    constexpr uint32_t kMask = kHalf ? 0x03C003C0u : 0x00780078u;
+    constexpr int kAt = kHalf ? 6 : 3;  // where nibble 0 has to go
+    const uint32_t x = w ^ 0x88888888u;
+    // (shifted & mask) | 16.0 as one instruction: the mask travels in a scalar register and 16.0 (`one`, from
+    // int4_biased_one, once per kernel) in a vector register: the instruction's encoding takes no literal constants,
+    // and one scalar operand at most
+    auto place = [&](uint32_t shifted) {
+        uint32_t r;
+        asm("v_and_or_b32 %0, %1, %2, %3" : "=v"(r) : "v"(shifted), "s"(kMask), "v"(one));
+        return r;
+    };
+    uint4 r;
+    r.x = place(x << kAt);
+    r.y = place(kAt >= 4 ? x << (kAt - 4) : x >> (4 - kAt));
+    r.z = place(x >> (8 - kAt));
+    r.w = place(x >> (12 - kAt));
+    return r;
+}
+
 // Sixteen (eight) elements of an int4 cache at the doubled address `vptr` (see kKvInt4): the packed words, each in
 // the slot where the 8-bit formats keep the eight bytes of the same elements (the other word of the pair is unused).
 __device__ __forceinline__ uint4 kv4_load16(const void* vptr) {

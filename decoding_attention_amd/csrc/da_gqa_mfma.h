@@ -148,6 +148,20 @@ __device__ __forceinline__ void gqa_segment(const SweepParams& p, uint8_t* const
     // head's q row.  V[t][c] = a_v[t] (n[t][c] - z_v[t]) likewise: the probabilities are multiplied by a_v[t] on
     // their way into the second product, and sum_t p'[t] z_v[t], one number per head, comes off every column at the end.
     constexpr bool TOK = (KV8 & kKvPerToken) != 0;
+    // B4: an int4 cache.  Its nibbles reach the matrix instructions as kInt4Bias + n (int4x8_biased), the eight
+    // elements of a word in the order 0, 4, 1, 5, 2, 6, 3, 7: Q is gathered in that order, the bias leaves the scores
+    // through the sum of the head's q row and the outputs through the sum of the rounded probabilities, and the
+    // output columns, which come out in that order within every run of eight, are put right after the last tile.
+    constexpr bool B4 = FMT == kKvInt4;
+    const uint32_t b4_one = B4 ? int4_biased_one<Tag>() : 0u;
+    auto convert8 = [b4_one](uint2 w) __attribute__((always_inline)) {
+        if constexpr (B4)
+            return int4x8_biased<Tag>(w.x, b4_one);
+        else if constexpr (FMT != 0)
+            return kv8x8_to_16<Tag, FMT>(w);
+        else
+            return make_uint4(w.x, w.y, 0u, 0u);  // (16-bit K/V: never called)
+    };
     constexpr int KB = KV8 ? 1 : 2;                 // bytes per K/V element
     constexpr int KSR = KV8 ? KS / 2 : KS;          // K registers (16 bytes) per 16-token tile
     constexpr int CPRL = KV8 ? DV / 16 : CPR;       // 16-byte chunks per V row as loaded
@@ -194,19 +208,26 @@ __device__ __forceinline__ void gqa_segment(const SweepParams& p, uint8_t* const
             // k indices this lane contributes to k-step ks: those of the K fragment it will hold
             const int at = KV8 ? (ks >> 1) * 64 + g * 16 + (ks & 1) * 8 : ks * 32 + g * 8;
             qf[nt][ks] = __builtin_bit_cast(vec8, *reinterpret_cast<const uint4*>(qrow + at));
+            if constexpr (B4) qf[nt][ks] = __builtin_shufflevector(qf[nt][ks], qf[nt][ks], 0, 4, 1, 5, 2, 6, 3, 7);
         }
         slope[nt] = p.is_alibi ? alibi_slope_log2(p.slopes, h, p.head_q) : 0.0f;
     }
-    // (TOK) sum of each head's q row: the four 16-lane groups hold different elements of the same rows
+    // (TOK, B4) sum of each head's q row: the four 16-lane groups hold different elements of the same rows
     float qsum[NT];
-    if constexpr (TOK) {
+    if constexpr (TOK || B4) {
 #pragma unroll
         for (int nt = 0; nt < NT; ++nt) {
+            // (a dot product with ones: one instruction per pair of elements)
+            constexpr uint32_t kOnes = std::is_same<Tag, f16_tag>::value ? 0x3C003C00u : 0x3F803F80u;
             float acc_q = 0.0f;
 #pragma unroll
-            for (int ks = 0; ks < KS; ++ks)
-#pragma unroll
-                for (int j = 0; j < 8; ++j) acc_q += (float)qf[nt][ks][j];
+            for (int ks = 0; ks < KS; ++ks) {
+                const uint4 w = __builtin_bit_cast(uint4, qf[nt][ks]);
+                acc_q = EL::dot2(w.x, kOnes, acc_q);
+                acc_q = EL::dot2(w.y, kOnes, acc_q);
+                acc_q = EL::dot2(w.z, kOnes, acc_q);
+                acc_q = EL::dot2(w.w, kOnes, acc_q);
+            }
             acc_q += __shfl_xor(acc_q, 16);
             acc_q += __shfl_xor(acc_q, 32);
             qsum[nt] = acc_q;
@@ -232,8 +253,12 @@ __device__ __forceinline__ void gqa_segment(const SweepParams& p, uint8_t* const
     const uint8_t* const vbytes = reinterpret_cast<const uint8_t*>(p.v) + (size_t)hk * p.v_head * KB;
     const uint32_t k_row_b = (uint32_t)p.k_row * KB, v_row_b = (uint32_t)p.v_row * KB;
     // (an int4 cache's elements come out of the conversion times a power of two, divided out here)
-    const float sl = p.scale_log2 * head_scale(p.k_scale, hk) * kv_widening_inverse<FMT>();  // score scale, log2 units
-    const float vs = head_scale(p.v_scale, hk) * kv_widening_inverse<FMT>();
+    const float sl = p.scale_log2 * head_scale(p.k_scale, hk);  // score scale, log2 units
+    const float vs = head_scale(p.v_scale, hk);
+    // (B4, per-head factors) the bias' share of every score of head nt, in log2 units
+    float bias_q[NT];
+#pragma unroll
+    for (int nt = 0; nt < NT; ++nt) bias_q[nt] = (B4 && !TOK) ? kInt4Bias * sl * qsum[nt] : 0.0f;
 
     // wave-private V tile in LDS
     uint8_t* const vt = smem + wave * (kGqaTile * VP);
@@ -355,6 +380,9 @@ __device__ __forceinline__ void gqa_segment(const SweepParams& p, uint8_t* const
         load_tok(c0 + tw * kGqaTile, tr);
     }
 
+    // (A second register set, refilled two tiles ahead, was measured for the 8-bit and 4-bit formats, whose tiles are
+    // half and a quarter of the bytes: no gain at 4096 tokens, a loss at 128: GQA int4 batch 64 x 4096 62.0 us against
+    // 59.9, MHA int4 batch 512 x 128 68.5 against 63.2.)
     for (int t = tw; t < ntiles; t += NW) {
         const int tok0 = c0 + t * kGqaTile;
         const bool more = t + NW < ntiles;
@@ -368,9 +396,9 @@ __device__ __forceinline__ void gqa_segment(const SweepParams& p, uint8_t* const
             const int row = slot / CPRL, ch = slot % CPRL;
             if constexpr (KV8) {  // sixteen 8-bit elements become 32 bytes of the 16-bit tile
                 *reinterpret_cast<uint4*>(vt + row * VP + ch * 32) =
-                    kv8x8_to_16<Tag, FMT>(make_uint2(tr.v[i].x, tr.v[i].y));
+                    convert8(make_uint2(tr.v[i].x, tr.v[i].y));
                 *reinterpret_cast<uint4*>(vt + row * VP + ch * 32 + 16) =
-                    kv8x8_to_16<Tag, FMT>(make_uint2(tr.v[i].z, tr.v[i].w));
+                    convert8(make_uint2(tr.v[i].z, tr.v[i].w));
             } else {
                 *reinterpret_cast<uint4*>(vt + row * VP + ch * 16) = tr.v[i];
             }
@@ -390,7 +418,7 @@ __device__ __forceinline__ void gqa_segment(const SweepParams& p, uint8_t* const
                     uint4 kfrag;
                     if constexpr (KV8) {
                         const uint4 w = tr.k[mt][ks >> 1];
-                        kfrag = kv8x8_to_16<Tag, FMT>((ks & 1) ? make_uint2(w.z, w.w) : make_uint2(w.x, w.y));
+                        kfrag = convert8((ks & 1) ? make_uint2(w.z, w.w) : make_uint2(w.x, w.y));
                     } else {
                         kfrag = tr.k[mt][ks];
                     }
@@ -415,9 +443,9 @@ __device__ __forceinline__ void gqa_segment(const SweepParams& p, uint8_t* const
 #pragma unroll
                     for (int j = 0; j < DV / 64; ++j) {
                         const uint4 w = tr.k[mt][j];
-                        *reinterpret_cast<uint4*>(row + j * 128 + g * 32) = kv8x8_to_16<Tag, FMT>(make_uint2(w.x, w.y));
+                        *reinterpret_cast<uint4*>(row + j * 128 + g * 32) = convert8(make_uint2(w.x, w.y));
                         *reinterpret_cast<uint4*>(row + j * 128 + g * 32 + 16) =
-                            kv8x8_to_16<Tag, FMT>(make_uint2(w.z, w.w));
+                            convert8(make_uint2(w.z, w.w));
                     }
                 } else {
 #pragma unroll
@@ -432,8 +460,7 @@ __device__ __forceinline__ void gqa_segment(const SweepParams& p, uint8_t* const
         vec8 pf[NT];
         const bool tail = tok0 + kGqaTile > c1;
         float x[NT][8], mx[NT];
-        // (TOK) per token: A = score scale x a_k, Z = z_k in the score tile's units (the integers come out of the
-        // conversion times kv_widening_inverse()^-1); x = A (s - Z qsum)
+        // (TOK) per token: A = score scale x a_k, Z = z_k plus the conversion's bias; x = A (s - Z qsum)
         float tokA[TOK ? 8 : 1], tokZ[TOK ? 8 : 1], tokV[TOK ? 8 : 1], tokW[TOK ? 8 : 1], tokVinv[TOK ? 8 : 1];
         if constexpr (TOK) {
             float* const mine = tokbuf + (lane >> 5) * 64 + (lane & 31);
@@ -449,9 +476,9 @@ __device__ __forceinline__ void gqa_segment(const SweepParams& p, uint8_t* const
 #pragma unroll
                 for (int r = 0; r < 4; ++r) {
                     tokA[mt * 4 + r] = sl * ak[r];
-                    tokZ[mt * 4 + r] = zk[r] * (1.0f / kv_widening_inverse<FMT>());
+                    tokZ[mt * 4 + r] = zk[r] + (B4 ? kInt4Bias : 0.0f);
                     tokV[mt * 4 + r] = av[r];
-                    tokW[mt * 4 + r] = zv[r] * (1.0f / kv_widening_inverse<FMT>());
+                    tokW[mt * 4 + r] = zv[r] + (B4 ? kInt4Bias : 0.0f);
                     if constexpr (std::is_same<Tag, bf16_tag>::value)
                         tokVinv[mt * 4 + r] = __builtin_amdgcn_rcpf(av[r]);
                 }
@@ -488,7 +515,7 @@ __device__ __forceinline__ void gqa_segment(const SweepParams& p, uint8_t* const
 #pragma unroll
                     for (int r = 0; r < 4; ++r) {
                         const int tok = tok0 + mt * 16 + g * 4 + r;
-                        float v = s[mt][nt][r] * sl + slope[nt] * (float)(tok - (len - 1));
+                        float v = s[mt][nt][r] * sl + slope[nt] * (float)(tok - (len - 1)) - bias_q[nt];
                         if (tok >= c1) v = -INFINITY;
                         x[nt][mt * 4 + r] = v;
                         mx[nt] = fmaxf(mx[nt], v);
@@ -498,7 +525,7 @@ __device__ __forceinline__ void gqa_segment(const SweepParams& p, uint8_t* const
                 for (int mt = 0; mt < 2; ++mt)
 #pragma unroll
                     for (int r = 0; r < 4; ++r) {
-                        x[nt][mt * 4 + r] = s[mt][nt][r] * sl;
+                        x[nt][mt * 4 + r] = B4 ? __builtin_fmaf(s[mt][nt][r], sl, -bias_q[nt]) : s[mt][nt][r] * sl;
                         mx[nt] = fmaxf(mx[nt], x[nt][mt * 4 + r]);
                     }
             }
@@ -538,12 +565,24 @@ __device__ __forceinline__ void gqa_segment(const SweepParams& p, uint8_t* const
                         l[nt] += pe;
                     corr[nt] = __builtin_fmaf(pv, tokW[j], corr[nt]);
                     x[nt][j] = pv;
+                } else if constexpr (B4) {
+                    x[nt][j] = fast_exp2(x[nt][j] - m[nt]);  // (rounded by pack8; the denominator follows below)
                 } else {
                     x[nt][j] = as_second_operand<Tag>(fast_exp2(x[nt][j] - m[nt]));
                     l[nt] += x[nt][j];
                 }
             }
             pf[nt] = MM::pack8(x[nt]);  // k index j <-> token g*4+j (j<4), 16+g*4+(j-4) (j>=4)
+            if constexpr (B4 && !TOK) {
+                // the denominator sums the probabilities as rounded for the matrix instruction (it is also what the
+                // bias is taken out with): a dot product of the packed pairs with ones
+                constexpr uint32_t kOnes = std::is_same<Tag, f16_tag>::value ? 0x3C003C00u : 0x3F803F80u;
+                const uint4 pw = __builtin_bit_cast(uint4, pf[nt]);
+                l[nt] = EL::dot2(pw.x, kOnes, l[nt]);
+                l[nt] = EL::dot2(pw.y, kOnes, l[nt]);
+                l[nt] = EL::dot2(pw.z, kOnes, l[nt]);
+                l[nt] = EL::dot2(pw.w, kOnes, l[nt]);
+            }
         }
 
         // O^T += V^T . P^T
@@ -569,11 +608,35 @@ __device__ __forceinline__ void gqa_segment(const SweepParams& p, uint8_t* const
     for (int nt = 0; nt < NT; ++nt) {
         l[nt] += __shfl_xor(l[nt], 16);
         l[nt] += __shfl_xor(l[nt], 32);
-        if constexpr (TOK) {  // the zero points' share comes off every column of the head
+        if constexpr (TOK) {  // the zero points' share (and the bias') comes off every column of the head
             corr[nt] += __shfl_xor(corr[nt], 16);
             corr[nt] += __shfl_xor(corr[nt], 32);
 #pragma unroll
             for (int ct = 0; ct < CT; ++ct) acc[nt][ct] -= corr[nt];
+        } else if constexpr (B4) {  // sum_t p (bias + n) = sum_t p n + bias l
+            const float off = kInt4Bias * l[nt];
+#pragma unroll
+            for (int ct = 0; ct < CT; ++ct) acc[nt][ct] -= off;
+        }
+        if constexpr (B4) {
+            // Columns: a run of eight lies in the conversion's order 0, 4, 1, 5 (this lane, 16-lane group g even) and
+            // 2, 6, 3, 7 (lane + 16, g odd).  The even group keeps columns 0 and 1 and takes 2 and 3 from its
+            // neighbour, the odd one keeps 6 and 7 and takes 4 and 5.
+            // v_permlane16_swap(x, y) hands the odd groups' x the even groups' y (of lane - 16) and the even groups' y
+            // the odd groups' x (of lane + 16): two of them per tile of sixteen columns.
+#pragma unroll
+            for (int ct = 0; ct < CT; ++ct) {
+                // (elements are copied to scalars first: a bit cast applied to a vector element reads element 0)
+                const float a0 = acc[nt][ct][0], a1 = acc[nt][ct][1], a2 = acc[nt][ct][2], a3 = acc[nt][ct][3];
+                const auto s01 = __builtin_amdgcn_permlane16_swap(__builtin_bit_cast(unsigned, a0),
+                                                                  __builtin_bit_cast(unsigned, a1), false, false);
+                const unsigned c04 = s01[0], c26 = s01[1];
+                const auto s23 = __builtin_amdgcn_permlane16_swap(__builtin_bit_cast(unsigned, a2),
+                                                                  __builtin_bit_cast(unsigned, a3), false, false);
+                const unsigned c15 = s23[0], c37 = s23[1];
+                acc[nt][ct] = f32x4{__builtin_bit_cast(float, c04), __builtin_bit_cast(float, c15),
+                                    __builtin_bit_cast(float, c26), __builtin_bit_cast(float, c37)};
+            }
         }
     }
 

@@ -1,9 +1,10 @@
 """int4 K/V cache: q and o stay 16-bit, K/V are two's-complement four-bit integers (-8 .. 7), two to a byte (element
 2 i in the low half of byte i), with one symmetric scale per KV head.
 
-Every value converts exactly to fp16 and to bf16, so with unit scales the int4 call must agree with the int8 call on the
-same integers bit for bit (same kernels, the nibbles widened to bytes by the load); with scales it is checked against
-float64 attention on the de-quantised inputs at the usual tolerance (max-abs 2e-3 fp16 / 1e-2 bf16).  The packing
+Every value converts exactly to fp16 and to bf16; the call is checked against float64 attention on the de-quantised
+inputs at the usual tolerance (max-abs 2e-3 fp16 / 1e-2 bf16) and against the int8 call on the same integers (the same
+bits on the VALU sweep, within a quarter of the tolerance on the grouped kernel, whose int4 conversion adds a bias
+that its sums take out again).  The packing
 helper is checked on the CPU against a per-element restatement of the layout.
 """
 import pytest
@@ -101,12 +102,20 @@ def test_int4_kv_with_scales_matches_float64_attention(shape, dtype):
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
 @pytest.mark.parametrize("shape", [SHAPES[0], SHAPES[2], SHAPES[3], SHAPES[5], SHAPES[6]])
 def test_int4_equals_int8_on_the_same_integers(shape, dtype):
-    """The same integers as an int8 cache: same kernels, same plan, the load widens the nibbles: same bits."""
+    """The same integers as an int8 cache.  On the VALU sweep the nibbles are widened to sixteen times their value, a
+    power of two divided out of the per-head factors: the same bits as the int8 call.  On the grouped kernel the
+    nibbles enter the matrix instructions with a bias that the kernel takes out of its sums again (exact products,
+    fp32 sums in another order): a quarter of the acceptance tolerance."""
     w, k4, v4, ks, vs = _case(*shape, dtype)
     o4 = _run(w, k4, v4, ks, vs)
     o8 = decoding_attn_fwd(w.q.to(DEV), k4.to(DEV), v4.to(DEV), w.cu_seq_k.to(DEV), w.max_seq_k, w.dim_v, w.is_alibi,
                            k_scale=ks.to(DEV), v_scale=vs.to(DEV)).cpu()
-    assert torch.equal(o4.view(torch.int16), o8.view(torch.int16))
+    batch, head_q, head_k, dim, dim_v, _ = shape
+    kind = _lib.plan(w.max_seq_k, batch, head_q, head_k, dim, dim_v, total_k=int(k4.shape[0]), kv_bits=4)["kind"]
+    if kind == 1:
+        assert torch.equal(o4.view(torch.int16), o8.view(torch.int16))
+    else:
+        assert (o4.float() - o8.float()).abs().max().item() <= TOL[dtype] / 4
 
 
 @pytest.mark.gpu
