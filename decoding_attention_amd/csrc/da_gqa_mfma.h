@@ -381,8 +381,9 @@ __device__ __forceinline__ void gqa_segment(const SweepParams& p, uint8_t* const
     }
 
     // (A second register set, refilled two tiles ahead, was measured for the 8-bit and 4-bit formats, whose tiles are
-    // half and a quarter of the bytes: no gain at 4096 tokens, a loss at 128: GQA int4 batch 64 x 4096 62.0 us against
-    // 59.9, MHA int4 batch 512 x 128 68.5 against 63.2.)
+    // half and a quarter of the bytes, and for the 32-heads-per-wave form, whose CUs hold one wave per SIMD: no gain
+    // anywhere, a loss on short sequences.  GQA int4 batch 64 x 4096 62.0 us against 59.9, MHA int4 batch 512 x 128
+    // 68.5 against 63.2, MQA fp16 batch 32 x 4096 21.6 against 20.8.)
     for (int t = tw; t < ntiles; t += NW) {
         const int tok0 = c0 + t * kGqaTile;
         const bool more = t + NW < ntiles;
