@@ -35,6 +35,9 @@ EXPORTED_SYMBOLS = (
     "da_decoding_attn_int4kv_tok",
     "da_decoding_attn_paged_int4kv_tok",
     "da_workspace_bytes_int4kv_tok",
+    "da_decoding_attn_int8kv_tok",
+    "da_decoding_attn_paged_int8kv_tok",
+    "da_workspace_bytes_int8kv_tok",
     "da_supported_head_dims",
     "da_last_error",
     "da_version",
@@ -116,6 +119,12 @@ def _declare(lib):
     lib.da_decoding_attn_paged_int4kv_tok.argtypes = lib.da_decoding_attn_paged_fp8kv.argtypes
     lib.da_workspace_bytes_int4kv_tok.restype = sz
     lib.da_workspace_bytes_int4kv_tok.argtypes = lib.da_workspace_bytes_fp8kv.argtypes
+    lib.da_decoding_attn_int8kv_tok.restype = ci
+    lib.da_decoding_attn_int8kv_tok.argtypes = lib.da_decoding_attn_fp8kv.argtypes
+    lib.da_decoding_attn_paged_int8kv_tok.restype = ci
+    lib.da_decoding_attn_paged_int8kv_tok.argtypes = lib.da_decoding_attn_paged_fp8kv.argtypes
+    lib.da_workspace_bytes_int8kv_tok.restype = sz
+    lib.da_workspace_bytes_int8kv_tok.argtypes = lib.da_workspace_bytes_fp8kv.argtypes
     ip = ctypes.POINTER(ci)
     lib.da_plan.restype = ci
     lib.da_plan.argtypes = [sz, sz, sz, sz, sz, sz, ci, sz, ip, ip, ip, ip]
@@ -170,14 +179,15 @@ def last_error() -> str:
 
 
 KV_BITS_INT4_PER_TOKEN = 5  # DA_KV_BITS_INT4_PER_TOKEN of include/decoding_attn_hip.h
+KV_BITS_INT8_PER_TOKEN = 9  # DA_KV_BITS_INT8_PER_TOKEN
 
 
 def plan(max_seq_k, batch, head_q, head_k, dim, dim_v, is_bf16=False, total_k=0, distinct_v=False, page_size=0,
          kv_bits=16):
     """Launch plan of a call: dict(kind, nsplit, chunk, heads_per_group, balanced).  `distinct_v`: V passed as its own
-    buffer; `page_size`: pages of that many tokens (0 = packed); `kv_bits`: 16, 8 (FP8, int8), 4 (int4) or KV_BITS_INT4_PER_TOKEN
-    (int4 with per-token pairs; distinct_v is implied)."""
-    if kv_bits == KV_BITS_INT4_PER_TOKEN:
+    buffer; `page_size`: pages of that many tokens (0 = packed); `kv_bits`: 16, 8 (FP8, int8), 4 (int4) or
+    KV_BITS_INT4_PER_TOKEN / KV_BITS_INT8_PER_TOKEN (int4 / int8 with per-token pairs; distinct_v is implied)."""
+    if kv_bits in (KV_BITS_INT4_PER_TOKEN, KV_BITS_INT8_PER_TOKEN):
         distinct_v = True
     del is_bf16  # (the plan does not depend on it)
     lib = load()

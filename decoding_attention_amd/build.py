@@ -27,6 +27,7 @@ SOURCES = [
     "da_gqa_mfma_i8.hip",
     "da_gqa_mfma_i4.hip",
     "da_gqa_mfma_i4t.hip",
+    "da_gqa_mfma_i8t.hip",
 ]
 
 # libdecoding_attn_probe.so (measurement aids of bench.py, csrc/decoding_attn_probe.h): the same objects, with

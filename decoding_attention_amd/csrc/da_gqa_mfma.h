@@ -817,5 +817,8 @@ hipError_t launch_gqa_mfma_i4(const SweepParams& p, bool is_bf16, int dim, int h
 // ... and over an int4 one whose rows carry their own (scale, zero) pairs (SweepParams::k_tok, v_tok); dim 64, 128, 256
 hipError_t launch_gqa_mfma_i4t(const SweepParams& p, bool is_bf16, int dim, int heads_per_group, bool wave_per_head,
                                dim3 grid, hipStream_t stream);
+// ... and over an int8 one with such pairs
+hipError_t launch_gqa_mfma_i8t(const SweepParams& p, bool is_bf16, int dim, int heads_per_group, bool wave_per_head,
+                               dim3 grid, hipStream_t stream);
 
 }  // namespace da

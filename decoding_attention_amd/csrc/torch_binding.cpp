@@ -45,14 +45,14 @@ const float *scale_ptr(const std::optional<at::Tensor> &t, const at::Tensor &q, 
     return s.data_ptr<float>();
 }
 
-// int4 with a (scale, zero) pair per (token, KV head): k_scale and v_scale are then tensors shaped like the rows they
+// int4 or int8 with a (scale, zero) pair per (token, KV head): k_scale and v_scale are then tensors shaped like the rows they
 // belong to with a last dimension of 2 (`rows` = the leading dimensions of the K tensor) instead of head_k values.
 bool per_token_pairs(const std::optional<at::Tensor> &ks, const std::optional<at::Tensor> &vs, const at::Tensor &q,
                      const at::Tensor &k, int kv8) {
     const bool k_pairs = ks.has_value() && ks.value().dim() == k.dim();
     const bool v_pairs = vs.has_value() && vs.value().dim() == k.dim();
     if (!k_pairs && !v_pairs) return false;
-    TORCH_CHECK(kv8 == 3, "per-token (scale, zero) pairs apply to an int4 K/V cache only");
+    TORCH_CHECK(kv8 == 3 || kv8 == 2, "per-token (scale, zero) pairs apply to an int4 or int8 K/V cache only");
     TORCH_CHECK(k_pairs && v_pairs, "per-token (scale, zero) pairs must be given for both K and V");
     for (const at::Tensor *t : {&ks.value(), &vs.value()}) {
         TORCH_CHECK(t->dtype() == torch::kFloat32 && t->is_cuda() && t->device() == q.device() && t->is_contiguous(),
@@ -156,7 +156,8 @@ at::Tensor dmha_fwd(const at::Tensor &q, const at::Tensor &k, const std::optiona
 
     // k.size(0) is the sum of the key lengths: a free host-side hint for sizing the sequence splits
     const size_t ws_bytes =
-        kv8 ? (tok ? da_workspace_bytes_int4kv_tok : kv8 == 3 ? da_workspace_bytes_int4kv : da_workspace_bytes_fp8kv)(
+        kv8 ? (tok ? (kv8 == 3 ? da_workspace_bytes_int4kv_tok : da_workspace_bytes_int8kv_tok)
+                   : kv8 == 3 ? da_workspace_bytes_int4kv : da_workspace_bytes_fp8kv)(
                   (size_t)max_seq_k, (size_t)batch, (size_t)head_q, (size_t)head_k, (size_t)dim, (size_t)dim_v,
                   (size_t)total_k, 0)
             : da_workspace_bytes((size_t)max_seq_k, (size_t)batch, (size_t)head_q, (size_t)head_k, (size_t)dim,
@@ -165,7 +166,7 @@ at::Tensor dmha_fwd(const at::Tensor &q, const at::Tensor &k, const std::optiona
     if (ws_bytes > 0) ws = torch::empty({(int64_t)ws_bytes}, q.options().dtype(torch::kUInt8));
 
     const float scale = softmax_scale.has_value() ? (float)softmax_scale.value() : 0.0f;
-    const auto kv8_entry = tok        ? da_decoding_attn_int4kv_tok
+    const auto kv8_entry = tok        ? (kv8 == 3 ? da_decoding_attn_int4kv_tok : da_decoding_attn_int8kv_tok)
                            : kv8 == 3 ? da_decoding_attn_int4kv
                                       : (kv8 == 2 ? da_decoding_attn_int8kv : da_decoding_attn_fp8kv);
     const int rc =
@@ -274,7 +275,8 @@ at::Tensor dmha_fwd_paged(const at::Tensor &q, const at::Tensor &k_pages, const 
     const float *v_scale_ptr = tok ? v_scale.value().data_ptr<float>() : scale_ptr(v_scale, q, head_k, "v_scale", kv8);
     const size_t hint = total_k > 0 ? (size_t)total_k : 0;
     const size_t ws_bytes =
-        kv8 ? (tok ? da_workspace_bytes_int4kv_tok : kv8 == 3 ? da_workspace_bytes_int4kv : da_workspace_bytes_fp8kv)(
+        kv8 ? (tok ? (kv8 == 3 ? da_workspace_bytes_int4kv_tok : da_workspace_bytes_int8kv_tok)
+                   : kv8 == 3 ? da_workspace_bytes_int4kv : da_workspace_bytes_fp8kv)(
                   (size_t)max_seq_k, (size_t)batch, (size_t)head_q, (size_t)head_k, (size_t)dim, (size_t)dim_v, hint,
                   (size_t)page_size)
             : da_workspace_bytes_paged((size_t)max_seq_k, (size_t)batch, (size_t)head_q, (size_t)head_k, (size_t)dim,
@@ -283,7 +285,7 @@ at::Tensor dmha_fwd_paged(const at::Tensor &q, const at::Tensor &k_pages, const 
     if (ws_bytes > 0) ws = torch::empty({(int64_t)ws_bytes}, q.options().dtype(torch::kUInt8));
 
     const float scale = softmax_scale.has_value() ? (float)softmax_scale.value() : 0.0f;
-    const auto kv8_entry = tok        ? da_decoding_attn_paged_int4kv_tok
+    const auto kv8_entry = tok        ? (kv8 == 3 ? da_decoding_attn_paged_int4kv_tok : da_decoding_attn_paged_int8kv_tok)
                            : kv8 == 3 ? da_decoding_attn_paged_int4kv
                                       : (kv8 == 2 ? da_decoding_attn_paged_int8kv : da_decoding_attn_paged_fp8kv);
     const int rc =

@@ -79,6 +79,17 @@ def quantize_int4_per_token(x: torch.Tensor):
     return pack_int4(n), torch.cat([scale, zero], dim=-1).contiguous()
 
 
+def quantize_int8_per_token(x: torch.Tensor):
+    """The same with eight bits: returns (torch.int8 tensor, pairs) with x ~= pairs[..., 0] * (n - pairs[..., 1]), the
+    row's minimum at -128 and its maximum at 127."""
+    xf = x.float()
+    lo, hi = xf.amin(dim=-1, keepdim=True), xf.amax(dim=-1, keepdim=True)
+    scale = ((hi - lo) / 255.0).clamp_min(1e-8)
+    zero = -128.0 - lo / scale
+    n = torch.round(xf / scale + zero).clamp(-128, 127).to(torch.int8)
+    return n, torch.cat([scale, zero], dim=-1).contiguous()
+
+
 def decoding_attn_fwd(q: torch.Tensor, k: torch.Tensor, v: Optional[torch.Tensor], cu_seq_k: torch.Tensor,
                       max_seq_k: int, dim_v: int, is_alibi: bool, *, softmax_scale: Optional[float] = None,
                       alibi_slopes: Optional[torch.Tensor] = None, k_scale: Optional[torch.Tensor] = None,
@@ -97,8 +108,8 @@ def decoding_attn_fwd(q: torch.Tensor, k: torch.Tensor, v: Optional[torch.Tensor
         k_scale, v_scale (keyword only): k and v may be torch.float8_e4m3fn or torch.int8 (an 8-bit K/V cache; q
             stays 16-bit), or torch.uint8 holding pairs of int4 values (see pack_int4: last dimensions dim / 2 and
             dim_v / 2); these are then float32 [head_k] GPU tensors of de-quantisation factors (default 1):
-            K = k_scale * k.  For an int4 cache they may instead be float32 [total_k, head_k, 2] tensors of
-            (scale, zero) pairs, one per token and KV head (quantize_int4_per_token builds them):
+            K = k_scale * k.  For an int4 or int8 cache they may instead be float32 [total_k, head_k, 2] tensors of
+            (scale, zero) pairs, one per token and KV head (quantize_int4_per_token, quantize_int8_per_token):
             K[t, h] = k_scale[t, h, 0] * (k[t, h] - k_scale[t, h, 1]); head dims 64, 128 and 256, v required.
     Return:
         o: [total_q, head_q, dim_v], same dtype as q.
@@ -131,7 +142,7 @@ def decoding_attn_paged_fwd(q: torch.Tensor, k_pages: torch.Tensor, v_pages: Opt
         total_k (keyword only): sum of seq_lens if the host knows it; only a hint for sizing sequence splits.
         k_scale, v_scale (keyword only): as for decoding_attn_fwd, when the pools are torch.float8_e4m3fn, torch.int8
             or torch.uint8 holding pairs of int4 values (last dimensions dim / 2 and dim_v / 2); per-token
-            (scale, zero) pairs of an int4 cache are float32 [pages, page_size, head_k, 2].
+            (scale, zero) pairs of an int4 or int8 cache are float32 [pages, page_size, head_k, 2].
     Return:
         o: [batch, head_q, dim_v], same dtype as q.
     """

@@ -1,5 +1,5 @@
-"""int4 K/V cache with a (scale, zero) pair per (token, KV head): K[t, h, c] = scale[t, h] * (n[t, h, c] - zero[t, h]),
-n the stored integer (-8 .. 7), and V likewise.  q and o stay 16-bit.
+"""int4 and int8 K/V caches with a (scale, zero) pair per (token, KV head): K[t, h, c] = scale[t, h] * (n[t, h, c] -
+zero[t, h]), n the stored integer (-8 .. 7, or -128 .. 127), and V likewise.  q and o stay 16-bit.
 
 The kernel never builds the de-quantised rows: its matrix instructions run on the integers and the factors enter the
 score tile, the probabilities and a per-head correction at the end.  It is therefore checked against float64 attention
@@ -11,7 +11,7 @@ import pytest
 import torch
 
 from decoding_attention_amd import (_lib, decoding_attn_fwd, decoding_attn_paged_fwd, pack_int4,
-                                    quantize_int4_per_token)
+                                    quantize_int4_per_token, quantize_int8_per_token)
 from decoding_attention_amd import workloads as wl
 from oracle import oracle
 from tests.gpu_util import TOL, sub_workload
@@ -24,6 +24,25 @@ def _unpack(p):
     hi = (p >> 4).to(torch.int16)
     n = torch.stack([lo, hi], dim=-1).flatten(-2)
     return torch.where(n >= 8, n - 16, n).to(torch.int8)
+
+
+def _ints(cache, bits):
+    """The stored integers of a cache tensor."""
+    return _unpack(cache) if bits == 4 else cache
+
+
+def _cache(ints, bits):
+    return pack_int4(ints) if bits == 4 else ints.to(torch.int8)
+
+
+def test_quantize_int8_per_token_round_trip():
+    g = torch.Generator().manual_seed(1)
+    x = torch.randn(29, 2, 128, generator=g) * 3 + torch.randn(29, 2, 1, generator=g)
+    n, pairs = quantize_int8_per_token(x)
+    assert n.dtype == torch.int8 and n.shape == x.shape and pairs.shape == (29, 2, 2)
+    assert (n.amin(-1) == -128).all() and (n.amax(-1) == 127).all()
+    back = pairs[..., :1] * (n.float() - pairs[..., 1:])
+    assert ((back - x).abs() <= pairs[..., :1] * 0.5001).all()
 
 
 def test_quantize_int4_per_token_round_trip():
@@ -39,19 +58,21 @@ def test_quantize_int4_per_token_round_trip():
     assert ((back - x).abs() <= pairs[..., :1] * 0.5001).all()
 
 
-def _case(batch, head_q, head_k, dim, seq_k, dtype, *, is_alibi=False, seed=3, varlen=True):
+def _case(batch, head_q, head_k, dim, seq_k, dtype, *, is_alibi=False, seed=3, varlen=True, bits=4):
     w = wl.make_workload(batch, head_q, head_k, dim, dim, seq_k, dtype, seed=seed, varlen=varlen, is_alibi=is_alibi)
     g = torch.Generator().manual_seed(seed + 50)
     # rows of different spread and offset, so that scales and zero points differ from token to token and head to head
     k = w.k.float() * (0.5 + torch.rand(w.k.shape[0], head_k, 1, generator=g)) + torch.randn(w.k.shape[0], head_k, 1, generator=g)
     v = w.v.float() * (0.5 + torch.rand(w.v.shape[0], head_k, 1, generator=g)) + 0.5 * torch.randn(w.v.shape[0], head_k, 1, generator=g)
-    k4, kp = quantize_int4_per_token(k)
-    v4, vp = quantize_int4_per_token(v)
+    quant = quantize_int4_per_token if bits == 4 else quantize_int8_per_token
+    k4, kp = quant(k)
+    v4, vp = quant(v)
     return w, k4, v4, kp, vp
 
 
-def _dequant(p4, pairs):
-    return pairs[..., :1].double() * (_unpack(p4).double() - pairs[..., 1:].double())
+def _dequant(cache, pairs):
+    ints = _unpack(cache) if cache.dtype == torch.uint8 else cache
+    return pairs[..., :1].double() * (ints.double() - pairs[..., 1:].double())
 
 
 def _reference(w, k4, v4, kp, vp, **kw):
@@ -81,10 +102,11 @@ SHAPES = [
 
 
 @pytest.mark.gpu
+@pytest.mark.parametrize("bits", [4, 8])
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
 @pytest.mark.parametrize("shape", SHAPES)
-def test_per_token_int4_matches_float64_attention(shape, dtype):
-    w, k4, v4, kp, vp = _case(*shape, dtype)
+def test_per_token_cache_matches_float64_attention(shape, dtype, bits):
+    w, k4, v4, kp, vp = _case(*shape, dtype, bits=bits)
     o = _run(w, k4, v4, kp, vp)
     assert torch.isfinite(o.float()).all()
     if w.batch > 8:  # the large case: sampled sequences against float64
@@ -112,16 +134,18 @@ def test_uniform_batch_with_fixed_splits():
 
 
 @pytest.mark.gpu
+@pytest.mark.parametrize("bits", [4, 8])
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
-def test_shifting_integers_and_zero_points_together_changes_nothing(dtype):
+def test_shifting_integers_and_zero_points_together_changes_nothing(dtype, bits):
     """scale * ((n + 1) - (zero + 1)) is the same row: a sign error or a dropped zero-point term on either side of the
     kernel's algebra (score tile, per-head correction) shows as a difference of the size of the values."""
-    w, k4, v4, kp, vp = _case(4, 32, 8, 128, 900, dtype, seed=17, is_alibi=True)
-    nk, nv = _unpack(k4).clamp(max=6), _unpack(v4).clamp(max=6)
-    a = _run(w, pack_int4(nk), pack_int4(nv), kp, vp)
+    w, k4, v4, kp, vp = _case(4, 32, 8, 128, 900, dtype, seed=17, is_alibi=True, bits=bits)
+    top = 6 if bits == 4 else 126
+    nk, nv = _ints(k4, bits).clamp(max=top), _ints(v4, bits).clamp(max=top)
+    a = _run(w, _cache(nk, bits), _cache(nv, bits), kp, vp)
     shift = torch.tensor([0.0, 1.0])
-    b = _run(w, pack_int4(nk + 1), pack_int4(nv + 1), kp + shift, vp + shift)
-    ref = _reference(w, pack_int4(nk), pack_int4(nv), kp, vp)
+    b = _run(w, _cache(nk + 1, bits), _cache(nv + 1, bits), kp + shift, vp + shift)
+    ref = _reference(w, _cache(nk, bits), _cache(nv, bits), kp, vp)
     assert (a.float() - ref).abs().max().item() <= TOL[dtype]
     assert (b.float() - ref).abs().max().item() <= TOL[dtype]
     assert ref.abs().max().item() > 50 * TOL[dtype]  # the check has teeth: the values are far above the tolerance
@@ -140,12 +164,13 @@ def test_zero_points_of_zero_reduce_to_the_per_head_call():
 
 
 @pytest.mark.gpu
+@pytest.mark.parametrize("bits", [4, 8])
 @pytest.mark.parametrize("shape", [SHAPES[0], SHAPES[2], SHAPES[3]])
-def test_paged_pools(shape):
+def test_paged_pools(shape, bits):
     """Pairs in pools of their own, [pages, page_size, head_k, 2], addressed through the same block table: float64
     attention on the de-quantised rows, and the same bits at every page size (64: one lookup per tile, 16: one per
     run of 16 tokens, 4 and 1: one per row)."""
-    w, k4, v4, kp, vp = _case(*shape, torch.float16, seed=21)
+    w, k4, v4, kp, vp = _case(*shape, torch.float16, seed=21, bits=bits)
     w4 = wl.Workload(w.name, w.q, k4, v4, w.cu_seq_k, w.max_seq_k, w.dim_v, w.is_alibi, w.lengths)
     wp = wl.Workload(w.name, w.q, kp, vp, w.cu_seq_k, w.max_seq_k, w.dim_v, w.is_alibi, w.lengths)
     outs = {}
@@ -167,9 +192,9 @@ def test_argument_errors():
     q, cu = w.q.to(DEV), w.cu_seq_k.to(DEV)
     with pytest.raises(RuntimeError, match="both K and V"):
         decoding_attn_fwd(q, k4.to(DEV), v4.to(DEV), cu, w.max_seq_k, 128, False, k_scale=kp.to(DEV))
-    with pytest.raises(RuntimeError, match="int4 K/V cache only"):
-        decoding_attn_fwd(q, _unpack(k4).to(DEV), _unpack(v4).to(DEV), cu, w.max_seq_k, 128, False,
-                          k_scale=kp.to(DEV), v_scale=vp.to(DEV))
+    with pytest.raises(RuntimeError, match="int4 or int8 K/V cache only"):
+        decoding_attn_fwd(q, w.k.to(torch.float8_e4m3fn).to(DEV), w.v.to(torch.float8_e4m3fn).to(DEV), cu, w.max_seq_k,
+                          128, False, k_scale=kp.to(DEV), v_scale=vp.to(DEV))
     with pytest.raises(RuntimeError, match="leading dimensions"):
         decoding_attn_fwd(q, k4.to(DEV), v4.to(DEV), cu, w.max_seq_k, 128, False, k_scale=kp[:-1].to(DEV),
                           v_scale=vp[:-1].to(DEV))

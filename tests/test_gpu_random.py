@@ -10,7 +10,8 @@ import random
 import pytest
 import torch
 
-from decoding_attention_amd import decoding_attn_fwd, decoding_attn_paged_fwd, pack_int4, quantize_int4_per_token
+from decoding_attention_amd import (decoding_attn_fwd, decoding_attn_paged_fwd, pack_int4, quantize_int4_per_token,
+                                    quantize_int8_per_token)
 from decoding_attention_amd import workloads as wl
 from oracle import oracle
 from tests.gpu_util import TOL, run_hip_ex, sub_workload
@@ -25,8 +26,8 @@ CASES_PER_CHUNK = 12
 
 def _one_case(rng, seed, case, int4=False, per_token=False):
     """int4: the case runs over an int4 cache (whatever format the draws below pick; the stream of draws is the same
-    either way, so the other cases do not move).  per_token: an int4 cache with a (scale, zero) pair per token and KV
-    head (never the latent form, never d = 96, which that entry point does not serve)."""
+    either way, so the other cases do not move).  per_token (4 or 8): an int4 or int8 cache with a (scale, zero) pair
+    per token and KV head (never the latent form, never d = 96, which those entry points do not serve)."""
     latent = rng.random() < 0.3 and not per_token
     dtype = rng.choice([torch.float16, torch.bfloat16])
     if latent:
@@ -61,7 +62,7 @@ def _one_case(rng, seed, case, int4=False, per_token=False):
     int8 = fp8 and rng.random() < 0.4  # the 8-bit cache holds int8 instead of FP8
     kv8_dtype = torch.int8 if int8 else FP8
     if int4 or per_token:
-        fp8, int8, kv8_dtype = True, True, torch.uint8
+        fp8, int8, kv8_dtype = True, True, torch.int8 if per_token == 8 else torch.uint8
     desc = (f"seed {seed} case {case}: latent={latent} {hq}/{hk} d{d} {dtype} b{batch} max{maxlen} {mode} "
             f"alibi={alibi} fp8={fp8} int8={int8} {layout} page={page} total={total}")
     kw, k8, v8 = {}, None, None
@@ -70,10 +71,13 @@ def _one_case(rng, seed, case, int4=False, per_token=False):
         # rows of different spread and offset: the pairs differ from token to token and head to head
         k = k.float() * (0.5 + torch.rand(total, hk, 1, generator=g)) + torch.randn(total, hk, 1, generator=g)
         v = v.float() * (0.5 + torch.rand(total, hk, 1, generator=g)) + 0.5 * torch.randn(total, hk, 1, generator=g)
-        k8, kpairs = quantize_int4_per_token(k)
-        v8, vpairs = quantize_int4_per_token(v)
+        quant = quantize_int8_per_token if per_token == 8 else quantize_int4_per_token
+        k8, kpairs = quant(k)
+        v8, vpairs = quant(v)
 
         def unpack(p4):
+            if per_token == 8:
+                return p4.double()
             n = torch.stack([(p4 & 15).to(torch.int16), (p4 >> 4).to(torch.int16)], dim=-1).flatten(-2)
             return torch.where(n >= 8, n - 16, n).double()
 
@@ -146,7 +150,15 @@ def test_random_cases_over_an_int4_cache_with_per_token_pairs(chunk):
     seed = 13
     rng = random.Random(seed * 1000 + chunk)
     for i in range(CASES_PER_CHUNK):
-        _one_case(rng, seed, chunk * CASES_PER_CHUNK + i, per_token=True)
+        _one_case(rng, seed, chunk * CASES_PER_CHUNK + i, per_token=4)
+
+
+@pytest.mark.parametrize("chunk", range(2))
+def test_random_cases_over_an_int8_cache_with_per_token_pairs(chunk):
+    seed = 17
+    rng = random.Random(seed * 1000 + chunk)
+    for i in range(CASES_PER_CHUNK):
+        _one_case(rng, seed, chunk * CASES_PER_CHUNK + i, per_token=8)
 
 
 @pytest.mark.parametrize("chunk", range(8))
