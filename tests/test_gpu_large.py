@@ -99,3 +99,38 @@ def test_batch_beyond_one_grid_axis(kind):
         w = wl.Workload("batch70000_paged", q[rows].cpu(), torch.cat(ks), torch.cat(vs), wl.get_cu_seq(sub), int(sub.max()),
                         d, False, sub.tolist())
         check_against_oracle(w, o[rows].cpu())
+
+
+def test_batch_beyond_one_grid_axis_with_per_token_pairs():
+    """The same seam with an int4 cache whose rows carry their own (scale, zero) pairs: the second launch addresses
+    the packed rows and their pairs by absolute row number, q and o by the run's first sequence."""
+    from decoding_attention_amd import quantize_int4_per_token
+    from oracle import oracle
+
+    g = torch.Generator(device="cpu").manual_seed(19)
+    batch, seam, hq, hk, d, sk = 70000, 65528, 8, 2, 64, 20
+    lens = torch.randint(1, sk + 1, (batch,), generator=g, dtype=torch.int32)
+    cu = wl.get_cu_seq(lens)
+    total = int(cu[-1])
+    gd = torch.Generator(device=DEV).manual_seed(19)
+    q = torch.randn(batch, hq, d, generator=gd, device=DEV, dtype=torch.float16)
+    k = torch.randn(total, hk, d, generator=gd, device=DEV) * 2 + 0.5
+    v = torch.randn(total, hk, d, generator=gd, device=DEV) - 0.3
+    k4, kp = quantize_int4_per_token(k)
+    v4, vp = quantize_int4_per_token(v)
+    o = decoding_attn_fwd(q, k4, v4, cu.to(DEV), sk, d, False, k_scale=kp, v_scale=vp)
+    torch.cuda.synchronize()
+    assert torch.isfinite(o.float()).all()
+
+    def unpack(p4):
+        n = torch.stack([(p4 & 15).to(torch.int16), (p4 >> 4).to(torch.int16)], dim=-1).flatten(-2)
+        return torch.where(n >= 8, n - 16, n).double()
+
+    rows = [0, 1, seam - 1, seam, seam + 1, batch - 1]
+    cu_l = cu.tolist()
+    sel = torch.cat([torch.arange(cu_l[b], cu_l[b + 1]) for b in rows]).to(DEV)
+    kd = (kp[sel][..., :1].double() * (unpack(k4[sel]) - kp[sel][..., 1:].double())).cpu()
+    vd = (vp[sel][..., :1].double() * (unpack(v4[sel]) - vp[sel][..., 1:].double())).cpu()
+    sub = torch.tensor([int(lens[b]) for b in rows], dtype=torch.int32)
+    ref = torch.from_numpy(oracle.attn_f64(q[rows].cpu(), kd, vd, wl.get_cu_seq(sub), d, False)).float()
+    assert (o[rows].cpu().float() - ref).abs().max().item() <= 2e-3
