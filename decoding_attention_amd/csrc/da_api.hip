@@ -525,7 +525,13 @@ bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) ==
 // Workspace of da_decoding_attn_noalloc: a device array that exists on every GPU the library is loaded on, from
 // load to process end.  The largest workspace any plan asks for is 256 work-groups x 128 heads x 514 floats =
 // 67.4 MB (the latent kernel's split partials), except for the balanced grid on pathologically ragged batches.
+#ifdef DA_BUILD_PROBES
+// (the measurement build, which only the benchmark loads, holds no such array: its no-alloc entry point serves the
+// plans that need no workspace and refuses the rest)
+constexpr size_t kScratchBytes = 256;
+#else
 constexpr size_t kScratchBytes = (size_t)80 << 20;
+#endif
 static __device__ __align__(256) unsigned char scratch[kScratchBytes];
 
 namespace {

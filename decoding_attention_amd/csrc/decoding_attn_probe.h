@@ -1,7 +1,8 @@
 /*
  * Measurement aids of the benchmark (bench.py), exported by libdecoding_attn_probe.so only: a second build of the
- * library's sources with these entry points added.  None of this is part of the drop-in ABI
- * (decoding_attn_hip.h) and nothing here has a counterpart in the reference.
+ * library's sources with these entry points added (and without the static device array of
+ * da_decoding_attn_noalloc, which this build answers only for plans that need no workspace).  None of this is part of
+ * the drop-in ABI (decoding_attn_hip.h) and nothing here has a counterpart in the reference.
  */
 #ifndef DECODING_ATTN_PROBE_H_
 #define DECODING_ATTN_PROBE_H_
