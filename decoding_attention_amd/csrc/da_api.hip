@@ -144,9 +144,10 @@ int rows_per_trip(size_t dim) {
 // no_latent_kernel: the cache format has no form of the latent kernel (int4): the latent form then runs on the grouped
 // kernel whatever its size, as ceil(heads / 16) groups per sequence that read the same rows.
 // group_only: the call has a form on the grouped kernel only (per-token quantisation factors): every shape takes it.
+// 2 = a pair per 64 elements of a row: at d = 256 its 32-head form would not fit the registers, 16 heads per group.
 Plan make_plan(size_t max_seq_k, size_t batch, size_t head_q, size_t head_k, size_t dim, size_t dim_v,
                bool v_distinct, size_t total_k, size_t page_size = 0, bool kv_8bit = false,
-               bool no_latent_kernel = false, bool group_only = false) {
+               bool no_latent_kernel = false, int group_only = 0) {
     const bool packed = page_size == 0;
     Plan pl;
     const int ratio = (int)(head_q / head_k);
@@ -233,6 +234,7 @@ Plan make_plan(size_t max_seq_k, size_t batch, size_t head_q, size_t head_k, siz
         pl.kind = kKindGroup;
         pl.rt = ratio > 16 ? 32 : 16;
         if (tun().gqa_heads == 16 || tun().gqa_heads == 32) pl.rt = tun().gqa_heads;
+        if (group_only == 2 && dim == 256) pl.rt = 16;
         pl.wave_per_head = head_k % 4 == 0 && tun().wave_per_head;
         trip = pl.wave_per_head ? da::kGqaTile : 4 * da::kGqaTile;
         // d = 128, four waves sharing one KV head's tokens (MQA and other head counts that are no multiple of four): one
@@ -442,7 +444,7 @@ Plan make_plan(size_t max_seq_k, size_t batch, size_t head_q, size_t head_k, siz
 // Workspace bytes of a call: the plan's, or, for a batch beyond one launch (kMaxGridBatch), the largest of its runs'.
 size_t plan_ws_bytes(size_t max_seq_k, size_t batch, size_t head_q, size_t head_k, size_t dim, size_t dim_v,
                      bool v_distinct, size_t total_k, size_t page_size = 0, bool kv_8bit = false,
-                     bool no_latent_kernel = false, bool group_only = false) {
+                     bool no_latent_kernel = false, int group_only = 0) {
     if (batch <= kMaxGridBatch)
         return make_plan(max_seq_k, batch, head_q, head_k, dim, dim_v, v_distinct, total_k, page_size, kv_8bit,
                          no_latent_kernel, group_only).ws_bytes;
@@ -612,9 +614,11 @@ int da_plan_call(size_t max_seq_k, size_t batch, size_t head_q, size_t head_k, s
         return fail(DA_ERR_INVALID_ARGUMENT, "head_q (%zu) must be a multiple of head_k (%zu)", head_q, head_k);
     if (!supported_dims(dim, dim_v))
         return fail(DA_ERR_UNSUPPORTED, "unsupported head dims (dim %zu, dim_v %zu)", dim, dim_v);
-    const bool per_token = kv_bits == DA_KV_BITS_INT4_PER_TOKEN || kv_bits == DA_KV_BITS_INT8_PER_TOKEN;
+    const bool per64 = kv_bits == DA_KV_BITS_INT4_GROUP64;
+    const bool per_token = kv_bits == DA_KV_BITS_INT4_PER_TOKEN || kv_bits == DA_KV_BITS_INT8_PER_TOKEN || per64;
     if (kv_bits != 16 && kv_bits != 8 && kv_bits != 4 && !per_token)
-        return fail(DA_ERR_INVALID_ARGUMENT, "kv_bits (%d) must be 16, 8, 4 or one of DA_KV_BITS_INT*_PER_TOKEN", kv_bits);
+        return fail(DA_ERR_INVALID_ARGUMENT,
+                    "kv_bits (%d) must be 16, 8, 4, one of DA_KV_BITS_INT*_PER_TOKEN or DA_KV_BITS_INT4_GROUP64", kv_bits);
     if (per_token && (dim != dim_v || (dim != 64 && dim != 128 && dim != 256) || !distinct_v))
         return fail(DA_ERR_UNSUPPORTED, "per-token factors: head dims (64,64), (128,128) and (256,256), V of its own");
     if (page_size != 0 && (page_size & (page_size - 1)) != 0)
@@ -623,7 +627,8 @@ int da_plan_call(size_t max_seq_k, size_t batch, size_t head_q, size_t head_k, s
     const bool folded = batch > kMaxGridBatch;
     const Plan pl = make_plan(max_seq_k, folded ? kMaxGridBatch : batch, head_q, head_k, dim, dim_v, distinct_v != 0,
                               folded ? 0 : total_k, page_size, kv_bits != 16,
-                              kv_bits == 4 || kv_bits == DA_KV_BITS_INT4_PER_TOKEN, per_token);
+                              kv_bits == 4 || kv_bits == DA_KV_BITS_INT4_PER_TOKEN || per64,
+                              per64 ? 2 : (per_token ? 1 : 0));
     if (kernel_kind) *kernel_kind = pl.kind;
     if (nsplit) *nsplit = pl.nsplit;
     if (chunk) *chunk = pl.chunk;
@@ -682,13 +687,15 @@ struct KvFormat {
     // (int4) a (scale, zero) pair per (token, KV head) instead of the per-head factors
     const float* k_tok = nullptr;
     const float* v_tok = nullptr;
+    bool tok_per64 = false;  // ... a pair per run of 64 elements of the row instead: [rows, head_k, dim / 64, 2]
 };
 
-KvFormat per_token_format(int fmt, const float* k_params, const float* v_params) {
+KvFormat per_token_format(int fmt, const float* k_params, const float* v_params, bool per64 = false) {
     KvFormat kf;
     kf.fmt = fmt;
     kf.k_tok = k_params;
     kf.v_tok = v_params;
+    kf.tok_per64 = per64;
     return kf;
 }
 
@@ -760,9 +767,12 @@ int run_attention(const void* q, const void* k, const void* v, void* o, const in
             return fail(DA_ERR_UNSUPPORTED, "per-token factors: head dims (64,64), (128,128) and (256,256) only");
         if ((reinterpret_cast<uintptr_t>(kf.k_tok) | reinterpret_cast<uintptr_t>(kf.v_tok)) & 7u)
             return fail(DA_ERR_INVALID_ARGUMENT, "k_params and v_params must be 8-byte aligned");
+        if (kf.tok_per64 && kf.fmt != da::kKvInt4)
+            return fail(DA_ERR_UNSUPPORTED, "a pair per 64 elements: int4 caches only");
     }
     const Plan pl = make_plan(max_seq_k, batch, head_q, head_k, dim, dim_v, v != nullptr, total_k,
-                              pg.table ? pg.page_size : 0, kf.fmt != 0, kf.fmt == da::kKvInt4, per_token);
+                              pg.table ? pg.page_size : 0, kf.fmt != 0, kf.fmt == da::kKvInt4,
+                              per_token ? (kf.tok_per64 ? 2 : 1) : 0);
     if (per_token && pl.kind != kKindGroup)  // (DA_FORCE_KIND=1 takes the grouped kernel away)
         return fail(DA_ERR_UNSUPPORTED, "per-token factors need the grouped kernel");
     if ((size_t)head_k * pl.groups > 65535)
@@ -855,6 +865,8 @@ int run_attention(const void* q, const void* k, const void* v, void* o, const in
             e = da::launch_mla_kv8(sp, kf.fmt, is_bf16 != 0, pl.rt, grid, stream);
         else if (pl.kind == kKindGroup && per_token && kf.fmt == da::kKvInt8)
             e = da::launch_gqa_mfma_i8t(sp, is_bf16 != 0, (int)dim, pl.rt, pl.wave_per_head, grid, stream);
+        else if (pl.kind == kKindGroup && per_token && kf.tok_per64 && dim > 64)  // (64: one run is the row)
+            e = da::launch_gqa_mfma_i4g(sp, is_bf16 != 0, (int)dim, pl.rt, pl.wave_per_head, grid, stream);
         else if (pl.kind == kKindGroup && per_token)
             e = da::launch_gqa_mfma_i4t(sp, is_bf16 != 0, (int)dim, pl.rt, pl.wave_per_head, grid, stream);
         else if (pl.kind == kKindGroup && kf.fmt == da::kKvInt8)
@@ -1117,6 +1129,40 @@ size_t da_workspace_bytes_int4kv_tok(size_t max_seq_k, size_t batch, size_t head
                                      size_t dim_v, size_t total_k, size_t page_size) {
     if (head_k == 0 || head_q % head_k != 0 || dim != dim_v || (dim != 64 && dim != 128 && dim != 256)) return 0;
     return plan_ws_bytes(max_seq_k, batch, head_q, head_k, dim, dim_v, true, total_k, page_size, true, true, true);
+}
+
+int da_decoding_attn_int4kv_grp64(const void* q, const void* k4, const void* v4, void* o, const int32_t* cu_seq_k,
+                                  size_t max_seq_k, size_t batch, size_t head_q, size_t head_k, size_t dim,
+                                  size_t dim_v, int is_alibi, int is_bf16, float softmax_scale,
+                                  const float* alibi_slopes, const float* k_params, const float* v_params,
+                                  size_t total_k, void* workspace, size_t workspace_bytes, void* hip_stream) {
+    if (!k_params || !v_params) return fail(DA_ERR_INVALID_ARGUMENT, "k_params or v_params is null");
+    return run_attention(q, k4, v4, o, cu_seq_k, Paging{}, per_token_format(da::kKvInt4, k_params, v_params, true),
+                         max_seq_k, batch, head_q, head_k, dim, dim_v, is_alibi, is_bf16, softmax_scale, alibi_slopes,
+                         total_k, workspace, workspace_bytes, hip_stream);
+}
+
+int da_decoding_attn_paged_int4kv_grp64(const void* q, const void* k_pages, const void* v_pages, void* o,
+                                        const int32_t* block_table, const int32_t* seq_lens, size_t max_seq_k,
+                                        size_t batch, size_t head_q, size_t head_k, size_t dim, size_t dim_v,
+                                        size_t page_size, size_t max_blocks_per_seq, size_t k_page_stride,
+                                        size_t v_page_stride, int is_alibi, int is_bf16, float softmax_scale,
+                                        const float* alibi_slopes, const float* k_params, const float* v_params,
+                                        size_t total_k, void* workspace, size_t workspace_bytes, void* hip_stream) {
+    if (!k_params || !v_params) return fail(DA_ERR_INVALID_ARGUMENT, "k_params or v_params is null");
+    Paging pg;
+    const int rc = check_paging(block_table, seq_lens, max_seq_k, head_k, dim, dim_v, page_size, max_blocks_per_seq,
+                                k_page_stride, v_page_stride, v_pages != nullptr, &pg);
+    if (rc != DA_OK) return rc;
+    return run_attention(q, k_pages, v_pages, o, nullptr, pg, per_token_format(da::kKvInt4, k_params, v_params, true),
+                         max_seq_k, batch, head_q, head_k, dim, dim_v, is_alibi, is_bf16, softmax_scale, alibi_slopes,
+                         total_k, workspace, workspace_bytes, hip_stream);
+}
+
+size_t da_workspace_bytes_int4kv_grp64(size_t max_seq_k, size_t batch, size_t head_q, size_t head_k, size_t dim,
+                                       size_t dim_v, size_t total_k, size_t page_size) {
+    if (head_k == 0 || head_q % head_k != 0 || dim != dim_v || (dim != 64 && dim != 128 && dim != 256)) return 0;
+    return plan_ws_bytes(max_seq_k, batch, head_q, head_k, dim, dim_v, true, total_k, page_size, true, true, 2);
 }
 
 int da_decoding_attn_int8kv_tok(const void* q, const void* k8, const void* v8, void* o, const int32_t* cu_seq_k,

@@ -128,6 +128,9 @@ constexpr int kKvInt4 = 3;
 // Flag on top of a format (grouped kernel's template argument only): every (token, KV head) row carries its own
 // (scale, zero) pair, element = scale * (integer - zero), instead of one factor per KV head (SweepParams::k_tok).
 constexpr int kKvPerToken = 8;
+// ... and on top of that: one pair per run of 64 elements of the row instead of one per row (head dims of 128 and 256:
+// two and four pairs; SweepParams::k_tok then holds [rows, head_k, dim / 64, 2] floats).
+constexpr int kKvGroup64 = 16;
 
 // Eight FP8 (OCP e4m3) values -> eight 16-bit elements of the compute type.  Both conversions are exact (e4m3
 // has 3 mantissa bits and |x| <= 448), so an FP8 K/V cache feeds the same arithmetic as a 16-bit one.

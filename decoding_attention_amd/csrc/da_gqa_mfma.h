@@ -100,13 +100,13 @@ constexpr int gqa_v_pitch() { return DV * 2 + 32; }  // LDS row pitch of the V t
 template <int DV>
 constexpr int gqa_merge_pitch() { return DV + 4; }  // floats per row of the merge area: conflict-free row writes
 
-constexpr int kGqaTokBytes = 512;  // per wave: the (scale, zero) pairs of a tile's tokens, K and V (per-token factors)
+constexpr int kGqaTokBytes = 512;  // per wave and pair of a row: the (scale, zero) pairs of a tile's tokens, K and V
 
 template <int DV>
-constexpr size_t gqa_lds_bytes(int nt, bool per_token = false) {
+constexpr size_t gqa_lds_bytes(int nt, int tok_pairs = 0) {
     // V tiles of the four waves (and, behind them, their tiles' per-token pairs), reused for the final merge
     // ([4][heads][pitch] floats + (m, l))
-    const size_t vt = 4 * (size_t)kGqaTile * gqa_v_pitch<DV>() + (per_token ? 4 * kGqaTokBytes : 0);
+    const size_t vt = 4 * (size_t)kGqaTile * gqa_v_pitch<DV>() + (size_t)tok_pairs * 4 * kGqaTokBytes;
     const size_t mg = 4 * (size_t)(16 * nt) * (gqa_merge_pitch<DV>() + 2) * sizeof(float);
     return vt > mg ? vt : mg;
 }
@@ -148,13 +148,19 @@ __device__ __forceinline__ void gqa_segment(const SweepParams& p, uint8_t* const
     // head's q row.  V[t][c] = a_v[t] (n[t][c] - z_v[t]) likewise: the probabilities are multiplied by a_v[t] on
     // their way into the second product, and sum_t p'[t] z_v[t], one number per head, comes off every column at the end.
     constexpr bool TOK = (KV8 & kKvPerToken) != 0;
+    // NG: pairs per row.  With kKvGroup64 every run of 64 elements of a row has its own pair: a run is what two
+    // consecutive k-steps of the score product cover (8-bit layouts) and what four 16-column tiles of the output
+    // cover, so the score tile is summed per run before the factors go on, and the second product takes a
+    // probability operand per run.
+    constexpr int NG = (TOK && (KV8 & kKvGroup64) != 0) ? D / 64 : 1;
+    static_assert(NG == 1 || (D == DV && D % 64 == 0), "one pair per 64 elements");
     // B4: an int4 cache.  Its nibbles reach the matrix instructions as kInt4Bias + n (int4x8_biased), the eight
     // elements of a word in the order 0, 4, 1, 5, 2, 6, 3, 7: Q is gathered in that order, the bias leaves the scores
     // through the sum of the head's q row and the outputs through the sum of the rounded probabilities, and the
     // output columns, which come out in that order within every run of eight, are put right after the last tile.
     constexpr bool B4 = FMT == kKvInt4;
     const uint32_t b4_one = B4 ? int4_biased_one<Tag>() : 0u;
-    auto convert8 = [b4_one](uint2 w) __attribute__((always_inline)) {
+    auto convert8 = [&](uint2 w) __attribute__((always_inline)) {
         if constexpr (B4)
             return int4x8_biased<Tag>(w.x, b4_one);
         else if constexpr (FMT != 0)
@@ -213,35 +219,43 @@ __device__ __forceinline__ void gqa_segment(const SweepParams& p, uint8_t* const
         slope[nt] = p.is_alibi ? alibi_slope_log2(p.slopes, h, p.head_q) : 0.0f;
     }
     // (TOK, B4) sum of each head's q row: the four 16-lane groups hold different elements of the same rows
-    float qsum[NT];
+    float qsum[NT][NG];  // (per run of the row when the pairs are)
     if constexpr (TOK || B4) {
 #pragma unroll
-        for (int nt = 0; nt < NT; ++nt) {
-            // (a dot product with ones: one instruction per pair of elements)
-            constexpr uint32_t kOnes = std::is_same<Tag, f16_tag>::value ? 0x3C003C00u : 0x3F803F80u;
-            float acc_q = 0.0f;
+        for (int nt = 0; nt < NT; ++nt)
 #pragma unroll
-            for (int ks = 0; ks < KS; ++ks) {
-                const uint4 w = __builtin_bit_cast(uint4, qf[nt][ks]);
-                acc_q = EL::dot2(w.x, kOnes, acc_q);
-                acc_q = EL::dot2(w.y, kOnes, acc_q);
-                acc_q = EL::dot2(w.z, kOnes, acc_q);
-                acc_q = EL::dot2(w.w, kOnes, acc_q);
+            for (int qg = 0; qg < NG; ++qg) {
+                // (a dot product with ones: one instruction per pair of elements)
+                constexpr uint32_t kOnes = std::is_same<Tag, f16_tag>::value ? 0x3C003C00u : 0x3F803F80u;
+                float acc_q = 0.0f;
+#pragma unroll
+                for (int ks = qg * (KS / NG); ks < (qg + 1) * (KS / NG); ++ks) {
+                    const uint4 w = __builtin_bit_cast(uint4, qf[nt][ks]);
+                    acc_q = EL::dot2(w.x, kOnes, acc_q);
+                    acc_q = EL::dot2(w.y, kOnes, acc_q);
+                    acc_q = EL::dot2(w.z, kOnes, acc_q);
+                    acc_q = EL::dot2(w.w, kOnes, acc_q);
+                }
+                acc_q += __shfl_xor(acc_q, 16);
+                acc_q += __shfl_xor(acc_q, 32);
+                qsum[nt][qg] = acc_q;
             }
-            acc_q += __shfl_xor(acc_q, 16);
-            acc_q += __shfl_xor(acc_q, 32);
-            qsum[nt] = acc_q;
-        }
     }
 
     f32x4 acc[NT][CT];
     float m[NT], l[NT];
-    float corr[NT];  // (TOK) sum over tokens of p'[t] z_v[t], in the accumulators' units
+    float corr[NT][NG];  // (TOK) sum over tokens of p'[t] z_v[t], in the accumulators' units
+    // (bf16, NG > 1) the denominators under the other runs' V scales: a probability rounded to eight bits for one run
+    // is not the one rounded for another, and each run's columns are divided by the sum of what they were multiplied
+    // by (the columns are brought to l's units after the last tile)
+    constexpr bool LQ = NG > 1 && std::is_same<Tag, bf16_tag>::value;
+    float lq[NT][NG];
 #pragma unroll
     for (int nt = 0; nt < NT; ++nt) {
         m[nt] = kNegBig;
         l[nt] = 0.0f;
-        corr[nt] = 0.0f;
+#pragma unroll
+        for (int qg = 0; qg < NG; ++qg) corr[nt][qg] = lq[nt][qg] = 0.0f;
 #pragma unroll
         for (int ct = 0; ct < CT; ++ct) acc[nt][ct] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
     }
@@ -258,7 +272,7 @@ __device__ __forceinline__ void gqa_segment(const SweepParams& p, uint8_t* const
     // (B4, per-head factors) the bias' share of every score of head nt, in log2 units
     float bias_q[NT];
 #pragma unroll
-    for (int nt = 0; nt < NT; ++nt) bias_q[nt] = (B4 && !TOK) ? kInt4Bias * sl * qsum[nt] : 0.0f;
+    for (int nt = 0; nt < NT; ++nt) bias_q[nt] = (B4 && !TOK) ? kInt4Bias * sl * qsum[nt][0] : 0.0f;
 
     // wave-private V tile in LDS
     uint8_t* const vt = smem + wave * (kGqaTile * VP);
@@ -273,7 +287,7 @@ __device__ __forceinline__ void gqa_segment(const SweepParams& p, uint8_t* const
     struct TileRegs {
         uint4 k[2][KSR];
         uint4 v[NVR];
-        float2 tokp;  // (TOK) lanes 0 .. 31: the K pair of the tile's token `lane`; 32 .. 63: the V pair of lane - 32
+        float2 tokp[NG];  // (TOK) lanes 0 .. 31: the K pairs of the tile's token `lane`; 32 .. 63: the V pairs of lane - 32
     };
     TileRegs tr;
 
@@ -327,8 +341,9 @@ __device__ __forceinline__ void gqa_segment(const SweepParams& p, uint8_t* const
         }
     };
     // (TOK) one pair per lane and tile, rows past the end as the last valid one; the wave passes them through its
-    // corner of LDS (tokbuf: K scales, K zeros, V scales, V zeros, 32 floats each) to the lanes that need them
-    float* const tokbuf = reinterpret_cast<float*>(smem + 4 * kGqaTile * VP + wave * kGqaTokBytes);
+    // corner of LDS (tokbuf: K scales, K zeros, V scales, V zeros, 32 floats each per run of the row) to the lanes
+    // that need them
+    float* const tokbuf = reinterpret_cast<float*>(smem + 4 * kGqaTile * VP + wave * (NG * kGqaTokBytes));
     auto load_tok = [&](int tok0, TileRegs& r) __attribute__((always_inline)) {
         if constexpr (TOK) {
             const int row = min(lane & 31, c1 - 1 - tok0);
@@ -343,7 +358,8 @@ __device__ __forceinline__ void gqa_segment(const SweepParams& p, uint8_t* const
                      (tok & ((1 << p.page_shift) - 1));
             }
             const float2* const pool = reinterpret_cast<const float2*>(lane < 32 ? p.k_tok : p.v_tok);
-            r.tokp = pool[at * p.head_k + hk];
+#pragma unroll
+            for (int qg = 0; qg < NG; ++qg) r.tokp[qg] = pool[(at * p.head_k + hk) * NG + qg];
         }
     };
     auto load_v = [&](int tok0, TileRegs& r) __attribute__((always_inline)) {
@@ -409,6 +425,7 @@ __device__ __forceinline__ void gqa_segment(const SweepParams& p, uint8_t* const
 
         // S^T = K . Q^T for the two 16-token tiles, then refill the K registers
         f32x4 s[2][NT];
+        f32x4 sq[2][NT][NG];  // (NG > 1) the sums of the row's runs, apart
 #pragma unroll
         for (int mt = 0; mt < 2; ++mt)
 #pragma unroll
@@ -416,6 +433,12 @@ __device__ __forceinline__ void gqa_segment(const SweepParams& p, uint8_t* const
                 f32x4 c = {0.0f, 0.0f, 0.0f, 0.0f};
 #pragma unroll
                 for (int ks = 0; ks < KS; ++ks) {
+                    if constexpr (NG > 1) {
+                        if (ks % (KS / NG) == 0 && ks != 0) {
+                            sq[mt][nt][ks / (KS / NG) - 1] = c;
+                            c = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+                        }
+                    }
                     uint4 kfrag;
                     if constexpr (KV8) {
                         const uint4 w = tr.k[mt][ks >> 1];
@@ -433,6 +456,7 @@ __device__ __forceinline__ void gqa_segment(const SweepParams& p, uint8_t* const
                 }
                 if constexpr (VK) settle(c);
                 s[mt][nt] = c;
+                sq[mt][nt][NG - 1] = c;
             }
         if constexpr (VK) {
             // the value columns of the tile, from the K registers: lane (n, g) holds 16-byte chunk ks * 4 + g of row
@@ -459,32 +483,47 @@ __device__ __forceinline__ void gqa_segment(const SweepParams& p, uint8_t* const
 
         // online softmax; token of s[mt][nt][r]: tok0 + mt*16 + g*4 + r, head nt*16 + n
         vec8 pf[NT];
+        vec8 pfg[NT][NG];  // (NG > 1) the probabilities under the V scales of the row's runs
         const bool tail = tok0 + kGqaTile > c1;
         float x[NT][8], mx[NT];
-        // (TOK) per token: A = score scale x a_k, Z = z_k plus the conversion's bias; x = A (s - Z qsum)
-        float tokA[TOK ? 8 : 1], tokZ[TOK ? 8 : 1], tokV[TOK ? 8 : 1], tokW[TOK ? 8 : 1], tokVinv[TOK ? 8 : 1];
+        // (TOK) per token (and run): A = score scale x a_k, Z = z_k plus the conversion's bias; x = sum A (s - Z qsum)
+        float tokA[NG][TOK ? 8 : 1], tokZ[NG][TOK ? 8 : 1], tokV[NG][TOK ? 8 : 1], tokW[NG][TOK ? 8 : 1], tokVinv[NG][TOK ? 8 : 1];
         if constexpr (TOK) {
-            float* const mine = tokbuf + (lane >> 5) * 64 + (lane & 31);
-            mine[0] = tr.tokp.x;
-            mine[32] = tr.tokp.y;
+            // tokbuf[((kind * NG + run) * 32 + token]: kind 0 K scale, 1 K zero, 2 V scale, 3 V zero
+            float* const mine = tokbuf + (lane >> 5) * (2 * NG * 32) + (lane & 31);
+#pragma unroll
+            for (int qg = 0; qg < NG; ++qg) {
+                mine[qg * 32] = tr.tokp[qg].x;
+                mine[(NG + qg) * 32] = tr.tokp[qg].y;
+            }
             if (PREFETCH && more) load_tok(tok_next, tr);
 #pragma unroll
-            for (int mt = 0; mt < 2; ++mt) {
-                const f32x4 ak = *reinterpret_cast<const f32x4*>(tokbuf + mt * 16 + g * 4);
-                const f32x4 zk = *reinterpret_cast<const f32x4*>(tokbuf + 32 + mt * 16 + g * 4);
-                const f32x4 av = *reinterpret_cast<const f32x4*>(tokbuf + 64 + mt * 16 + g * 4);
-                const f32x4 zv = *reinterpret_cast<const f32x4*>(tokbuf + 96 + mt * 16 + g * 4);
+            for (int qg = 0; qg < NG; ++qg)
 #pragma unroll
-                for (int r = 0; r < 4; ++r) {
-                    tokA[mt * 4 + r] = sl * ak[r];
-                    tokZ[mt * 4 + r] = zk[r] + (B4 ? kInt4Bias : 0.0f);
-                    tokV[mt * 4 + r] = av[r];
-                    tokW[mt * 4 + r] = zv[r] + (B4 ? kInt4Bias : 0.0f);
-                    if constexpr (std::is_same<Tag, bf16_tag>::value)
-                        tokVinv[mt * 4 + r] = __builtin_amdgcn_rcpf(av[r]);
+                for (int mt = 0; mt < 2; ++mt) {
+                    const f32x4 ak = *reinterpret_cast<const f32x4*>(tokbuf + (0 * NG + qg) * 32 + mt * 16 + g * 4);
+                    const f32x4 zk = *reinterpret_cast<const f32x4*>(tokbuf + (1 * NG + qg) * 32 + mt * 16 + g * 4);
+                    const f32x4 av = *reinterpret_cast<const f32x4*>(tokbuf + (2 * NG + qg) * 32 + mt * 16 + g * 4);
+                    const f32x4 zv = *reinterpret_cast<const f32x4*>(tokbuf + (3 * NG + qg) * 32 + mt * 16 + g * 4);
+#pragma unroll
+                    for (int r = 0; r < 4; ++r) {
+                        tokA[qg][mt * 4 + r] = sl * ak[r];
+                        tokZ[qg][mt * 4 + r] = zk[r] + (B4 ? kInt4Bias : 0.0f);
+                        tokV[qg][mt * 4 + r] = av[r];
+                        tokW[qg][mt * 4 + r] = zv[r] + (B4 ? kInt4Bias : 0.0f);
+                        if constexpr (std::is_same<Tag, bf16_tag>::value)
+                            tokVinv[qg][mt * 4 + r] = __builtin_amdgcn_rcpf(av[r]);
+                    }
                 }
-            }
         }
+        // the score of token j = mt * 4 + r under the pairs: sum over the row's runs
+        auto tok_score = [&](int mt, int nt, int r) __attribute__((always_inline)) {
+            float v = (sq[mt][nt][0][r] - tokZ[0][mt * 4 + r] * qsum[nt][0]) * tokA[0][mt * 4 + r];
+#pragma unroll
+            for (int qg = 1; qg < NG; ++qg)
+                v = __builtin_fmaf(sq[mt][nt][qg][r] - tokZ[qg][mt * 4 + r] * qsum[nt][qg], tokA[qg][mt * 4 + r], v);
+            return v;
+        };
 #pragma unroll
         for (int nt = 0; nt < NT; ++nt) {
             mx[nt] = -INFINITY;
@@ -495,8 +534,7 @@ __device__ __forceinline__ void gqa_segment(const SweepParams& p, uint8_t* const
 #pragma unroll
                         for (int r = 0; r < 4; ++r) {
                             const int tok = tok0 + mt * 16 + g * 4 + r;
-                            float v = (s[mt][nt][r] - tokZ[mt * 4 + r] * qsum[nt]) * tokA[mt * 4 + r] +
-                                      slope[nt] * (float)(tok - (len - 1));
+                            float v = tok_score(mt, nt, r) + slope[nt] * (float)(tok - (len - 1));
                             if (tok >= c1) v = -INFINITY;
                             x[nt][mt * 4 + r] = v;
                             mx[nt] = fmaxf(mx[nt], v);
@@ -506,7 +544,7 @@ __device__ __forceinline__ void gqa_segment(const SweepParams& p, uint8_t* const
                     for (int mt = 0; mt < 2; ++mt)
 #pragma unroll
                         for (int r = 0; r < 4; ++r) {
-                            x[nt][mt * 4 + r] = (s[mt][nt][r] - tokZ[mt * 4 + r] * qsum[nt]) * tokA[mt * 4 + r];
+                            x[nt][mt * 4 + r] = tok_score(mt, nt, r);
                             mx[nt] = fmaxf(mx[nt], x[nt][mt * 4 + r]);
                         }
                 }
@@ -546,26 +584,41 @@ __device__ __forceinline__ void gqa_segment(const SweepParams& p, uint8_t* const
                 const float alpha = fast_exp2(m[nt] - mn);
                 m[nt] = mn;
                 l[nt] *= alpha;
-                if constexpr (TOK) corr[nt] *= alpha;
+                if constexpr (TOK) {
+#pragma unroll
+                    for (int qg = 0; qg < NG; ++qg) {
+                        corr[nt][qg] *= alpha;
+                        if constexpr (LQ) lq[nt][qg] *= alpha;
+                    }
+                }
 #pragma unroll
                 for (int ct = 0; ct < CT; ++ct) acc[nt][ct] *= alpha;
             }
         }
 #pragma unroll
         for (int nt = 0; nt < NT; ++nt) {
+            float xg[NG][8];  // (NG > 1) probabilities under the other runs' V scales
 #pragma unroll
             for (int j = 0; j < 8; ++j) {
                 if constexpr (TOK) {
                     // the second product's operand is p a_v[t], rounded to 16 bits; the zero-point sum uses the
                     // rounded value, and so does the denominator where the rounding is coarse (bf16)
                     const float pe = fast_exp2(x[nt][j] - m[nt]);
-                    const float pv = round16<Tag>(pe * tokV[j]);
+                    const float pv = round16<Tag>(pe * tokV[0][j]);
+                    // (a scale of zero: the row adds nothing to the columns and its whole probability to the sum)
                     if constexpr (std::is_same<Tag, bf16_tag>::value)
-                        l[nt] += pv * tokVinv[j];
+                        l[nt] += tokV[0][j] != 0.0f ? pv * tokVinv[0][j] : pe;
                     else
                         l[nt] += pe;
-                    corr[nt] = __builtin_fmaf(pv, tokW[j], corr[nt]);
+                    corr[nt][0] = __builtin_fmaf(pv, tokW[0][j], corr[nt][0]);
                     x[nt][j] = pv;
+#pragma unroll
+                    for (int qg = 1; qg < NG; ++qg) {
+                        const float pq = round16<Tag>(pe * tokV[qg][j]);
+                        corr[nt][qg] = __builtin_fmaf(pq, tokW[qg][j], corr[nt][qg]);
+                        if constexpr (LQ) lq[nt][qg] += tokV[qg][j] != 0.0f ? pq * tokVinv[qg][j] : pe;
+                        xg[qg][j] = pq;
+                    }
                 } else if constexpr (B4) {
                     x[nt][j] = fast_exp2(x[nt][j] - m[nt]);  // (rounded by pack8; the denominator follows below)
                 } else {
@@ -574,6 +627,9 @@ __device__ __forceinline__ void gqa_segment(const SweepParams& p, uint8_t* const
                 }
             }
             pf[nt] = MM::pack8(x[nt]);  // k index j <-> token g*4+j (j<4), 16+g*4+(j-4) (j>=4)
+            pfg[nt][0] = pf[nt];
+#pragma unroll
+            for (int qg = 1; qg < NG; ++qg) pfg[nt][qg] = MM::pack8(xg[qg]);
             if constexpr (B4 && !TOK) {
                 // the denominator sums the probabilities as rounded for the matrix instruction (it is also what the
                 // bias is taken out with): a dot product of the packed pairs with ones
@@ -594,7 +650,7 @@ __device__ __forceinline__ void gqa_segment(const SweepParams& p, uint8_t* const
             const s16x8_t both = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
             const vec8 a = __builtin_bit_cast(vec8, both);
 #pragma unroll
-            for (int nt = 0; nt < NT; ++nt) acc[nt][ct] = MM::mma(a, pf[nt], acc[nt][ct]);
+            for (int nt = 0; nt < NT; ++nt) acc[nt][ct] = MM::mma(a, pfg[nt][NG > 1 ? ct / (CT / NG) : 0], acc[nt][ct]);
         }
 
         if (!PREFETCH && more) {
@@ -610,10 +666,29 @@ __device__ __forceinline__ void gqa_segment(const SweepParams& p, uint8_t* const
         l[nt] += __shfl_xor(l[nt], 16);
         l[nt] += __shfl_xor(l[nt], 32);
         if constexpr (TOK) {  // the zero points' share (and the bias') comes off every column of the head
-            corr[nt] += __shfl_xor(corr[nt], 16);
-            corr[nt] += __shfl_xor(corr[nt], 32);
 #pragma unroll
-            for (int ct = 0; ct < CT; ++ct) acc[nt][ct] -= corr[nt];
+            for (int qg = 0; qg < NG; ++qg) {
+                corr[nt][qg] += __shfl_xor(corr[nt][qg], 16);
+                corr[nt][qg] += __shfl_xor(corr[nt][qg], 32);
+            }
+            float to_l[NG];  // (LQ) run's denominator -> l
+            to_l[0] = 1.0f;
+            if constexpr (LQ) {
+#pragma unroll
+                for (int qg = 1; qg < NG; ++qg) {
+                    float d = lq[nt][qg];
+                    d += __shfl_xor(d, 16);
+                    d += __shfl_xor(d, 32);
+                    to_l[qg] = d > 0.0f ? l[nt] * __builtin_amdgcn_rcpf(d) : 1.0f;
+                }
+            }
+#pragma unroll
+            for (int ct = 0; ct < CT; ++ct) {
+                const int qg = NG > 1 ? ct / (CT / NG) : 0;
+                acc[nt][ct] -= corr[nt][qg];
+                if constexpr (LQ)
+                    if (qg > 0) acc[nt][ct] *= to_l[qg];
+            }
         } else if constexpr (B4) {  // sum_t p (bias + n) = sum_t p n + bias l
             const float off = kInt4Bias * l[nt];
 #pragma unroll
@@ -816,6 +891,9 @@ hipError_t launch_gqa_mfma_i4(const SweepParams& p, bool is_bf16, int dim, int h
                               dim3 grid, hipStream_t stream);
 // ... and over an int4 one whose rows carry their own (scale, zero) pairs (SweepParams::k_tok, v_tok); dim 64, 128, 256
 hipError_t launch_gqa_mfma_i4t(const SweepParams& p, bool is_bf16, int dim, int heads_per_group, bool wave_per_head,
+                               dim3 grid, hipStream_t stream);
+// ... and over an int4 one with a pair per run of 64 elements of each row ([rows, head_k, dim / 64, 2]); dim 128, 256
+hipError_t launch_gqa_mfma_i4g(const SweepParams& p, bool is_bf16, int dim, int heads_per_group, bool wave_per_head,
                                dim3 grid, hipStream_t stream);
 // ... and over an int8 one with such pairs
 hipError_t launch_gqa_mfma_i8t(const SweepParams& p, bool is_bf16, int dim, int heads_per_group, bool wave_per_head,

@@ -1,6 +1,6 @@
 // Launch helpers of the grouped-head MFMA sweep, shared by the translation units that instantiate it (16-bit
-// K/V in da_gqa_mfma.hip, FP8 in da_gqa_mfma_kv8.hip, int8 in da_gqa_mfma_i8.hip, int4 in da_gqa_mfma_i4.hip, the per-token forms in da_gqa_mfma_i4t.hip and da_gqa_mfma_i8t.hip; separate units so that the sets
-// compile in parallel).
+// K/V in da_gqa_mfma.hip, FP8 in da_gqa_mfma_kv8.hip, int8 in da_gqa_mfma_i8.hip, int4 in da_gqa_mfma_i4.hip, the per-token forms in da_gqa_mfma_i4t.hip and da_gqa_mfma_i8t.hip, int4 with a pair per 64 elements in
+// da_gqa_mfma_i4g.hip; separate units so that the sets compile in parallel).
 #pragma once
 #include "da_gqa_mfma.h"
 
@@ -15,7 +15,7 @@ hipError_t launch_form(const SweepParams& p, dim3 grid, hipStream_t stream) {
     constexpr bool kPrefetch = D <= 128 || D == 576;
     constexpr int kMinWaves = (D <= 128 && (NT == 1 || D <= 64)) ? 2 : 1;
     auto kern = gqa_mfma_kernel<Tag, D, DV, NT, kPrefetch, WH, kMinWaves, KV8, PGM>;
-    const size_t lds = gqa_lds_bytes<DV>(NT, (KV8 & kKvPerToken) != 0);
+    const size_t lds = gqa_lds_bytes<DV>(NT, (KV8 & kKvPerToken) == 0 ? 0 : ((KV8 & kKvGroup64) != 0 ? D / 64 : 1));
     if (lds > 48 * 1024) {
         static std::atomic<uint64_t> devices_done{0};
         const hipError_t attr_err = ensure_lds_limit(reinterpret_cast<const void*>(kern), lds, devices_done);
@@ -38,15 +38,20 @@ template <typename Tag, int D, int KV8>
 hipError_t launch_dim(const SweepParams& p, int heads_per_group, bool wh, dim3 grid, hipStream_t stream) {
     if (heads_per_group == 16)
         return wh ? launch_one<Tag, D, 1, true, KV8>(p, grid, stream) : launch_one<Tag, D, 1, false, KV8>(p, grid, stream);
-    if (heads_per_group == 32)
-        return wh ? launch_one<Tag, D, 2, true, KV8>(p, grid, stream) : launch_one<Tag, D, 2, false, KV8>(p, grid, stream);
+    // (a pair per 64 elements at d = 256: four sets of factors and 32 heads do not fit a wave's registers)
+    if constexpr (!((KV8 & kKvGroup64) != 0 && D == 256))
+        if (heads_per_group == 32)
+            return wh ? launch_one<Tag, D, 2, true, KV8>(p, grid, stream)
+                      : launch_one<Tag, D, 2, false, KV8>(p, grid, stream);
     return hipErrorInvalidValue;
 }
 
 template <typename Tag, int KV8>
 hipError_t launch_tag(const SweepParams& p, int dim, int heads_per_group, bool wh, dim3 grid, hipStream_t stream) {
     switch (dim) {
-        case 64: return launch_dim<Tag, 64, KV8>(p, heads_per_group, wh, grid, stream);
+        case 64:  // (one pair per 64 elements is one pair per row here: the per-token instantiation serves it)
+            if constexpr ((KV8 & kKvGroup64) == 0) return launch_dim<Tag, 64, KV8>(p, heads_per_group, wh, grid, stream);
+            return hipErrorInvalidValue;
         case 96:
             if constexpr (!KV8) return launch_dim<Tag, 96, 0>(p, heads_per_group, wh, grid, stream);
             return hipErrorInvalidValue;  // 8-bit loads pair up k-steps: head dims that are multiples of 64 only

@@ -47,21 +47,29 @@ const float *scale_ptr(const std::optional<at::Tensor> &t, const at::Tensor &q, 
 
 // int4 or int8 with a (scale, zero) pair per (token, KV head): k_scale and v_scale are then tensors shaped like the rows they
 // belong to with a last dimension of 2 (`rows` = the leading dimensions of the K tensor) instead of head_k values.
-bool per_token_pairs(const std::optional<at::Tensor> &ks, const std::optional<at::Tensor> &vs, const at::Tensor &q,
-                     const at::Tensor &k, int kv8) {
-    const bool k_pairs = ks.has_value() && ks.value().dim() == k.dim();
-    const bool v_pairs = vs.has_value() && vs.value().dim() == k.dim();
-    if (!k_pairs && !v_pairs) return false;
+// One dimension more, [..., head_k, dim / 64, 2], is a pair per run of 64 elements of every row (int4 only).
+// Returns 0 (per-head factors), 1 (a pair per row) or 2 (a pair per 64 elements).
+int per_token_pairs(const std::optional<at::Tensor> &ks, const std::optional<at::Tensor> &vs, const at::Tensor &q,
+                    const at::Tensor &k, int kv8) {
+    const int64_t kd = k.dim();
+    const auto form = [kd](const std::optional<at::Tensor> &t) {
+        return !t.has_value() ? 0 : (t.value().dim() == kd ? 1 : (t.value().dim() == kd + 1 ? 2 : 0));
+    };
+    const int k_form = form(ks), v_form = form(vs);
+    if (k_form == 0 && v_form == 0) return 0;
     TORCH_CHECK(kv8 == 3 || kv8 == 2, "per-token (scale, zero) pairs apply to an int4 or int8 K/V cache only");
-    TORCH_CHECK(k_pairs && v_pairs, "per-token (scale, zero) pairs must be given for both K and V");
+    TORCH_CHECK(k_form == v_form, "per-token (scale, zero) pairs must be given for both K and V, in the same form");
+    TORCH_CHECK(k_form == 1 || kv8 == 3, "a (scale, zero) pair per 64 elements applies to an int4 K/V cache only");
     for (const at::Tensor *t : {&ks.value(), &vs.value()}) {
         TORCH_CHECK(t->dtype() == torch::kFloat32 && t->is_cuda() && t->device() == q.device() && t->is_contiguous(),
                     "per-token pairs must be contiguous float32 GPU tensors");
-        for (int64_t d = 0; d + 1 < k.dim(); ++d)
+        for (int64_t d = 0; d + 1 < kd; ++d)
             TORCH_CHECK(t->size(d) == k.size(d), "per-token pairs must have the K tensor's leading dimensions");
-        TORCH_CHECK(t->size(k.dim() - 1) == 2, "per-token pairs must have a last dimension of 2 (scale, zero)");
+        if (k_form == 2)
+            TORCH_CHECK(t->size(kd - 1) * 64 == q.size(-1), "pairs per 64 elements: [..., head_k, dim / 64, 2]");
+        TORCH_CHECK(t->size(-1) == 2, "per-token pairs must have a last dimension of 2 (scale, zero)");
     }
-    return true;
+    return k_form;
 }
 
 at::Tensor dmha_fwd(const at::Tensor &q, const at::Tensor &k, const std::optional<at::Tensor> &v_,
@@ -149,14 +157,15 @@ at::Tensor dmha_fwd(const at::Tensor &q, const at::Tensor &k, const std::optiona
     c10::hip::HIPGuardMasqueradingAsCUDA guard(q.device());
     hipStream_t stream = c10::hip::getCurrentHIPStreamMasqueradingAsCUDA(q.device().index()).stream();
 
-    const bool tok = per_token_pairs(k_scale, v_scale, q, k, kv8);
+    const int tok = per_token_pairs(k_scale, v_scale, q, k, kv8);
     TORCH_CHECK(!tok || v_ptr != nullptr, "per-token pairs need a V cache of its own");
     const float *k_scale_ptr = tok ? k_scale.value().data_ptr<float>() : scale_ptr(k_scale, q, head_k, "k_scale", kv8);
     const float *v_scale_ptr = tok ? v_scale.value().data_ptr<float>() : scale_ptr(v_scale, q, head_k, "v_scale", kv8);
 
     // k.size(0) is the sum of the key lengths: a free host-side hint for sizing the sequence splits
     const size_t ws_bytes =
-        kv8 ? (tok ? (kv8 == 3 ? da_workspace_bytes_int4kv_tok : da_workspace_bytes_int8kv_tok)
+        kv8 ? (tok == 2 ? da_workspace_bytes_int4kv_grp64
+               : tok ? (kv8 == 3 ? da_workspace_bytes_int4kv_tok : da_workspace_bytes_int8kv_tok)
                    : kv8 == 3 ? da_workspace_bytes_int4kv : da_workspace_bytes_fp8kv)(
                   (size_t)max_seq_k, (size_t)batch, (size_t)head_q, (size_t)head_k, (size_t)dim, (size_t)dim_v,
                   (size_t)total_k, 0)
@@ -166,7 +175,8 @@ at::Tensor dmha_fwd(const at::Tensor &q, const at::Tensor &k, const std::optiona
     if (ws_bytes > 0) ws = torch::empty({(int64_t)ws_bytes}, q.options().dtype(torch::kUInt8));
 
     const float scale = softmax_scale.has_value() ? (float)softmax_scale.value() : 0.0f;
-    const auto kv8_entry = tok        ? (kv8 == 3 ? da_decoding_attn_int4kv_tok : da_decoding_attn_int8kv_tok)
+    const auto kv8_entry = tok == 2   ? da_decoding_attn_int4kv_grp64
+                           : tok      ? (kv8 == 3 ? da_decoding_attn_int4kv_tok : da_decoding_attn_int8kv_tok)
                            : kv8 == 3 ? da_decoding_attn_int4kv
                                       : (kv8 == 2 ? da_decoding_attn_int8kv : da_decoding_attn_fp8kv);
     const int rc =
@@ -269,13 +279,14 @@ at::Tensor dmha_fwd_paged(const at::Tensor &q, const at::Tensor &k_pages, const 
     c10::hip::HIPGuardMasqueradingAsCUDA guard(q.device());
     hipStream_t stream = c10::hip::getCurrentHIPStreamMasqueradingAsCUDA(q.device().index()).stream();
 
-    const bool tok = per_token_pairs(k_scale, v_scale, q, k_pages, kv8);
+    const int tok = per_token_pairs(k_scale, v_scale, q, k_pages, kv8);
     TORCH_CHECK(!tok || v_ptr != nullptr, "per-token pairs need a V cache of its own");
     const float *k_scale_ptr = tok ? k_scale.value().data_ptr<float>() : scale_ptr(k_scale, q, head_k, "k_scale", kv8);
     const float *v_scale_ptr = tok ? v_scale.value().data_ptr<float>() : scale_ptr(v_scale, q, head_k, "v_scale", kv8);
     const size_t hint = total_k > 0 ? (size_t)total_k : 0;
     const size_t ws_bytes =
-        kv8 ? (tok ? (kv8 == 3 ? da_workspace_bytes_int4kv_tok : da_workspace_bytes_int8kv_tok)
+        kv8 ? (tok == 2 ? da_workspace_bytes_int4kv_grp64
+               : tok ? (kv8 == 3 ? da_workspace_bytes_int4kv_tok : da_workspace_bytes_int8kv_tok)
                    : kv8 == 3 ? da_workspace_bytes_int4kv : da_workspace_bytes_fp8kv)(
                   (size_t)max_seq_k, (size_t)batch, (size_t)head_q, (size_t)head_k, (size_t)dim, (size_t)dim_v, hint,
                   (size_t)page_size)
@@ -285,7 +296,8 @@ at::Tensor dmha_fwd_paged(const at::Tensor &q, const at::Tensor &k_pages, const 
     if (ws_bytes > 0) ws = torch::empty({(int64_t)ws_bytes}, q.options().dtype(torch::kUInt8));
 
     const float scale = softmax_scale.has_value() ? (float)softmax_scale.value() : 0.0f;
-    const auto kv8_entry = tok        ? (kv8 == 3 ? da_decoding_attn_paged_int4kv_tok : da_decoding_attn_paged_int8kv_tok)
+    const auto kv8_entry = tok == 2   ? da_decoding_attn_paged_int4kv_grp64
+                           : tok      ? (kv8 == 3 ? da_decoding_attn_paged_int4kv_tok : da_decoding_attn_paged_int8kv_tok)
                            : kv8 == 3 ? da_decoding_attn_paged_int4kv
                                       : (kv8 == 2 ? da_decoding_attn_paged_int8kv : da_decoding_attn_paged_fp8kv);
     const int rc =

@@ -152,6 +152,19 @@ def test_shifting_integers_and_zero_points_together_changes_nothing(dtype, bits)
 
 
 @pytest.mark.gpu
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+def test_rows_with_a_scale_of_zero(dtype):
+    """A constant row may come with a scale of exactly zero: it is a row of zeros, and its probability still counts."""
+    w, k4, v4, kp, vp = _case(3, 16, 4, 128, 400, dtype, seed=41)
+    g = torch.Generator().manual_seed(4)
+    kp[torch.rand(kp.shape[:2], generator=g) < 0.2, 0] = 0.0
+    vp[torch.rand(vp.shape[:2], generator=g) < 0.2, 0] = 0.0
+    o = _run(w, k4, v4, kp, vp)
+    assert torch.isfinite(o.float()).all()
+    assert (o.float() - _reference(w, k4, v4, kp, vp)).abs().max().item() <= TOL[dtype]
+
+
+@pytest.mark.gpu
 def test_zero_points_of_zero_reduce_to_the_per_head_call():
     w = wl.make_workload(5, 32, 8, 128, 128, 1100, torch.float16, seed=23, varlen=True)
     ks, vs = torch.full((8,), 3.0 / 7), torch.linspace(0.3, 0.5, 8)

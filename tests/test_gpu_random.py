@@ -10,8 +10,8 @@ import random
 import pytest
 import torch
 
-from decoding_attention_amd import (decoding_attn_fwd, decoding_attn_paged_fwd, pack_int4, quantize_int4_per_token,
-                                    quantize_int8_per_token)
+from decoding_attention_amd import (decoding_attn_fwd, decoding_attn_paged_fwd, pack_int4, quantize_int4_per_group,
+                                    quantize_int4_per_token, quantize_int8_per_token)
 from decoding_attention_amd import workloads as wl
 from oracle import oracle
 from tests.gpu_util import TOL, run_hip_ex, sub_workload
@@ -27,7 +27,8 @@ CASES_PER_CHUNK = 12
 def _one_case(rng, seed, case, int4=False, per_token=False):
     """int4: the case runs over an int4 cache (whatever format the draws below pick; the stream of draws is the same
     either way, so the other cases do not move).  per_token (4 or 8): an int4 or int8 cache with a (scale, zero) pair
-    per token and KV head (never the latent form, never d = 96, which those entry points do not serve)."""
+    per token and KV head (never the latent form, never d = 96, which those entry points do not serve); 64: an int4
+    cache with a pair per run of 64 elements of each row."""
     latent = rng.random() < 0.3 and not per_token
     dtype = rng.choice([torch.float16, torch.bfloat16])
     if latent:
@@ -69,11 +70,17 @@ def _one_case(rng, seed, case, int4=False, per_token=False):
     k_true, v_true = k.float(), None if v is None else v.float()
     if per_token:
         # rows of different spread and offset: the pairs differ from token to token and head to head
-        k = k.float() * (0.5 + torch.rand(total, hk, 1, generator=g)) + torch.randn(total, hk, 1, generator=g)
-        v = v.float() * (0.5 + torch.rand(total, hk, 1, generator=g)) + 0.5 * torch.randn(total, hk, 1, generator=g)
-        quant = quantize_int8_per_token if per_token == 8 else quantize_int4_per_token
+        runs = d // 64 if per_token == 64 else 1  # (per_token == 64: every run of 64 elements likewise)
+        shape = (total, hk, runs, 1)
+        k = (k.float().unflatten(-1, (runs, -1)) * (0.5 + torch.rand(shape, generator=g))
+             + torch.randn(shape, generator=g)).flatten(-2)
+        v = (v.float().unflatten(-1, (runs, -1)) * (0.5 + torch.rand(shape, generator=g))
+             + 0.5 * torch.randn(shape, generator=g)).flatten(-2)
+        quant = {8: quantize_int8_per_token, 4: quantize_int4_per_token, 64: quantize_int4_per_group}[per_token]
         k8, kpairs = quant(k)
         v8, vpairs = quant(v)
+        if per_token != 64:
+            kpairs, vpairs = kpairs.unsqueeze(-2), vpairs.unsqueeze(-2)  # [total, hk, runs, 2] from here on
 
         def unpack(p4):
             if per_token == 8:
@@ -81,9 +88,10 @@ def _one_case(rng, seed, case, int4=False, per_token=False):
             n = torch.stack([(p4 & 15).to(torch.int16), (p4 >> 4).to(torch.int16)], dim=-1).flatten(-2)
             return torch.where(n >= 8, n - 16, n).double()
 
-        k_true = kpairs[..., :1].double() * (unpack(k8) - kpairs[..., 1:].double())
-        v_true = vpairs[..., :1].double() * (unpack(v8) - vpairs[..., 1:].double())
-        kw = dict(k_scale=kpairs.to(DEV), v_scale=vpairs.to(DEV))
+        k_true = (kpairs[..., :1].double() * (unpack(k8).unflatten(-1, (runs, -1)) - kpairs[..., 1:].double())).flatten(-2)
+        v_true = (vpairs[..., :1].double() * (unpack(v8).unflatten(-1, (runs, -1)) - vpairs[..., 1:].double())).flatten(-2)
+        as_passed = (lambda t: t) if per_token == 64 else (lambda t: t.squeeze(-2))  # noqa: E731
+        kw = dict(k_scale=as_passed(kpairs).to(DEV), v_scale=as_passed(vpairs).to(DEV))
     elif fp8:
         def quantise(x, scale):
             y = x.float() / scale.view(1, -1, 1)
@@ -112,9 +120,10 @@ def _one_case(rng, seed, case, int4=False, per_token=False):
                           lens.tolist())
         pk = wl.to_pages(src, page, seed=case, poison=not fp8).to(DEV)
         if per_token:  # the pairs in pools of their own, numbered like the pages (same seed)
-            pp = wl.to_pages(wl.Workload("pp", q, kpairs, vpairs, cu, max_seq_k, dv, alibi, lens.tolist()), page,
-                             seed=case).to(DEV)
-            kw = dict(k_scale=pp.k_pages, v_scale=pp.v_pages)
+            pp = wl.to_pages(wl.Workload("pp", q, kpairs.flatten(-2), vpairs.flatten(-2), cu, max_seq_k, dv, alibi,
+                                         lens.tolist()), page, seed=case).to(DEV)
+            kw = dict(k_scale=as_passed(pp.k_pages.unflatten(-1, (runs, 2))),
+                      v_scale=as_passed(pp.v_pages.unflatten(-1, (runs, 2))))
         kp = pk.k_pages.view(kv8_dtype) if fp8 else pk.k_pages
         vp = None if pk.v_pages is None else (pk.v_pages.view(kv8_dtype) if fp8 else pk.v_pages)
         o = decoding_attn_paged_fwd(q.to(DEV), kp, vp, pk.block_table, pk.seq_lens, max_seq_k, dv, alibi,
@@ -167,3 +176,11 @@ def test_random_cases(chunk):
     rng = random.Random(seed * 1000 + chunk)
     for i in range(CASES_PER_CHUNK):
         _one_case(rng, seed, chunk * CASES_PER_CHUNK + i)
+
+
+@pytest.mark.parametrize("chunk", range(3))
+def test_random_cases_over_an_int4_cache_with_pairs_per_64_elements(chunk):
+    seed = 19
+    rng = random.Random(seed * 1000 + chunk)
+    for i in range(CASES_PER_CHUNK):
+        _one_case(rng, seed, chunk * CASES_PER_CHUNK + i, per_token=64)
