@@ -248,12 +248,18 @@ __device__ __forceinline__ uint4 int4x8_biased(uint32_t w, uint32_t one) {
 
 // Sixteen (eight) elements of an int4 cache at the doubled address `vptr` (see kKvInt4): the packed words, each in
 // the slot where the 8-bit formats keep the eight bytes of the same elements (the other word of the pair is unused).
+// The halved address is cast to the global address space by hand: an address that went through integer arithmetic
+// is a generic one to the compiler, and a generic (flat) load counts against the LDS counter as well, so that every
+// wait for an LDS read would also wait for the K/V loads in flight.
 __device__ __forceinline__ uint4 kv4_load16(const void* vptr) {
-    const uint2 w = *reinterpret_cast<const uint2*>(reinterpret_cast<uintptr_t>(vptr) >> 1);
+    typedef unsigned int u32x2 __attribute__((ext_vector_type(2)));
+    typedef const u32x2 __attribute__((address_space(1))) * global_u32x2_ptr;
+    const u32x2 w = *(global_u32x2_ptr)(reinterpret_cast<uintptr_t>(vptr) >> 1);
     return make_uint4(w.x, 0u, w.y, 0u);
 }
 __device__ __forceinline__ uint2 kv4_load8(const void* vptr) {
-    return make_uint2(*reinterpret_cast<const uint32_t*>(reinterpret_cast<uintptr_t>(vptr) >> 1), 0u);
+    typedef const uint32_t __attribute__((address_space(1))) * global_u32_ptr;
+    return make_uint2(*(global_u32_ptr)(reinterpret_cast<uintptr_t>(vptr) >> 1), 0u);
 }
 
 // Eight elements of an 8-bit K/V cache of format FMT -> eight 16-bit elements of the compute type (an int4 cache's

@@ -420,6 +420,11 @@ __device__ __forceinline__ void gqa_segment(const SweepParams& p, uint8_t* const
                 *reinterpret_cast<uint4*>(vt + row * VP + ch * 16) = tr.v[i];
             }
         }
+        // The K registers of this tile, the only loads still in flight, are needed right after: wait for them here,
+        // before the V loads of the next tile are issued (on both sides of the branch: the compiler's bookkeeping
+        // joins them).  Left to itself the compiler puts a wait for everything behind those V loads, which holds
+        // the wave for a whole memory latency every tile.
+        if constexpr (PREFETCH) __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0), the other counters untouched
         if (PREFETCH && more) load_v(tok_next, tr);
         }
 
