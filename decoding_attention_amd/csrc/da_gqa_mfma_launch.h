@@ -12,7 +12,9 @@ namespace gqa_launch {
 template <typename Tag, int D, int NT, bool WH, int KV8, int PGM>
 hipError_t launch_form(const SweepParams& p, dim3 grid, hipStream_t stream) {
     constexpr int DV = D == 576 ? 512 : D;  // (576, 512): the latent form, V inside the K rows
-    constexpr bool kPrefetch = D <= 128 || D == 576;
+    // the next tile's loads issued as soon as this tile's registers are free, not after its last matrix instruction
+    // (d = 256 with 32 heads a group: the longer live ranges do not fit 512 registers, 41 to 78 of them spilled)
+    constexpr bool kPrefetch = D <= 128 || D == 576 || (D == 256 && NT == 1);
     constexpr int kMinWaves = (D <= 128 && (NT == 1 || D <= 64)) ? 2 : 1;
     auto kern = gqa_mfma_kernel<Tag, D, DV, NT, kPrefetch, WH, kMinWaves, KV8, PGM>;
     const size_t lds = gqa_lds_bytes<DV>(NT, (KV8 & kKvPerToken) == 0 ? 0 : ((KV8 & kKvGroup64) != 0 ? D / 64 : 1));
