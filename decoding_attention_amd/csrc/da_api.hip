@@ -219,6 +219,12 @@ Plan make_plan(size_t max_seq_k, size_t batch, size_t head_q, size_t head_k, siz
                (ratio >= tun().group_min_ratio || group_only ||
                 (tun().group_min_ratio > 1 && (max_seq_k >= 1024 || dim <= 96) &&
                  (long long)batch * (long long)head_k * (long long)max_seq_k >= (1ll << 21)) ||
+                // ... and over long sequences of a small batch (measured, 32 heads, 16-bit / FP8: batch 1 x 8192 tokens
+                // 26.3 -> 23.9 / 17.8 -> 14.9 us, 1 x 16384 47.9 -> 42.7 / 27.6 -> 24.8, 2 x 4096 25.0 -> 23.7 /
+                // 17.7 -> 15.3, 4 x 8192 89.8 -> 82.1 / 46.4 -> 44.6, d 64 1 x 16384 27.7 -> 24.6 / 18.8 -> 15.7; a
+                // tie at 1 x 4096 and 1 x 6144; d 256 stays: 1 x 8192 24.9 against 35.2)
+                (tun().group_min_ratio > 1 && dim <= 128 && max_seq_k >= 4096 &&
+                 (long long)batch * (long long)head_k * (long long)max_seq_k >= (3ll << 16)) ||
                 // an int4 cache (the format without a latent kernel): the VALU sweep pays more per nibble than the
                 // matrix kernel's word-wise conversion does (measured, MHA 32 heads d 128: batch 512 x 128 tokens 92.0
                 // -> 54.8 us, batch 2048 x 128 397 -> 254, batch 32 x 1024 50.5 -> 30.8, batch 32 x 128 8.7 -> 6.8,
