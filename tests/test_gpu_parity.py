@@ -46,7 +46,7 @@ def test_reference_grid_mla(head_q, batch, seq_k, dtype):
 
 
 @pytest.mark.parametrize("batch,seq_k", [(1, 128), (8, 128), (32, 128), (128, 128), (512, 128), (1, 512), (1, 1536),
-                                          (1, 4096), (1, 8192)])
+                                          (1, 4096), (1, 6144), (2, 4096), (1, 8192)])
 def test_config1_mha_sweep_points(batch, seq_k):
     """Every point of the two sweeps (batch 2048 below), every row against the oracle."""
     w = wl.config_mha_sweep(batch, seq_k)

@@ -179,6 +179,12 @@ def test_plan_of_every_call_form():
         assert _lib.plan(128, 512, 32, 32, 128, 128, kv_bits=bits)["kind"] == 3
         with pytest.raises(RuntimeError):
             _lib.plan(128, 512, 32, 32, 96, 96, kv_bits=bits)
+    # one query head per KV head: the grouped kernel over long sequences of a small batch at d <= 128, else the VALU sweep
+    assert _lib.plan(8192, 1, 32, 32, 128, 128, distinct_v=True)["kind"] == 3
+    assert _lib.plan(6144, 1, 32, 32, 128, 128, distinct_v=True)["kind"] == 3
+    assert _lib.plan(4096, 1, 32, 32, 128, 128, distinct_v=True)["kind"] == 1
+    assert _lib.plan(8192, 1, 16, 16, 256, 256, distinct_v=True)["kind"] == 1
+    assert _lib.plan(128, 512, 32, 32, 128, 128, distinct_v=True)["kind"] == 1
     for bad in (dict(kv_bits=12), dict(page_size=48)):
         with pytest.raises(RuntimeError):
             _lib.plan(*shape, **bad)
