@@ -94,7 +94,7 @@ def _device_copies(torch, w, dev, min_total_bytes=768 << 20):
 
 
 def measure(torch, w, steps, warmup, page_size=0, kv_fp8=False, kv_int8=False, kv_int4=False, kv_int4_tok=False,
-            kv_int8_tok=False, kv_int4_g64=False):
+            kv_int8_tok=False, kv_int4_g64=False, kv_int8_g64=False):
     from decoding_attention_amd import _lib, decoding_attn_fwd
     from decoding_attention_amd import workloads as wl
 
@@ -103,10 +103,10 @@ def measure(torch, w, steps, warmup, page_size=0, kv_fp8=False, kv_int8=False, k
     outs = []
 
     def make(c):
-        if kv_int4_tok or kv_int8_tok or kv_int4_g64:  # a (scale, zero) pair per (token, KV head), or per 64 elements
+        if kv_int4_tok or kv_int8_tok or kv_int4_g64 or kv_int8_g64:  # a (scale, zero) pair per row, or per 64 elements
             from decoding_attention_amd import (quantize_int4_per_group, quantize_int4_per_token,
-                                                quantize_int8_per_token)
-            quant = (quantize_int4_per_group if kv_int4_g64 else
+                                                quantize_int8_per_group, quantize_int8_per_token)
+            quant = (quantize_int4_per_group if kv_int4_g64 else quantize_int8_per_group if kv_int8_g64 else
                      quantize_int4_per_token if kv_int4_tok else quantize_int8_per_token)
             k4, kp = quant(c.k)
             v4, vp = quant(c.v)
@@ -152,18 +152,19 @@ def measure(torch, w, steps, warmup, page_size=0, kv_fp8=False, kv_int8=False, k
     mean_ms, min_ms = _time_calls(torch, fns, steps, warmup)
     assert torch.isfinite(outs[0].float()).all()
     nbytes = wl.workload_bytes(w)
-    if kv_fp8 or kv_int8 or kv_int4 or kv_int4_tok or kv_int8_tok or kv_int4_g64:  # one byte (half a byte) per K/V element
+    per64 = kv_int4_g64 or kv_int8_g64
+    if kv_fp8 or kv_int8 or kv_int4 or kv_int4_tok or kv_int8_tok or per64:  # one byte (half a byte) per K/V element
         kv_elems = int(w.k.numel() + (w.v.numel() if w.v is not None else 0))
         nbytes = wl.algorithmic_bytes(w.batch, w.head_q, w.head_k, w.dim, w.dim_v, int(w.k.shape[0]), w.v is not None,
                                       elem_bytes=2) - (kv_elems * 3 // 2 if (kv_int4 or kv_int4_tok or kv_int4_g64) else kv_elems)
-        if kv_int4_tok or kv_int8_tok or kv_int4_g64:  # two float pairs per (token, KV head), or per 64 elements of it
-            nbytes += int(w.k.shape[0]) * w.head_k * 16 * (w.dim // 64 if kv_int4_g64 else 1)
+        if kv_int4_tok or kv_int8_tok or per64:  # two float pairs per (token, KV head), or per 64 elements of it
+            nbytes += int(w.k.shape[0]) * w.head_k * 16 * (w.dim // 64 if per64 else 1)
     flops = wl.workload_flops(w)
     # the plan of the call that was timed
     plan = _lib.plan(w.max_seq_k, w.batch, w.head_q, w.head_k, w.dim, w.dim_v,
                      total_k=int(w.k.shape[0]),
                      distinct_v=w.v is not None and w.dim != w.dim_v, page_size=page_size,
-                     kv_bits=_lib.KV_BITS_INT4_GROUP64 if kv_int4_g64 else
+                     kv_bits=_lib.KV_BITS_INT4_GROUP64 if kv_int4_g64 else _lib.KV_BITS_INT8_GROUP64 if kv_int8_g64 else
                      _lib.KV_BITS_INT4_PER_TOKEN if kv_int4_tok else _lib.KV_BITS_INT8_PER_TOKEN if kv_int8_tok else
                      4 if kv_int4 else 8 if (kv_fp8 or kv_int8) else 16)
     return {
@@ -502,6 +503,7 @@ def run_sweep(args, measure_fn=None, workload_fn=None, out=None):
                 shapes += [(None, "kv-int4-tok", w, {"kv_int4_tok": True})]
                 shapes += [(None, "kv-int8-tok", w, {"kv_int8_tok": True})]
                 shapes += [(None, "kv-int4-g64", w, {"kv_int4_g64": True})]
+                shapes += [(None, "kv-int8-g64", w, {"kv_int8_g64": True})]
     results = []
     for marker, tag, spec, kw in shapes:
         if marker == SEQ_MARKER:

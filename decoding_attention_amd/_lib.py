@@ -38,6 +38,9 @@ EXPORTED_SYMBOLS = (
     "da_decoding_attn_int4kv_grp64",
     "da_decoding_attn_paged_int4kv_grp64",
     "da_workspace_bytes_int4kv_grp64",
+    "da_decoding_attn_int8kv_grp64",
+    "da_decoding_attn_paged_int8kv_grp64",
+    "da_workspace_bytes_int8kv_grp64",
     "da_decoding_attn_int8kv_tok",
     "da_decoding_attn_paged_int8kv_tok",
     "da_workspace_bytes_int8kv_tok",
@@ -124,6 +127,12 @@ def _declare(lib):
     lib.da_decoding_attn_int4kv_grp64.argtypes = lib.da_decoding_attn_fp8kv.argtypes
     lib.da_decoding_attn_paged_int4kv_grp64.restype = ci
     lib.da_decoding_attn_paged_int4kv_grp64.argtypes = lib.da_decoding_attn_paged_fp8kv.argtypes
+    lib.da_decoding_attn_int8kv_grp64.restype = ci
+    lib.da_decoding_attn_int8kv_grp64.argtypes = lib.da_decoding_attn_fp8kv.argtypes
+    lib.da_decoding_attn_paged_int8kv_grp64.restype = ci
+    lib.da_decoding_attn_paged_int8kv_grp64.argtypes = lib.da_decoding_attn_paged_fp8kv.argtypes
+    lib.da_workspace_bytes_int8kv_grp64.restype = sz
+    lib.da_workspace_bytes_int8kv_grp64.argtypes = lib.da_workspace_bytes_fp8kv.argtypes
     lib.da_workspace_bytes_int4kv_grp64.restype = sz
     lib.da_workspace_bytes_int4kv_grp64.argtypes = lib.da_workspace_bytes_fp8kv.argtypes
     lib.da_workspace_bytes_int4kv_tok.restype = sz
@@ -190,15 +199,16 @@ def last_error() -> str:
 KV_BITS_INT4_PER_TOKEN = 5  # DA_KV_BITS_INT4_PER_TOKEN of include/decoding_attn_hip.h
 KV_BITS_INT8_PER_TOKEN = 9  # DA_KV_BITS_INT8_PER_TOKEN
 KV_BITS_INT4_GROUP64 = 6  # DA_KV_BITS_INT4_GROUP64
+KV_BITS_INT8_GROUP64 = 10  # DA_KV_BITS_INT8_GROUP64
 
 
 def plan(max_seq_k, batch, head_q, head_k, dim, dim_v, is_bf16=False, total_k=0, distinct_v=False, page_size=0,
          kv_bits=16):
     """Launch plan of a call: dict(kind, nsplit, chunk, heads_per_group, balanced).  `distinct_v`: V passed as its own
     buffer; `page_size`: pages of that many tokens (0 = packed); `kv_bits`: 16, 8 (FP8, int8), 4 (int4) or
-    KV_BITS_INT4_PER_TOKEN / KV_BITS_INT8_PER_TOKEN (int4 / int8 with per-token pairs) or KV_BITS_INT4_GROUP64 (int4
-    with a pair per 64 elements); distinct_v is implied for these."""
-    if kv_bits in (KV_BITS_INT4_PER_TOKEN, KV_BITS_INT8_PER_TOKEN, KV_BITS_INT4_GROUP64):
+    KV_BITS_INT4_PER_TOKEN / KV_BITS_INT8_PER_TOKEN (int4 / int8 with per-token pairs) or KV_BITS_INT4_GROUP64 /
+    KV_BITS_INT8_GROUP64 (a pair per 64 elements); distinct_v is implied for these."""
+    if kv_bits in (KV_BITS_INT4_PER_TOKEN, KV_BITS_INT8_PER_TOKEN, KV_BITS_INT4_GROUP64, KV_BITS_INT8_GROUP64):
         distinct_v = True
     del is_bf16  # (the plan does not depend on it)
     lib = load()

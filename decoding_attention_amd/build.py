@@ -28,6 +28,7 @@ SOURCES = [
     "da_gqa_mfma_i4.hip",
     "da_gqa_mfma_i4t.hip",
     "da_gqa_mfma_i4g.hip",
+    "da_gqa_mfma_i8g.hip",
     "da_gqa_mfma_i8t.hip",
 ]
 

@@ -620,11 +620,11 @@ int da_plan_call(size_t max_seq_k, size_t batch, size_t head_q, size_t head_k, s
         return fail(DA_ERR_INVALID_ARGUMENT, "head_q (%zu) must be a multiple of head_k (%zu)", head_q, head_k);
     if (!supported_dims(dim, dim_v))
         return fail(DA_ERR_UNSUPPORTED, "unsupported head dims (dim %zu, dim_v %zu)", dim, dim_v);
-    const bool per64 = kv_bits == DA_KV_BITS_INT4_GROUP64;
+    const bool per64 = kv_bits == DA_KV_BITS_INT4_GROUP64 || kv_bits == DA_KV_BITS_INT8_GROUP64;
     const bool per_token = kv_bits == DA_KV_BITS_INT4_PER_TOKEN || kv_bits == DA_KV_BITS_INT8_PER_TOKEN || per64;
     if (kv_bits != 16 && kv_bits != 8 && kv_bits != 4 && !per_token)
         return fail(DA_ERR_INVALID_ARGUMENT,
-                    "kv_bits (%d) must be 16, 8, 4, one of DA_KV_BITS_INT*_PER_TOKEN or DA_KV_BITS_INT4_GROUP64", kv_bits);
+                    "kv_bits (%d) must be 16, 8, 4 or one of DA_KV_BITS_INT*_PER_TOKEN and DA_KV_BITS_INT*_GROUP64", kv_bits);
     if (per_token && (dim != dim_v || (dim != 64 && dim != 128 && dim != 256) || !distinct_v))
         return fail(DA_ERR_UNSUPPORTED, "per-token factors: head dims (64,64), (128,128) and (256,256), V of its own");
     if (page_size != 0 && (page_size & (page_size - 1)) != 0)
@@ -633,7 +633,7 @@ int da_plan_call(size_t max_seq_k, size_t batch, size_t head_q, size_t head_k, s
     const bool folded = batch > kMaxGridBatch;
     const Plan pl = make_plan(max_seq_k, folded ? kMaxGridBatch : batch, head_q, head_k, dim, dim_v, distinct_v != 0,
                               folded ? 0 : total_k, page_size, kv_bits != 16,
-                              kv_bits == 4 || kv_bits == DA_KV_BITS_INT4_PER_TOKEN || per64,
+                              kv_bits == 4 || kv_bits == DA_KV_BITS_INT4_PER_TOKEN || kv_bits == DA_KV_BITS_INT4_GROUP64,
                               per64 ? 2 : (per_token ? 1 : 0));
     if (kernel_kind) *kernel_kind = pl.kind;
     if (nsplit) *nsplit = pl.nsplit;
@@ -773,8 +773,6 @@ int run_attention(const void* q, const void* k, const void* v, void* o, const in
             return fail(DA_ERR_UNSUPPORTED, "per-token factors: head dims (64,64), (128,128) and (256,256) only");
         if ((reinterpret_cast<uintptr_t>(kf.k_tok) | reinterpret_cast<uintptr_t>(kf.v_tok)) & 7u)
             return fail(DA_ERR_INVALID_ARGUMENT, "k_params and v_params must be 8-byte aligned");
-        if (kf.tok_per64 && kf.fmt != da::kKvInt4)
-            return fail(DA_ERR_UNSUPPORTED, "a pair per 64 elements: int4 caches only");
     }
     const Plan pl = make_plan(max_seq_k, batch, head_q, head_k, dim, dim_v, v != nullptr, total_k,
                               pg.table ? pg.page_size : 0, kf.fmt != 0, kf.fmt == da::kKvInt4,
@@ -869,10 +867,12 @@ int run_attention(const void* q, const void* k, const void* v, void* o, const in
     if (kf.fmt != 0) {
         if (pl.kind == kKindMfma)
             e = da::launch_mla_kv8(sp, kf.fmt, is_bf16 != 0, pl.rt, grid, stream);
-        else if (pl.kind == kKindGroup && per_token && kf.fmt == da::kKvInt8)
+        else if (pl.kind == kKindGroup && per_token && kf.fmt == da::kKvInt8 && !(kf.tok_per64 && dim > 64))
             e = da::launch_gqa_mfma_i8t(sp, is_bf16 != 0, (int)dim, pl.rt, pl.wave_per_head, grid, stream);
         else if (pl.kind == kKindGroup && per_token && kf.tok_per64 && dim > 64)  // (64: one run is the row)
-            e = da::launch_gqa_mfma_i4g(sp, is_bf16 != 0, (int)dim, pl.rt, pl.wave_per_head, grid, stream);
+            e = kf.fmt == da::kKvInt8
+                    ? da::launch_gqa_mfma_i8g(sp, is_bf16 != 0, (int)dim, pl.rt, pl.wave_per_head, grid, stream)
+                    : da::launch_gqa_mfma_i4g(sp, is_bf16 != 0, (int)dim, pl.rt, pl.wave_per_head, grid, stream);
         else if (pl.kind == kKindGroup && per_token)
             e = da::launch_gqa_mfma_i4t(sp, is_bf16 != 0, (int)dim, pl.rt, pl.wave_per_head, grid, stream);
         else if (pl.kind == kKindGroup && kf.fmt == da::kKvInt8)
@@ -1169,6 +1169,40 @@ size_t da_workspace_bytes_int4kv_grp64(size_t max_seq_k, size_t batch, size_t he
                                        size_t dim_v, size_t total_k, size_t page_size) {
     if (head_k == 0 || head_q % head_k != 0 || dim != dim_v || (dim != 64 && dim != 128 && dim != 256)) return 0;
     return plan_ws_bytes(max_seq_k, batch, head_q, head_k, dim, dim_v, true, total_k, page_size, true, true, 2);
+}
+
+int da_decoding_attn_int8kv_grp64(const void* q, const void* k8, const void* v8, void* o, const int32_t* cu_seq_k,
+                                  size_t max_seq_k, size_t batch, size_t head_q, size_t head_k, size_t dim,
+                                  size_t dim_v, int is_alibi, int is_bf16, float softmax_scale,
+                                  const float* alibi_slopes, const float* k_params, const float* v_params,
+                                  size_t total_k, void* workspace, size_t workspace_bytes, void* hip_stream) {
+    if (!k_params || !v_params) return fail(DA_ERR_INVALID_ARGUMENT, "k_params or v_params is null");
+    return run_attention(q, k8, v8, o, cu_seq_k, Paging{}, per_token_format(da::kKvInt8, k_params, v_params, true),
+                         max_seq_k, batch, head_q, head_k, dim, dim_v, is_alibi, is_bf16, softmax_scale, alibi_slopes,
+                         total_k, workspace, workspace_bytes, hip_stream);
+}
+
+int da_decoding_attn_paged_int8kv_grp64(const void* q, const void* k_pages, const void* v_pages, void* o,
+                                        const int32_t* block_table, const int32_t* seq_lens, size_t max_seq_k,
+                                        size_t batch, size_t head_q, size_t head_k, size_t dim, size_t dim_v,
+                                        size_t page_size, size_t max_blocks_per_seq, size_t k_page_stride,
+                                        size_t v_page_stride, int is_alibi, int is_bf16, float softmax_scale,
+                                        const float* alibi_slopes, const float* k_params, const float* v_params,
+                                        size_t total_k, void* workspace, size_t workspace_bytes, void* hip_stream) {
+    if (!k_params || !v_params) return fail(DA_ERR_INVALID_ARGUMENT, "k_params or v_params is null");
+    Paging pg;
+    const int rc = check_paging(block_table, seq_lens, max_seq_k, head_k, dim, dim_v, page_size, max_blocks_per_seq,
+                                k_page_stride, v_page_stride, v_pages != nullptr, &pg);
+    if (rc != DA_OK) return rc;
+    return run_attention(q, k_pages, v_pages, o, nullptr, pg, per_token_format(da::kKvInt8, k_params, v_params, true),
+                         max_seq_k, batch, head_q, head_k, dim, dim_v, is_alibi, is_bf16, softmax_scale, alibi_slopes,
+                         total_k, workspace, workspace_bytes, hip_stream);
+}
+
+size_t da_workspace_bytes_int8kv_grp64(size_t max_seq_k, size_t batch, size_t head_q, size_t head_k, size_t dim,
+                                       size_t dim_v, size_t total_k, size_t page_size) {
+    if (head_k == 0 || head_q % head_k != 0 || dim != dim_v || (dim != 64 && dim != 128 && dim != 256)) return 0;
+    return plan_ws_bytes(max_seq_k, batch, head_q, head_k, dim, dim_v, true, total_k, page_size, true, false, 2);
 }
 
 int da_decoding_attn_int8kv_tok(const void* q, const void* k8, const void* v8, void* o, const int32_t* cu_seq_k,

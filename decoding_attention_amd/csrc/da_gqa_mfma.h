@@ -900,6 +900,9 @@ hipError_t launch_gqa_mfma_i4t(const SweepParams& p, bool is_bf16, int dim, int 
 // ... and over an int4 one with a pair per run of 64 elements of each row ([rows, head_k, dim / 64, 2]); dim 128, 256
 hipError_t launch_gqa_mfma_i4g(const SweepParams& p, bool is_bf16, int dim, int heads_per_group, bool wave_per_head,
                                dim3 grid, hipStream_t stream);
+// ... and over an int8 one with a pair per run of 64 elements
+hipError_t launch_gqa_mfma_i8g(const SweepParams& p, bool is_bf16, int dim, int heads_per_group, bool wave_per_head,
+                               dim3 grid, hipStream_t stream);
 // ... and over an int8 one with such pairs
 hipError_t launch_gqa_mfma_i8t(const SweepParams& p, bool is_bf16, int dim, int heads_per_group, bool wave_per_head,
                                dim3 grid, hipStream_t stream);

@@ -1,6 +1,6 @@
 // Launch helpers of the grouped-head MFMA sweep, shared by the translation units that instantiate it (16-bit
-// K/V in da_gqa_mfma.hip, FP8 in da_gqa_mfma_kv8.hip, int8 in da_gqa_mfma_i8.hip, int4 in da_gqa_mfma_i4.hip, the per-token forms in da_gqa_mfma_i4t.hip and da_gqa_mfma_i8t.hip, int4 with a pair per 64 elements in
-// da_gqa_mfma_i4g.hip; separate units so that the sets compile in parallel).
+// K/V in da_gqa_mfma.hip, FP8 in da_gqa_mfma_kv8.hip, int8 in da_gqa_mfma_i8.hip, int4 in da_gqa_mfma_i4.hip, the per-token forms in da_gqa_mfma_i4t.hip and da_gqa_mfma_i8t.hip, int4 and int8 with a pair per 64 elements in
+// da_gqa_mfma_i4g.hip and da_gqa_mfma_i8g.hip; separate units so that the sets compile in parallel).
 #pragma once
 #include "da_gqa_mfma.h"
 

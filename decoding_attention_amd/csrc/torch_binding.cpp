@@ -47,7 +47,7 @@ const float *scale_ptr(const std::optional<at::Tensor> &t, const at::Tensor &q, 
 
 // int4 or int8 with a (scale, zero) pair per (token, KV head): k_scale and v_scale are then tensors shaped like the rows they
 // belong to with a last dimension of 2 (`rows` = the leading dimensions of the K tensor) instead of head_k values.
-// One dimension more, [..., head_k, dim / 64, 2], is a pair per run of 64 elements of every row (int4 only).
+// One dimension more, [..., head_k, dim / 64, 2], is a pair per run of 64 elements of every row.
 // Returns 0 (per-head factors), 1 (a pair per row) or 2 (a pair per 64 elements).
 int per_token_pairs(const std::optional<at::Tensor> &ks, const std::optional<at::Tensor> &vs, const at::Tensor &q,
                     const at::Tensor &k, int kv8) {
@@ -59,7 +59,6 @@ int per_token_pairs(const std::optional<at::Tensor> &ks, const std::optional<at:
     if (k_form == 0 && v_form == 0) return 0;
     TORCH_CHECK(kv8 == 3 || kv8 == 2, "per-token (scale, zero) pairs apply to an int4 or int8 K/V cache only");
     TORCH_CHECK(k_form == v_form, "per-token (scale, zero) pairs must be given for both K and V, in the same form");
-    TORCH_CHECK(k_form == 1 || kv8 == 3, "a (scale, zero) pair per 64 elements applies to an int4 K/V cache only");
     for (const at::Tensor *t : {&ks.value(), &vs.value()}) {
         TORCH_CHECK(t->dtype() == torch::kFloat32 && t->is_cuda() && t->device() == q.device() && t->is_contiguous(),
                     "per-token pairs must be contiguous float32 GPU tensors");
@@ -164,7 +163,7 @@ at::Tensor dmha_fwd(const at::Tensor &q, const at::Tensor &k, const std::optiona
 
     // k.size(0) is the sum of the key lengths: a free host-side hint for sizing the sequence splits
     const size_t ws_bytes =
-        kv8 ? (tok == 2 ? da_workspace_bytes_int4kv_grp64
+        kv8 ? (tok == 2 ? (kv8 == 3 ? da_workspace_bytes_int4kv_grp64 : da_workspace_bytes_int8kv_grp64)
                : tok ? (kv8 == 3 ? da_workspace_bytes_int4kv_tok : da_workspace_bytes_int8kv_tok)
                    : kv8 == 3 ? da_workspace_bytes_int4kv : da_workspace_bytes_fp8kv)(
                   (size_t)max_seq_k, (size_t)batch, (size_t)head_q, (size_t)head_k, (size_t)dim, (size_t)dim_v,
@@ -175,7 +174,7 @@ at::Tensor dmha_fwd(const at::Tensor &q, const at::Tensor &k, const std::optiona
     if (ws_bytes > 0) ws = torch::empty({(int64_t)ws_bytes}, q.options().dtype(torch::kUInt8));
 
     const float scale = softmax_scale.has_value() ? (float)softmax_scale.value() : 0.0f;
-    const auto kv8_entry = tok == 2   ? da_decoding_attn_int4kv_grp64
+    const auto kv8_entry = tok == 2   ? (kv8 == 3 ? da_decoding_attn_int4kv_grp64 : da_decoding_attn_int8kv_grp64)
                            : tok      ? (kv8 == 3 ? da_decoding_attn_int4kv_tok : da_decoding_attn_int8kv_tok)
                            : kv8 == 3 ? da_decoding_attn_int4kv
                                       : (kv8 == 2 ? da_decoding_attn_int8kv : da_decoding_attn_fp8kv);
@@ -285,7 +284,7 @@ at::Tensor dmha_fwd_paged(const at::Tensor &q, const at::Tensor &k_pages, const 
     const float *v_scale_ptr = tok ? v_scale.value().data_ptr<float>() : scale_ptr(v_scale, q, head_k, "v_scale", kv8);
     const size_t hint = total_k > 0 ? (size_t)total_k : 0;
     const size_t ws_bytes =
-        kv8 ? (tok == 2 ? da_workspace_bytes_int4kv_grp64
+        kv8 ? (tok == 2 ? (kv8 == 3 ? da_workspace_bytes_int4kv_grp64 : da_workspace_bytes_int8kv_grp64)
                : tok ? (kv8 == 3 ? da_workspace_bytes_int4kv_tok : da_workspace_bytes_int8kv_tok)
                    : kv8 == 3 ? da_workspace_bytes_int4kv : da_workspace_bytes_fp8kv)(
                   (size_t)max_seq_k, (size_t)batch, (size_t)head_q, (size_t)head_k, (size_t)dim, (size_t)dim_v, hint,
@@ -296,7 +295,7 @@ at::Tensor dmha_fwd_paged(const at::Tensor &q, const at::Tensor &k_pages, const 
     if (ws_bytes > 0) ws = torch::empty({(int64_t)ws_bytes}, q.options().dtype(torch::kUInt8));
 
     const float scale = softmax_scale.has_value() ? (float)softmax_scale.value() : 0.0f;
-    const auto kv8_entry = tok == 2   ? da_decoding_attn_paged_int4kv_grp64
+    const auto kv8_entry = tok == 2   ? (kv8 == 3 ? da_decoding_attn_paged_int4kv_grp64 : da_decoding_attn_paged_int8kv_grp64)
                            : tok      ? (kv8 == 3 ? da_decoding_attn_paged_int4kv_tok : da_decoding_attn_paged_int8kv_tok)
                            : kv8 == 3 ? da_decoding_attn_paged_int4kv
                                       : (kv8 == 2 ? da_decoding_attn_paged_int8kv : da_decoding_attn_paged_fp8kv);

@@ -93,6 +93,19 @@ def quantize_int4_per_group(x: torch.Tensor, group: int = 64):
     return pack_int4(n.flatten(-2)), torch.cat([scale, zero], dim=-1).contiguous()
 
 
+def quantize_int8_per_group(x: torch.Tensor, group: int = 64):
+    """The same with eight bits: returns (torch.int8 tensor, pairs [..., dim / 64, 2]), each run's minimum at -128 and
+    its maximum at 127."""
+    if group != 64 or x.shape[-1] % 64 != 0:
+        raise ValueError("groups of 64 elements, last dimension a multiple of 64")
+    xf = x.float().unflatten(-1, (x.shape[-1] // 64, 64))
+    lo, hi = xf.amin(dim=-1, keepdim=True), xf.amax(dim=-1, keepdim=True)
+    scale = ((hi - lo) / 255.0).clamp_min(1e-8)
+    zero = -128.0 - lo / scale
+    n = torch.round(xf / scale + zero).clamp(-128, 127).to(torch.int8)
+    return n.flatten(-2), torch.cat([scale, zero], dim=-1).contiguous()
+
+
 def quantize_int8_per_token(x: torch.Tensor):
     """The same with eight bits: returns (torch.int8 tensor, pairs) with x ~= pairs[..., 0] * (n - pairs[..., 1]), the
     row's minimum at -128 and its maximum at 127."""
@@ -125,8 +138,8 @@ def decoding_attn_fwd(q: torch.Tensor, k: torch.Tensor, v: Optional[torch.Tensor
             K = k_scale * k.  For an int4 or int8 cache they may instead be float32 [total_k, head_k, 2] tensors of
             (scale, zero) pairs, one per token and KV head (quantize_int4_per_token, quantize_int8_per_token):
             K[t, h] = k_scale[t, h, 0] * (k[t, h] - k_scale[t, h, 1]); head dims 64, 128 and 256, v required.
-            For an int4 cache, float32 [total_k, head_k, dim / 64, 2] gives every run of 64 elements of a row its own
-            pair (quantize_int4_per_group).
+            float32 [total_k, head_k, dim / 64, 2] gives every run of 64 elements of a row its own pair
+            (quantize_int4_per_group, quantize_int8_per_group).
     Return:
         o: [total_q, head_q, dim_v], same dtype as q.
     """
@@ -159,7 +172,7 @@ def decoding_attn_paged_fwd(q: torch.Tensor, k_pages: torch.Tensor, v_pages: Opt
         k_scale, v_scale (keyword only): as for decoding_attn_fwd, when the pools are torch.float8_e4m3fn, torch.int8
             or torch.uint8 holding pairs of int4 values (last dimensions dim / 2 and dim_v / 2); per-token
             (scale, zero) pairs of an int4 or int8 cache are float32 [pages, page_size, head_k, 2], pairs per 64
-            elements of an int4 cache [pages, page_size, head_k, dim / 64, 2].
+            elements [pages, page_size, head_k, dim / 64, 2].
     Return:
         o: [batch, head_q, dim_v], same dtype as q.
     """

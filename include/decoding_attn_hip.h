@@ -263,6 +263,24 @@ int da_decoding_attn_paged_int4kv_grp64(const void *q, const void *k_pages, cons
 size_t da_workspace_bytes_int4kv_grp64(size_t max_seq_k, size_t batch, size_t head_q, size_t head_k, size_t dim,
                                        size_t dim_v, size_t total_k, size_t page_size);
 
+/* The same with an int8 cache (k8 and v8 as for da_decoding_attn_int8kv). */
+int da_decoding_attn_int8kv_grp64(const void *q, const void *k8, const void *v8, void *o, const int32_t *cu_seq_k,
+                                  size_t max_seq_k, size_t batch, size_t head_q, size_t head_k, size_t dim,
+                                  size_t dim_v, int is_alibi, int is_bf16, float softmax_scale,
+                                  const float *alibi_slopes, const float *k_params, const float *v_params,
+                                  size_t total_k, void *workspace, size_t workspace_bytes, void *hip_stream);
+
+int da_decoding_attn_paged_int8kv_grp64(const void *q, const void *k_pages, const void *v_pages, void *o,
+                                        const int32_t *block_table, const int32_t *seq_lens, size_t max_seq_k,
+                                        size_t batch, size_t head_q, size_t head_k, size_t dim, size_t dim_v,
+                                        size_t page_size, size_t max_blocks_per_seq, size_t k_page_stride,
+                                        size_t v_page_stride, int is_alibi, int is_bf16, float softmax_scale,
+                                        const float *alibi_slopes, const float *k_params, const float *v_params,
+                                        size_t total_k, void *workspace, size_t workspace_bytes, void *hip_stream);
+
+size_t da_workspace_bytes_int8kv_grp64(size_t max_seq_k, size_t batch, size_t head_q, size_t head_k, size_t dim,
+                                       size_t dim_v, size_t total_k, size_t page_size);
+
 /*
  * The same per-token scheme over an int8 cache: k8 and v8 as for da_decoding_attn_int8kv (both required),
  * K[t, hk, c] = k_params[t, hk, 0] * (int8 value - k_params[t, hk, 1]), V likewise.  Arguments, layouts, head dims and
@@ -323,14 +341,15 @@ int da_plan_is_balanced(size_t max_seq_k, size_t batch, size_t head_q, size_t he
  * The plan of any call of this library, for benchmarks that report it beside a measurement: page_size 0 = packed
  * layout, else pages of page_size tokens; distinct_v != 0 = V passed as a buffer of its own; kv_bits 16 = fp16/bf16
  * K/V, 8 = the FP8 and int8 caches, 4 = the int4 cache, DA_KV_BITS_INT4_PER_TOKEN / DA_KV_BITS_INT8_PER_TOKEN = the
- * int4 / int8 cache with per-token (scale, zero) pairs, DA_KV_BITS_INT4_GROUP64 = the int4 cache with a pair per 64
- * elements (distinct_v must be set for the three).  Outputs as da_plan's, balanced as da_plan_is_balanced's result;
+ * int4 / int8 cache with per-token (scale, zero) pairs, DA_KV_BITS_INT4_GROUP64 / DA_KV_BITS_INT8_GROUP64 = the int4 /
+ * int8 cache with a pair per 64 elements (distinct_v must be set for the four).  Outputs as da_plan's, balanced as da_plan_is_balanced's result;
  * any output pointer may be NULL.  No counterpart in the reference (one tile shape per head dim,
  * csrc/kernel/decoding_attn/decoding_fwd_hd*.cu).
  */
 #define DA_KV_BITS_INT4_PER_TOKEN 5
 #define DA_KV_BITS_INT8_PER_TOKEN 9
 #define DA_KV_BITS_INT4_GROUP64 6
+#define DA_KV_BITS_INT8_GROUP64 10
 int da_plan_call(size_t max_seq_k, size_t batch, size_t head_q, size_t head_k, size_t dim, size_t dim_v, size_t total_k,
                  size_t page_size, int distinct_v, int kv_bits, int *kernel_kind, int *nsplit, int *chunk,
                  int *heads_per_group, int *balanced);

@@ -1,4 +1,4 @@
-"""int4 K/V cache with a (scale, zero) pair per run of 64 elements of every (token, KV head) row:
+"""int4 and int8 K/V caches with a (scale, zero) pair per run of 64 elements of every (token, KV head) row:
 K[t, h, c] = scale[t, h, c // 64] * (n[t, h, c] - zero[t, h, c // 64]), V likewise.  q and o stay 16-bit.
 
 As for the per-token form the kernel works on the integers, so it is checked against float64 attention on the
@@ -13,7 +13,7 @@ import pytest
 import torch
 
 from decoding_attention_amd import (_lib, decoding_attn_fwd, decoding_attn_paged_fwd, quantize_int4_per_group,
-                                    quantize_int4_per_token)
+                                    quantize_int4_per_token, quantize_int8_per_group, quantize_int8_per_token)
 from decoding_attention_amd import workloads as wl
 from oracle import oracle
 from tests.gpu_util import TOL, sub_workload
@@ -36,7 +36,18 @@ def test_quantize_int4_per_group_round_trip():
         quantize_int4_per_group(torch.zeros(2, 96))
 
 
-def _case(batch, head_q, head_k, dim, seq_k, dtype, *, is_alibi=False, seed=3, varlen=True):
+def test_quantize_int8_per_group_round_trip():
+    g = torch.Generator().manual_seed(2)
+    x = (torch.randn(11, 2, 2, 64, generator=g) * 3 + torch.randn(11, 2, 2, 1, generator=g)).flatten(-2)
+    n, pairs = quantize_int8_per_group(x)
+    assert n.dtype == torch.int8 and n.shape == x.shape and pairs.shape == (11, 2, 2, 2)
+    runs = n.unflatten(-1, (2, 64))
+    assert (runs.amin(-1) == -128).all() and (runs.amax(-1) == 127).all()
+    back = pairs[..., :1] * (runs.float() - pairs[..., 1:])
+    assert ((back - x.unflatten(-1, (2, 64))).abs() <= pairs[..., :1] * 0.5001).all()
+
+
+def _case(batch, head_q, head_k, dim, seq_k, dtype, *, is_alibi=False, seed=3, varlen=True, bits=4):
     w = wl.make_workload(batch, head_q, head_k, dim, dim, seq_k, dtype, seed=seed, varlen=varlen, is_alibi=is_alibi)
     g = torch.Generator().manual_seed(seed + 70)
     rows, ng = w.k.shape[0], dim // 64
@@ -46,13 +57,14 @@ def _case(batch, head_q, head_k, dim, seq_k, dtype, *, is_alibi=False, seed=3, v
         x = x * (0.3 + 1.5 * torch.rand(rows, head_k, ng, 1, generator=g)) + offset * torch.randn(rows, head_k, ng, 1, generator=g)
         return x.flatten(-2)
 
-    k4, kp = quantize_int4_per_group(spread(w.k, 1.0))
-    v4, vp = quantize_int4_per_group(spread(w.v, 0.5))
+    quant = quantize_int4_per_group if bits == 4 else quantize_int8_per_group
+    k4, kp = quant(spread(w.k, 1.0))
+    v4, vp = quant(spread(w.v, 0.5))
     return w, k4, v4, kp, vp
 
 
 def _dequant(cache, pairs):
-    n = _unpack(cache).double().unflatten(-1, (pairs.shape[-2], 64))
+    n = (_unpack(cache) if cache.dtype == torch.uint8 else cache).double().unflatten(-1, (pairs.shape[-2], 64))
     return (pairs[..., :1].double() * (n - pairs[..., 1:].double())).flatten(-2)
 
 
@@ -84,10 +96,11 @@ SHAPES = [
 
 
 @pytest.mark.gpu
+@pytest.mark.parametrize("bits", [4, 8])
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
 @pytest.mark.parametrize("shape", SHAPES)
-def test_per_group_cache_matches_float64_attention(shape, dtype):
-    w, k4, v4, kp, vp = _case(*shape, dtype, is_alibi=shape[0] == 6)
+def test_per_group_cache_matches_float64_attention(shape, dtype, bits):
+    w, k4, v4, kp, vp = _case(*shape, dtype, is_alibi=shape[0] == 6, bits=bits)
     o = _run(w, k4, v4, kp, vp)
     assert torch.isfinite(o.float()).all()
     if w.batch > 8:  # the large case: sampled sequences against float64
@@ -107,10 +120,11 @@ def test_per_group_cache_matches_float64_attention(shape, dtype):
 
 
 @pytest.mark.gpu
+@pytest.mark.parametrize("bits", [4, 8])
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
-def test_runs_with_a_scale_of_zero(dtype):
+def test_runs_with_a_scale_of_zero(dtype, bits):
     """A constant run may come with a scale of exactly zero: a run of zeros, whose row still counts in the sums."""
-    w, k4, v4, kp, vp = _case(3, 16, 4, 128, 400, dtype, seed=41)
+    w, k4, v4, kp, vp = _case(3, 16, 4, 128, 400, dtype, seed=41, bits=bits)
     g = torch.Generator().manual_seed(4)
     kp[torch.rand(kp.shape[:3], generator=g) < 0.2, 0] = 0.0
     vp[torch.rand(vp.shape[:3], generator=g) < 0.2, 0] = 0.0
@@ -125,25 +139,29 @@ def _swap_runs(x, ng, unit):
 
 
 @pytest.mark.gpu
+@pytest.mark.parametrize("bits", [4, 8])
 @pytest.mark.parametrize("dim", [128, 256])
-def test_exchanging_runs(dim):
-    w, k4, v4, kp, vp = _case(3, 16, 4, dim, 600, torch.float16, seed=31)
+def test_exchanging_runs(dim, bits):
+    w, k4, v4, kp, vp = _case(3, 16, 4, dim, 600, torch.float16, seed=31, bits=bits)
     ng = dim // 64
+    unit = 32 if bits == 4 else 64  # cache entries per run
     base = _run(w, k4, v4, kp, vp)
     # V: the output's column runs follow, bit for bit (each run's columns see the same arithmetic wherever they sit)
-    o = _run(w, k4, _swap_runs(v4, ng, 32), kp, vp.flip(-2).contiguous())
+    o = _run(w, k4, _swap_runs(v4, ng, unit), kp, vp.flip(-2).contiguous())
     assert torch.equal(_swap_runs(o, ng, 64).view(torch.int16), base.view(torch.int16))
     # K with q: the same scores (summed over the runs in another order)
-    o = _run(w, _swap_runs(k4, ng, 32), v4, kp.flip(-2).contiguous(), vp, q=_swap_runs(w.q, ng, 64))
+    o = _run(w, _swap_runs(k4, ng, unit), v4, kp.flip(-2).contiguous(), vp, q=_swap_runs(w.q, ng, 64))
     assert (o.float() - base.float()).abs().max().item() <= TOL[torch.float16] / 4
 
 
 @pytest.mark.gpu
+@pytest.mark.parametrize("bits", [4, 8])
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
-def test_equal_pairs_in_every_run_reduce_to_the_per_token_call(dtype):
+def test_equal_pairs_in_every_run_reduce_to_the_per_token_call(dtype, bits):
     w = wl.make_workload(4, 32, 8, 128, 128, 1000, dtype, seed=5, varlen=True)
-    k4, kp = quantize_int4_per_token(w.k)
-    v4, vp = quantize_int4_per_token(w.v)
+    quant = quantize_int4_per_token if bits == 4 else quantize_int8_per_token
+    k4, kp = quant(w.k)
+    v4, vp = quant(w.v)
     per_token = _run(w, k4, v4, kp, vp)
     twice = lambda p: p.unsqueeze(-2).expand(-1, -1, 2, -1).contiguous()  # noqa: E731
     per_group = _run(w, k4, v4, twice(kp), twice(vp))
@@ -151,11 +169,12 @@ def test_equal_pairs_in_every_run_reduce_to_the_per_token_call(dtype):
 
 
 @pytest.mark.gpu
+@pytest.mark.parametrize("bits", [4, 8])
 @pytest.mark.parametrize("shape", [SHAPES[0], SHAPES[2], SHAPES[5]])
-def test_paged_pools(shape):
+def test_paged_pools(shape, bits):
     """Pairs in pools of their own, [pages, page_size, head_k, dim / 64, 2], addressed through the same block table:
     float64 attention on the de-quantised rows at 64-token pages, and the same bits at every page size."""
-    w, k4, v4, kp, vp = _case(*shape, torch.float16, seed=21)
+    w, k4, v4, kp, vp = _case(*shape, torch.float16, seed=21, bits=bits)
     w4 = wl.Workload(w.name, w.q, k4, v4, w.cu_seq_k, w.max_seq_k, w.dim_v, w.is_alibi, w.lengths)
     flat = lambda p: p.flatten(-2)  # noqa: E731  (to_pages handles [rows, head_k, x])
     wp = wl.Workload(w.name, w.q, flat(kp), flat(vp), w.cu_seq_k, w.max_seq_k, w.dim_v, w.is_alibi, w.lengths)
@@ -177,6 +196,7 @@ def test_paged_pools(shape):
 def test_plan_takes_sixteen_heads_a_group_at_256():
     """Four sets of factors for 32 heads do not fit a wave's registers: d = 256 runs as groups of 16 heads."""
     assert _lib.plan(1024, 8, 32, 1, 256, 256, kv_bits=_lib.KV_BITS_INT4_GROUP64)["heads_per_group"] == 16
+    assert _lib.plan(1024, 8, 32, 1, 256, 256, kv_bits=_lib.KV_BITS_INT8_GROUP64)["heads_per_group"] == 16
     assert _lib.plan(1024, 8, 32, 1, 256, 256, kv_bits=_lib.KV_BITS_INT4_PER_TOKEN)["heads_per_group"] == 32
     assert _lib.plan(1024, 8, 32, 1, 128, 128, kv_bits=_lib.KV_BITS_INT4_GROUP64)["heads_per_group"] == 32
 
@@ -185,8 +205,8 @@ def test_plan_takes_sixteen_heads_a_group_at_256():
 def test_argument_errors():
     w, k4, v4, kp, vp = _case(2, 8, 2, 128, 100, torch.float16)
     q, cu = w.q.to(DEV), w.cu_seq_k.to(DEV)
-    k8 = _unpack(k4).to(DEV)
-    with pytest.raises(RuntimeError, match="int4 K/V cache only"):
+    k8 = _unpack(k4).float().to(torch.float8_e4m3fn).to(DEV)
+    with pytest.raises(RuntimeError, match="int4 or int8 K/V cache only"):
         decoding_attn_fwd(q, k8, k8, cu, w.max_seq_k, 128, False, k_scale=kp.to(DEV), v_scale=vp.to(DEV))
     with pytest.raises(RuntimeError, match="same form"):
         decoding_attn_fwd(q, k4.to(DEV), v4.to(DEV), cu, w.max_seq_k, 128, False, k_scale=kp.to(DEV),

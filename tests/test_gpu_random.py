@@ -11,7 +11,7 @@ import pytest
 import torch
 
 from decoding_attention_amd import (decoding_attn_fwd, decoding_attn_paged_fwd, pack_int4, quantize_int4_per_group,
-                                    quantize_int4_per_token, quantize_int8_per_token)
+                                    quantize_int4_per_token, quantize_int8_per_group, quantize_int8_per_token)
 from decoding_attention_amd import workloads as wl
 from oracle import oracle
 from tests.gpu_util import TOL, run_hip_ex, sub_workload
@@ -24,11 +24,11 @@ HEADS = [(32, 8), (32, 32), (32, 1), (8, 2), (28, 4), (16, 16), (64, 8), (12, 4)
 CASES_PER_CHUNK = 12
 
 
-def _one_case(rng, seed, case, int4=False, per_token=False):
+def _one_case(rng, seed, case, int4=False, per_token=False, per64=False):
     """int4: the case runs over an int4 cache (whatever format the draws below pick; the stream of draws is the same
     either way, so the other cases do not move).  per_token (4 or 8): an int4 or int8 cache with a (scale, zero) pair
-    per token and KV head (never the latent form, never d = 96, which those entry points do not serve); 64: an int4
-    cache with a pair per run of 64 elements of each row."""
+    per token and KV head (never the latent form, never d = 96, which those entry points do not serve); with per64 the
+    pairs are per run of 64 elements of each row."""
     latent = rng.random() < 0.3 and not per_token
     dtype = rng.choice([torch.float16, torch.bfloat16])
     if latent:
@@ -70,16 +70,17 @@ def _one_case(rng, seed, case, int4=False, per_token=False):
     k_true, v_true = k.float(), None if v is None else v.float()
     if per_token:
         # rows of different spread and offset: the pairs differ from token to token and head to head
-        runs = d // 64 if per_token == 64 else 1  # (per_token == 64: every run of 64 elements likewise)
+        runs = d // 64 if per64 else 1  # (per64: every run of 64 elements likewise)
         shape = (total, hk, runs, 1)
         k = (k.float().unflatten(-1, (runs, -1)) * (0.5 + torch.rand(shape, generator=g))
              + torch.randn(shape, generator=g)).flatten(-2)
         v = (v.float().unflatten(-1, (runs, -1)) * (0.5 + torch.rand(shape, generator=g))
              + 0.5 * torch.randn(shape, generator=g)).flatten(-2)
-        quant = {8: quantize_int8_per_token, 4: quantize_int4_per_token, 64: quantize_int4_per_group}[per_token]
+        quant = {(8, False): quantize_int8_per_token, (4, False): quantize_int4_per_token,
+                 (4, True): quantize_int4_per_group, (8, True): quantize_int8_per_group}[(per_token, per64)]
         k8, kpairs = quant(k)
         v8, vpairs = quant(v)
-        if per_token != 64:
+        if not per64:
             kpairs, vpairs = kpairs.unsqueeze(-2), vpairs.unsqueeze(-2)  # [total, hk, runs, 2] from here on
 
         def unpack(p4):
@@ -90,7 +91,7 @@ def _one_case(rng, seed, case, int4=False, per_token=False):
 
         k_true = (kpairs[..., :1].double() * (unpack(k8).unflatten(-1, (runs, -1)) - kpairs[..., 1:].double())).flatten(-2)
         v_true = (vpairs[..., :1].double() * (unpack(v8).unflatten(-1, (runs, -1)) - vpairs[..., 1:].double())).flatten(-2)
-        as_passed = (lambda t: t) if per_token == 64 else (lambda t: t.squeeze(-2))  # noqa: E731
+        as_passed = (lambda t: t) if per64 else (lambda t: t.squeeze(-2))  # noqa: E731
         kw = dict(k_scale=as_passed(kpairs).to(DEV), v_scale=as_passed(vpairs).to(DEV))
     elif fp8:
         def quantise(x, scale):
@@ -183,4 +184,12 @@ def test_random_cases_over_an_int4_cache_with_pairs_per_64_elements(chunk):
     seed = 19
     rng = random.Random(seed * 1000 + chunk)
     for i in range(CASES_PER_CHUNK):
-        _one_case(rng, seed, chunk * CASES_PER_CHUNK + i, per_token=64)
+        _one_case(rng, seed, chunk * CASES_PER_CHUNK + i, per_token=4, per64=True)
+
+
+@pytest.mark.parametrize("chunk", range(2))
+def test_random_cases_over_an_int8_cache_with_pairs_per_64_elements(chunk):
+    seed = 23
+    rng = random.Random(seed * 1000 + chunk)
+    for i in range(CASES_PER_CHUNK):
+        _one_case(rng, seed, chunk * CASES_PER_CHUNK + i, per_token=8, per64=True)

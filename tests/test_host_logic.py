@@ -175,7 +175,8 @@ def test_plan_of_every_call_form():
     ragged = _lib.plan(8192, 64, 32, 8, 128, 128, total_k=300000, page_size=64)
     assert ragged["balanced"] == bool(lib.da_plan_is_balanced(8192, 64, 32, 8, 128, 128, 300000, 64))
     # per-token pairs and pairs per 64 elements: the grouped kernel whatever the shape
-    for bits in (_lib.KV_BITS_INT4_PER_TOKEN, _lib.KV_BITS_INT8_PER_TOKEN, _lib.KV_BITS_INT4_GROUP64):
+    for bits in (_lib.KV_BITS_INT4_PER_TOKEN, _lib.KV_BITS_INT8_PER_TOKEN, _lib.KV_BITS_INT4_GROUP64,
+                 _lib.KV_BITS_INT8_GROUP64):
         assert _lib.plan(128, 512, 32, 32, 128, 128, kv_bits=bits)["kind"] == 3
         with pytest.raises(RuntimeError):
             _lib.plan(128, 512, 32, 32, 96, 96, kv_bits=bits)
