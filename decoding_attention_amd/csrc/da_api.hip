@@ -243,19 +243,18 @@ Plan make_plan(size_t max_seq_k, size_t batch, size_t head_q, size_t head_k, siz
         if (group_only == 2 && dim == 256) pl.rt = 16;
         pl.wave_per_head = head_k % 4 == 0 && tun().wave_per_head;
         trip = pl.wave_per_head ? da::kGqaTile : 4 * da::kGqaTile;
-        // d = 128, four waves sharing one KV head's tokens (MQA and other head counts that are no multiple of four): one
-        // work-group per CU already saturates what this form can pull, and half as many splits halve the merge
-        // (measured, 256 against 512 work-groups: MQA 32/1, batch 64 x 4096 tokens 35.7 -> 29.6 us; 16/2 heads, batch 32
-        // x 4096 a tie).  With one wave per KV head the usual 512 do better since the K/V loads are non-temporal
-        // (32/8 heads, batch 64 x 4096 tokens 170.4 -> 166.1 us, batch 128 x 2048 167.4 -> 165.0; with ordinary loads it
-        // was the other way round, 181.8 against 183.8).
-        // (16-bit K/V in whole tiles or 16-token runs only: the 8-bit forms and the per-row page lookups keep fewer
-        // bytes in flight per work-group and need the 512; FP8, batch 64 x 4096 tokens: 96 us against 110)
-        if (dim == 128 && !kv_8bit && (packed || page_size >= 16) && !pl.wave_per_head) target_wgs = tun().group_target_wgs_d128;
-        // d = 96 (rows of 192 bytes, ordinary loads, the slowest stream of the four head dims): 256 work-groups, half
-        // the merge (measured, 32/8 heads: batch 64 x 4096 tokens 144.1 -> 142.0 us, batch 32 x 8192 145.6 -> 142.6,
-        // batch 128 x 2048 142.5 -> 138.1; 16/4 heads, batch 64 x 4096 75.6 -> 74.3)
-        if (dim == 96 && !kv_8bit && (packed || page_size >= 16)) target_wgs = tun().group_target_wgs_d128;
+        // 16-bit K/V in whole tiles or 16-token runs, rows of 192 bytes and more (d = 96, 128, 256): one work-group per
+        // CU saturates what the kernel can pull, and half as many splits halve the partials and the merge.  Measured,
+        // 256 against 512 work-groups, bf16: 32/8 heads d 128, batch 64 x 4096 tokens 165.4 -> 159.4 us, batch 128 x 2048
+        // 164.4 -> 156.2, batch 32 x 4096 84.5 -> 80.7; 64/8 heads 169.0 -> 160.8; 32/4 heads 88.0 -> 82.9; over 16-token
+        // pages 169.9 -> 164.1; MQA 32/1, batch 64 x 4096 35.7 -> 29.6; d 256, 32/8 heads, batch 64 x 4096 317.7 -> 309.0,
+        // batch 128 x 2048 320.7 -> 305.7; d 96, 32/8 heads, batch 64 x 4096 144.1 -> 142.0, batch 128 x 2048 142.5 ->
+        // 138.1.  (Before the kernel waited for a tile's K registers ahead of issuing the next tile's V loads, the
+        // form with one wave per KV head needed the second work-group per CU to hide that wait: 170.4 against 166.1.)
+        // Not at d = 64, whose work-groups stream too few bytes for one per CU (batch 32 x 4096: 47.0 -> 52.2 us), and
+        // not over 8-bit K/V or per-row page lookups, which keep fewer bytes in flight per work-group (FP8, 32/8 heads,
+        // batch 32 x 4096 tokens 47.8 -> 53.1 us, batch 48 69.3 -> 80.2; int4 30.4 -> 34.3 and 43.8 -> 49.4).
+        if (dim >= 96 && !kv_8bit && (packed || page_size >= 16)) target_wgs = tun().group_target_wgs_d128;
     } else {
         pl.kind = kKindSweep;
         const int max_rt = dim > 256 ? 2 : 4;
@@ -276,16 +275,20 @@ Plan make_plan(size_t max_seq_k, size_t batch, size_t head_q, size_t head_k, siz
     const double kv_bytes = (double)total_k * (double)head_k * (double)(dim + dim_v) * (kv_8bit ? 1.0 : 2.0);
     if (pl.kind == kKindGroup && tun().flat_wgs > 0 && batch >= 2) {
         const long long ygrid = base / (long long)batch;
-        // (without a count: the work-groups the fixed-split plan of this shape aims at, so that a uniform batch is cut
-        // the same way -- MQA at d = 128, 256 instead of 512: batch 64 x 4096 tokens 42.1 -> 29.5 us)
-        long long w = std::max<long long>(1, (total_k == 0 ? std::min(target_wgs, tun().flat_wgs) : tun().flat_wgs) / ygrid);
+        // (the work-groups the fixed-split plan of this shape aims at, so that a uniform batch without a count is cut
+        // the same way -- MQA at d = 128, 256 instead of 512: batch 64 x 4096 tokens 42.1 -> 29.5 us -- and a ragged one
+        // gains what the uniform one gains: 32/8 heads d 128 bf16, batch 64 x 1..8192 tokens 209.3 -> 202.0 us, batch
+        // 128 x 1..4096 170.6 -> 166.7, 64/8 heads, batch 32 x 1..16384 182.5 -> 175.5; over 16-token pages 197.6 ->
+        // 194.8, 177.7 -> 172.0, 185.1 -> 177.6)
+        long long w = std::max<long long>(1, std::min(target_wgs, tun().flat_wgs) / ygrid);
         const long long unit = packed ? 1 : da::kGqaTile;
         const long long step = std::max<long long>(1, trip / unit);  // a work-group's waves advance `trip` tokens together
         const long long mn = std::max<long long>(tun().flat_min_tokens / unit, step);
         const bool counted = ragged && total_k < ((size_t)1 << 30) && total_k >= 64 * batch &&
                              (packed || kv_bytes >= (double)tun().flat_paged_min_mb * 1e6);
         const bool uncounted = total_k == 0 && packed && !latent_group && tun().flat_uncounted &&
-                               (long long)batch * (long long)max_seq_k >= w * (long long)tun().flat_uncounted_min &&
+                               (long long)batch * (long long)max_seq_k >=
+                                   std::max<long long>(1, tun().flat_wgs / ygrid) * (long long)tun().flat_uncounted_min &&
                                (long long)batch * (long long)max_seq_k < (1ll << 30);
         if (counted || uncounted) {
             pl.flat_step = (int)step;

@@ -83,14 +83,14 @@ def test_plan_total_k_hint_changes_the_splits_and_never_the_kernel():
     full = _lib.plan(sk, batch, 32, 8, 128, 128, total_k=batch * sk)
     ragged = _lib.plan(sk, batch, 32, 8, 128, 128, total_k=batch * sk // 2)
     assert full["kind"] == base["kind"] and full["chunk"] >= base["chunk"] and full["nsplit"] <= base["nsplit"]
-    # grouped kernel: equal shares of the concatenated tokens, 512 work-groups over the 2 groups of 4 KV heads
+    # grouped kernel: equal shares of the concatenated tokens, 256 work-groups over the 2 groups of 4 KV heads
     assert ragged["kind"] == base["kind"] == 3 and ragged["balanced"] and not full["balanced"]
-    assert ragged["nsplit"] == 256 and ragged["chunk"] == batch * sk // 2 // 256
+    assert ragged["nsplit"] == 128 and ragged["chunk"] == batch * sk // 2 // 128
     # a partial slot per (share, sequence) pair that can occur: shares + sequences
     ws = _lib.load().da_workspace_bytes(sk, batch, 32, 8, 128, 128, batch * sk // 2)
     assert ws == (ragged["nsplit"] + batch) * 32 * (128 + 2) * 4
     # without a count the same grid, the share left to the device
-    assert base["balanced"] and base["nsplit"] == 256 and base["chunk"] == 0
+    assert base["balanced"] and base["nsplit"] == 128 and base["chunk"] == 0
     # VALU sweep (one query head per KV head, short sequences): shorter fixed splits
     sk, batch = 2048, 16
     base = _lib.plan(sk, batch, 32, 32, 256, 256)
@@ -101,13 +101,13 @@ def test_plan_total_k_hint_changes_the_splits_and_never_the_kernel():
 
 def test_plan_without_a_token_count_at_d128():
     """The reference-signature entry point passes no token count: a batch large enough for whole shares then takes the
-    balanced grid, which cuts a uniform batch exactly as the counted plan's fixed splits do (256 shares of 64 x 4096 /
-    256 = 1024 tokens, the share derived on the device); smaller problems keep fixed splits of up to 2048 tokens."""
+    balanced grid, which cuts a uniform batch exactly as the counted plan's fixed splits do (128 shares of 64 x 4096 /
+    128 = 2048 tokens, the share derived on the device); smaller problems keep fixed splits of up to 2048 tokens."""
     blind = _lib.plan(4096, 64, 32, 8, 128, 128)
     counted = _lib.plan(4096, 64, 32, 8, 128, 128, total_k=64 * 4096)
     assert blind["kind"] == counted["kind"] == 3
-    assert (counted["nsplit"], counted["chunk"], counted["balanced"]) == (4, 1024, False)
-    assert (blind["nsplit"], blind["chunk"], blind["balanced"]) == (256, 0, True)
+    assert (counted["nsplit"], counted["chunk"], counted["balanced"]) == (2, 2048, False)
+    assert (blind["nsplit"], blind["chunk"], blind["balanced"]) == (128, 0, True)
     # a single long sequence: nothing to balance, the cap sets the cut
     one = _lib.plan(16384, 1, 32, 8, 128, 128)
     assert not one["balanced"] and one["chunk"] <= 2048
