@@ -248,7 +248,8 @@ Plan make_plan(size_t max_seq_k, size_t batch, size_t head_q, size_t head_k, siz
         // 256 against 512 work-groups, bf16: 32/8 heads d 128, batch 64 x 4096 tokens 165.4 -> 159.4 us, batch 128 x 2048
         // 164.4 -> 156.2, batch 32 x 4096 84.5 -> 80.7; 64/8 heads 169.0 -> 160.8; 32/4 heads 88.0 -> 82.9; over 16-token
         // pages 169.9 -> 164.1; MQA 32/1, batch 64 x 4096 35.7 -> 29.6; d 256, 32/8 heads, batch 64 x 4096 317.7 -> 309.0,
-        // batch 128 x 2048 320.7 -> 305.7; d 96, 32/8 heads, batch 64 x 4096 144.1 -> 142.0, batch 128 x 2048 142.5 ->
+        // batch 128 x 2048 320.7 -> 305.7, 16/1 heads, batch 64 x 4096 53.8 -> 46.2, 64/1 heads 93.5 -> 77.9, 32/2 heads
+        // 95.7 -> 87.3; d 96, 32/8 heads, batch 64 x 4096 144.1 -> 142.0, batch 128 x 2048 142.5 ->
         // 138.1.  (Before the kernel waited for a tile's K registers ahead of issuing the next tile's V loads, the
         // form with one wave per KV head needed the second work-group per CU to hide that wait: 170.4 against 166.1.)
         // Not at d = 64, whose work-groups stream too few bytes for one per CU (batch 32 x 4096: 47.0 -> 52.2 us), and
